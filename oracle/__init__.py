@@ -1,0 +1,247 @@
+"""ctypes binding of the CPU oracle (oracle/oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py``.  The product (``refactorgraph_amd``) never imports it.
+
+Each wrapper takes and returns numpy arrays; the reference file:line every function follows
+is listed in oracle/oracle.h.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "liboracle.so")
+
+F32, U8, I8, U16, I16, I32, F64 = 1, 2, 3, 4, 5, 6, 11
+_NP2CODE = {np.dtype(np.uint8): U8, np.dtype(np.int8): I8, np.dtype(np.uint16): U16,
+            np.dtype(np.int16): I16, np.dtype(np.int32): I32}
+
+
+def build() -> str:
+    """Compile oracle.c with the committed Makefile."""
+    subprocess.run(["make", "-C", _HERE, "-s"], check=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        sz, vp, i32, f32 = C.c_size_t, C.c_void_p, C.c_int, C.c_float
+        L.oracle_rms_norm_f32.argtypes = [vp, vp, vp, sz, sz, f32, i32]
+        L.oracle_rms_norm_f64.argtypes = [vp, vp, vp, sz, sz, f32, i32]
+        L.oracle_softmax_f32.argtypes = [vp, vp, sz, sz, sz, i32]
+        L.oracle_softmax_f64.argtypes = [vp, vp, sz, sz, sz, i32]
+        L.oracle_softmax_literal_f32.argtypes = [vp, vp, sz, sz, sz]
+        L.oracle_softmax_causal_f32.argtypes = [vp, vp, sz, sz, sz, i32]
+        L.oracle_matmul_integer.argtypes = [vp, vp, vp, vp, i32, i32, vp, i32, i32,
+                                            sz, sz, sz, sz, vp, vp, sz, sz, i32]
+        L.oracle_dequantize_linear.argtypes = [vp, vp, vp, vp, sz, sz, sz, i32, sz, i32]
+        L.oracle_dequantize_linear.restype = i32
+        L.oracle_matmul_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, f32]
+        L.oracle_mul_f32.argtypes = [vp, vp, vp, sz, sz]
+        L.oracle_attention_head_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, f32, i32, vp]
+        L.oracle_rope_f32.argtypes = [vp, vp, vp, i32, sz, sz, sz, sz, f32, i32]
+        for name in ("oracle_rms_norm_f32", "oracle_rms_norm_f64", "oracle_softmax_f32",
+                     "oracle_softmax_f64", "oracle_softmax_literal_f32", "oracle_softmax_causal_f32",
+                     "oracle_matmul_integer", "oracle_matmul_f32", "oracle_mul_f32",
+                     "oracle_attention_head_f32", "oracle_rope_f32"):
+            getattr(L, name).restype = None
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype=None):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def rms_norm(x, w, eps, threads=1):
+    x = _c(x)
+    assert x.dtype in (np.float32, np.float64)
+    w = _c(w, x.dtype)
+    cols = x.shape[-1]
+    rows = x.size // cols if cols else 0
+    y = np.empty_like(x)
+    fn = lib().oracle_rms_norm_f32 if x.dtype == np.float32 else lib().oracle_rms_norm_f64
+    fn(_p(y), _p(x), _p(w), rows, cols, float(eps), threads)
+    return y
+
+
+def _pre_mid_post(shape, axis):
+    pre = int(np.prod(shape[:axis], dtype=np.int64))
+    post = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return pre, int(shape[axis]), post
+
+
+def softmax(x, axis=-1, threads=1):
+    x = _c(x)
+    assert x.dtype in (np.float32, np.float64)
+    axis = axis % x.ndim
+    pre, mid, post = _pre_mid_post(x.shape, axis)
+    y = np.empty_like(x)
+    fn = lib().oracle_softmax_f32 if x.dtype == np.float32 else lib().oracle_softmax_f64
+    fn(_p(y), _p(x), pre, mid, post, threads)
+    return y
+
+
+def softmax_literal(x, axis=-1):
+    x = _c(x, np.float32)
+    axis = axis % x.ndim
+    pre, mid, post = _pre_mid_post(x.shape, axis)
+    y = np.empty_like(x)
+    lib().oracle_softmax_literal_f32(_p(y), _p(x), pre, mid, post)
+    return y
+
+
+def softmax_causal(x, threads=1):
+    x = _c(x, np.float32)
+    rows, cols = x.shape[-2], x.shape[-1]
+    batch = x.size // (rows * cols)
+    y = np.empty_like(x)
+    lib().oracle_softmax_causal_f32(_p(y), _p(x), batch, rows, cols, threads)
+    return y
+
+
+def batch_offsets(a_batch_shape, b_batch_shape):
+    """Operand matrix index for every output batch under multidirectional broadcasting
+    (independent of the host-side Broadcaster: numpy's own broadcasting does the work)."""
+    na = int(np.prod(a_batch_shape, dtype=np.int64))
+    nb = int(np.prod(b_batch_shape, dtype=np.int64))
+    ia = np.arange(na, dtype=np.uint32).reshape(a_batch_shape)
+    ib = np.arange(nb, dtype=np.uint32).reshape(b_batch_shape)
+    oa, ob = np.broadcast_arrays(ia, ib)
+    return _c(oa.reshape(-1)), _c(ob.reshape(-1)), na, nb
+
+
+def matmul_integer(a, b, a_zp=None, b_zp=None, threads=1):
+    """a [..., m, k], b [..., k, n] of uint8/int8; zero points: None, 1-element array, or
+    per-row arrays as the reference reads them (A: [batch*m], B: [batch*k])."""
+    a, b = _c(a), _c(b)
+    assert a.dtype in (np.uint8, np.int8) and b.dtype in (np.uint8, np.int8)
+    m, k = a.shape[-2:]
+    k2, n = b.shape[-2:]
+    assert k == k2
+    oa, ob, na, nb = batch_offsets(a.shape[:-2], b.shape[:-2])
+    batch = oa.size
+    out_batch_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    y = np.empty(out_batch_shape + (m, n), dtype=np.int32)
+
+    def zp_args(zp):
+        if zp is None:
+            return None, 1, 1
+        zp = _c(zp)
+        assert zp.dtype in (np.uint8, np.int8)
+        return zp, int(zp.dtype == np.int8), int(zp.size == 1)
+
+    az, az_s, az_sc = zp_args(a_zp)
+    bz, bz_s, bz_sc = zp_args(b_zp)
+    lib().oracle_matmul_integer(_p(y), _p(a), _p(b), _p(az), az_s, az_sc, _p(bz), bz_s, bz_sc,
+                                batch, m, k, n, _p(oa), _p(ob), na, nb, threads)
+    return y
+
+
+def dequantize_linear(x, scale, zp=None, axis=1, threads=1):
+    x = _c(x)
+    code = _NP2CODE[x.dtype]
+    scale = _c(scale, np.float32).reshape(-1)
+    if zp is not None:
+        zp = _c(zp, x.dtype).reshape(-1)
+        assert zp.size == scale.size
+    if scale.size == 1:
+        outer, axis_len, inner = 1, 1, x.size
+    else:
+        axis = axis % x.ndim
+        outer, axis_len, inner = _pre_mid_post(x.shape, axis)
+        assert scale.size == axis_len
+    y = np.empty(x.shape, dtype=np.float32)
+    rc = lib().oracle_dequantize_linear(_p(y), _p(x), _p(scale), _p(zp), outer, axis_len, inner,
+                                        code, scale.size, threads)
+    assert rc == 0
+    return y
+
+
+def matmul_f32(a, b, trans_b=False, alpha=1.0):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    M, K = a.shape
+    if trans_b:
+        N = b.shape[0]
+        sb0, sb1 = 1, K
+    else:
+        N = b.shape[1]
+        sb0, sb1 = N, 1
+    y = np.empty((M, N), dtype=np.float32)
+    lib().oracle_matmul_f32(_p(y), _p(a), _p(b), M, K, N, K, 1, sb0, sb1, float(alpha))
+    return y
+
+
+def mul_f32(a, b):
+    a, b = _c(a, np.float32), _c(b, np.float32)
+    y = np.empty(a.shape if a.size >= b.size else b.shape, dtype=np.float32)
+    lib().oracle_mul_f32(_p(y), _p(a), _p(b), a.size, b.size)
+    return y
+
+
+def attention_head(q, kc, vc, past, scale, causal=True):
+    """q [seq, D]; kc/vc [past+seq, D] (history followed by the new rows), float32."""
+    q, kc, vc = _c(q, np.float32), _c(kc, np.float32), _c(vc, np.float32)
+    seq, D = q.shape
+    assert kc.shape == (past + seq, D) and vc.shape == (past + seq, D)
+    o = np.empty((seq, D), dtype=np.float32)
+    scratch = np.empty(2 * seq * (past + seq), dtype=np.float32)
+    lib().oracle_attention_head_f32(_p(o), _p(q), _p(kc), _p(vc), seq, int(past), D,
+                                    float(scale), int(causal), _p(scratch))
+    return o
+
+
+def attention_kvcache(q, k, v, k_cache, v_cache, past_lens, scale, heads=None):
+    """Composed attention with cache append, fp32 math on already up-cast inputs.
+
+    q [N,H,seq,D]; k,v [N,Hkv,seq,D]; caches [N,Hkv,S,D] (updated copies are returned);
+    past_lens: int array [N] (or one value).  ``heads``: optional iterable of (b, h) pairs to
+    evaluate (others are left as NaN) so large shapes can be spot-checked.
+    Returns (o, k_cache_out, v_cache_out)."""
+    q = _c(q, np.float32)
+    N, H, seq, D = q.shape
+    Hkv = k.shape[1]
+    g = H // Hkv
+    past_lens = np.broadcast_to(np.asarray(past_lens, dtype=np.int64).reshape(-1), (N,))
+    kc = np.array(k_cache, copy=True)
+    vc = np.array(v_cache, copy=True)
+    for b in range(N):
+        p = int(past_lens[b])
+        kc[b, :, p:p + seq, :] = k[b]
+        vc[b, :, p:p + seq, :] = v[b]
+    o = np.full(q.shape, np.nan, dtype=np.float32)
+    pairs = heads if heads is not None else [(b, h) for b in range(N) for h in range(H)]
+    for b, h in pairs:
+        p = int(past_lens[b])
+        kh = h // g
+        o[b, h] = attention_head(q[b, h], kc[b, kh, :p + seq].astype(np.float32),
+                                 vc[b, kh, :p + seq].astype(np.float32), p, scale, True)
+    return o, kc, vc
+
+
+def rope(x, pos, theta=10000.0, threads=1):
+    """x [batch, seq, heads, D] float32 (already up-cast); pos int64 [batch, seq] or [seq]."""
+    x = _c(x, np.float32)
+    batch, seq, heads, D = x.shape
+    pos = _c(pos, np.int64)
+    per_batch = int(pos.ndim == 2)
+    assert pos.shape == ((batch, seq) if per_batch else (seq,))
+    y = np.empty_like(x)
+    lib().oracle_rope_f32(_p(y), _p(x), _p(pos), per_batch, batch, seq, heads, D, float(theta), threads)
+    return y

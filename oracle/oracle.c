@@ -1,0 +1,390 @@
+/*
+ * CPU oracle (test infrastructure, never on the product path): see oracle.h for
+ * the reference file:line each function follows and for what pins it.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ threads */
+
+typedef void (*range_fn)(size_t begin, size_t end, void *ctx);
+
+struct span_job {
+    range_fn fn;
+    void *ctx;
+    size_t begin, end;
+};
+
+static void *span_entry(void *p) {
+    struct span_job *j = (struct span_job *) p;
+    j->fn(j->begin, j->end, j->ctx);
+    return NULL;
+}
+
+/* Split [0, n) into contiguous spans, one per thread. The arithmetic done for
+ * an index never depends on the split. */
+static void for_spans(size_t n, int threads, range_fn fn, void *ctx) {
+    if (threads <= 1 || n < 2) {
+        fn(0, n, ctx);
+        return;
+    }
+    if ((size_t) threads > n) threads = (int) n;
+    pthread_t *tid = (pthread_t *) malloc(sizeof(pthread_t) * (size_t) threads);
+    struct span_job *jobs = (struct span_job *) malloc(sizeof(struct span_job) * (size_t) threads);
+    size_t chunk = (n + (size_t) threads - 1) / (size_t) threads;
+    int started = 0;
+    for (int t = 0; t < threads; ++t) {
+        size_t b = (size_t) t * chunk, e = b + chunk > n ? n : b + chunk;
+        if (b >= e) break;
+        jobs[t].fn = fn;
+        jobs[t].ctx = ctx;
+        jobs[t].begin = b;
+        jobs[t].end = e;
+        if (pthread_create(&tid[t], NULL, span_entry, &jobs[t]) != 0) {
+            fn(b, e, ctx);
+            tid[t] = 0;
+            jobs[t].fn = NULL;
+        }
+        started = t + 1;
+    }
+    for (int t = 0; t < started; ++t)
+        if (jobs[t].fn) pthread_join(tid[t], NULL);
+    free(jobs);
+    free(tid);
+}
+
+/* ----------------------------------------------------------------- rms norm */
+
+struct rms_ctx {
+    void *y;
+    const void *x, *w;
+    size_t cols;
+    float eps;
+};
+
+static void rms_rows_f32(size_t r0, size_t r1, void *p) {
+    struct rms_ctx *c = (struct rms_ctx *) p;
+    const float *w = (const float *) c->w;
+    for (size_t r = r0; r < r1; ++r) {
+        const float *x = (const float *) c->x + r * c->cols;
+        float *y = (float *) c->y + r * c->cols;
+        float ss = 0.0f;
+        for (size_t j = 0; j < c->cols; ++j) ss = ss + x[j] * x[j];
+        ss = ss / (float) c->cols;
+        ss = ss + c->eps;
+        /* double division of 1 by the float square root, rounded back to float */
+        ss = (float) (1.0 / (double) sqrtf(ss));
+        for (size_t j = 0; j < c->cols; ++j) y[j] = x[j] * ss * w[j];
+    }
+}
+
+static void rms_rows_f64(size_t r0, size_t r1, void *p) {
+    struct rms_ctx *c = (struct rms_ctx *) p;
+    const double *w = (const double *) c->w;
+    for (size_t r = r0; r < r1; ++r) {
+        const double *x = (const double *) c->x + r * c->cols;
+        double *y = (double *) c->y + r * c->cols;
+        double ss = 0.0;
+        for (size_t j = 0; j < c->cols; ++j) ss = ss + x[j] * x[j];
+        ss = ss / (double) c->cols;
+        ss = ss + (double) c->eps;
+        ss = 1.0 / sqrt(ss);
+        for (size_t j = 0; j < c->cols; ++j) y[j] = x[j] * ss * w[j];
+    }
+}
+
+void oracle_rms_norm_f32(float *y, const float *x, const float *w,
+                         size_t rows, size_t cols, float eps, int threads) {
+    struct rms_ctx c = {y, x, w, cols, eps};
+    for_spans(rows, threads, rms_rows_f32, &c);
+}
+
+void oracle_rms_norm_f64(double *y, const double *x, const double *w,
+                         size_t rows, size_t cols, float eps, int threads) {
+    struct rms_ctx c = {y, x, w, cols, eps};
+    for_spans(rows, threads, rms_rows_f64, &c);
+}
+
+/* ------------------------------------------------------------------ softmax */
+
+struct softmax_ctx {
+    void *y;
+    const void *x;
+    size_t mid, post;
+    size_t rows, cols; /* causal form */
+};
+
+/* slice i of pre*post: first element at (i - i%post)*mid + i%post, step post */
+#define SOFTMAX_BODY(T, EXP)                                                   \
+    struct softmax_ctx *c = (struct softmax_ctx *) p;                          \
+    const T *x = (const T *) c->x;                                             \
+    T *y = (T *) c->y;                                                         \
+    size_t mid = c->mid, post = c->post;                                       \
+    for (size_t i = i0; i < i1; ++i) {                                         \
+        size_t base = (i - i % post) * mid + i % post;                         \
+        size_t arg = 0;                                                        \
+        for (size_t j = 1; j < mid; ++j)                                       \
+            if (x[base + arg * post] < x[base + j * post]) arg = j;            \
+        T mx = x[base + arg * post];                                           \
+        T sum = 0;                                                             \
+        for (size_t j = 0; j < mid; ++j) {                                     \
+            T e = EXP(x[base + j * post] - mx);                                \
+            y[base + j * post] = e;                                            \
+            sum = sum + e;                                                     \
+        }                                                                      \
+        for (size_t j = 0; j < mid; ++j) y[base + j * post] = y[base + j * post] / sum; \
+    }
+
+static void softmax_slices_f32(size_t i0, size_t i1, void *p) { SOFTMAX_BODY(float, expf) }
+static void softmax_slices_f64(size_t i0, size_t i1, void *p) { SOFTMAX_BODY(double, exp) }
+
+void oracle_softmax_f32(float *y, const float *x, size_t pre, size_t mid, size_t post, int threads) {
+    struct softmax_ctx c = {y, x, mid, post, 0, 0};
+    for_spans(pre * post, threads, softmax_slices_f32, &c);
+}
+
+void oracle_softmax_f64(double *y, const double *x, size_t pre, size_t mid, size_t post, int threads) {
+    struct softmax_ctx c = {y, x, mid, post, 0, 0};
+    for_spans(pre * post, threads, softmax_slices_f64, &c);
+}
+
+void oracle_softmax_literal_f32(float *y, const float *x, size_t pre, size_t mid, size_t post) {
+    for (size_t i = 0; i < pre * post; ++i) {
+        size_t base = (i - i % post) * mid + i % post;
+        size_t arg = 0;
+        for (size_t j = 1; j < mid; ++j)
+            if (x[base + arg * post] < x[base + j * post]) arg = j;
+        float mx = x[base + arg * post];
+        int sum = 0; /* the reference's accumulator type: every addend < 1 is truncated away */
+        for (size_t j = 0; j < mid; ++j) {
+            float e = expf(x[base + j * post] - mx);
+            y[base + j * post] = e;
+            sum = (int) ((float) sum + e);
+        }
+        for (size_t j = 0; j < mid; ++j) y[base + j * post] = y[base + j * post] / (float) sum;
+    }
+}
+
+static void softmax_causal_rows_f32(size_t i0, size_t i1, void *p) {
+    struct softmax_ctx *c = (struct softmax_ctx *) p;
+    size_t rows = c->rows, cols = c->cols;
+    for (size_t i = i0; i < i1; ++i) {
+        const float *x = (const float *) c->x + i * cols;
+        float *y = (float *) c->y + i * cols;
+        size_t r = i % rows;
+        size_t keep = r + (cols - rows) + 1; /* columns 0 .. r + (cols - rows) */
+        if (keep > cols) keep = cols;
+        float mx = x[0];
+        for (size_t j = 1; j < keep; ++j)
+            if (mx < x[j]) mx = x[j];
+        float sum = 0.0f;
+        for (size_t j = 0; j < keep; ++j) {
+            float e = expf(x[j] - mx);
+            y[j] = e;
+            sum = sum + e;
+        }
+        for (size_t j = 0; j < keep; ++j) y[j] = y[j] / sum;
+        for (size_t j = keep; j < cols; ++j) y[j] = 0.0f;
+    }
+}
+
+void oracle_softmax_causal_f32(float *y, const float *x, size_t batch, size_t rows, size_t cols, int threads) {
+    struct softmax_ctx c = {y, x, 0, 0, rows, cols};
+    for_spans(batch * rows, threads, softmax_causal_rows_f32, &c);
+}
+
+/* ----------------------------------------------------------- matmul integer */
+
+/* the reference's subtraction: int8 - int8 wraps to int8; uint8 - uint8 goes
+ * through int16 and is truncated to int8. Both are "difference modulo 256". */
+static int8_t zp_sub(int is_signed, uint8_t v, uint8_t z) {
+    if (is_signed) return (int8_t) ((int) (int8_t) v - (int) (int8_t) z);
+    return (int8_t) (int16_t) ((int16_t) v - (int16_t) z);
+}
+
+struct mmi_ctx {
+    int32_t *y;
+    const int8_t *a, *b;
+    size_t m, k, n;
+};
+
+static void mmi_rows(size_t i0, size_t i1, void *p) {
+    struct mmi_ctx *c = (struct mmi_ctx *) p;
+    size_t k = c->k, n = c->n;
+    for (size_t i = i0; i < i1; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            int32_t sum = 0;
+            for (size_t q = 0; q < k; ++q)
+                sum += (int32_t) ((int) c->a[i * k + q] * (int) c->b[q * n + j]);
+            c->y[i * n + j] = sum;
+        }
+}
+
+void oracle_matmul_integer(int32_t *y, const void *a_, const void *b_,
+                           const void *a_zp_, int a_zp_signed, int a_zp_scalar,
+                           const void *b_zp_, int b_zp_signed, int b_zp_scalar,
+                           size_t batch, size_t m, size_t k, size_t n,
+                           const uint32_t *a_off, const uint32_t *b_off,
+                           size_t a_batch, size_t b_batch, int threads) {
+    const uint8_t *a = (const uint8_t *) a_, *b = (const uint8_t *) b_;
+    const uint8_t *a_zp = (const uint8_t *) a_zp_, *b_zp = (const uint8_t *) b_zp_;
+    int8_t *aw = NULL, *bw = NULL; /* the reference's workspace: zero-point-adjusted copies */
+    if (a_zp) {
+        aw = (int8_t *) malloc(a_batch * m * k + 1);
+        for (size_t i = 0; i < a_batch; ++i)
+            for (size_t r = 0; r < m; ++r)
+                for (size_t q = 0; q < k; ++q) {
+                    uint8_t z = a_zp_scalar ? a_zp[0] : a_zp[i * m + r];
+                    aw[(i * m + r) * k + q] = zp_sub(a_zp_signed, a[(i * m + r) * k + q], z);
+                }
+    }
+    if (b_zp) {
+        bw = (int8_t *) malloc(b_batch * k * n + 1);
+        for (size_t i = 0; i < b_batch; ++i)
+            for (size_t r = 0; r < k; ++r)
+                for (size_t q = 0; q < n; ++q) {
+                    /* as written in the reference: one zero point per ROW of B */
+                    uint8_t z = b_zp_scalar ? b_zp[0] : b_zp[i * k + r];
+                    bw[(i * k + r) * n + q] = zp_sub(b_zp_signed, b[(i * k + r) * n + q], z);
+                }
+    }
+    const int8_t *as = aw ? aw : (const int8_t *) a;
+    const int8_t *bs = bw ? bw : (const int8_t *) b;
+    for (size_t i = 0; i < batch; ++i) {
+        size_t ia = a_off ? a_off[i] : i, ib = b_off ? b_off[i] : i;
+        struct mmi_ctx c = {y + i * m * n, as + ia * m * k, bs + ib * k * n, m, k, n};
+        for_spans(m, threads, mmi_rows, &c);
+    }
+    free(aw);
+    free(bw);
+}
+
+/* -------------------------------------------------------- dequantize linear */
+
+struct dq_ctx {
+    float *y;
+    const void *x, *zp;
+    const float *scale;
+    size_t axis_len, inner, scale_count;
+    int dtype;
+};
+
+#define DQ_LOOP(TI)                                                            \
+    {                                                                          \
+        const TI *x = (const TI *) c->x;                                       \
+        const TI *zp = (const TI *) c->zp;                                     \
+        for (size_t e = e0; e < e1; ++e) {                                     \
+            size_t a = c->scale_count == 1 ? 0 : (e / c->inner) % c->axis_len; \
+            float s = c->scale[a];                                             \
+            /* the zero constant of the reference is an int when absent */     \
+            if (zp) c->y[e] = (float) (x[e] - zp[a]) * s;                      \
+            else c->y[e] = (float) (x[e] - 0) * s;                             \
+        }                                                                      \
+    }
+
+static void dq_span(size_t e0, size_t e1, void *p) {
+    struct dq_ctx *c = (struct dq_ctx *) p;
+    switch (c->dtype) {
+        case ORACLE_U8: DQ_LOOP(uint8_t) break;
+        case ORACLE_I8: DQ_LOOP(int8_t) break;
+        case ORACLE_U16: DQ_LOOP(uint16_t) break;
+        case ORACLE_I16: DQ_LOOP(int16_t) break;
+        case ORACLE_I32: DQ_LOOP(int32_t) break;
+        default: break;
+    }
+}
+
+int oracle_dequantize_linear(float *y, const void *x, const float *scale, const void *zp,
+                             size_t outer, size_t axis_len, size_t inner,
+                             int in_dtype, size_t scale_count, int threads) {
+    switch (in_dtype) {
+        case ORACLE_U8: case ORACLE_I8: case ORACLE_U16: case ORACLE_I16: case ORACLE_I32: break;
+        default: return -1;
+    }
+    if (scale_count != 1 && scale_count != axis_len) return -1;
+    struct dq_ctx c = {y, x, zp, scale, axis_len, inner, scale_count, in_dtype};
+    for_spans(outer * axis_len * inner, threads, dq_span, &c);
+    return 0;
+}
+
+/* ------------------------------------------------------- float matmul + mul */
+
+void oracle_matmul_f32(float *y, const float *a, const float *b,
+                       size_t M, size_t K, size_t N,
+                       size_t sa0, size_t sa1, size_t sb0, size_t sb1, float alpha) {
+    for (size_t i = 0; i < M; ++i)
+        for (size_t j = 0; j < N; ++j) {
+            float sum = 0.0f;
+            for (size_t q = 0; q < K; ++q) sum += a[i * sa0 + q * sa1] * b[q * sb0 + j * sb1];
+            y[i * N + j] = alpha * sum; /* beta == 0: the stale y is not read */
+        }
+}
+
+void oracle_mul_f32(float *y, const float *a, const float *b, size_t n_a, size_t n_b) {
+    size_t n = n_a > n_b ? n_a : n_b;
+    for (size_t i = 0; i < n; ++i) y[i] = a[n_a == 1 ? 0 : i] * b[n_b == 1 ? 0 : i];
+}
+
+/* ---------------------------------------------------------------- attention */
+
+void oracle_attention_head_f32(float *o, const float *q, const float *kc, const float *vc,
+                               size_t seq, size_t past, size_t D, float scale, int causal,
+                               float *scratch) {
+    size_t len = past + seq;
+    float *s = scratch, *pbuf = scratch + seq * len;
+    /* S = Q K^T (transB), then the "scale" kernel */
+    oracle_matmul_f32(s, q, kc, seq, D, len, D, 1, 1, D, 1.0f);
+    oracle_mul_f32(s, s, &scale, seq * len, 1);
+    if (causal)
+        for (size_t r = 0; r < seq; ++r)
+            for (size_t cidx = past + r + 1; cidx < len; ++cidx) s[r * len + cidx] = -INFINITY;
+    oracle_softmax_f32(pbuf, s, seq, len, 1, 1);
+    /* O = P V */
+    oracle_matmul_f32(o, pbuf, vc, seq, len, D, len, 1, D, 1, 1.0f);
+}
+
+/* --------------------------------------------------------------------- rope */
+
+struct rope_ctx {
+    float *y;
+    const float *x;
+    const int64_t *pos;
+    const float *inv_freq;
+    int pos_per_batch;
+    size_t seq, heads, D;
+};
+
+static void rope_tokens(size_t t0, size_t t1, void *p) {
+    struct rope_ctx *c = (struct rope_ctx *) p;
+    size_t half = c->D / 2;
+    for (size_t t = t0; t < t1; ++t) {
+        size_t s = t % c->seq;
+        int64_t position = c->pos_per_batch ? c->pos[t] : c->pos[s];
+        for (size_t i = 0; i < half; ++i) {
+            float angle = (float) position * c->inv_freq[i];
+            float cs = (float) cos((double) angle), sn = (float) sin((double) angle);
+            for (size_t h = 0; h < c->heads; ++h) {
+                const float *x = c->x + (t * c->heads + h) * c->D;
+                float *y = c->y + (t * c->heads + h) * c->D;
+                float lo = x[i], hi = x[i + half];
+                y[i] = lo * cs - hi * sn;
+                y[i + half] = hi * cs + lo * sn;
+            }
+        }
+    }
+}
+
+void oracle_rope_f32(float *y, const float *x, const int64_t *pos, int pos_per_batch,
+                     size_t batch, size_t seq, size_t heads, size_t D, float theta, int threads) {
+    size_t half = D / 2;
+    float *inv_freq = (float *) malloc(sizeof(float) * (half ? half : 1));
+    for (size_t i = 0; i < half; ++i)
+        inv_freq[i] = (float) pow((double) theta, -2.0 * (double) i / (double) D);
+    struct rope_ctx c = {y, x, pos, inv_freq, pos_per_batch, seq, heads, D};
+    for_spans(batch * seq, threads, rope_tokens, &c);
+    free(inv_freq);
+}

@@ -1,0 +1,364 @@
+"""Pins the CPU oracle (oracle/oracle.c) before anything is compared with it.
+
+Each oracle function is checked against (1) the known-answer vectors held by the reference's
+own tests (tests/golden/reference_kats.json) and (2) independent mathematics chosen so that a
+plausible mistake (dropped term, wrong sign/index, transposed operand) fails: float64 brute
+force, closed forms, invariants, numpy/torch library routines.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+
+
+def ulp_close(a, b, ulps=4):
+    """gtest's EXPECT_FLOAT_EQ: within 4 units in the last place."""
+    a = np.asarray(a, np.float32)
+    b = np.asarray(b, np.float32)
+    ai = a.view(np.int32).astype(np.int64)
+    bi = b.view(np.int32).astype(np.int64)
+    ai = np.where(ai < 0, -(ai & 0x7FFFFFFF), ai)
+    bi = np.where(bi < 0, -(bi & 0x7FFFFFFF), bi)
+    return np.all(np.abs(ai - bi) <= ulps)
+
+
+# ------------------------------------------------------------------ RmsNormalization
+
+def test_rms_kat_iota():
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    w = np.array([1, 2, 3, 4], dtype=np.float32)
+    y = oracle.rms_norm(x, w, 0.0)
+    # the reference test's inline formula, evaluated in float64
+    ref = np.zeros_like(x, dtype=np.float64)
+    for i in range(6):
+        row = x.reshape(6, 4)[i].astype(np.float64)
+        rms = 1.0 / np.sqrt((row * row).sum() / 4) if (row * row).sum() else np.inf
+        ref.reshape(6, 4)[i] = row * rms * w
+    assert ulp_close(y.reshape(-1)[4:], ref.astype(np.float32).reshape(-1)[4:])
+
+
+def test_rms_kat_constant_row():
+    x = np.full((2, 3, 4096), 2.0, np.float32)
+    w = np.full((4096,), 3.0, np.float32)
+    y = oracle.rms_norm(x, w, 0.0)
+    assert np.all(y == 3.0)
+
+
+def test_rms_recorded_vector():
+    rec = [c for c in GOLDEN["rms_normalization"] if c["kind"] == "recorded"][0]
+    y = oracle.rms_norm(np.array(rec["x"], np.float32).reshape(rec["shape"]),
+                        np.array(rec["w"], np.float32), rec["eps"])
+    assert ulp_close(y.reshape(-1), np.array(rec["expect"], np.float32), ulps=1)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_rms_against_float64_brute_force_and_invariants(dtype):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((7, 5, 333)).astype(dtype)
+    w = rng.uniform(0.5, 1.5, 333).astype(dtype)
+    eps = 1e-5
+    y = oracle.rms_norm(x, w, eps)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    ms = (x64 * x64).mean(-1, keepdims=True)
+    ref = x64 / np.sqrt(ms + np.float64(np.float32(eps))) * w64
+    tol = 1e-5 if dtype == np.float32 else 1e-12
+    assert np.all(np.abs(y - ref) <= tol * np.abs(ref) + 1e-30)
+    # invariant: sum_j (y_j / w_j)^2 == D * ms / (ms + eps)
+    lhs = ((y.astype(np.float64) / w64) ** 2).sum(-1)
+    rhs = 333 * ms[..., 0] / (ms[..., 0] + eps)
+    assert np.allclose(lhs, rhs, rtol=1e-4 if dtype == np.float32 else 1e-10)
+    # threads do not change a bit
+    assert np.array_equal(y, oracle.rms_norm(x, w, eps, threads=3))
+
+
+def test_rms_serial_float_accumulation_is_followed():
+    # 2^24 + 1 is not representable: a serial float sum of ones saturates, a pairwise one does not
+    # (cols chosen so the per-row serial sum of squares hits the float spacing).
+    x = np.ones((1, 1 << 12), np.float32) * np.float32(4096.0)  # x^2 = 2^24
+    x[0, 1:] = 1.0  # every later addend (1.0) is below half the spacing of 2^24 -> absorbed
+    y = oracle.rms_norm(x, np.ones(1 << 12, np.float32), 0.0)
+    expect_first = np.float32(4096.0) * np.float32(1.0 / np.sqrt(np.float64(np.float32(2.0 ** 24) / np.float32(4096))))
+    assert y[0, 0] == expect_first
+
+
+# ------------------------------------------------------------------ Softmax
+
+def test_softmax_kat_zeros_axis1_f64():
+    c = GOLDEN["softmax"][0]
+    x = np.zeros(c["shape"], np.float64)
+    y = oracle.softmax(x, axis=c["axis"])
+    assert np.all(y == 1.0 / 3)
+
+
+def test_softmax_literal_defect_vectors():
+    for case in GOLDEN["softmax"][1]["cases"]:
+        y = oracle.softmax_literal(np.array(case["x"], np.float32))
+        assert np.allclose(y, case["expect"], atol=5e-5)
+        # and the corrected oracle deliberately differs (it is a true softmax)
+        z = oracle.softmax(np.array(case["x"], np.float32))
+        assert abs(z.sum() - 1) < 1e-6 and not np.allclose(y, z, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("axis", [0, 1, 2, 3])
+def test_softmax_against_float64_textbook_all_axes(dtype, axis):
+    rng = np.random.default_rng(3)
+    x = (3 * rng.standard_normal((3, 4, 5, 6))).astype(dtype)
+    y = oracle.softmax(x, axis=axis)
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+    ref = e / e.sum(axis=axis, keepdims=True)
+    assert np.allclose(y, ref, rtol=2e-6 if dtype == np.float32 else 1e-14, atol=0)
+    assert np.allclose(y.sum(axis=axis), 1.0, atol=1e-6)
+    # shift invariance and thread independence
+    assert np.allclose(oracle.softmax((x + dtype(7)).astype(dtype), axis=axis), y, rtol=1e-5)
+    assert np.array_equal(y, oracle.softmax(x, axis=axis, threads=4))
+
+
+def test_softmax_matches_torch_library():
+    import torch
+    rng = np.random.default_rng(4)
+    x = (3 * rng.standard_normal((2, 3, 64, 257))).astype(np.float32)
+    ref = torch.softmax(torch.from_numpy(x).double(), dim=-1).numpy()
+    assert np.allclose(oracle.softmax(x), ref, rtol=3e-6, atol=1e-12)
+
+
+def test_softmax_causal_equals_data_masked_and_structure():
+    rng = np.random.default_rng(5)
+    for rows, cols in [(6, 6), (4, 9), (1, 5)]:
+        x = (3 * rng.standard_normal((2, 3, rows, cols))).astype(np.float32)
+        y = oracle.softmax_causal(x)
+        masked = x.copy()
+        r = np.arange(rows)[:, None]
+        c = np.arange(cols)[None, :]
+        masked[..., c > r + (cols - rows)] = -np.inf
+        assert np.array_equal(y, oracle.softmax(masked))  # exp(-inf) = 0 exactly, sums identical
+        assert np.all(y[..., c > r + (cols - rows)] == 0)
+        if rows == cols:
+            assert np.all(y[..., 0, 0] == 1.0)  # row 0 is one-hot
+        assert np.allclose(y.sum(-1), 1.0, atol=1e-6)
+
+
+# ------------------------------------------------------------------ MatMulInteger
+
+def _i8(a, zp, signed):
+    """mathematical restatement: difference modulo 256 read as int8."""
+    if signed:
+        d = a.astype(np.int8).astype(np.int64) - np.asarray(zp).astype(np.int8).astype(np.int64)
+    else:
+        d = a.astype(np.uint8).astype(np.int64) - np.asarray(zp).astype(np.uint8).astype(np.int64)
+    return ((d + 128) % 256) - 128
+
+
+def test_matmul_integer_kats():
+    k0, k1, k2, k3 = GOLDEN["mat_mul_integer"]
+    y = oracle.matmul_integer(np.array(k0["a"], np.uint8).reshape(k0["a_shape"]),
+                              np.array(k0["b"], np.uint8).reshape(k0["b_shape"]))
+    assert y.reshape(-1).tolist() == k0["expect"]
+    a = np.arange(1, 5, dtype=np.uint8).reshape(1, 4)
+    b = np.tile(np.arange(1, 13, dtype=np.uint8), (4, 1))
+    assert oracle.matmul_integer(a, b).reshape(-1).tolist() == [10 * i for i in range(1, 13)]
+    for rec in (k2, k3):
+        a = np.array(rec["a"], np.uint8).reshape(rec["a_shape"])
+        b = np.array(rec["b"], np.int8).reshape(rec["b_shape"])
+        az = np.array([rec["a_zp"]], np.uint8) if "a_zp" in rec else None
+        bz = np.array([rec["b_zp"]], np.int8) if "b_zp" in rec else None
+        assert oracle.matmul_integer(a, b, az, bz).reshape(-1).tolist() == rec["expect"]
+
+
+def test_matmul_integer_against_int64_brute_force():
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (37, 53), dtype=np.uint8)
+    b = rng.integers(-128, 128, (53, 29), dtype=np.int8)
+    az = np.array([128], np.uint8)
+    bz = np.array([0], np.int8)
+    y = oracle.matmul_integer(a, b, az, bz, threads=3)
+    ref = (a.astype(np.int64) - 128) @ b.astype(np.int64)
+    assert np.array_equal(y, ref)
+    # a - 128 == int8(a ^ 0x80): the identity the HIP kernel's fused zero point relies on
+    assert np.array_equal((a ^ 0x80).view(np.int8).astype(np.int64), a.astype(np.int64) - 128)
+    # non-square, transposition-sensitive: A @ B != (B.T @ A.T) unless transposed back
+    assert not np.array_equal(y, ref.T.copy().reshape(ref.shape)) or ref.shape[0] == ref.shape[1]
+
+
+def test_matmul_integer_extremes_and_wrap():
+    a = np.full((2, 4096), 0, np.uint8)      # a - 128 = -128
+    b = np.full((4096, 3), -128, np.int8)
+    y = oracle.matmul_integer(a, b, np.array([128], np.uint8), None)
+    assert np.all(y == 2 ** 26)
+    # outside the representable range the reference WRAPS (255 - 1 = 254 -> -2), it does not saturate
+    a = np.array([[255, 0]], np.uint8)
+    b = np.array([[1], [1]], np.int8)
+    y = oracle.matmul_integer(a, b, np.array([1], np.uint8), None)
+    assert y.item() == (-2) + (-1)
+
+
+def test_matmul_integer_zero_point_variants_and_broadcast():
+    rng = np.random.default_rng(6)
+    a = rng.integers(0, 256, (2, 1, 5, 7), dtype=np.uint8)
+    b = rng.integers(0, 256, (1, 3, 7, 4), dtype=np.uint8)
+    # per-row zero point for A: one per (batch, row); for B as written: one per (batch, row of B)
+    az = rng.integers(0, 256, (2 * 5,), dtype=np.uint8)
+    bz = rng.integers(-128, 128, (3 * 7,), dtype=np.int8)  # I8 zero point => B bytes read signed
+    y = oracle.matmul_integer(a, b, az, bz)
+    A = _i8(a, az.reshape(2, 1, 5, 1), signed=False)
+    B = _i8(b, bz.reshape(1, 3, 7, 1), signed=True)
+    ref = np.einsum("abik,abkj->abij", np.broadcast_to(A, (2, 3, 5, 7)), np.broadcast_to(B, (2, 3, 7, 4)))
+    assert y.shape == (2, 3, 5, 4) and np.array_equal(y, ref)
+
+
+# ------------------------------------------------------------------ DequantizeLinear
+
+def test_dequantize_kat():
+    c = GOLDEN["dequantize_linear"][0]
+    y = oracle.dequantize_linear(np.array(c["x"], np.uint8), np.float32(c["scale"]), np.array([c["zp"]], np.uint8))
+    assert y.tolist() == c["expect"]
+
+
+@pytest.mark.parametrize("dt", [np.uint8, np.int8, np.uint16, np.int16, np.int32])
+def test_dequantize_scalar_and_per_axis_closed_form(dt):
+    rng = np.random.default_rng(7)
+    info = np.iinfo(dt)
+    lo, hi = max(info.min, -(1 << 20)), min(info.max, 1 << 20)
+    x = rng.integers(lo, hi + 1, (3, 5, 4), dtype=dt)
+    zp1 = rng.integers(lo, hi + 1, (1,), dtype=dt)
+    s1 = np.float32(0.0123)
+    y = oracle.dequantize_linear(x, s1, zp1)
+    ref = (x.astype(np.int64) - int(zp1[0])).astype(np.float32) * s1
+    assert np.array_equal(y, ref)
+    for axis in (0, 1, 2):
+        n = x.shape[axis]
+        s = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+        zp = rng.integers(lo, hi + 1, (n,), dtype=dt)
+        shape = [1, 1, 1]
+        shape[axis] = n
+        ref = (x.astype(np.int64) - zp.astype(np.int64).reshape(shape)).astype(np.float32) * s.reshape(shape)
+        assert np.array_equal(oracle.dequantize_linear(x, s, zp, axis=axis, threads=2), ref)
+        assert np.array_equal(oracle.dequantize_linear(x, s, None, axis=axis),
+                              x.astype(np.float32) * s.reshape(shape))
+
+
+# ------------------------------------------------------------------ MatMul / Mul (oracle blocks)
+
+def test_matmul_f32_exact_on_integer_operands_and_transb():
+    rng = np.random.default_rng(8)
+    a = rng.integers(-8, 9, (5, 11)).astype(np.float32)
+    b = rng.integers(-8, 9, (11, 7)).astype(np.float32)
+    assert np.array_equal(oracle.matmul_f32(a, b), (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32))
+    bt = np.ascontiguousarray(b.T)
+    assert np.array_equal(oracle.matmul_f32(a, bt, trans_b=True), oracle.matmul_f32(a, b))
+    assert np.array_equal(oracle.matmul_f32(a, b, alpha=0.5), 0.5 * oracle.matmul_f32(a, b))
+    assert np.array_equal(oracle.mul_f32(a, np.float32(0.25)), a * np.float32(0.25))
+
+
+# ------------------------------------------------------------------ Attention (parity unpinned by the reference)
+
+def _attention_f64(q, kc, vc, past, scale):
+    seq = q.shape[0]
+    s = (q.astype(np.float64) @ kc.astype(np.float64).T) * scale
+    cols = np.arange(past + seq)[None, :]
+    rows = np.arange(seq)[:, None]
+    s[cols > past + rows] = -np.inf
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    return p @ vc.astype(np.float64)
+
+
+def test_attention_head_vs_float64_brute_force_tiny():
+    rng = np.random.default_rng(9)
+    for seq, past, D in [(1, 0, 8), (1, 5, 8), (4, 3, 8), (7, 0, 16)]:
+        q = rng.standard_normal((seq, D)).astype(np.float32)
+        kc = rng.standard_normal((past + seq, D)).astype(np.float32)
+        vc = rng.standard_normal((past + seq, D)).astype(np.float32)
+        o = oracle.attention_head(q, kc, vc, past, 1 / np.sqrt(D))
+        assert np.allclose(o, _attention_f64(q, kc, vc, past, 1 / np.sqrt(D)), rtol=1e-5, atol=1e-6)
+
+
+def test_attention_invariants():
+    rng = np.random.default_rng(10)
+    D = 16
+    # seq=1, past=0 => O = V
+    q = rng.standard_normal((1, D)).astype(np.float32)
+    k = rng.standard_normal((1, D)).astype(np.float32)
+    v = rng.standard_normal((1, D)).astype(np.float32)
+    assert np.array_equal(oracle.attention_head(q, k, v, 0, 0.25), v)
+    # uniform K => O = mean(V)
+    L = 9
+    kc = np.tile(k, (L, 1))
+    vc = rng.standard_normal((L, D)).astype(np.float32)
+    o = oracle.attention_head(q, kc, vc, L - 1, 0.25)
+    assert np.allclose(o[0], vc.mean(0), rtol=1e-5, atol=1e-6)
+    # permuting past positions leaves a decode output unchanged (up to summation order)
+    kc = rng.standard_normal((L, D)).astype(np.float32)
+    perm = np.concatenate([rng.permutation(L - 1), [L - 1]])
+    o1 = oracle.attention_head(q, kc, vc, L - 1, 0.25)
+    o2 = oracle.attention_head(q, kc[perm], vc[perm], L - 1, 0.25)
+    assert np.allclose(o1, o2, rtol=1e-5, atol=1e-6)
+
+
+def test_attention_kvcache_vs_torch_sdpa_gqa():
+    import torch
+    rng = np.random.default_rng(11)
+    N, H, Hkv, seq, D, S = 2, 4, 2, 3, 8, 10
+    q = rng.standard_normal((N, H, seq, D)).astype(np.float32)
+    k = rng.standard_normal((N, Hkv, seq, D)).astype(np.float32)
+    v = rng.standard_normal((N, Hkv, seq, D)).astype(np.float32)
+    kc = rng.standard_normal((N, Hkv, S, D)).astype(np.float32)
+    vc = rng.standard_normal((N, Hkv, S, D)).astype(np.float32)
+    past = np.array([4, 6])
+    o, kco, vco = oracle.attention_kvcache(q, k, v, kc, vc, past, 1 / np.sqrt(D))
+    for b in range(N):
+        p = past[b]
+        assert np.array_equal(kco[b, :, p:p + seq], k[b]) and np.array_equal(vco[b, :, p:p + seq], v[b])
+        assert np.array_equal(kco[b, :, :p], kc[b, :, :p]) and np.array_equal(kco[b, :, p + seq:], kc[b, :, p + seq:])
+        L = p + seq
+        mask = torch.ones(seq, L, dtype=torch.bool).tril(diagonal=int(p))
+        kk = torch.from_numpy(kco[b, :, :L]).repeat_interleave(H // Hkv, dim=0)
+        vv = torch.from_numpy(vco[b, :, :L]).repeat_interleave(H // Hkv, dim=0)
+        ref = torch.nn.functional.scaled_dot_product_attention(
+            torch.from_numpy(q[b]).double(), kk.double(), vv.double(), attn_mask=mask)
+        assert np.allclose(o[b], ref.numpy(), rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------------------------ RoPE (parity unpinned by the reference)
+
+def _rope_hf_f64(x, pos, theta):
+    """Independent HF-style rotate_half formulation in float64."""
+    D = x.shape[-1]
+    inv = 1.0 / (theta ** (np.arange(0, D, 2, dtype=np.float64) / D))
+    ang = pos[..., None].astype(np.float64) * inv           # [B, S, D/2]
+    emb = np.concatenate([ang, ang], -1)[:, :, None, :]      # [B, S, 1, D]
+    x64 = x.astype(np.float64)
+    rot = np.concatenate([-x64[..., D // 2:], x64[..., :D // 2]], -1)
+    return x64 * np.cos(emb) + rot * np.sin(emb)
+
+
+def test_rope_vs_independent_float64_and_invariants():
+    rng = np.random.default_rng(12)
+    B, S, H, D = 2, 50, 3, 16
+    x = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    pos = np.tile(np.arange(S, dtype=np.int64), (B, 1))
+    y = oracle.rope(x, pos, 10000.0)
+    assert np.allclose(y, _rope_hf_f64(x, pos, 10000.0), atol=2e-5)
+    # [seq] positions broadcast over batch
+    assert np.array_equal(y, oracle.rope(x, pos[0], 10000.0))
+    # pos 0 => identity
+    assert np.array_equal(oracle.rope(x, np.zeros((B, S), np.int64)), x)
+    # pairwise norm preserved
+    n_in = x[..., :D // 2] ** 2 + x[..., D // 2:] ** 2
+    n_out = y[..., :D // 2] ** 2 + y[..., D // 2:] ** 2
+    assert np.allclose(n_in, n_out, rtol=1e-5, atol=1e-6)
+    # R(p1) R(p2) = R(p1 + p2); inverse by negated position
+    p1 = rng.integers(0, 100, (B, S)).astype(np.int64)
+    p2 = rng.integers(0, 100, (B, S)).astype(np.int64)
+    assert np.allclose(oracle.rope(oracle.rope(x, p1), p2), oracle.rope(x, p1 + p2), atol=1e-4)
+    assert np.allclose(oracle.rope(oracle.rope(x, p1), -p1), x, atol=1e-5)
+    # large positions (the config's range) still within 1e-3 of float64 angles
+    big = np.full((B, S), 2047, np.int64)
+    assert np.allclose(oracle.rope(x, big), _rope_hf_f64(x, big, 10000.0), atol=1e-3)
+    assert np.array_equal(oracle.rope(x, p1, threads=4), oracle.rope(x, p1))
