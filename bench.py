@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X kernel backend for RefactorGraph's LLM-operator hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|headline] [--no-cpu]
+
+Prints ONE JSON line.  The headline metric is AttentionKVCache decode throughput (algorithmic
+GB/s, fp16, N=32, 32 query / 8 kv heads, D=128, cache capacity 4096, per-row history lengths
+~U{1024..4095}) with all inputs resident in HBM before the timed region.  A "step" is one
+decode call (cache append + attention for the whole batch).  The same line carries
+  roofline      the decode call against the 8 TB/s HBM peak,
+  cpu_baseline  the CPU oracle (a C restatement of the reference's CPU kernels) timed on a
+                bounded sample of the same workload on this host,
+  ops           the other hot-path kernels at their BASELINE.json configs, each with its own
+                roofline entry (MatMulInteger against the 5.0 POP/s dense int8 MFMA peak).
+One GPU only: --gpus N with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published
+FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 MFMA, published
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--ops", default="all", choices=["all", "headline"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only", default="", help="comma-separated op names to run besides the headline")
+    return ap.parse_args()
+
+
+def time_steps(torch, fn, steps, warmup, n_sets):
+    """Runs fn(i % n_sets) warmup+steps times; returns (wall ms per step over the timed region,
+    mean device ms per call from HIP events on the launch stream, min device ms)."""
+    for i in range(warmup):
+        fn(i % n_sets)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn(i % n_sets)
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev = [a.elapsed_time(b) for a, b in zip(starts, stops)]
+    return wall_ms, float(np.mean(dev)), float(np.min(dev))
+
+
+def hbm_entry(bytes_per_call, dev_ms):
+    gbs = bytes_per_call / (dev_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the path shards without exchange; "
+              "no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from refactorgraph_amd import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = "cuda"
+    torch.cuda.set_device(0)
+    only = set(filter(None, args.only.split(",")))
+
+    def want(name):
+        return args.ops == "all" and (not only or name in only)
+
+    # ------------------------------------------------------------ headline: decode
+    N, H, Hkv, D, cap = 32, 32, 8, 128, 4096
+    scale = 1.0 / math.sqrt(D)
+    past_np = np.random.default_rng(14).integers(1024, 4096, N).astype(np.int64)
+    sum_past = int(past_np.sum())
+    decode_bytes = 4096 * sum_past + 786432  # K,V history read + new rows read/written + Q read + O write
+    n_sets = 2                                # 2 x 537 MB of caches: nothing survives in the 256 MB MALL
+    gen = torch.Generator(device=dev)
+
+    def randn16(shape, seed):
+        gen.manual_seed(seed)
+        return torch.randn(shape, generator=gen, device=dev, dtype=torch.float32).half()
+
+    sets = []
+    for s in range(n_sets):
+        sets.append(dict(
+            q=randn16((N, H, 1, D), 9 + 100 * s), k=randn16((N, Hkv, 1, D), 10 + 100 * s),
+            v=randn16((N, Hkv, 1, D), 11 + 100 * s), kc=randn16((N, Hkv, cap, D), 12 + 100 * s),
+            vc=randn16((N, Hkv, cap, D), 13 + 100 * s), o=torch.empty((N, H, 1, D), device=dev, dtype=torch.float16)))
+    past = torch.from_numpy(past_np).to(dev)
+    ws = ops.attention_workspace(N, H, Hkv, 1, cap, D, dev)
+
+    def decode(i):
+        t = sets[i]
+        ops.attention_kvcache(t["q"], t["k"], t["v"], t["kc"], t["vc"], past, scale, out=t["o"], workspace=ws)
+
+    wall_ms, dev_ms, dev_min = time_steps(torch, decode, args.steps, args.warmup, n_sets)
+    value = decode_bytes / (wall_ms * 1e-3) / 1e9
+    roofline = hbm_entry(decode_bytes, dev_ms)
+    roofline["kernel"] = "attn_split+attn_merge (one rg_hip_attention_kvcache call)"
+    roofline["algorithmic_bytes"] = decode_bytes
+    roofline["device_ms_mean"] = round(dev_ms, 5)
+    roofline["device_ms_min"] = round(dev_min, 5)
+
+    result = {
+        "metric": "AttentionKVCache decode GB/s (% HBM peak); MatMulInteger int8 TOPS (% MFMA)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "AttentionKVCache decode fp16 N=32 H=32 Hkv=8 D=128 cap=4096 "
+                               "past~U{1024..4095} (seed 14), scale 1/sqrt(128)",
+                   "sum_past": sum_past, "cache_sets_rotated": n_sets},
+        "roofline": roofline,
+    }
+
+    # ------------------------------------------------------------ CPU baseline (bounded sample)
+    if not args.no_cpu:
+        import oracle
+        t = sets[0]
+        rows = [0, 1]                       # two batch rows, all 32 heads each
+        f = lambda x: x.float().cpu().numpy()
+        q, kc, vc = f(t["q"][rows]), f(t["kc"][rows]), f(t["vc"][rows])
+        k, v = f(t["k"][rows]), f(t["v"][rows])
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 10.0:
+            oracle.attention_kvcache(q, k, v, kc, vc, past_np[rows], scale)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        sample_bytes = 4096 * int(past_np[rows].sum()) + 786432 * len(rows) // N
+        result["cpu_baseline"] = {
+            "value": round(sample_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"batch rows {rows} of the same workload (all 32 heads, {reps} repetitions, "
+                      f"{cpu_s * 1e3:.1f} ms each); composed MatMul/scale/softmax/MatMul oracle in fp32"}
+
+    # ------------------------------------------------------------ the other hot-path kernels
+    ops_out = {}
+    steps, warmup = args.steps, args.warmup
+
+    if want("rms_norm"):
+        nb = 5  # 5 x (134 MB in + 134 MB out): beyond the 256 MB MALL
+        xs = [torch.randn((32, 128, 4096), device=dev) for _ in range(nb)]
+        ys = [torch.empty_like(xs[0]) for _ in range(nb)]
+        w = torch.rand(4096, device=dev) + 0.5
+        wall, dms, dmin = time_steps(torch, lambda i: ops.rms_norm(xs[i], w, 1e-5, out=ys[i]), steps, warmup, nb)
+        e = hbm_entry(134234112, dms)
+        e.update(workload="RmsNormalization f32 [32,128,4096]", device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5))
+        ops_out["rms_norm"] = e
+        del xs, ys
+
+    if want("softmax"):
+        x = (3 * torch.randn((8, 32, 2048, 2048), device=dev)).half()
+        y = torch.empty_like(x)
+        for causal, nbytes, name in ((False, 4294967296, "softmax"), (True, 3221749760, "softmax_causal")):
+            wall, dms, dmin = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 2, 5), 3, 1)
+            e = hbm_entry(nbytes, dms)
+            e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_mean=round(dms, 5),
+                     device_ms_min=round(dmin, 5))
+            ops_out[name] = e
+        del x, y
+
+    if want("rope"):
+        nb = 2
+        xs = [torch.randn((16, 2048, 32, 128), device=dev).half() for _ in range(nb)]
+        ys = [torch.empty_like(xs[0]) for _ in range(nb)]
+        pos = torch.arange(2048, device=dev, dtype=torch.int64).repeat(16, 1).contiguous()
+        wall, dms, dmin = time_steps(torch, lambda i: ops.rope(xs[i], pos, 10000.0, out=ys[i]), steps, warmup, nb)
+        e = hbm_entry(537133056, dms)
+        e.update(workload="RotaryEmbedding fp16 [16,2048,32,128]", device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5))
+        ops_out["rope"] = e
+        del xs, ys
+
+    if want("dequantize_linear"):
+        nb = 8  # 8 x 84 MB
+        xs = [torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8) for _ in range(nb)]
+        ys = [torch.empty((4096, 4096), device=dev) for _ in range(nb)]
+        sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
+        wall, dms, dmin = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
+        e = hbm_entry(83902464, dms)
+        e.update(workload="DequantizeLinear i8->f32 [4096,4096] per-axis scale", device_ms_mean=round(dms, 5),
+                 device_ms_min=round(dmin, 5))
+        ops_out["dequantize_linear"] = e
+        del xs, ys
+
+    if want("matmul_integer"):
+        a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
+        b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
+        az = torch.tensor([128], device=dev, dtype=torch.uint8)
+        bz = torch.tensor([0], device=dev, dtype=torch.int8)
+        y = torch.empty((4096, 4096), device=dev, dtype=torch.int32)
+        wall, dms, dmin = time_steps(torch, lambda i: ops.matmul_integer(a, b, az, bz, out=y), steps, warmup, 1)
+        tops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
+        ops_out["matmul_integer"] = {
+            "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+            "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
+            "workload": "MatMulInteger u8 x i8 -> i32 4096^3, a_zp=128 b_zp=0",
+            "device_ms_mean": round(dms, 5), "device_ms_min": round(dmin, 5)}
+        if not args.no_cpu:
+            import oracle
+            m = 64
+            an, bn = a[:m].cpu().numpy(), b.cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.matmul_integer(an, bn, np.array([128], np.uint8), np.array([0], np.int8), threads=1)
+            dt = time.perf_counter() - t0
+            ops_out["matmul_integer"]["cpu_baseline"] = {
+                "value": round(2 * m * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
+                "sample": f"first {m} rows of A against all of B ({dt:.1f} s)"}
+        del a, b, y
+
+    if want("attention_prefill"):
+        Np, seq = 32, 512
+        q = torch.randn((Np, H, seq, D), device=dev).half()
+        k = torch.randn((Np, Hkv, seq, D), device=dev).half()
+        v = torch.randn((Np, Hkv, seq, D), device=dev).half()
+        kc = torch.zeros((Np, Hkv, cap, D), device=dev, dtype=torch.float16)
+        vc = torch.zeros_like(kc)
+        o = torch.empty_like(q)
+        zero = torch.zeros(Np, device=dev, dtype=torch.int64)
+        wsp = ops.attention_workspace(Np, H, Hkv, seq, cap, D, dev)
+        wall, dms, dmin = time_steps(
+            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp),
+            max(steps // 5, 3), 2, 1)
+        e = hbm_entry(402653184, dms)
+        flops = 68853694464
+        e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=128",
+                 device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5),
+                 mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
+                 mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
+        ops_out["attention_prefill"] = e
+
+    if ops_out:
+        result["ops"] = ops_out
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

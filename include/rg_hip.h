@@ -1,0 +1,150 @@
+/*
+ * rg_hip.h — C ABI of the gfx950 (MI355X) kernel library behind RefactorGraph's
+ * 04kernel plugin surface.
+ *
+ * The reference links its CUDA kernels as C++ into the kernel library; here the
+ * device code lives in one shared object (librg_hip.so) and the host-side
+ * `Kernel::lower(Resources&)` closures are its only callers.  Each entry point
+ * below names the reference interface it stands in for (paths relative to the
+ * reference tree).
+ *
+ * Conventions
+ *   - every pointer named y/x/a/b/... is a DEVICE address unless said otherwise;
+ *   - `dtype` is the reference's DataType code
+ *     (src/00common/include/common/data_type.h:19-36): F32=1 U8=2 I8=3 U16=4
+ *     I16=5 I32=6 I64=7 FP16=10 F64=11 BF16=16;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream, which
+ *     is what a Routine uses: src/03runtime/src/stream.cc:60-69);
+ *   - launchers only enqueue work: no synchronisation, no allocation, no throw;
+ *   - the return value is a hipError_t as int (0 = success), or one of the
+ *     negative RG_HIP_E_* codes for requests the library does not handle.
+ */
+#ifndef RG_HIP_H
+#define RG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    RG_F32 = 1, RG_U8 = 2, RG_I8 = 3, RG_U16 = 4, RG_I16 = 5, RG_I32 = 6, RG_I64 = 7,
+    RG_FP16 = 10, RG_F64 = 11, RG_BF16 = 16,
+};
+
+enum {
+    RG_HIP_E_UNSUPPORTED = -1, /* dtype / shape combination has no kernel */
+    RG_HIP_E_ARGUMENT = -2,    /* null pointer, zero/odd size, misaligned operand */
+    RG_HIP_E_WORKSPACE = -3,   /* workspace smaller than the matching *_workspace() query */
+};
+
+/* ---- device + memory: what a hardware::Device / hardware::Memory backend needs -------------
+ * replaces the CUDA runtime calls in src/02hardware/src/devices/nvidia/device.cc:17-47
+ * (cudaGetDeviceCount, cudaSetDevice, cudaMemGetInfo, cudaGetDeviceProperties) and
+ * src/02hardware/src/devices/nvidia/memory.cc:14-38 (cudaMalloc, cudaFree, cudaMemcpy x3);
+ * rg_hip_sync stands in for kernel::cuda::sync (src/04kernel/cuda/src/functions.cu:13-15). */
+int rg_hip_device_count(int *count);
+int rg_hip_set_device(int card);
+int rg_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
+int rg_hip_device_name(char *buf, size_t len);
+int rg_hip_malloc(void **ptr, size_t bytes);
+int rg_hip_free(void *ptr);
+int rg_hip_memcpy_h2d(void *dst, const void *src, size_t bytes); /* blocking, like cudaMemcpy */
+int rg_hip_memcpy_d2h(void *dst, const void *src, size_t bytes); /* blocking */
+int rg_hip_memcpy_d2d(void *dst, const void *src, size_t bytes); /* blocking */
+int rg_hip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stream);
+int rg_hip_sync(void);
+const char *rg_hip_error_string(int status);
+
+/* ---- RmsNormalization --------------------------------------------------------------------
+ * replaces the NVRTC kernel + launch of
+ * src/04kernel/src/kernels/rms_normalization/cuda_kernel.cc:53-88,128-130;
+ * arithmetic contract: src/04kernel/src/kernels/rms_normalization/cpu_kernel.cc:47-65.
+ * y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * w.  dtype: F32, F64, FP16, BF16
+ * (sums in float for FP16/BF16).  y may alias x. */
+int rg_hip_rms_norm(void *y, const void *x, const void *w,
+                    size_t rows, size_t cols, float eps, int dtype, void *stream);
+
+/* ---- Softmax -----------------------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/softmax/cuda_kernel.cu:21-125 (and the cuDNN path
+ * cudnn_kernel.cc:37-76); shape digest as SoftmaxInfo
+ * (src/04kernel/src/attributes/softmax_info.cc:6-13): softmax along `mid` of [pre, mid, post].
+ * dtype: F32, F64, FP16, BF16 (exp/sum in float for FP16/BF16).
+ * causal_rows == 0: plain softmax.  causal_rows == R > 0 (requires post == 1, pre % R == 0,
+ * mid >= R): rows are grouped in [R, mid] matrices and row r keeps columns
+ * c <= r + (mid - R); masked inputs are not read and masked outputs are exactly 0. */
+int rg_hip_softmax(void *y, const void *x, size_t pre, size_t mid, size_t post,
+                   int dtype, size_t causal_rows, void *stream);
+
+/* ---- RotaryEmbedding ---------------------------------------------------------------------
+ * no counterpart exists in the reference (no rotary operator or kernel anywhere in src/);
+ * rotate-half pairing (i, i + dim/2), angle = pos * theta^(-2i/dim), on x[batch, seq, heads, dim].
+ * pos: int64 [batch, seq] when pos_per_batch != 0, else [seq].  dtype: FP16, BF16, F32.
+ * dim even, <= 512.  y may alias x. */
+int rg_hip_rope(void *y, const void *x, const int64_t *pos, int pos_per_batch,
+                size_t batch, size_t seq, size_t heads, size_t dim,
+                float theta, int dtype, void *stream);
+
+/* ---- DequantizeLinear --------------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/dequantize_linear/cuda_kernel.cc:50-86; arithmetic
+ * contract src/04kernel/src/kernels/dequantize_linear/cpu_kernel.cc:43-56:
+ * y = (float)((int)x - (int)zp) * scale.  x viewed as [outer, axis_len, inner];
+ * per_axis == 0: scale/zp hold one element (the reference path);
+ * per_axis != 0: scale/zp hold axis_len elements.  zp may be NULL (= 0).
+ * in_dtype: U8, I8, U16, I16, I32; output float. */
+int rg_hip_dequantize_linear(float *y, const void *x, const float *scale, const void *zp,
+                             size_t outer, size_t axis_len, size_t inner,
+                             int in_dtype, int per_axis, void *stream);
+
+/* ---- MatMulInteger -----------------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust
+ * zero-point pre-pass + cublasGemmEx); arithmetic contract
+ * src/04kernel/src/kernels/mat_mul_integer/cpu_kernel.cc:26-146:
+ * Y[i,j] = sum_k int8(A[i,k] - a_zp) * int8(B[k,j] - b_zp), differences taken modulo 256.
+ * a [a_batch, m, k], b [b_batch, k, n] bytes (row-major), y int32 [batch, m, n].
+ * a_zp / b_zp: NULL, or device pointers to one byte (RG_MMI_*_ZP_SCALAR) or to one byte per
+ * (batch, row) of the operand, as the reference's CPU kernel reads them.
+ * a_index / b_index: HOST arrays [batch] giving the operand matrix used by each output batch
+ * (the Broadcaster's locate(), src/04kernel/src/attributes/broadcaster.cc:87-100); NULL = i.
+ * The zero points are fused into the tile loads: no workspace is needed and
+ * rg_hip_matmul_integer_workspace() returns 0 (the reference needs m*k [+ k*n] bytes). */
+enum {
+    RG_MMI_A_ZP_SCALAR = 1u,
+    RG_MMI_B_ZP_SCALAR = 2u,
+};
+size_t rg_hip_matmul_integer_workspace(size_t batch, size_t m, size_t k, size_t n, unsigned flags);
+int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b,
+                          const void *a_zp, const void *b_zp, unsigned flags,
+                          size_t batch, size_t m, size_t k, size_t n,
+                          const uint32_t *a_index, const uint32_t *b_index,
+                          void *workspace, void *stream);
+
+/* ---- Attention with KV cache ---------------------------------------------------------------
+ * the reference declares this kernel but never defines it
+ * (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-25); the parameter block follows
+ * AttentionCuda::info and the tensor layouts follow src/08-01llm/README.md:29-63:
+ *   q, o [N, n_head, seq, D]; k, v [N, n_kv_head, seq, D]; caches [N, n_kv_head, cap, D].
+ * For batch row b with past = past_lens[past_per_row ? b : 0] (int64, read on the device):
+ *   the new k/v rows are written to cache[b, :, past .. past+seq), then query row r attends
+ *   cache positions 0 .. past + r with scores scaled by `scale` (causal decoder mask);
+ *   cache rows >= past + seq are left untouched.  past + seq > cap is clamped on the device
+ *   (rows that do not fit are dropped), never written out of bounds.
+ * k_cache == v_cache == NULL: no cache (past = 0, attends k/v directly).  past_lens == NULL: 0.
+ * n_head % n_kv_head == 0; D in {64, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
+ * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials for decode). */
+size_t rg_hip_attention_kvcache_workspace(size_t N, size_t n_head, size_t n_kv_head,
+                                          size_t seq, size_t cap, size_t D);
+int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *v,
+                             void *k_cache, void *v_cache,
+                             const int64_t *past_lens, int past_per_row,
+                             size_t N, size_t n_head, size_t n_kv_head,
+                             size_t seq, size_t cap, size_t D,
+                             float scale, int dtype,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RG_HIP_H */

@@ -1,0 +1,135 @@
+// RmsNormalization for gfx950.
+//
+// Arithmetic contract: src/04kernel/src/kernels/rms_normalization/cpu_kernel.cc:47-65 of the
+// reference (y = x * 1/sqrt(mean(x^2) + eps) * w, normalised over the last axis).
+// HBM-bound: one read of x, one write of y.  A row is held in registers between the
+// sum-of-squares pass and the scaling pass, so x is fetched from memory exactly once;
+// all global accesses are 128-bit and wave-contiguous.
+#include "common.hpp"
+
+namespace rg {
+namespace {
+
+// GROUP threads (one wavefront, or the whole 256-thread workgroup) own one row and keep up to
+// NV 16-byte vectors of it per thread.
+template <class T, int GROUP, int NV>
+__global__ __launch_bounds__(256) void rms_norm_rows(T *__restrict__ y, const T *__restrict__ x,
+                                                     const T *__restrict__ w, uint32_t rows,
+                                                     uint32_t cols, float eps) {
+    using CT = typename Compute<T>::type;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int ROWS_PER_BLOCK = 256 / GROUP;
+    __shared__ CT smem[4];
+
+    const uint32_t t = threadIdx.x % GROUP;
+    const size_t row = static_cast<size_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / GROUP;
+    const bool live = row < rows;  // only ever false for GROUP == 64 (no block barrier there)
+    const uint32_t nvec = cols / VEC;
+    const T *xr = x + row * cols;
+    T *yr = y + row * cols;
+
+    Vec16<T> xv[NV];
+    CT acc = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = t + i * GROUP;
+        if (live && idx < nvec) {
+            xv[i] = load16(xr + static_cast<size_t>(idx) * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const CT f = to_compute(xv[i].v[e]);
+                acc += f * f;
+            }
+        }
+    }
+    if constexpr (GROUP == kWave) {
+        acc = wave_sum(acc);
+    } else {
+        acc = block_allreduce<GROUP / kWave>(
+            acc, smem, [](CT v) { return wave_sum(v); }, [](CT a, CT b) { return a + b; });
+    }
+    const CT scale = CT(1) / sqrt(acc / static_cast<CT>(cols) + static_cast<CT>(eps));
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = t + i * GROUP;
+        if (live && idx < nvec) {
+            const Vec16<T> wv = load16(w + static_cast<size_t>(idx) * VEC);
+            Vec16<T> out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                out.v[e] = from_compute<T>(to_compute(xv[i].v[e]) * scale * to_compute(wv.v[e]));
+            store16(yr + static_cast<size_t>(idx) * VEC, out);
+        }
+    }
+}
+
+// Any row length / alignment: one workgroup per row, two passes over x (second one from cache).
+template <class T>
+__global__ __launch_bounds__(256) void rms_norm_generic(T *__restrict__ y, const T *__restrict__ x,
+                                                        const T *__restrict__ w, uint32_t cols,
+                                                        float eps) {
+    using CT = typename Compute<T>::type;
+    __shared__ CT smem[4];
+    const T *xr = x + static_cast<size_t>(blockIdx.x) * cols;
+    T *yr = y + static_cast<size_t>(blockIdx.x) * cols;
+    CT acc = 0;
+    for (uint32_t j = threadIdx.x; j < cols; j += 256) {
+        const CT f = to_compute(xr[j]);
+        acc += f * f;
+    }
+    acc = block_allreduce<4>(
+        acc, smem, [](CT v) { return wave_sum(v); }, [](CT a, CT b) { return a + b; });
+    const CT scale = CT(1) / sqrt(acc / static_cast<CT>(cols) + static_cast<CT>(eps));
+    for (uint32_t j = threadIdx.x; j < cols; j += 256)
+        yr[j] = from_compute<T>(to_compute(xr[j]) * scale * to_compute(w[j]));
+}
+
+template <class T, int GROUP, int NV>
+void launch_rows(T *y, const T *x, const T *w, size_t rows, size_t cols, float eps, hipStream_t s) {
+    constexpr int ROWS_PER_BLOCK = 256 / GROUP;
+    const unsigned grid = static_cast<unsigned>((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
+    rms_norm_rows<T, GROUP, NV><<<grid, 256, 0, s>>>(y, x, w, static_cast<uint32_t>(rows),
+                                                     static_cast<uint32_t>(cols), eps);
+}
+
+template <class T>
+int dispatch(void *y_, const void *x_, const void *w_, size_t rows, size_t cols, float eps,
+             hipStream_t s) {
+    auto *y = static_cast<T *>(y_);
+    auto *x = static_cast<const T *>(x_);
+    auto *w = static_cast<const T *>(w_);
+    constexpr size_t VEC = Vec16<T>::N;
+    const bool vec_ok = cols % VEC == 0 && aligned16(y) && aligned16(x) && aligned16(w);
+    const size_t nvec = cols / VEC;
+    if (vec_ok && nvec <= 64 * 2) {
+        if (nvec <= 64) launch_rows<T, 64, 1>(y, x, w, rows, cols, eps, s);
+        else launch_rows<T, 64, 2>(y, x, w, rows, cols, eps, s);
+    } else if (vec_ok && nvec <= 256 * 8) {
+        if (nvec <= 256) launch_rows<T, 256, 1>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 512) launch_rows<T, 256, 2>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 1024) launch_rows<T, 256, 4>(y, x, w, rows, cols, eps, s);
+        else launch_rows<T, 256, 8>(y, x, w, rows, cols, eps, s);
+    } else {
+        rms_norm_generic<T><<<static_cast<unsigned>(rows), 256, 0, s>>>(
+            y, x, w, static_cast<uint32_t>(cols), eps);
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace rg
+
+extern "C" int rg_hip_rms_norm(void *y, const void *x, const void *w, size_t rows, size_t cols,
+                               float eps, int dtype, void *stream) {
+    if (!y || !x || !w) return RG_HIP_E_ARGUMENT;
+    if (rows == 0 || cols == 0) return 0;
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+    hipStream_t s = rg::as_stream(stream);
+    switch (dtype) {
+        case RG_F32: return rg::dispatch<float>(y, x, w, rows, cols, eps, s);
+        case RG_F64: return rg::dispatch<double>(y, x, w, rows, cols, eps, s);
+        case RG_FP16: return rg::dispatch<__half>(y, x, w, rows, cols, eps, s);
+        case RG_BF16: return rg::dispatch<__hip_bfloat16>(y, x, w, rows, cols, eps, s);
+        default: return RG_HIP_E_UNSUPPORTED;
+    }
+}

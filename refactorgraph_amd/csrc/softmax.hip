@@ -1,0 +1,196 @@
+// Softmax along one axis of a [pre, mid, post] view, optional causal mask, for gfx950.
+//
+// Arithmetic contract: src/04kernel/src/kernels/softmax/cpu_kernel.cc:27-60 of the reference,
+// with a floating accumulator (the reference's own CUDA kernel, cuda_kernel.cu:29-55, computes
+// the same true softmax).  HBM-bound: a row is read once with 128-bit loads, kept in registers
+// through max / exp / sum, and written once.  FP16/BF16 rows are evaluated in float and rounded
+// once on store.
+#include "common.hpp"
+
+namespace rg {
+namespace {
+
+template <class CT> __device__ __forceinline__ CT neg_inf();
+template <> __device__ __forceinline__ float neg_inf<float>() { return -__builtin_inff(); }
+template <> __device__ __forceinline__ double neg_inf<double>() { return -__builtin_inf(); }
+
+// exp(d) for d <= 0.  16-bit storage: hardware exp2 on d*log2(e) (relative error ~1e-6 at
+// |d| < 30, far below the storage precision); F32/F64: the library routine.
+template <class T> struct Exp {
+    static __device__ __forceinline__ float eval(float d) {
+        return __builtin_amdgcn_exp2f(d * 1.4426950408889634f);
+    }
+};
+template <> struct Exp<float> {
+    static __device__ __forceinline__ float eval(float d) { return expf(d); }
+};
+template <> struct Exp<double> {
+    static __device__ __forceinline__ double eval(double d) { return exp(d); }
+};
+
+// e / sum.  16-bit storage multiplies by one reciprocal per row (the extra rounding is ~1e-7
+// relative); F32/F64 divide, as the reference does.
+template <class T> struct Normalise {
+    float inv;
+    __device__ __forceinline__ explicit Normalise(float sum) : inv(1.0f / sum) {}
+    __device__ __forceinline__ float operator()(float e) const { return e * inv; }
+};
+template <> struct Normalise<float> {
+    float sum;
+    __device__ __forceinline__ explicit Normalise(float s) : sum(s) {}
+    __device__ __forceinline__ float operator()(float e) const { return e / sum; }
+};
+template <> struct Normalise<double> {
+    double sum;
+    __device__ __forceinline__ explicit Normalise(double s) : sum(s) {}
+    __device__ __forceinline__ double operator()(double e) const { return e / sum; }
+};
+
+// GROUP threads own one contiguous row (post == 1), NV 16-byte vectors per thread.
+// causal_rows == 0: plain.  Otherwise row r of each [causal_rows, mid] matrix keeps the first
+// r + (mid - causal_rows) + 1 columns; vectors wholly beyond that are neither loaded nor
+// computed, only zero-filled.
+template <class T, int GROUP, int NV>
+__global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *__restrict__ x,
+                                                    uint64_t rows, uint32_t mid,
+                                                    uint32_t causal_rows) {
+    using CT = typename Compute<T>::type;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int ROWS_PER_BLOCK = 256 / GROUP;
+    __shared__ CT smem[4];
+
+    const uint32_t t = threadIdx.x % GROUP;
+    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / GROUP;
+    const bool live = row < rows;
+    const uint32_t nvec = mid / VEC;
+    uint32_t keep = mid;  // number of unmasked leading columns
+    if (causal_rows) keep = static_cast<uint32_t>(row % causal_rows) + (mid - causal_rows) + 1;
+    const T *xr = x + row * mid;
+    T *yr = y + row * mid;
+
+    CT f[NV][VEC];
+    CT mx = neg_inf<CT>();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = t + i * GROUP;
+        const uint32_t c0 = idx * VEC;
+        if (live && idx < nvec && c0 < keep) {
+            const Vec16<T> xv = load16(xr + c0);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                f[i][e] = c0 + e < keep ? to_compute(xv.v[e]) : neg_inf<CT>();
+                mx = mx < f[i][e] ? f[i][e] : mx;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) f[i][e] = neg_inf<CT>();
+        }
+    }
+    auto wmax = [](CT v) { return wave_max(v); };
+    auto wsum = [](CT v) { return wave_sum(v); };
+    if constexpr (GROUP == kWave) mx = wave_max(mx);
+    else mx = block_allreduce<GROUP / kWave>(mx, smem, wmax, [](CT a, CT b) { return a < b ? b : a; });
+
+    CT sum = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            // masked / padding slots hold -inf: exp gives exactly 0
+            f[i][e] = Exp<T>::eval(f[i][e] - mx);
+            sum += f[i][e];
+        }
+    if constexpr (GROUP == kWave) sum = wave_sum(sum);
+    else sum = block_allreduce<GROUP / kWave>(sum, smem, wsum, [](CT a, CT b) { return a + b; });
+
+    const Normalise<T> norm(sum);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = t + i * GROUP;
+        if (live && idx < nvec) {
+            Vec16<T> out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out.v[e] = from_compute<T>(norm(f[i][e]));
+            store16(yr + static_cast<size_t>(idx) * VEC, out);
+        }
+    }
+}
+
+// Any mid / post / alignment: one thread per (pre, post) slice, three passes, neighbouring
+// threads touch neighbouring `post` positions.
+template <class T>
+__global__ __launch_bounds__(256) void softmax_generic(T *__restrict__ y, const T *__restrict__ x,
+                                                       uint64_t slices, uint32_t mid, uint64_t post,
+                                                       uint32_t causal_rows) {
+    using CT = typename Compute<T>::type;
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= slices) return;
+    const uint64_t base = (i - i % post) * mid + i % post;
+    uint32_t keep = mid;
+    if (causal_rows) keep = static_cast<uint32_t>(i % causal_rows) + (mid - causal_rows) + 1;
+    CT mx = neg_inf<CT>();
+    for (uint32_t j = 0; j < keep; ++j) {
+        const CT v = to_compute(x[base + j * post]);
+        mx = mx < v ? v : mx;
+    }
+    CT sum = 0;
+    for (uint32_t j = 0; j < keep; ++j) sum += Exp<T>::eval(to_compute(x[base + j * post]) - mx);
+    for (uint32_t j = 0; j < keep; ++j)
+        y[base + j * post] = from_compute<T>(Exp<T>::eval(to_compute(x[base + j * post]) - mx) / sum);
+    for (uint32_t j = keep; j < mid; ++j) y[base + j * post] = from_compute<T>(CT(0));
+}
+
+template <class T, int GROUP, int NV>
+void launch_rows(T *y, const T *x, size_t rows, size_t mid, size_t causal_rows, hipStream_t s) {
+    constexpr int ROWS_PER_BLOCK = 256 / GROUP;
+    const unsigned grid = static_cast<unsigned>((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
+    softmax_rows<T, GROUP, NV><<<grid, 256, 0, s>>>(y, x, rows, static_cast<uint32_t>(mid),
+                                                    static_cast<uint32_t>(causal_rows));
+}
+
+template <class T>
+int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size_t causal_rows,
+             hipStream_t s) {
+    auto *y = static_cast<T *>(y_);
+    auto *x = static_cast<const T *>(x_);
+    constexpr size_t VEC = Vec16<T>::N;
+    const size_t nvec = mid / VEC;
+    const bool rows_ok = post == 1 && mid % VEC == 0 && aligned16(y) && aligned16(x) &&
+                         (pre + 3) / 4 <= 0x7fffffffu;
+    if (rows_ok && nvec <= 64 * 4) {
+        if (nvec <= 64) launch_rows<T, 64, 1>(y, x, pre, mid, causal_rows, s);
+        else if (nvec <= 128) launch_rows<T, 64, 2>(y, x, pre, mid, causal_rows, s);
+        else launch_rows<T, 64, 4>(y, x, pre, mid, causal_rows, s);
+    } else if (rows_ok && nvec <= 256 * 4) {
+        if (nvec <= 256) launch_rows<T, 256, 1>(y, x, pre, mid, causal_rows, s);
+        else if (nvec <= 512) launch_rows<T, 256, 2>(y, x, pre, mid, causal_rows, s);
+        else launch_rows<T, 256, 4>(y, x, pre, mid, causal_rows, s);
+    } else {
+        const uint64_t slices = static_cast<uint64_t>(pre) * post;
+        const uint64_t grid = (slices + 255) / 256;
+        if (grid > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+        softmax_generic<T><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+            y, x, slices, static_cast<uint32_t>(mid), post, static_cast<uint32_t>(causal_rows));
+    }
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace rg
+
+extern "C" int rg_hip_softmax(void *y, const void *x, size_t pre, size_t mid, size_t post,
+                              int dtype, size_t causal_rows, void *stream) {
+    if (!y || !x) return RG_HIP_E_ARGUMENT;
+    if (pre == 0 || mid == 0 || post == 0) return 0;
+    if (mid > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+    if (causal_rows && (post != 1 || pre % causal_rows != 0 || mid < causal_rows))
+        return RG_HIP_E_ARGUMENT;
+    hipStream_t s = rg::as_stream(stream);
+    switch (dtype) {
+        case RG_F32: return rg::dispatch<float>(y, x, pre, mid, post, causal_rows, s);
+        case RG_F64: return rg::dispatch<double>(y, x, pre, mid, post, causal_rows, s);
+        case RG_FP16: return rg::dispatch<__half>(y, x, pre, mid, post, causal_rows, s);
+        case RG_BF16: return rg::dispatch<__hip_bfloat16>(y, x, pre, mid, post, causal_rows, s);
+        default: return RG_HIP_E_UNSUPPORTED;
+    }
+}

@@ -1,0 +1,153 @@
+"""Test/benchmark driver: calls the C ABI on torch CUDA(HIP) tensors.
+
+Every function hands raw device pointers to librg_hip.so and enqueues on torch's current
+stream.  Argument meaning follows include/rg_hip.h; outputs are allocated with torch.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+import torch
+
+from . import abi
+from .abi import check, lib
+
+_T2CODE = {
+    torch.float32: abi.F32, torch.float64: abi.F64, torch.float16: abi.FP16, torch.bfloat16: abi.BF16,
+    torch.uint8: abi.U8, torch.int8: abi.I8, torch.int16: abi.I16, torch.int32: abi.I32,
+    torch.int64: abi.I64,
+}
+if hasattr(torch, "uint16"):
+    _T2CODE[torch.uint16] = abi.U16
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _need_gpu(*ts):
+    for t in ts:
+        if t is not None and (not t.is_cuda or not t.is_contiguous()):
+            raise ValueError("operands must be contiguous device tensors")
+
+
+def rms_norm(x, w, eps=1e-5, out=None):
+    _need_gpu(x, w)
+    y = torch.empty_like(x) if out is None else out
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    check(lib().rg_hip_rms_norm(_ptr(y), _ptr(x), _ptr(w), rows, cols, float(eps), _T2CODE[x.dtype], _stream()),
+          "rg_hip_rms_norm")
+    return y
+
+
+def softmax(x, axis=-1, causal=False, out=None):
+    _need_gpu(x)
+    axis = axis % x.dim()
+    pre = math.prod(x.shape[:axis])
+    mid = x.shape[axis]
+    post = math.prod(x.shape[axis + 1:])
+    causal_rows = x.shape[-2] if causal else 0
+    y = torch.empty_like(x) if out is None else out
+    check(lib().rg_hip_softmax(_ptr(y), _ptr(x), pre, mid, post, _T2CODE[x.dtype], causal_rows, _stream()),
+          "rg_hip_softmax")
+    return y
+
+
+def rope(x, pos, theta=10000.0, out=None):
+    _need_gpu(x, pos)
+    assert pos.dtype == torch.int64
+    batch, seq, heads, dim = x.shape
+    per_batch = int(pos.dim() == 2)
+    y = torch.empty_like(x) if out is None else out
+    check(lib().rg_hip_rope(_ptr(y), _ptr(x), _ptr(pos), per_batch, batch, seq, heads, dim, float(theta),
+                            _T2CODE[x.dtype], _stream()), "rg_hip_rope")
+    return y
+
+
+def dequantize_linear(x, scale, zp=None, axis=1, out=None):
+    _need_gpu(x, scale, zp)
+    assert scale.dtype == torch.float32
+    per_axis = int(scale.numel() != 1)
+    if per_axis:
+        axis = axis % x.dim()
+        outer, axis_len, inner = math.prod(x.shape[:axis]), x.shape[axis], math.prod(x.shape[axis + 1:])
+        assert scale.numel() == axis_len
+    else:
+        outer, axis_len, inner = 1, 1, x.numel()
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device) if out is None else out
+    check(lib().rg_hip_dequantize_linear(_ptr(y), _ptr(x), _ptr(scale), _ptr(zp), outer, axis_len, inner,
+                                         _T2CODE[x.dtype], per_axis, _stream()), "rg_hip_dequantize_linear")
+    return y
+
+
+def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):
+    """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
+    (batch, row) of the operand as the reference's CPU kernel reads them."""
+    _need_gpu(a, b, a_zp, b_zp)
+    m, k = a.shape[-2:]
+    k2, n = b.shape[-2:]
+    assert k == k2
+    ab, bb = tuple(a.shape[:-2]), tuple(b.shape[:-2])
+    ob = tuple(np.broadcast_shapes(ab, bb))
+    batch = math.prod(ob)
+    a_idx = b_idx = None
+    if ab != bb:
+        na, nb = math.prod(ab), math.prod(bb)
+        ia = np.arange(na, dtype=np.uint32).reshape(ab)
+        ib = np.arange(nb, dtype=np.uint32).reshape(bb)
+        oa, obb = np.broadcast_arrays(ia, ib)
+        a_idx = np.ascontiguousarray(oa.reshape(-1))
+        b_idx = np.ascontiguousarray(obb.reshape(-1))
+    flags = 0
+    if a_zp is not None and a_zp.numel() == 1:
+        flags |= abi.MMI_A_ZP_SCALAR
+    if b_zp is not None and b_zp.numel() == 1:
+        flags |= abi.MMI_B_ZP_SCALAR
+    y = torch.empty(ob + (m, n), dtype=torch.int32, device=a.device) if out is None else out
+    check(lib().rg_hip_matmul_integer(
+        _ptr(y), _ptr(a), _ptr(b), _ptr(a_zp), _ptr(b_zp), flags, batch, m, k, n,
+        None if a_idx is None else a_idx.ctypes.data_as(C.c_void_p),
+        None if b_idx is None else b_idx.ctypes.data_as(C.c_void_p),
+        None, _stream()), "rg_hip_matmul_integer")
+    return y
+
+
+_ws_cache = {}
+
+
+def attention_workspace(N, H, Hkv, seq, cap, D, device):
+    nbytes = lib().rg_hip_attention_kvcache_workspace(N, H, Hkv, seq, cap, D)
+    key = (nbytes, str(device))
+    if key not in _ws_cache:
+        _ws_cache[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return _ws_cache[key]
+
+
+def attention_kvcache(q, k, v, k_cache=None, v_cache=None, past_lens=None, scale=None, out=None,
+                      workspace=None):
+    """q [N,H,seq,D]; k, v [N,Hkv,seq,D]; caches [N,Hkv,cap,D] are updated in place;
+    past_lens: int64 device tensor with 1 or N elements (None = 0)."""
+    _need_gpu(q, k, v, k_cache, v_cache, past_lens)
+    N, H, seq, D = q.shape
+    Hkv = k.shape[1]
+    cap = k_cache.shape[2] if k_cache is not None else 0
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    per_row = 0
+    if past_lens is not None:
+        assert past_lens.dtype == torch.int64 and past_lens.numel() in (1, N)
+        per_row = int(past_lens.numel() == N and N > 1)
+    o = torch.empty_like(q) if out is None else out
+    ws = attention_workspace(N, H, Hkv, seq, cap, D, q.device) if workspace is None else workspace
+    check(lib().rg_hip_attention_kvcache(
+        _ptr(o), _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache), _ptr(v_cache), _ptr(past_lens), per_row,
+        N, H, Hkv, seq, cap, D, float(scale), _T2CODE[q.dtype], _ptr(ws), ws.numel(), _stream()),
+        "rg_hip_attention_kvcache")
+    return o

@@ -1,0 +1,386 @@
+"""Parity of the HIP kernels (called through the C ABI) against the CPU oracle.
+
+Bars: bit-exact for MatMulInteger / DequantizeLinear; <= 1e-5 relative for fp32 RmsNormalization
+and fp32 Softmax; <= 2e-3 absolute for fp16 paths (oracle in fp32 on up-cast inputs).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from refactorgraph_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+REL_F32 = 1e-5
+ABS_F16 = 2e-3
+DEV = "cuda"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_rel(y, ref, rel):
+    y = y.astype(np.float64)
+    ref = ref.astype(np.float64)
+    err = np.abs(y - ref)
+    bad = err > rel * np.abs(ref) + 1e-30
+    assert not bad.any(), f"max rel err {np.max(err / (np.abs(ref) + 1e-30)):.3e}"
+
+
+# ------------------------------------------------------------------ RmsNormalization
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (2, 3, 4096), (5, 7, 100), (3, 8192), (2, 10000), (4, 4097),
+                                   (64, 128, 512)])
+def test_rms_norm_f32(shape):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(shape).astype(np.float32)
+    w = np.random.default_rng(2).uniform(0.5, 1.5, shape[-1]).astype(np.float32)
+    y = host(ops.rms_norm(dev(x), dev(w), 1e-5))
+    assert_rel(y, oracle.rms_norm(x, w, 1e-5, threads=8), REL_F32)
+
+
+def test_rms_norm_reference_kats():
+    # reference tests: iota [2,3,4] with eps 0; x=2, w=3 on [2,3,4096] -> exactly 3
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    w = np.arange(1, 5, dtype=np.float32)
+    y = host(ops.rms_norm(dev(x), dev(w), 0.0))
+    assert_rel(y[0, 1:], oracle.rms_norm(x, w, 0.0)[0, 1:], 4 * 1.2e-7)
+    x = np.full((2, 3, 4096), 2.0, np.float32)
+    w = np.full(4096, 3.0, np.float32)
+    assert np.all(host(ops.rms_norm(dev(x), dev(w), 0.0)) == 3.0)
+
+
+def test_rms_norm_f64_and_halves():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((33, 1024))
+    w = rng.uniform(0.5, 1.5, 1024)
+    y = host(ops.rms_norm(dev(x), dev(w), 1e-5))
+    assert_rel(y, oracle.rms_norm(x, w, 1e-5), 1e-12)
+    for dt in (torch.float16, torch.bfloat16):
+        xt = dev(x.astype(np.float32)).to(dt)
+        wt = dev(w.astype(np.float32)).to(dt)
+        y = ops.rms_norm(xt, wt, 1e-5).float()
+        ref = oracle.rms_norm(host(xt.float()), host(wt.float()), 1e-5)
+        tol = ABS_F16 if dt == torch.float16 else 4e-2
+        assert np.max(np.abs(host(y) - ref)) <= tol * max(1.0, np.abs(ref).max() / 2)
+
+
+def test_rms_norm_full_config_in_place():
+    # BASELINE config [32,128,4096] fp32, checked on a row sample against the oracle and fully
+    # through the invariant sum_j (y_j/w_j)^2 = D*ms/(ms+eps)
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((32, 128, 4096), dtype=np.float32)
+    w = np.random.default_rng(2).uniform(0.5, 1.5, 4096).astype(np.float32)
+    xd = dev(x)
+    y = host(ops.rms_norm(xd, dev(w), 1e-5, out=xd))  # y aliases x
+    rows = np.random.default_rng(0).choice(32 * 128, 256, replace=False)
+    assert_rel(y.reshape(-1, 4096)[rows], oracle.rms_norm(x.reshape(-1, 4096)[rows], w, 1e-5), REL_F32)
+    ms = (x.astype(np.float64) ** 2).mean(-1)
+    lhs = ((y.astype(np.float64) / w) ** 2).sum(-1)
+    assert np.allclose(lhs, 4096 * ms / (ms + 1e-5), rtol=1e-5)
+
+
+# ------------------------------------------------------------------ Softmax
+
+@pytest.mark.parametrize("shape,axis", [((2, 3, 2, 4), 1), ((4, 5, 2048), 2), ((3, 1000), 1), ((6, 7, 33), 2),
+                                        ((2, 64, 5), 1), ((8, 4096), 1), ((2, 3, 9000), 2), ((5, 6), 0)])
+def test_softmax_f32(shape, axis):
+    rng = np.random.default_rng(3)
+    x = (3 * rng.standard_normal(shape)).astype(np.float32)
+    y = host(ops.softmax(dev(x), axis))
+    assert_rel(y, oracle.softmax(x, axis, threads=8), REL_F32)
+
+
+def test_softmax_reference_kat_and_f64():
+    x = np.zeros((2, 3, 2, 4), np.float64)
+    assert np.all(host(ops.softmax(dev(x), 1)) == 1.0 / 3)
+    x = 3 * np.random.default_rng(3).standard_normal((17, 513))
+    assert_rel(host(ops.softmax(dev(x), 1)), oracle.softmax(x, 1), 1e-13)
+
+
+@pytest.mark.parametrize("dt,tol", [(torch.float16, ABS_F16), (torch.bfloat16, 8e-3)])
+def test_softmax_16bit_plain_and_causal(dt, tol):
+    rng = np.random.default_rng(3)
+    for shape in [(2, 3, 256, 256), (1, 2, 64, 2048), (3, 130, 136), (2, 2048, 2048)]:
+        x16 = dev((3 * rng.standard_normal(shape)).astype(np.float32)).to(dt)
+        x32 = host(x16.float())
+        y = host(ops.softmax(x16).float())
+        assert np.max(np.abs(y - oracle.softmax(x32, threads=8))) <= tol
+        # causal flag == data-masked input, bit for bit, and both match the oracle
+        yc = ops.softmax(x16, causal=True)
+        R, Cc = shape[-2], shape[-1]
+        mask = torch.arange(Cc, device=DEV)[None, :] > torch.arange(R, device=DEV)[:, None] + (Cc - R)
+        ym = ops.softmax(x16.masked_fill(mask, float("-inf")))
+        assert torch.equal(yc, ym)
+        assert np.max(np.abs(host(yc.float()) - oracle.softmax_causal(x32, threads=8))) <= tol
+        assert torch.all(yc[..., mask] == 0)
+
+
+def test_softmax_full_config_properties():
+    # [8,32,2048,2048] fp16: a slab against the oracle, the whole tensor through row sums
+    g = torch.Generator(device=DEV).manual_seed(3)
+    x = (3 * torch.randn((8, 32, 2048, 2048), generator=g, device=DEV, dtype=torch.float32)).half()
+    y = ops.softmax(x)
+    yc = ops.softmax(x, causal=True)
+    sums = y.float().sum(-1)
+    assert float((sums - 1).abs().max()) < 2e-2  # 2048 roundings of fp16 outputs
+    assert float((yc.float().sum(-1) - 1).abs().max()) < 2e-2
+    assert torch.all(yc[0, 0].triu(1) == 0) and torch.all(yc[7, 31].triu(1) == 0)
+    slab = host(x[5, 17, 1000:1064].float())
+    assert np.max(np.abs(host(y[5, 17, 1000:1064].float()) - oracle.softmax(slab))) <= ABS_F16
+    ref_c = oracle.softmax_causal(host(x[2, 9].float()), threads=8)
+    assert np.max(np.abs(host(yc[2, 9].float()) - ref_c)) <= ABS_F16
+
+
+# ------------------------------------------------------------------ RotaryEmbedding
+
+@pytest.mark.parametrize("B,S,H,D", [(2, 50, 3, 16), (1, 33, 32, 128), (3, 17, 8, 64), (2, 9, 40, 256),
+                                     (2, 7, 5, 6), (1, 2048, 4, 128)])
+def test_rope_f16(B, S, H, D):
+    rng = np.random.default_rng(4)
+    x16 = dev(rng.standard_normal((B, S, H, D)).astype(np.float32)).half()
+    pos = np.tile(np.arange(S, dtype=np.int64), (B, 1))
+    ref = oracle.rope(host(x16.float()), pos, 10000.0, threads=8)
+    y = host(ops.rope(x16, dev(pos), 10000.0).float())
+    assert np.max(np.abs(y - ref)) <= ABS_F16
+    # [seq] positions broadcast; in place
+    y2 = ops.rope(x16.clone(), dev(pos[0]), 10000.0)
+    assert np.array_equal(host(y2.float()), y)
+    xin = x16.clone()
+    ops.rope(xin, dev(pos), 10000.0, out=xin)
+    assert np.array_equal(host(xin.float()), y)
+
+
+def test_rope_f32_random_positions_and_bf16():
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((2, 40, 6, 128)).astype(np.float32)
+    pos = rng.integers(0, 4096, (2, 40)).astype(np.int64)
+    ref = oracle.rope(x, pos, 10000.0)
+    y = host(ops.rope(dev(x), dev(pos), 10000.0))
+    assert np.max(np.abs(y - ref)) <= 2e-5
+    xb = dev(x).bfloat16()
+    yb = host(ops.rope(xb, dev(pos), 500000.0).float())
+    assert np.max(np.abs(yb - oracle.rope(host(xb.float()), pos, 500000.0))) <= 2e-2
+
+
+def test_rope_full_config_properties():
+    # [16,2048,32,128] fp16: pos 0 rows are the identity, pair norms are preserved, a token slab
+    # matches the oracle
+    g = torch.Generator(device=DEV).manual_seed(4)
+    x = torch.randn((16, 2048, 32, 128), generator=g, device=DEV, dtype=torch.float32).half()
+    pos = torch.arange(2048, device=DEV, dtype=torch.int64).repeat(16, 1)
+    y = ops.rope(x, pos)
+    assert torch.equal(y[:, 0], x[:, 0])
+    n_in = x[3].float()[..., :64] ** 2 + x[3].float()[..., 64:] ** 2
+    n_out = y[3].float()[..., :64] ** 2 + y[3].float()[..., 64:] ** 2
+    assert float((n_in - n_out).abs().max()) < 4e-2
+    sl = slice(1990, 2048)
+    ref = oracle.rope(host(x[11:12, sl].float()), host(pos[11:12, sl]), 10000.0, threads=8)
+    assert np.max(np.abs(host(y[11:12, sl].float()) - ref)) <= ABS_F16
+
+
+# ------------------------------------------------------------------ DequantizeLinear (bit-exact)
+
+def test_dequantize_reference_kat():
+    y = ops.dequantize_linear(dev(np.array([0, 3, 128, 255], np.uint8)), dev(np.array([2.0], np.float32)),
+                              dev(np.array([128], np.uint8)))
+    assert host(y).tolist() == [-256, -250, 0, 254]
+
+
+@pytest.mark.parametrize("dt", [np.uint8, np.int8, np.int16, np.int32])
+@pytest.mark.parametrize("shape,axis", [((4096,), 0), ((3, 5, 4), 1), ((16, 64), 1), ((7, 33), 1), ((8, 12, 6), 0),
+                                        ((256, 1024), 1)])
+def test_dequantize_bit_exact(dt, shape, axis):
+    rng = np.random.default_rng(7)
+    info = np.iinfo(dt)
+    lo, hi = max(info.min, -(1 << 20)), min(info.max, 1 << 20)
+    x = rng.integers(lo, hi + 1, shape, dtype=dt)
+    # scalar (reference path), with and without zero point
+    s1 = np.array([0.0123], np.float32)
+    z1 = rng.integers(lo, hi + 1, (1,), dtype=dt)
+    assert np.array_equal(host(ops.dequantize_linear(dev(x), dev(s1), dev(z1))), oracle.dequantize_linear(x, s1, z1))
+    assert np.array_equal(host(ops.dequantize_linear(dev(x), dev(s1))), oracle.dequantize_linear(x, s1))
+    # per-axis
+    n = shape[axis]
+    s = np.random.default_rng(8).uniform(1e-3, 1e-2, n).astype(np.float32)
+    z = rng.integers(lo, hi + 1, (n,), dtype=dt)
+    assert np.array_equal(host(ops.dequantize_linear(dev(x), dev(s), dev(z), axis=axis)),
+                          oracle.dequantize_linear(x, s, z, axis=axis))
+    assert np.array_equal(host(ops.dequantize_linear(dev(x), dev(s), axis=axis)),
+                          oracle.dequantize_linear(x, s, None, axis=axis))
+
+
+def test_dequantize_full_config_bit_exact():
+    x = np.random.default_rng(7).integers(-128, 128, (4096, 4096), dtype=np.int8)
+    s = np.random.default_rng(8).uniform(1e-3, 1e-2, 4096).astype(np.float32)
+    y = host(ops.dequantize_linear(dev(x), dev(s), axis=1))
+    assert np.array_equal(y, oracle.dequantize_linear(x, s, None, axis=1, threads=8))
+
+
+# ------------------------------------------------------------------ MatMulInteger (bit-exact)
+
+def test_matmul_integer_reference_kats():
+    a = np.array([[1, 2, 3], [4, 5, 6]], np.uint8)
+    b = np.array([[1], [2], [3]], np.uint8)
+    assert host(ops.matmul_integer(dev(a), dev(b))).reshape(-1).tolist() == [14, 32]
+    a = np.arange(1, 5, dtype=np.uint8).reshape(1, 4)
+    b = np.tile(np.arange(1, 13, dtype=np.uint8), (4, 1))
+    assert host(ops.matmul_integer(dev(a), dev(b))).reshape(-1).tolist() == [10 * i for i in range(1, 13)]
+    a = np.array([0, 128, 255, 1, 127, 200], np.uint8).reshape(2, 3)
+    b = np.array([-128, 127, 1, -1, 5, 7], np.int8).reshape(3, 2)
+    y = ops.matmul_integer(dev(a), dev(b), dev(np.array([128], np.uint8)), dev(np.array([0], np.int8)))
+    assert host(y).reshape(-1).tolist() == [17019, -15367, 16615, -15624]
+    assert host(ops.matmul_integer(dev(a), dev(b))).reshape(-1).tolist() == [-133, 121, -281, -392]
+
+
+@pytest.mark.parametrize("m,k,n", [(37, 53, 29), (256, 64, 256), (256, 192, 512), (512, 1024, 256), (300, 64, 256),
+                                   (1, 4096, 1), (768, 128, 768)])
+def test_matmul_integer_bit_exact_config_zero_points(m, k, n):
+    a = np.random.default_rng(5).integers(0, 256, (m, k), dtype=np.uint8)
+    b = np.random.default_rng(6).integers(-128, 128, (k, n), dtype=np.int8)
+    az, bz = np.array([128], np.uint8), np.array([0], np.int8)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz)))
+    assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
+
+
+@pytest.mark.parametrize("m,k,n", [(20, 33, 17), (256, 128, 256)])
+def test_matmul_integer_zero_point_variants_and_broadcast(m, k, n):
+    rng = np.random.default_rng(6)
+    a = rng.integers(0, 256, (2, 1, m, k), dtype=np.uint8)
+    b = rng.integers(0, 256, (1, 3, k, n), dtype=np.uint8)
+    variants = [
+        (None, None),
+        (rng.integers(0, 256, (1,), dtype=np.uint8), rng.integers(-128, 128, (1,), dtype=np.int8)),
+        (rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (3 * k,), dtype=np.int8)),
+        (rng.integers(-128, 128, (2 * m,), dtype=np.int8), None),
+    ]
+    for az, bz in variants:
+        y = host(ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz)))
+        assert y.shape == (2, 3, m, n)
+        assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
+    # equal batch shapes: the strided (grid.z) path
+    a2 = rng.integers(0, 256, (3, m, k), dtype=np.uint8)
+    b2 = rng.integers(-128, 128, (3, k, n), dtype=np.int8)
+    az = rng.integers(0, 256, (3 * m,), dtype=np.uint8)
+    y = host(ops.matmul_integer(dev(a2), dev(b2), dev(az), None))
+    assert np.array_equal(y, oracle.matmul_integer(a2, b2, az, None, threads=8))
+
+
+def test_matmul_integer_extremes():
+    a = np.zeros((256, 4096), np.uint8)
+    b = np.full((4096, 256), -128, np.int8)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(np.array([128], np.uint8)), None))
+    assert np.all(y == 2 ** 26)
+
+
+def test_matmul_integer_full_config():
+    # 4096^3: exact float64 BLAS product as the full-size check (all partial sums < 2^53), a
+    # sample of rows against the oracle itself
+    a = np.random.default_rng(5).integers(0, 256, (4096, 4096), dtype=np.uint8)
+    b = np.random.default_rng(6).integers(-128, 128, (4096, 4096), dtype=np.int8)
+    az, bz = np.array([128], np.uint8), np.array([0], np.int8)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz)))
+    ref = (a.astype(np.float64) - 128.0) @ b.astype(np.float64)
+    assert np.array_equal(y.astype(np.float64), ref)
+    rows = [0, 1, 255, 256, 2047, 4095]
+    assert np.array_equal(y[rows], oracle.matmul_integer(a[rows], b, az, bz, threads=8))
+
+
+# ------------------------------------------------------------------ AttentionKVCache
+
+def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_row=True, pairs=None):
+    rng = np.random.default_rng(seed)
+    mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).to(dt)
+    q, k, v = mk((N, H, seq, D)), mk((N, Hkv, seq, D)), mk((N, Hkv, seq, D))
+    kc, vc = mk((N, Hkv, cap, D)), mk((N, Hkv, cap, D))
+    past = np.asarray(past, dtype=np.int64).reshape(-1)
+    kc0, vc0 = kc.clone(), vc.clone()
+    o = ops.attention_kvcache(q, k, v, kc, vc, dev(past), 1 / math.sqrt(D))
+    f = lambda t: host(t.float())
+    ref_o, ref_kc, ref_vc = oracle.attention_kvcache(f(q), f(k), f(v), f(kc0), f(vc0), past, 1 / math.sqrt(D),
+                                                     heads=pairs)
+    return f(o), ref_o, f(kc), ref_kc, f(vc), ref_vc
+
+
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,past", [
+    (2, 4, 2, 1, 64, 64, [5, 40]),
+    (3, 8, 2, 1, 300, 128, [0, 17, 299]),
+    (4, 32, 8, 1, 1024, 128, [1, 100, 640, 1023]),
+    (2, 6, 2, 1, 128, 128, [64, 3]),        # group of 3 heads: 2 + 1 launches
+    (2, 4, 4, 1, 128, 64, [100, 9]),        # MHA
+    (2, 8, 2, 5, 64, 128, [0, 20]),         # several new rows with history
+    (1, 4, 1, 16, 16, 64, [0]),             # prefill into an exactly fitting cache
+])
+def test_attention_decode_and_small_prefill(N, H, Hkv, seq, cap, D, past):
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past)
+    assert np.max(np.abs(o - ref_o)) <= ABS_F16
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)  # appended rows, rest untouched
+
+
+def test_attention_scalar_past_no_cache_and_bf16():
+    o, ref_o, kc, ref_kc, _, _ = _attention_case(2, 8, 2, 1, 200, 128, [77])
+    assert np.max(np.abs(o - ref_o)) <= ABS_F16 and np.array_equal(kc, ref_kc)
+    o, ref_o, kc, ref_kc, _, _ = _attention_case(2, 8, 4, 1, 256, 128, [200, 13], dt=torch.bfloat16)
+    assert np.max(np.abs(o - ref_o)) <= 2e-2 and np.array_equal(kc, ref_kc)
+    # no cache: plain causal self-attention over the new rows
+    rng = np.random.default_rng(10)
+    mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).half()
+    q, k, v = mk((2, 4, 9, 64)), mk((2, 2, 9, 64)), mk((2, 2, 9, 64))
+    o = host(ops.attention_kvcache(q, k, v, scale=0.125).float())
+    f = lambda t: host(t.float())
+    ref, _, _ = oracle.attention_kvcache(f(q), f(k), f(v), np.zeros((2, 2, 9, 64), np.float32),
+                                         np.zeros((2, 2, 9, 64), np.float32), [0, 0], 0.125)
+    assert np.max(np.abs(o - ref)) <= ABS_F16
+
+
+def test_attention_decode_full_config():
+    # N=32, 32 q heads / 8 kv heads, D=128, cap 4096, past ~ U{1024..4095}
+    past = np.random.default_rng(14).integers(1024, 4096, 32)
+    pairs = [(b, h) for b in (0, 7, 19, 31) for h in (0, 5, 14, 31)]
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(32, 32, 8, 1, 4096, 128, past, pairs=pairs)
+    for b, h in pairs:
+        assert np.max(np.abs(o[b, h] - ref_o[b, h])) <= ABS_F16
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+    assert np.isfinite(o).all()
+
+
+def test_attention_decode_invariants_full_size():
+    # uniform K => O = mean(V); permuting history positions leaves O unchanged (to rounding)
+    N, H, Hkv, cap, D = 4, 32, 8, 4096, 128
+    g = torch.Generator(device=DEV).manual_seed(12)
+    rnd = lambda shape: torch.randn(shape, generator=g, device=DEV).half()
+    q, k, v = rnd((N, H, 1, D)), rnd((N, Hkv, 1, D)), rnd((N, Hkv, 1, D))
+    vc = rnd((N, Hkv, cap, D))
+    past = torch.tensor([4095, 2048, 1024, 3000], device=DEV)
+    kc = k.expand(N, Hkv, cap, D).contiguous()
+    o = ops.attention_kvcache(q, k, v, kc, vc.clone(), past)
+    for b in range(N):
+        L = int(past[b]) + 1
+        vv = torch.cat([vc[b, :, :L - 1], v[b]], dim=1).float().mean(1)          # [Hkv, D]
+        assert float((o[b, :, 0].float() - vv.repeat_interleave(4, 0)).abs().max()) <= ABS_F16
+    kc = rnd((N, Hkv, cap, D))
+    o1 = ops.attention_kvcache(q, k, v, kc.clone(), vc.clone(), past)
+    perm = torch.randperm(1024, generator=torch.Generator().manual_seed(1)).to(DEV)
+    kc2, vc2 = kc.clone(), vc.clone()
+    kc2[:, :, :1024] = kc[:, :, perm]
+    vc2[:, :, :1024] = vc[:, :, perm]
+    o2 = ops.attention_kvcache(q, k, v, kc2, vc2, past)
+    assert float((o1.float() - o2.float()).abs().max()) <= ABS_F16
+
+
+def test_attention_prefill_config_sample():
+    # seq 512, past 0, causal, 32/8 heads, D=128 (batch cut to 2 so the oracle finishes in seconds)
+    pairs = [(0, 0), (0, 13), (1, 31)]
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(2, 32, 8, 512, 4096, 128, [0, 0], pairs=pairs)
+    for b, h in pairs:
+        assert np.max(np.abs(o[b, h] - ref_o[b, h])) <= ABS_F16
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
