@@ -42,23 +42,41 @@ def parse():
 
 
 def time_steps(torch, fn, steps, warmup, n_sets):
-    """Runs fn(i % n_sets) warmup+steps times; returns (wall ms per step over the timed region,
-    mean device ms per call from HIP events on the launch stream, min device ms)."""
+    """Times `steps` calls fn(i % n_sets) after `warmup` untimed ones.
+
+    The timed calls are captured once into a HIP graph (plain kernel launches on the capture
+    stream) and replayed, so the device sees them back to back and host launch overhead does not
+    enter; the replay is bracketed by device synchronisation for the wall clock and by HIP events
+    on the replay stream for the device time.  Returns (wall ms per step, device ms per step,
+    "graph" | "eager")."""
     for i in range(warmup):
         fn(i % n_sets)
     torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    mode = "graph"
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(steps):
+                fn(i % n_sets)
+        run = graph.replay
+        run()                      # one untimed replay (graph upload)
+    except Exception as exc:       # capture unavailable: time eager launches instead
+        sys.stderr.write(f"bench.py: graph capture failed ({exc}); timing eager launches\n")
+        mode = "eager"
+
+        def run():
+            for i in range(steps):
+                fn(i % n_sets)
     torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for i in range(steps):
-        starts[i].record()
-        fn(i % n_sets)
-        stops[i].record()
+    start.record()
+    run()
+    stop.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    dev = [a.elapsed_time(b) for a, b in zip(starts, stops)]
-    return wall_ms, float(np.mean(dev)), float(np.min(dev))
+    dev_ms = start.elapsed_time(stop) / steps
+    return wall_ms, dev_ms, mode
 
 
 def hbm_entry(bytes_per_call, dev_ms):
@@ -108,18 +126,20 @@ def main():
             vc=randn16((N, Hkv, cap, D), 13 + 100 * s), o=torch.empty((N, H, 1, D), device=dev, dtype=torch.float16)))
     past = torch.from_numpy(past_np).to(dev)
     ws = ops.attention_workspace(N, H, Hkv, 1, cap, D, dev)
+    state = ops.attention_state(dev)   # persistent ticket counters: the call is a single launch
 
     def decode(i):
         t = sets[i]
-        ops.attention_kvcache(t["q"], t["k"], t["v"], t["kc"], t["vc"], past, scale, out=t["o"], workspace=ws)
+        ops.attention_kvcache(t["q"], t["k"], t["v"], t["kc"], t["vc"], past, scale, out=t["o"], workspace=ws,
+                              sync_state=state)
 
-    wall_ms, dev_ms, dev_min = time_steps(torch, decode, args.steps, args.warmup, n_sets)
+    wall_ms, dev_ms, mode = time_steps(torch, decode, args.steps, args.warmup, n_sets)
     value = decode_bytes / (wall_ms * 1e-3) / 1e9
     roofline = hbm_entry(decode_bytes, dev_ms)
-    roofline["kernel"] = "attn_split+attn_merge (one rg_hip_attention_kvcache call)"
+    roofline["kernel"] = "attn_split (one rg_hip_attention_kvcache call = one launch)"
     roofline["algorithmic_bytes"] = decode_bytes
-    roofline["device_ms_mean"] = round(dev_ms, 5)
-    roofline["device_ms_min"] = round(dev_min, 5)
+    roofline["device_ms_per_launch"] = round(dev_ms, 5)
+    roofline["timing"] = mode
 
     result = {
         "metric": "AttentionKVCache decode GB/s (% HBM peak); MatMulInteger int8 TOPS (% MFMA)",
@@ -161,9 +181,9 @@ def main():
         xs = [torch.randn((32, 128, 4096), device=dev) for _ in range(nb)]
         ys = [torch.empty_like(xs[0]) for _ in range(nb)]
         w = torch.rand(4096, device=dev) + 0.5
-        wall, dms, dmin = time_steps(torch, lambda i: ops.rms_norm(xs[i], w, 1e-5, out=ys[i]), steps, warmup, nb)
+        wall, dms, mode = time_steps(torch, lambda i: ops.rms_norm(xs[i], w, 1e-5, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(134234112, dms)
-        e.update(workload="RmsNormalization f32 [32,128,4096]", device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5))
+        e.update(workload="RmsNormalization f32 [32,128,4096]", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["rms_norm"] = e
         del xs, ys
 
@@ -171,10 +191,9 @@ def main():
         x = (3 * torch.randn((8, 32, 2048, 2048), device=dev)).half()
         y = torch.empty_like(x)
         for causal, nbytes, name in ((False, 4294967296, "softmax"), (True, 3221749760, "softmax_causal")):
-            wall, dms, dmin = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 2, 5), 3, 1)
+            wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 2, 5), 3, 1)
             e = hbm_entry(nbytes, dms)
-            e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_mean=round(dms, 5),
-                     device_ms_min=round(dmin, 5))
+            e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_per_launch=round(dms, 5), timing=mode)
             ops_out[name] = e
         del x, y
 
@@ -183,9 +202,9 @@ def main():
         xs = [torch.randn((16, 2048, 32, 128), device=dev).half() for _ in range(nb)]
         ys = [torch.empty_like(xs[0]) for _ in range(nb)]
         pos = torch.arange(2048, device=dev, dtype=torch.int64).repeat(16, 1).contiguous()
-        wall, dms, dmin = time_steps(torch, lambda i: ops.rope(xs[i], pos, 10000.0, out=ys[i]), steps, warmup, nb)
+        wall, dms, mode = time_steps(torch, lambda i: ops.rope(xs[i], pos, 10000.0, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(537133056, dms)
-        e.update(workload="RotaryEmbedding fp16 [16,2048,32,128]", device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5))
+        e.update(workload="RotaryEmbedding fp16 [16,2048,32,128]", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["rope"] = e
         del xs, ys
 
@@ -194,10 +213,9 @@ def main():
         xs = [torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8) for _ in range(nb)]
         ys = [torch.empty((4096, 4096), device=dev) for _ in range(nb)]
         sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
-        wall, dms, dmin = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
+        wall, dms, mode = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(83902464, dms)
-        e.update(workload="DequantizeLinear i8->f32 [4096,4096] per-axis scale", device_ms_mean=round(dms, 5),
-                 device_ms_min=round(dmin, 5))
+        e.update(workload="DequantizeLinear i8->f32 [4096,4096] per-axis scale", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["dequantize_linear"] = e
         del xs, ys
 
@@ -207,13 +225,13 @@ def main():
         az = torch.tensor([128], device=dev, dtype=torch.uint8)
         bz = torch.tensor([0], device=dev, dtype=torch.int8)
         y = torch.empty((4096, 4096), device=dev, dtype=torch.int32)
-        wall, dms, dmin = time_steps(torch, lambda i: ops.matmul_integer(a, b, az, bz, out=y), steps, warmup, 1)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul_integer(a, b, az, bz, out=y), steps, warmup, 1)
         tops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
         ops_out["matmul_integer"] = {
             "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
             "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
             "workload": "MatMulInteger u8 x i8 -> i32 4096^3, a_zp=128 b_zp=0",
-            "device_ms_mean": round(dms, 5), "device_ms_min": round(dmin, 5)}
+            "device_ms_per_launch": round(dms, 5), "timing": mode}
         if not args.no_cpu:
             import oracle
             m = 64
@@ -236,13 +254,14 @@ def main():
         o = torch.empty_like(q)
         zero = torch.zeros(Np, device=dev, dtype=torch.int64)
         wsp = ops.attention_workspace(Np, H, Hkv, seq, cap, D, dev)
-        wall, dms, dmin = time_steps(
-            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp),
+        wall, dms, mode = time_steps(
+            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp,
+                                                   sync_state=state),
             max(steps // 5, 3), 2, 1)
         e = hbm_entry(402653184, dms)
         flops = 68853694464
         e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=128",
-                 device_ms_mean=round(dms, 5), device_ms_min=round(dmin, 5),
+                 device_ms_per_launch=round(dms, 5), timing=mode,
                  mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
                  mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
         ops_out["attention_prefill"] = e

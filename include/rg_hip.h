@@ -133,16 +133,24 @@ int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b,
  *   (rows that do not fit are dropped), never written out of bounds.
  * k_cache == v_cache == NULL: no cache (past = 0, attends k/v directly).  past_lens == NULL: 0.
  * n_head % n_kv_head == 0; D in {64, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
- * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials for decode). */
+ * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials), contents irrelevant.
+ * sync_state: NULL, or rg_hip_attention_kvcache_state_bytes() bytes of device memory that the
+ *   caller zeroed once and keeps for this purpose (a runtime::Resource of the stream, like the
+ *   reference's library handles, src/04kernel/src/utilities/cuda/cublas_context.cu:18-31); the
+ *   kernel uses it for ticket counters and leaves it zero.  With it the whole call is one
+ *   kernel launch; without it a small clearing launch precedes the kernel.  Calls that share
+ *   one sync_state must not overlap (a Stream runs its routines in order on one queue). */
 size_t rg_hip_attention_kvcache_workspace(size_t N, size_t n_head, size_t n_kv_head,
                                           size_t seq, size_t cap, size_t D);
+size_t rg_hip_attention_kvcache_state_bytes(void);
 int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *v,
                              void *k_cache, void *v_cache,
                              const int64_t *past_lens, int past_per_row,
                              size_t N, size_t n_head, size_t n_kv_head,
                              size_t seq, size_t cap, size_t D,
                              float scale, int dtype,
-                             void *workspace, size_t workspace_bytes, void *stream);
+                             void *workspace, size_t workspace_bytes, void *sync_state,
+                             void *stream);
 
 #ifdef __cplusplus
 }

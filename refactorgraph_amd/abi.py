@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG, "lib", "librg_hip.so")
+# RG_HIP_LIBRARY overrides the in-tree library (e.g. to compare builds)
+LIB_PATH = os.environ.get("RG_HIP_LIBRARY") or os.path.join(PKG, "lib", "librg_hip.so")
 HOST_LIB_PATH = os.path.join(PKG, "lib", "librg_host.so")
 HOST_TESTS_PATH = os.path.join(PKG, "lib", "rg_host_tests")
 
@@ -36,8 +37,9 @@ SIGNATURES = {
     "rg_hip_matmul_integer_workspace": (_sz, [_sz, _sz, _sz, _sz, _u]),
     "rg_hip_matmul_integer": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
     "rg_hip_attention_kvcache_workspace": (_sz, [_sz, _sz, _sz, _sz, _sz, _sz]),
+    "rg_hip_attention_kvcache_state_bytes": (_sz, []),
     "rg_hip_attention_kvcache": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _sz,
-                                      _f, _i, _vp, _sz, _vp]),
+                                      _f, _i, _vp, _sz, _vp, _vp]),
 }
 
 

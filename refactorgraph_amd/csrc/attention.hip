@@ -15,8 +15,9 @@
 // load is 1 KiB contiguous.  QK^T uses packed-half dot products followed by a DPP reduction
 // over the 16 lanes of a key row, which leaves every lane holding the scores it needs for the
 // PV update of its own slice of the head dimension; softmax is the online (running max / sum)
-// form in float.  Segments that end up in more than one range leave (max, sum, unnormalised O)
-// partials that a second small kernel merges.
+// form in float.  A segment that ends up in more than one range leaves (max, sum, unnormalised
+// O) partials; the workgroup that finishes such a segment last (a ticket counter per segment)
+// merges them, so one launch does everything.
 #include "common.hpp"
 
 namespace rg {
@@ -24,6 +25,7 @@ namespace {
 
 constexpr int kMaxBatch = 1024;     // rows of the batch whose lengths a workgroup scans
 constexpr float kMinusBig = -1e30f; // running-max sentinel (finite: keeps exp2 arguments defined)
+constexpr float kSlack = 6.0f;      // log2 headroom of the softmax reference before it is raised
 
 struct AttnParams {
     const void *q, *k, *v;
@@ -36,6 +38,7 @@ struct AttnParams {
     int append;          // write the new k/v rows into the caches
     float scale_log2e;   // scale * log2(e)
     float *part;         // partial slots: 2 per workgroup, each G*(D+2) floats
+    uint32_t *counters;  // one ticket counter per workgroup, zero between launches
     uint32_t n_workgroups;
 };
 
@@ -54,7 +57,7 @@ __device__ __forceinline__ uint64_t keys_before_row(uint32_t Hkv, uint32_t base,
 }
 
 // Fills `part` (shared memory) and returns the total key count.  Called by every thread.
-__device__ uint64_t build_partition(const AttnParams &p, Partition part, uint64_t *scan_tmp) {
+__device__ uint64_t build_partition(const AttnParams &p, Partition part) {
     const uint32_t t = threadIdx.x;
     // clamp so that the seq new rows always fit the cache; no cache: no history
     for (uint32_t b = t; b < p.N; b += blockDim.x) {
@@ -66,16 +69,28 @@ __device__ uint64_t build_partition(const AttnParams &p, Partition part, uint64_
         part.base[b] = static_cast<uint32_t>(raw);
     }
     __syncthreads();
-    // exclusive scan of per-batch-row key counts; N <= kMaxBatch, blockDim.x-strided chunks
-    if (t == 0) {
-        uint64_t run = 0;
-        for (uint32_t b = 0; b < p.N; ++b) {
-            part.prefix[b] = run;
-            run += keys_before_row(p.Hkv, part.base[b], p.seq);
+    // exclusive scan of per-batch-row key counts by the first wavefront: each lane sums a
+    // contiguous run of rows, the lane totals are scanned with shuffles
+    if (t < kWave) {
+        const uint32_t per_lane = (p.N + kWave - 1) / kWave;
+        const uint32_t b0 = t * per_lane;
+        uint64_t mine = 0;
+        for (uint32_t i = 0; i < per_lane; ++i)
+            if (b0 + i < p.N) mine += keys_before_row(p.Hkv, part.base[b0 + i], p.seq);
+        uint64_t incl = mine;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const uint64_t up = __shfl_up(incl, d, kWave);
+            if (t >= static_cast<uint32_t>(d)) incl += up;
         }
-        part.prefix[p.N] = run;
+        uint64_t run = incl - mine;
+        for (uint32_t i = 0; i < per_lane; ++i)
+            if (b0 + i < p.N) {
+                part.prefix[b0 + i] = run;
+                run += keys_before_row(p.Hkv, part.base[b0 + i], p.seq);
+            }
+        if (t == kWave - 1) part.prefix[p.N] = incl;
     }
-    (void) scan_tmp;
     __syncthreads();
     return part.prefix[p.N];
 }
@@ -165,24 +180,92 @@ __device__ __forceinline__ float row_sum(float v) {
     return v;
 }
 
+// Device-scope (all XCDs) visible accesses for the split-KV partials: the store is written
+// through, the load does not hit a stale line of another XCD's L2.
+__device__ __forceinline__ void store_coherent(float *p, float v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float *p) {
+    return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT));
+}
+
 // ---------------------------------------------------------------- split kernel
 
+// Merge of the partials of one cut segment (pieces held by workgroups first..last), one
+// (head, d) output per thread iteration.  Loads of a batch of partials are independent.
 template <class T, int D, int G>
-__global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
+__device__ void merge_segment(const AttnParams &p, const Segment &sg, uint64_t W, uint64_t first,
+                              uint64_t last) {
+    T *O = static_cast<T *>(p.o);
+    constexpr int B = 8;
+    for (uint32_t idx = threadIdx.x; idx < G * D; idx += 256) {
+        const uint32_t g = idx / D, d = idx % D;
+        float M = kMinusBig, o_sum = 0.f, l_sum = 0.f;
+        for (uint64_t w0 = first; w0 <= last; w0 += B) {
+            float pm[B], po[B], pl[B];
+#pragma unroll
+            for (int j = 0; j < B; ++j) {
+                const uint64_t w = w0 + j;
+                pm[j] = kMinusBig;
+                po[j] = 0.f;
+                pl[j] = 0.f;
+                if (w <= last) {
+                    const uint64_t piece_start = sg.start > w * W ? sg.start : w * W;
+                    const uint64_t slot = w * 2 + (piece_start == w * W ? 0 : 1);
+                    const float *ps = p.part + slot * (G * (D + 2)) + g * (D + 2);
+                    pm[j] = load_coherent(ps + D);
+                    po[j] = load_coherent(ps + d);
+                    pl[j] = load_coherent(ps + D + 1);
+                }
+            }
+            float mn = M;
+#pragma unroll
+            for (int j = 0; j < B; ++j) mn = fmaxf(mn, pm[j]);
+            const float alpha = __builtin_amdgcn_exp2f(M - mn);
+            o_sum *= alpha;
+            l_sum *= alpha;
+            M = mn;
+#pragma unroll
+            for (int j = 0; j < B; ++j) {
+                const float wgt = __builtin_amdgcn_exp2f(pm[j] - mn);
+                o_sum = fmaf(wgt, po[j], o_sum);
+                l_sum = fmaf(wgt, pl[j], l_sum);
+            }
+        }
+        const uint32_t h = sg.kvh * p.group + p.head0 + g;
+        T *dst = O + ((static_cast<uint64_t>(sg.b) * p.H + h) * p.seq + sg.r) * D + d;
+        *reinterpret_cast<uint16_t *>(dst) = Elem<T>::pack(o_sum / l_sum);
+    }
+}
+
+#ifndef RG_ATTN_MINWAVES
+#define RG_ATTN_MINWAVES 1
+#endif
+#ifndef RG_ATTN_U
+#define RG_ATTN_U 4
+#endif
+#ifndef RG_ATTN_DB
+#define RG_ATTN_DB 1
+#endif
+template <class T, int D, int G>
+__global__ __launch_bounds__(256, RG_ATTN_MINWAVES) void attn_split(const AttnParams p) {
     constexpr int LPR = D / 8;          // lanes per key row
     constexpr int KPW = kWave / LPR;    // key rows per wavefront load
     constexpr int KPB = KPW * 4;        // key rows per workgroup step
-    constexpr int STATES = KPB;         // independent online-softmax states per workgroup
-    constexpr int U = 4;                // steps in flight
+    constexpr int U = RG_ATTN_U;        // steps per register set
+    constexpr uint32_t SPAN = KPB * U;  // keys per step group
 
     __shared__ uint64_t sh_prefix[kMaxBatch + 1];
     __shared__ uint32_t sh_base[kMaxBatch];
-    __shared__ float sh_o[STATES][G][D];
-    __shared__ float sh_m[STATES][G];
-    __shared__ float sh_l[STATES][G];
+    __shared__ float sh_o[4][G][D];
+    __shared__ float sh_m[4][G];
+    __shared__ float sh_l[4][G];
+    __shared__ uint32_t sh_last;
 
     const Partition part{sh_prefix, sh_base};
-    const uint64_t total = build_partition(p, part, nullptr);
+    const uint64_t total = build_partition(p, part);
     const uint64_t W = range_width(total, p.n_workgroups);
     const uint64_t range_begin = static_cast<uint64_t>(blockIdx.x) * W;
     if (range_begin >= total) return;
@@ -190,6 +273,7 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
 
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t row = lane / LPR, chunk = lane % LPR;  // key row within a wavefront load, 16-byte slice
+    const uint32_t key_in_span = wave * KPW + row;
     const T *Q = static_cast<const T *>(p.q);
     const T *Kn = static_cast<const T *>(p.k);
     const T *Vn = static_cast<const T *>(p.v);
@@ -204,6 +288,7 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
         const uint64_t left = range_end - f;
         const uint32_t len = static_cast<uint32_t>(left < sg.len - pos0 ? left : sg.len - pos0);
         const bool whole = pos0 == 0 && len == sg.len;
+        const uint32_t end = pos0 + len;
 
         // this lane's slice of the G query rows
         uint32_t qv[G][4];
@@ -216,77 +301,66 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
             for (int e = 0; e < 4; ++e) qv[g][e] = raw.w[e];
         }
         const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
-        const T *k_hist = Kc ? Kc + kv_head * p.cap * D : nullptr;
-        const T *v_hist = Vc ? Vc + kv_head * p.cap * D : nullptr;
-        const T *k_new = Kn + kv_head * p.seq * D;
-        const T *v_new = Vn + kv_head * p.seq * D;
-        // only the last query row's segment appends, and only on the launch that owns it
-        const bool do_append = p.append && Kc && sg.r + 1 == p.seq;
 
         float m[G], l[G], acc[G][8];
+        bool fresh = true;  // no step group consumed yet (wave-uniform)
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            m[g] = kMinusBig;
+            m[g] = 0.f;
             l[g] = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
         }
 
-        const uint32_t end = pos0 + len;
-        for (uint32_t step0 = pos0; step0 < end; step0 += KPB * U) {
-            Raw16 kk[U], vv[U];
-            bool valid[U];
+        // Online-softmax update with one step group; keys >= limit are masked out.  The running
+        // reference m[g] is only raised (and the accumulators rescaled) when some score exceeds
+        // it by more than kSlack, a wave-uniform and rare event after the first group; otherwise
+        // p = exp2(s - m) <= 2^kSlack is accumulated directly.
+        auto consume = [&](uint32_t step0, uint32_t limit, const Raw16(&kk)[U], const Raw16(&vv)[U]) {
+            float t[U][G];  // score - reference, log2 units
+            float over = -__builtin_inff();
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const uint32_t key = step0 + u * KPB + wave * KPW + row;
-                valid[u] = key < end;
-                kk[u] = Raw16{{0, 0, 0, 0}};
-                vv[u] = Raw16{{0, 0, 0, 0}};
-                if (valid[u]) {
-                    if (key >= sg.base) {  // one of the new rows
-                        const uint64_t off = static_cast<uint64_t>(key - sg.base) * D + chunk * 8;
-                        kk[u] = *reinterpret_cast<const Raw16 *>(k_new + off);
-                        vv[u] = *reinterpret_cast<const Raw16 *>(v_new + off);
-                        if (do_append) {
-                            const uint64_t coff = (kv_head * p.cap + key) * D + chunk * 8;
-                            *reinterpret_cast<Raw16 *>(Kc + coff) = kk[u];
-                            *reinterpret_cast<Raw16 *>(Vc + coff) = vv[u];
-                        }
-                    } else {
-                        const uint64_t off = static_cast<uint64_t>(key) * D + chunk * 8;
-                        kk[u] = *reinterpret_cast<const Raw16 *>(k_hist + off);
-                        vv[u] = *reinterpret_cast<const Raw16 *>(v_hist + off);
-                    }
-                }
-            }
-            float s[U][G];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
+                const bool valid = step0 + u * KPB + key_in_span < limit;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     float d = 0.f;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) d = Elem<T>::dot2(qv[g][e], kk[u].w[e], d);
-                    d = row_sum<LPR>(d) * p.scale_log2e;
-                    s[u][g] = valid[u] ? d : -__builtin_inff();
+                    d = fmaf(row_sum<LPR>(d), p.scale_log2e, -m[g]);
+                    t[u][g] = valid ? d : -__builtin_inff();
+                    over = fmaxf(over, t[u][g]);
                 }
+            }
+            if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    // how far the reference moves: to the group maximum the first time (the
+                    // reference starts at 0 with empty accumulators), never down afterwards
+                    float up = fresh ? kMinusBig : 0.f;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) up = fmaxf(up, t[u][g]);
+                    const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
+                    m[g] += up;
+                    l[g] *= alpha;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) t[u][g] -= up;
+                }
+                fresh = false;
+            }
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                float mn = m[g];
-#pragma unroll
-                for (int u = 0; u < U; ++u) mn = fmaxf(mn, s[u][g]);
-                const float alpha = __builtin_amdgcn_exp2f(m[g] - mn);
-                m[g] = mn;
-                float pr[U], ps = 0.f;
+                float pr[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    pr[u] = __builtin_amdgcn_exp2f(s[u][g] - mn);
-                    ps += pr[u];
+                    pr[u] = __builtin_amdgcn_exp2f(t[u][g]);
+                    l[g] += pr[u];
                 }
-                l[g] = l[g] * alpha + ps;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float a0 = acc[g][2 * e] * alpha, a1 = acc[g][2 * e + 1] * alpha;
+                    float a0 = acc[g][2 * e], a1 = acc[g][2 * e + 1];
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         a0 = fmaf(pr[u], Elem<T>::lo(vv[u].w[e]), a0);
@@ -296,18 +370,108 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
                     acc[g][2 * e + 1] = a1;
                 }
             }
+        };
+
+        // ---- history rows [pos0, hist_end): unconditional, clamped, streaming loads from the
+        // caches; two register sets keep the next step group in flight while one is consumed
+        const uint32_t hist_end = end < sg.base ? end : sg.base;
+        if (pos0 < hist_end) {
+            const T *k_hist = Kc + kv_head * p.cap * D + chunk * 8;
+            const T *v_hist = Vc + kv_head * p.cap * D + chunk * 8;
+            auto issue = [&](uint32_t step0, Raw16(&kk)[U], Raw16(&vv)[U]) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t key = step0 + u * KPB + key_in_span;
+                    key = key < hist_end ? key : hist_end - 1;
+                    const uint64_t off = static_cast<uint64_t>(key) * D;
+                    kk[u] = __builtin_bit_cast(
+                        Raw16, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(k_hist + off)));
+                    vv[u] = __builtin_bit_cast(
+                        Raw16, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(v_hist + off)));
+                }
+            };
+#if RG_ATTN_DB
+            Raw16 kA[U], vA[U], kB[U], vB[U];
+            issue(pos0, kA, vA);
+            for (uint32_t step0 = pos0; step0 < hist_end; step0 += 2 * SPAN) {
+                if (step0 + SPAN < hist_end) issue(step0 + SPAN, kB, vB);
+                consume(step0, hist_end, kA, vA);
+                if (step0 + SPAN < hist_end) {
+                    if (step0 + 2 * SPAN < hist_end) issue(step0 + 2 * SPAN, kA, vA);
+                    consume(step0 + SPAN, hist_end, kB, vB);
+                }
+            }
+#else
+            Raw16 kA[U], vA[U];
+            for (uint32_t step0 = pos0; step0 < hist_end; step0 += SPAN) {
+                issue(step0, kA, vA);
+                consume(step0, hist_end, kA, vA);
+            }
+#endif
         }
 
-        // merge the STATES row states of the workgroup
-        const uint32_t st = wave * KPW + row;
-        __syncthreads();  // previous piece finished reading
+        // ---- new rows [max(pos0, base), end): read from the k/v inputs; the segment of the last
+        // query row also writes them into the caches
+        if (end > sg.base) {
+            const T *k_new = Kn + kv_head * p.seq * D + chunk * 8;
+            const T *v_new = Vn + kv_head * p.seq * D + chunk * 8;
+            const bool do_append = p.append && Kc && sg.r + 1 == p.seq;
+            const uint32_t new0 = pos0 > sg.base ? pos0 : sg.base;
+            for (uint32_t step0 = new0; step0 < end; step0 += SPAN) {
+                Raw16 kk[U], vv[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t key = step0 + u * KPB + key_in_span;
+                    kk[u] = Raw16{{0, 0, 0, 0}};
+                    vv[u] = Raw16{{0, 0, 0, 0}};
+                    if (key < end) {
+                        const uint64_t off = static_cast<uint64_t>(key - sg.base) * D;
+                        kk[u] = *reinterpret_cast<const Raw16 *>(k_new + off);
+                        vv[u] = *reinterpret_cast<const Raw16 *>(v_new + off);
+                        if (do_append) {
+                            const uint64_t coff = (kv_head * p.cap + key) * D + chunk * 8;
+                            *reinterpret_cast<Raw16 *>(Kc + coff) = kk[u];
+                            *reinterpret_cast<Raw16 *>(Vc + coff) = vv[u];
+                        }
+                    }
+                }
+                consume(step0, end, kk, vv);
+            }
+        }
+
+        // ---- merge the four key rows of each wavefront with shuffles, then the four wavefronts
+        // through LDS
 #pragma unroll
         for (int g = 0; g < G; ++g) {
+            float M = fmaxf(m[g], __shfl_xor(m[g], LPR, kWave));
+            if constexpr (KPW >= 4) M = fmaxf(M, __shfl_xor(M, 2 * LPR, kWave));
+            if constexpr (KPW >= 8) M = fmaxf(M, __shfl_xor(M, 4 * LPR, kWave));
+            const float w = __builtin_amdgcn_exp2f(m[g] - M);
+            m[g] = M;
+            float lv = l[g] * w;
+            lv += __shfl_xor(lv, LPR, kWave);
+            if constexpr (KPW >= 4) lv += __shfl_xor(lv, 2 * LPR, kWave);
+            if constexpr (KPW >= 8) lv += __shfl_xor(lv, 4 * LPR, kWave);
+            l[g] = lv;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) sh_o[st][g][chunk * 8 + e] = acc[g][e];
-            if (chunk == 0) {
-                sh_m[st][g] = m[g];
-                sh_l[st][g] = l[g];
+            for (int e = 0; e < 8; ++e) {
+                float a = acc[g][e] * w;
+                a += __shfl_xor(a, LPR, kWave);
+                if constexpr (KPW >= 4) a += __shfl_xor(a, 2 * LPR, kWave);
+                if constexpr (KPW >= 8) a += __shfl_xor(a, 4 * LPR, kWave);
+                acc[g][e] = a;
+            }
+        }
+        __syncthreads();  // the previous piece has finished reading the shared state
+        if (row == 0) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sh_o[wave][g][chunk * 8 + e] = acc[g][e];
+                if (chunk == 0) {
+                    sh_m[wave][g] = m[g];
+                    sh_l[wave][g] = l[g];
+                }
             }
         }
         __syncthreads();
@@ -317,10 +481,10 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
             const uint32_t g = idx / D, d = idx % D;
             float M = kMinusBig;
 #pragma unroll
-            for (int s2 = 0; s2 < STATES; ++s2) M = fmaxf(M, sh_m[s2][g]);
+            for (int s2 = 0; s2 < 4; ++s2) M = fmaxf(M, sh_m[s2][g]);
             float o_sum = 0.f, l_sum = 0.f;
 #pragma unroll
-            for (int s2 = 0; s2 < STATES; ++s2) {
+            for (int s2 = 0; s2 < 4; ++s2) {
                 const float w = __builtin_amdgcn_exp2f(sh_m[s2][g] - M);
                 o_sum = fmaf(w, sh_o[s2][g][d], o_sum);
                 l_sum = fmaf(w, sh_l[s2][g], l_sum);
@@ -330,57 +494,38 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
                 T *dst = O + ((static_cast<uint64_t>(sg.b) * p.H + h) * p.seq + sg.r) * D + d;
                 *reinterpret_cast<uint16_t *>(dst) = Elem<T>::pack(o_sum / l_sum);
             } else {
-                pslot[g * (D + 2) + d] = o_sum;
+                store_coherent(pslot + g * (D + 2) + d, o_sum);
                 if (d == 0) {
-                    pslot[g * (D + 2) + D] = M;
-                    pslot[g * (D + 2) + D + 1] = l_sum;
+                    store_coherent(pslot + g * (D + 2) + D, M);
+                    store_coherent(pslot + g * (D + 2) + D + 1, l_sum);
                 }
             }
+        }
+        if (!whole) {
+            // The workgroup that completes a cut segment last merges its partials.  The partials
+            // are written through to device-coherent memory and read back past the per-XCD L2
+            // (device-scope atomic accesses), so only this wavefront's outstanding stores have to
+            // drain before the ticket is taken; no cache-wide write-back or invalidate is issued.
+            const uint64_t first = sg.start / W, last = (sg.start + sg.len - 1) / W;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const uint32_t ticket = __hip_atomic_fetch_add(p.counters + first, 1u, __ATOMIC_RELAXED,
+                                                               __HIP_MEMORY_SCOPE_AGENT);
+                const uint32_t is_last = ticket == static_cast<uint32_t>(last - first);
+                if (is_last) p.counters[first] = 0;  // leave the counters as they were found
+                sh_last = is_last;
+            }
+            __syncthreads();
+            if (sh_last) merge_segment<T, D, G>(p, sg, W, first, last);
         }
         f += len;
     }
 }
 
-// One workgroup per segment; merges the partials of segments that were cut.
-template <class T, int D, int G>
-__global__ __launch_bounds__(256) void attn_merge(const AttnParams p) {
-    __shared__ uint64_t sh_prefix[kMaxBatch + 1];
-    __shared__ uint32_t sh_base[kMaxBatch];
-    const Partition part{sh_prefix, sh_base};
-    const uint64_t total = build_partition(p, part, nullptr);
-    const uint64_t W = range_width(total, p.n_workgroups);
-
-    const uint32_t kvh = blockIdx.x % p.Hkv;
-    const uint32_t br = blockIdx.x / p.Hkv;
-    const uint32_t r = br % p.seq, b = br / p.seq;
-    const uint32_t base = part.base[b];
-    const uint32_t len = base + r + 1;
-    const uint64_t start = part.prefix[b] + keys_before_row(p.Hkv, base, r) + static_cast<uint64_t>(kvh) * len;
-    const uint64_t first = start / W, last = (start + len - 1) / W;
-    if (first == last) return;  // finished by the split kernel
-
-    T *O = static_cast<T *>(p.o);
-    for (uint32_t idx = threadIdx.x; idx < G * D; idx += 256) {
-        const uint32_t g = idx / D, d = idx % D;
-        float M = kMinusBig;
-        for (uint64_t w = first; w <= last; ++w) {
-            const uint64_t piece_start = start > w * W ? start : w * W;
-            const uint64_t slot = w * 2 + (piece_start == w * W ? 0 : 1);
-            M = fmaxf(M, p.part[slot * (G * (D + 2)) + g * (D + 2) + D]);
-        }
-        float o_sum = 0.f, l_sum = 0.f;
-        for (uint64_t w = first; w <= last; ++w) {
-            const uint64_t piece_start = start > w * W ? start : w * W;
-            const uint64_t slot = w * 2 + (piece_start == w * W ? 0 : 1);
-            const float *ps = p.part + slot * (G * (D + 2)) + g * (D + 2);
-            const float wgt = __builtin_amdgcn_exp2f(ps[D] - M);
-            o_sum = fmaf(wgt, ps[d], o_sum);
-            l_sum = fmaf(wgt, ps[D + 1], l_sum);
-        }
-        const uint32_t h = kvh * p.group + p.head0 + g;
-        T *dst = O + ((static_cast<uint64_t>(b) * p.H + h) * p.seq + r) * D + d;
-        *reinterpret_cast<uint16_t *>(dst) = Elem<T>::pack(o_sum / l_sum);
-    }
+// Zeroes the ticket counters when the caller supplies no persistent (already zero) ones.
+__global__ __launch_bounds__(256) void attn_clear(uint32_t *counters, uint32_t n) {
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) counters[i] = 0;
 }
 
 // ---------------------------------------------------------------- host side
@@ -422,10 +567,6 @@ int launch(AttnParams p, hipStream_t s) {
     if (wgs > kMaxWorkgroups) wgs = kMaxWorkgroups;
     p.n_workgroups = wgs;
     attn_split<T, D, G><<<wgs, 256, 0, s>>>(p);
-    int rc = launch_status();
-    if (rc) return rc;
-    const uint64_t segments = static_cast<uint64_t>(p.N) * p.seq * p.Hkv;
-    attn_merge<T, D, G><<<static_cast<unsigned>(segments), 256, 0, s>>>(p);
     return launch_status();
 }
 
@@ -453,9 +594,12 @@ int dispatch_group(AttnParams p, hipStream_t s) {
     return 0;
 }
 
+constexpr size_t kCounterBytes = kMaxWorkgroups * sizeof(uint32_t);
+
 size_t workspace_bytes(size_t D) {
-    // two partial slots per workgroup, sized for the widest head group (4)
-    return static_cast<size_t>(kMaxWorkgroups) * 2 * 4 * (D + 2) * sizeof(float);
+    // ticket counters (used when the caller passes no persistent ones), then two partial slots
+    // per workgroup sized for the widest head group (4)
+    return kCounterBytes + static_cast<size_t>(kMaxWorkgroups) * 2 * 4 * (D + 2) * sizeof(float);
 }
 
 }  // namespace
@@ -465,11 +609,14 @@ extern "C" size_t rg_hip_attention_kvcache_workspace(size_t, size_t, size_t, siz
     return rg::workspace_bytes(D);
 }
 
+extern "C" size_t rg_hip_attention_kvcache_state_bytes(void) { return rg::kCounterBytes; }
+
 extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *v,
                                         void *k_cache, void *v_cache, const int64_t *past_lens,
                                         int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
                                         size_t seq, size_t cap, size_t D, float scale, int dtype,
-                                        void *workspace, size_t workspace_bytes, void *stream) {
+                                        void *workspace, size_t workspace_bytes, void *sync_state,
+                                        void *stream) {
     using namespace rg;
     if (!o || !q || !k || !v) return RG_HIP_E_ARGUMENT;
     if ((k_cache == nullptr) != (v_cache == nullptr)) return RG_HIP_E_ARGUMENT;
@@ -496,8 +643,16 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
     p.cap = static_cast<uint32_t>(cap);
     p.group = p.H / p.Hkv;
     p.scale_log2e = scale * 1.4426950408889634f;
-    p.part = static_cast<float *>(workspace);
+    p.part = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
     hipStream_t s = as_stream(stream);
+    if (sync_state) {
+        p.counters = static_cast<uint32_t *>(sync_state);
+    } else {
+        p.counters = static_cast<uint32_t *>(workspace);
+        attn_clear<<<4, 256, 0, s>>>(p.counters, kMaxWorkgroups);
+        const int rc = launch_status();
+        if (rc) return rc;
+    }
     if (dtype == RG_FP16) {
         return D == 128 ? dispatch_group<__half, 128>(p, s) : dispatch_group<__half, 64>(p, s);
     }

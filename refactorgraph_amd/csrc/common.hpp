@@ -103,6 +103,19 @@ __device__ __forceinline__ void store16(T *p, const Vec16<T> &v) {
     *reinterpret_cast<Vec16<T> *>(p) = v;
 }
 
+// Streaming variants: data touched once, marked non-temporal so it does not displace reusable
+// lines in L2 / the memory-side cache.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <class T>
+__device__ __forceinline__ Vec16<T> load16_stream(const T *p) {
+    const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return __builtin_bit_cast(Vec16<T>, raw);
+}
+template <class T>
+__device__ __forceinline__ void store16_stream(T *p, const Vec16<T> &v) {
+    __builtin_nontemporal_store(__builtin_bit_cast(u32x4, v), reinterpret_cast<u32x4 *>(p));
+}
+
 // ---------------------------------------------------------------- storage <-> compute type
 
 template <class T> struct Compute { using type = float; };

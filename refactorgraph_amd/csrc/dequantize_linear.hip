@@ -17,6 +17,7 @@ struct alignas(4) Bytes4 {
 struct alignas(16) Float4 {
     float v[4];
 };
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <class TI> __device__ __forceinline__ int widen(uint8_t raw);
 template <> __device__ __forceinline__ int widen<uint8_t>(uint8_t raw) { return raw; }
@@ -35,7 +36,8 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint64_t g = g0 + u * 256;
-        if (g < groups) in[u] = *reinterpret_cast<const Bytes4 *>(x + g * 4);
+        if (g < groups)
+            in[u] = __builtin_bit_cast(Bytes4, __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(x + g * 4)));
     }
     float s_scalar = 0.f;
     int z_scalar = 0;
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
                 for (int e = 0; e < 4; ++e)
                     out.v[e] = static_cast<float>(widen<TI>(in[u].b[e]) - z_scalar) * s_scalar;
             }
-            *reinterpret_cast<Float4 *>(y + g * 4) = out;
+            __builtin_nontemporal_store(__builtin_bit_cast(f32x4, out), reinterpret_cast<f32x4 *>(y + g * 4));
         }
     }
 }

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void rms_norm_rows(T *__restrict__ y, const T 
     for (int i = 0; i < NV; ++i) {
         const uint32_t idx = t + i * GROUP;
         if (live && idx < nvec) {
-            xv[i] = load16(xr + static_cast<size_t>(idx) * VEC);
+            xv[i] = load16_stream(xr + static_cast<size_t>(idx) * VEC);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const CT f = to_compute(xv[i].v[e]);
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void rms_norm_rows(T *__restrict__ y, const T 
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
                 out.v[e] = from_compute<T>(to_compute(xv[i].v[e]) * scale * to_compute(wv.v[e]));
-            store16(yr + static_cast<size_t>(idx) * VEC, out);
+            store16_stream(yr + static_cast<size_t>(idx) * VEC, out);
         }
     }
 }
@@ -101,9 +101,13 @@ int dispatch(void *y_, const void *x_, const void *w_, size_t rows, size_t cols,
     constexpr size_t VEC = Vec16<T>::N;
     const bool vec_ok = cols % VEC == 0 && aligned16(y) && aligned16(x) && aligned16(w);
     const size_t nvec = cols / VEC;
-    if (vec_ok && nvec <= 64 * 2) {
+    if (vec_ok && nvec <= 64 * 16) {
+        // one wavefront per row: no workgroup barrier, up to 16 loads in flight per lane
         if (nvec <= 64) launch_rows<T, 64, 1>(y, x, w, rows, cols, eps, s);
-        else launch_rows<T, 64, 2>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 128) launch_rows<T, 64, 2>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 256) launch_rows<T, 64, 4>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 512) launch_rows<T, 64, 8>(y, x, w, rows, cols, eps, s);
+        else launch_rows<T, 64, 16>(y, x, w, rows, cols, eps, s);
     } else if (vec_ok && nvec <= 256 * 8) {
         if (nvec <= 256) launch_rows<T, 256, 1>(y, x, w, rows, cols, eps, s);
         else if (nvec <= 512) launch_rows<T, 256, 2>(y, x, w, rows, cols, eps, s);

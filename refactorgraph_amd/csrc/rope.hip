@@ -53,8 +53,8 @@ __global__ __launch_bounds__(256) void rope_tokens(T *__restrict__ y, const T *_
             const uint32_t tk = u / units_per_token, r = u % units_per_token;
             const uint32_t h = r / slices, sl = r % slices;
             const T *p = x + ((tok0 + tk) * heads + h) * D + sl * VEC;
-            lo[it] = load16(p);
-            hi[it] = load16(p + half);
+            lo[it] = load16_stream(p);
+            hi[it] = load16_stream(p + half);
         }
     }
 
@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256) void rope_tokens(T *__restrict__ y, const T *_
                 ohi.v[e] = from_compute<T>(b * cs + a * sn);
             }
             T *q = y + ((tok0 + tk) * heads + h) * D + sl * VEC;
-            store16(q, olo);
-            store16(q + half, ohi);
+            store16_stream(q, olo);
+            store16_stream(q + half, ohi);
         }
     }
 }

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *
         const uint32_t idx = t + i * GROUP;
         const uint32_t c0 = idx * VEC;
         if (live && idx < nvec && c0 < keep) {
-            const Vec16<T> xv = load16(xr + c0);
+            const Vec16<T> xv = load16_stream(xr + c0);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 f[i][e] = c0 + e < keep ? to_compute(xv.v[e]) : neg_inf<CT>();
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *
             Vec16<T> out;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) out.v[e] = from_compute<T>(norm(f[i][e]));
-            store16(yr + static_cast<size_t>(idx) * VEC, out);
+            store16_stream(yr + static_cast<size_t>(idx) * VEC, out);
         }
     }
 }

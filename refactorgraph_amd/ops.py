@@ -130,8 +130,19 @@ def attention_workspace(N, H, Hkv, seq, cap, D, device):
     return _ws_cache[key]
 
 
+_state_cache = {}
+
+
+def attention_state(device):
+    """Persistent, zero-initialised ticket counters (one buffer per device, calls must not overlap)."""
+    key = str(device)
+    if key not in _state_cache:
+        _state_cache[key] = torch.zeros(lib().rg_hip_attention_kvcache_state_bytes(), dtype=torch.uint8, device=device)
+    return _state_cache[key]
+
+
 def attention_kvcache(q, k, v, k_cache=None, v_cache=None, past_lens=None, scale=None, out=None,
-                      workspace=None):
+                      workspace=None, sync_state=None):
     """q [N,H,seq,D]; k, v [N,Hkv,seq,D]; caches [N,Hkv,cap,D] are updated in place;
     past_lens: int64 device tensor with 1 or N elements (None = 0)."""
     _need_gpu(q, k, v, k_cache, v_cache, past_lens)
@@ -148,6 +159,7 @@ def attention_kvcache(q, k, v, k_cache=None, v_cache=None, past_lens=None, scale
     ws = attention_workspace(N, H, Hkv, seq, cap, D, q.device) if workspace is None else workspace
     check(lib().rg_hip_attention_kvcache(
         _ptr(o), _ptr(q), _ptr(k), _ptr(v), _ptr(k_cache), _ptr(v_cache), _ptr(past_lens), per_row,
-        N, H, Hkv, seq, cap, D, float(scale), _T2CODE[q.dtype], _ptr(ws), ws.numel(), _stream()),
+        N, H, Hkv, seq, cap, D, float(scale), _T2CODE[q.dtype], _ptr(ws), ws.numel(), _ptr(sync_state),
+        _stream()),
         "rg_hip_attention_kvcache")
     return o

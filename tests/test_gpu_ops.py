@@ -297,14 +297,15 @@ def test_matmul_integer_full_config():
 
 # ------------------------------------------------------------------ AttentionKVCache
 
-def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_row=True, pairs=None):
+def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_row=True, pairs=None,
+                    sync_state=None):
     rng = np.random.default_rng(seed)
     mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).to(dt)
     q, k, v = mk((N, H, seq, D)), mk((N, Hkv, seq, D)), mk((N, Hkv, seq, D))
     kc, vc = mk((N, Hkv, cap, D)), mk((N, Hkv, cap, D))
     past = np.asarray(past, dtype=np.int64).reshape(-1)
     kc0, vc0 = kc.clone(), vc.clone()
-    o = ops.attention_kvcache(q, k, v, kc, vc, dev(past), 1 / math.sqrt(D))
+    o = ops.attention_kvcache(q, k, v, kc, vc, dev(past), 1 / math.sqrt(D), sync_state=sync_state)
     f = lambda t: host(t.float())
     ref_o, ref_kc, ref_vc = oracle.attention_kvcache(f(q), f(k), f(v), f(kc0), f(vc0), past, 1 / math.sqrt(D),
                                                      heads=pairs)
@@ -351,6 +352,20 @@ def test_attention_decode_full_config():
         assert np.max(np.abs(o[b, h] - ref_o[b, h])) <= ABS_F16
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
     assert np.isfinite(o).all()
+
+
+def test_attention_persistent_sync_state_is_left_zero():
+    # with caller-owned ticket counters the call is one launch; the counters must come back zero
+    # so that consecutive calls (different shapes) can share them
+    state = ops.attention_state(DEV)
+    for shape in [(4, 32, 8, 1, 1024, 128, [1, 100, 640, 1023]), (2, 8, 2, 5, 64, 128, [0, 20]),
+                  (32, 32, 8, 1, 4096, 128, np.random.default_rng(14).integers(1024, 4096, 32))]:
+        pairs = [(0, 0), (1, 3)] if shape[0] == 32 else None
+        o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(*shape, pairs=pairs, sync_state=state)
+        ok = np.isfinite(ref_o)
+        assert np.max(np.abs(o[ok] - ref_o[ok])) <= ABS_F16
+        assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+        assert int(state.sum()) == 0
 
 
 def test_attention_decode_invariants_full_size():
