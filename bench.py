@@ -33,8 +33,8 @@ FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 MFMA, published
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=4000)
     ap.add_argument("--ops", default="all", choices=["all", "headline"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma-separated op names to run besides the headline")
@@ -42,36 +42,42 @@ def parse():
 
 
 def time_steps(torch, fn, steps, warmup, n_sets):
-    """Times `steps` calls fn(i % n_sets) after `warmup` untimed ones.
+    """Times exactly `steps` calls fn(i % n_sets) after at least `warmup` untimed ones.
 
-    The timed calls are captured once into a HIP graph (plain kernel launches on the capture
-    stream) and replayed, so the device sees them back to back and host launch overhead does not
-    enter; the replay is bracketed by device synchronisation for the wall clock and by HIP events
-    on the replay stream for the device time.  Returns (wall ms per step, device ms per step,
-    "graph" | "eager")."""
-    for i in range(warmup):
+    The calls are captured into a HIP graph of `chunk` steps (chunk divides `steps`; plain kernel
+    launches on the capture stream) that is replayed steps/chunk times, so the device sees the
+    launches back to back and host launch overhead does not enter.  Warm-up replays the same
+    graph: the GPU leaves its idle clocks only after a few hundred milliseconds of load, so a
+    short warm-up would time the clock ramp, not the kernel.  The timed region is bracketed by
+    device synchronisation (wall clock) and by HIP events on the replay stream (device time).
+    Returns (wall ms per step, device ms per step, "graph" | "eager")."""
+    chunk = max(d for d in range(1, min(steps, 100) + 1) if steps % d == 0)
+    for i in range(min(warmup, 3)):
         fn(i % n_sets)
     torch.cuda.synchronize()
     mode = "graph"
     try:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            for i in range(steps):
+            for i in range(chunk):
                 fn(i % n_sets)
         run = graph.replay
-        run()                      # one untimed replay (graph upload)
+        run()                      # graph upload
     except Exception as exc:       # capture unavailable: time eager launches instead
         sys.stderr.write(f"bench.py: graph capture failed ({exc}); timing eager launches\n")
         mode = "eager"
 
         def run():
-            for i in range(steps):
+            for i in range(chunk):
                 fn(i % n_sets)
+    for _ in range((warmup + chunk - 1) // chunk):
+        run()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    run()
+    for _ in range(steps // chunk):
+        run()
     stop.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
@@ -191,7 +197,7 @@ def main():
         x = (3 * torch.randn((8, 32, 2048, 2048), device=dev)).half()
         y = torch.empty_like(x)
         for causal, nbytes, name in ((False, 4294967296, "softmax"), (True, 3221749760, "softmax_causal")):
-            wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 2, 5), 3, 1)
+            wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 4, 5), max(warmup // 8, 3), 1)
             e = hbm_entry(nbytes, dms)
             e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_per_launch=round(dms, 5), timing=mode)
             ops_out[name] = e
@@ -257,7 +263,7 @@ def main():
         wall, dms, mode = time_steps(
             torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp,
                                                    sync_state=state),
-            max(steps // 5, 3), 2, 1)
+            max(steps // 40, 3), max(warmup // 80, 2), 1)
         e = hbm_entry(402653184, dms)
         flops = 68853694464
         e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=128",
