@@ -240,21 +240,12 @@ __device__ void merge_segment(const AttnParams &p, const Segment &sg, uint64_t W
     }
 }
 
-#ifndef RG_ATTN_MINWAVES
-#define RG_ATTN_MINWAVES 1
-#endif
-#ifndef RG_ATTN_U
-#define RG_ATTN_U 4
-#endif
-#ifndef RG_ATTN_DB
-#define RG_ATTN_DB 1
-#endif
 template <class T, int D, int G>
-__global__ __launch_bounds__(256, RG_ATTN_MINWAVES) void attn_split(const AttnParams p) {
+__global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
     constexpr int LPR = D / 8;          // lanes per key row
     constexpr int KPW = kWave / LPR;    // key rows per wavefront load
     constexpr int KPB = KPW * 4;        // key rows per workgroup step
-    constexpr int U = RG_ATTN_U;        // steps per register set
+    constexpr int U = 4;                // steps per register set
     constexpr uint32_t SPAN = KPB * U;  // keys per step group
 
     __shared__ uint64_t sh_prefix[kMaxBatch + 1];
@@ -390,7 +381,6 @@ __global__ __launch_bounds__(256, RG_ATTN_MINWAVES) void attn_split(const AttnPa
                         Raw16, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(v_hist + off)));
                 }
             };
-#if RG_ATTN_DB
             Raw16 kA[U], vA[U], kB[U], vB[U];
             issue(pos0, kA, vA);
             for (uint32_t step0 = pos0; step0 < hist_end; step0 += 2 * SPAN) {
@@ -401,13 +391,6 @@ __global__ __launch_bounds__(256, RG_ATTN_MINWAVES) void attn_split(const AttnPa
                     consume(step0 + SPAN, hist_end, kB, vB);
                 }
             }
-#else
-            Raw16 kA[U], vA[U];
-            for (uint32_t step0 = pos0; step0 < hist_end; step0 += SPAN) {
-                issue(step0, kA, vA);
-                consume(step0, hist_end, kA, vA);
-            }
-#endif
         }
 
         // ---- new rows [max(pos0, base), end): read from the k/v inputs; the segment of the last
