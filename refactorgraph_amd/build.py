@@ -4,7 +4,6 @@
     librg_host.so    C++ host layer mirroring the reference's plugin surface
                      (hardware::Device, runtime::Resources/Routine, kernel::Kernel,
                      collectors); links librg_hip.so
-    rg_host_tests    C++ test driver for the host layer (run by tests/ on a GPU box)
 
 hipcc cross-compiles for gfx950 without a GPU, so this runs anywhere the ROCm toolchain is
 installed.  Usage: ``python -m refactorgraph_amd.build [--jobs N]``.
@@ -79,11 +78,6 @@ def build_host(jobs=8):
         objs = list(ex.map(_compile_host, srcs))
     out = os.path.join(LIB, "librg_host.so")
     _run(["g++", "-shared", "-fPIC", *objs, "-o", out, f"-L{LIB}", "-lrg_hip", "-Wl,-rpath,$ORIGIN"])
-    tests = sorted(glob.glob(os.path.join(HOST, "test", "*.cc")))
-    if tests:
-        exe = os.path.join(LIB, "rg_host_tests")
-        _run(["g++", *HOST_FLAGS, *tests, "-o", exe, f"-L{LIB}", "-lrg_host", "-lrg_hip",
-              "-Wl,-rpath,$ORIGIN", "-lpthread"])
     return out
 
 

@@ -1,0 +1,56 @@
+// Per-operator kernel selectors of the hot path, each with a case for Device::Type::Amd.
+// Constructor arguments and filter() contracts follow
+// src/04kernel/include/kernel/collectors/{rms_normalization.h, softmax.h, mat_mul_integer.h,
+// dequantize_linear.h, attention.h}; RotaryEmbeddingCollector has no counterpart there.
+#pragma once
+
+#include "rg_mirror/kernel.h"
+
+namespace refactor::kernel {
+
+    struct RmsNormalizationCollector final : public InfoCollector {
+        float epsilon;
+        constexpr RmsNormalizationCollector(hardware::Device::Type target, float epsilon_) noexcept
+            : InfoCollector(target), epsilon(epsilon_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    struct SoftmaxCollector final : public InfoCollector {
+        dim_t axis;
+        bool causal;// extension: decoder mask over the last two axes (needs axis == rank - 1)
+        constexpr SoftmaxCollector(hardware::Device::Type target, dim_t axis_, bool causal_ = false) noexcept
+            : InfoCollector(target), axis(axis_), causal(causal_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    struct MatMulIntegerCollector final : public InfoCollector {
+        constexpr explicit MatMulIntegerCollector(hardware::Device::Type target) noexcept
+            : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    struct DequantizeLinearCollector final : public InfoCollector {
+        int axis;// used only when the scale has more than one element (ONNX default 1)
+        explicit DequantizeLinearCollector(hardware::Device::Type target, int axis_ = 1) noexcept
+            : InfoCollector(target), axis(axis_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: query, key, value [, past_seq_len [, k_cache, v_cache]]; outputs: output
+    // [, k_cache, v_cache] (src/08-01llm/README.md:29-63).
+    struct AttentionCollector final : public InfoCollector {
+        dim_t maxSeqLen;
+        AttentionCollector(hardware::Device::Type target, dim_t maxSeqLen_) noexcept
+            : InfoCollector(target), maxSeqLen(maxSeqLen_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: x [batch, seq, heads, dim], positions int64 [batch, seq] or [seq]; outputs: y like x
+    struct RotaryEmbeddingCollector final : public InfoCollector {
+        float theta;
+        constexpr RotaryEmbeddingCollector(hardware::Device::Type target, float theta_) noexcept
+            : InfoCollector(target), theta(theta_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+}// namespace refactor::kernel

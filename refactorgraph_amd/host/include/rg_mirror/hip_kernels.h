@@ -1,0 +1,111 @@
+// The gfx950 kernels behind the collectors: one Kernel subclass per operator, each lowering to
+// a Routine that calls one rg_hip_* launcher of include/rg_hip.h on the default stream.
+// build() is noexcept and returns nullptr when the kernel does not apply, as the reference's
+// CUDA kernels do (e.g. src/04kernel/src/kernels/softmax/cuda_kernel.cc:9-17).
+#pragma once
+
+#include "rg_mirror/attributes.h"
+
+namespace refactor::kernel {
+
+    struct RmsNormalizationHip final : public Kernel {
+        float epsilon;
+        DataType dataType;
+        dim_t blockCount, blockSize;
+
+        RmsNormalizationHip(float, DataType, dim_t, dim_t) noexcept;
+        static KernelBox build(float epsilon, Tensor const &x) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    struct SoftmaxHip final : public Kernel {
+        SoftmaxInfo info;
+        dim_t causalRows;// 0: plain softmax
+
+        SoftmaxHip(SoftmaxInfo, dim_t causalRows) noexcept;
+        static KernelBox build(SoftmaxInfo, dim_t causalRows = 0) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    struct MatMulIntegerHip final : public Kernel {
+        MatMulIntegerInfo info;
+
+        explicit MatMulIntegerHip(MatMulIntegerInfo) noexcept;
+        static KernelBox build(MatMulIntegerInfo) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    struct DequantizeLinearHip final : public Kernel {
+        DataType from;
+        size_t outer, axisLen, inner;
+        bool perAxis, withZeroPoint;
+
+        DequantizeLinearHip(DataType, size_t, size_t, size_t, bool, bool) noexcept;
+        // scale with one element: the reference's per-tensor path; with more: one per index of `axis`
+        static KernelBox build(TensorRefs const &inputs, Tensor const &output, int axis = 1) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    struct AttentionHip final : public Kernel {
+        // the reference's parameter block (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-14)
+        // plus what it leaves to the run time: where past_seq_len comes from
+        struct Info {
+            DataType dataType;
+            dim_t batch, nHead, nKVHead, pastSeqLen, seqLen, cacheLen, headDim;
+            bool resetCache;   // 6-input form: copy the input caches into the output caches first
+            bool pastFromInput;// inputs[3] holds past_seq_len (read on the device at run time)
+            dim_t pastCount;   // its element count: 1 (reference contract) or batch (per row)
+        } info;
+
+        explicit AttentionHip(Info) noexcept;
+        static KernelBox build(Info) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    struct RotaryEmbeddingHip final : public Kernel {
+        DataType dataType;
+        dim_t batch, seq, heads, dim;
+        bool posPerBatch;
+        float theta;
+
+        RotaryEmbeddingHip(DataType, dim_t, dim_t, dim_t, dim_t, bool, float) noexcept;
+        static KernelBox build(float theta, Tensor const &x, Tensor const &pos) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    // Per-stream device state kept in Resources, in the way the reference keeps its library
+    // handles there (src/04kernel/src/utilities/cuda/cublas_context.cu:18-31): the zeroed ticket
+    // counters that let the attention kernel finish in a single launch.
+    class HipAttentionState final : public runtime::Resource {
+        void *_counters;
+
+    public:
+        HipAttentionState();
+        ~HipAttentionState();
+        HipAttentionState(HipAttentionState const &) = delete;
+        static size_t typeId() noexcept;
+        static runtime::ResourceBox build();
+        size_t resourceTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        void *counters() const noexcept { return _counters; }
+    };
+
+}// namespace refactor::kernel

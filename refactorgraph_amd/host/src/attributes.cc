@@ -1,0 +1,108 @@
+#include "rg_mirror/attributes.h"
+#include <algorithm>
+#include <numeric>
+
+namespace refactor::kernel {
+
+    SoftmaxInfo::SoftmaxInfo(Tensor const &data, dim_t axis) noexcept
+        : pre(1), mid(data.shape[axis]), post(1), type(data.dataType) {
+        for (dim_t i = 0; i < axis; ++i) { pre *= data.shape[i]; }
+        for (size_t i = axis + 1; i < data.shape.size(); ++i) { post *= data.shape[i]; }
+    }
+
+    // The shapes are right-aligned and walked from the last dimension to the first.  A dimension
+    // is described by which inputs really extend along it (size != 1); a run of dimensions with
+    // the same description collapses into one entry.
+    Broadcaster::Broadcaster(std::vector<std::vector<dim_t>> const &inputShapes)
+        : strides{}, outputsCount(1), inputsCount(static_cast<dim_t>(inputShapes.size())) {
+        ASSERT(inputsCount > 0, "Broadcaster: no inputs");
+        size_t rank = 0;
+        for (auto const &s : inputShapes) { rank = std::max(rank, s.size()); }
+
+        std::vector<bool> pattern(inputsCount, false), here(inputsCount);
+        std::vector<dim_t> extent(inputsCount, 1);// elements each input spans so far
+        std::vector<std::vector<dim_t>> entries;  // innermost first: per-input strides + output stride
+        for (size_t back = 0; back < rank; ++back) {
+            dim_t size = 1;
+            for (dim_t i = 0; i < inputsCount; ++i) {
+                auto const &s = inputShapes[i];
+                dim_t d = back < s.size() ? s[s.size() - 1 - back] : 1;
+                here[i] = d != 1;
+                if (d != 1) {
+                    ASSERT(size == 1 || size == d, "Broadcaster: shape mismatch");
+                    size = d;
+                }
+            }
+            if (size == 1) { continue; }
+            if (here != pattern) {
+                pattern = here;
+                std::vector<dim_t> entry(inputsCount + 1, 0);
+                for (dim_t i = 0; i < inputsCount; ++i) {
+                    if (pattern[i]) { entry[i] = extent[i]; }
+                }
+                entry[inputsCount] = outputsCount;
+                entries.push_back(std::move(entry));
+            }
+            for (dim_t i = 0; i < inputsCount; ++i) {
+                if (pattern[i]) { extent[i] *= size; }
+            }
+            outputsCount *= size;
+        }
+        // a single entry where every input walks with the output: nothing is broadcast
+        if (entries.size() == 1 && std::all_of(entries[0].begin(), entries[0].end(), [](dim_t x) { return x == 1; })) {
+            return;
+        }
+        for (auto it = entries.rbegin(); it != entries.rend(); ++it) {
+            strides.insert(strides.end(), it->begin(), it->end());
+        }
+    }
+
+    Broadcaster::Broadcaster(TensorRefs const &inputs)
+        : Broadcaster([&] {
+              std::vector<std::vector<dim_t>> shapes;
+              for (auto const &t : inputs) { shapes.emplace_back(t.get().shape.begin(), t.get().shape.end()); }
+              return shapes;
+          }()) {}
+
+    void Broadcaster::locate(dim_t k, dim_t ans[]) const noexcept {
+        if (strides.empty()) {
+            std::fill_n(ans, inputsCount, k);
+            return;
+        }
+        std::fill_n(ans, inputsCount, 0);
+        auto const width = inputsCount + 1;
+        for (size_t at = 0; at < strides.size(); at += width) {
+            auto const q = k / strides[at + inputsCount];
+            k %= strides[at + inputsCount];
+            for (dim_t j = 0; j < inputsCount; ++j) { ans[j] += strides[at + j] * q; }
+        }
+    }
+
+    MatMulIntegerInfo::Input::Input(TensorRefs const &inputs, size_t i) noexcept
+        : withZeroPoint(false), signed_(true), scalar(true) {
+        if (inputs.size() <= i + 2) { return; }
+        auto const &zp = inputs[i + 2].get();
+        auto const count = zp.elementsSize();
+        if (zp.data) {
+            // a constant zero point of all zeros needs no work
+            auto bytes = zp.data->get<uint8_t>();
+            if (std::all_of(bytes, bytes + count, [](uint8_t x) { return x == 0; })) { return; }
+        }
+        withZeroPoint = true;
+        signed_ = zp.dataType == DataType::I8;
+        scalar = count == 1;
+    }
+
+    static std::vector<dim_t> batchDims(Tensor const &t) {
+        return std::vector<dim_t>(t.shape.begin(), t.shape.end() - 2);
+    }
+
+    MatMulIntegerInfo::MatMulIntegerInfo(TensorRefs const &inputs) noexcept
+        : a(inputs, 0),
+          b(inputs, 1),
+          m(inputs[0].get().shape.rbegin()[1]),
+          k(inputs[0].get().shape.rbegin()[0]),
+          n(inputs[1].get().shape.rbegin()[0]),
+          broadcaster({batchDims(inputs[0].get()), batchDims(inputs[1].get())}) {}
+
+}// namespace refactor::kernel

@@ -1,0 +1,136 @@
+#include "rg_mirror/collectors.h"
+#include "rg_mirror/hip_kernels.h"
+
+// The reference's CPU kernels are not part of this build (the CPU target has no candidates here);
+// the Amd case of every collector offers the gfx950 kernel.
+namespace refactor::kernel {
+
+    using Target = hardware::Device::Type;
+
+#define ADD(PTR)                                  \
+    if (auto ptr = (PTR); ptr) {                  \
+        ans.emplace_back(std::move(ptr));         \
+    }
+
+    std::vector<KernelBox>
+    RmsNormalizationCollector::filter(TensorRefs inputs, TensorRefs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(RmsNormalizationHip::build(epsilon, inputs[0]))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    SoftmaxCollector::filter(TensorRefs inputs, TensorRefs) const {
+        auto const &x = inputs[0].get();
+        SoftmaxInfo info(x, axis);
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd: {
+                dim_t causalRows = 0;
+                if (causal) {
+                    // the mask is defined over the last two axes
+                    if (x.rank() < 2 || axis + 1 != static_cast<dim_t>(x.rank())) { break; }
+                    causalRows = x.shape[x.rank() - 2];
+                }
+                ADD(SoftmaxHip::build(info, causalRows))
+            } break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    MatMulIntegerCollector::filter(TensorRefs inputs, TensorRefs) const {
+        MatMulIntegerInfo info(inputs);
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(MatMulIntegerHip::build(info))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    DequantizeLinearCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(DequantizeLinearHip::build(inputs, outputs[0], axis))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    AttentionCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
+        auto const &query = inputs[0].get();
+        auto const &key = inputs[1].get();
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd: {
+                AttentionHip::Info info{
+                    .dataType = query.dataType,
+                    .batch = query.shape[0],
+                    .nHead = query.shape[1],
+                    .nKVHead = key.shape[1],
+                    .pastSeqLen = 0,
+                    .seqLen = query.shape[2],
+                    .cacheLen = outputs.size() == 1 ? 0 : outputs[1].get().shape[2],
+                    .headDim = query.shape[3],
+                    .resetCache = inputs.size() == 6,
+                    .pastFromInput = inputs.size() > 3,
+                    .pastCount = 0,
+                };
+                if (info.pastFromInput) {
+                    // past_seq_len is operator input 3 (after query, key, value); it is read on the
+                    // device at run time, a constant value is only recorded for the description
+                    auto const &past = inputs[3].get();
+                    info.pastCount = static_cast<dim_t>(past.elementsSize());
+                    if (past.data) { info.pastSeqLen = static_cast<dim_t>(*past.data->get<int64_t>()); }
+                }
+                ADD(AttentionHip::build(info))
+            } break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    RotaryEmbeddingCollector::filter(TensorRefs inputs, TensorRefs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(RotaryEmbeddingHip::build(theta, inputs[0], inputs[1]))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+}// namespace refactor::kernel
