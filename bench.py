@@ -29,6 +29,21 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published
 FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 MFMA, published
 
+# HBM-side bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, one run each,
+# KiB per dispatch) on the workloads below and scaled by what the same counters read for a plain
+# 256 MiB device copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  They are
+# properties of the kernels at these shapes, not of a particular run; the counter summaries are
+# kept in profiles/.
+MEASURED_TRAFFIC = {
+    "decode": (2 * 172652 + 2271) * 1024,
+    "rms_norm": (2 * 32867 + 65619) * 1024,
+    "softmax": (2 * 1048617 + 2097156) * 1024,
+    "softmax_causal": (2 * 540713 + 2097158) * 1024,
+    "rope": (2 * 131646 + 262167) * 1024,
+    "dequantize_linear": (2 * 8292 + 65569) * 1024,
+    "matmul_integer": (2 * 52558 + 71295) * 1024,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -38,6 +53,9 @@ def parse():
     ap.add_argument("--ops", default="all", choices=["all", "headline"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma-separated op names to run besides the headline")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also launch one plain device copy of 256 MiB (a reference point for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters into bytes)")
     return ap.parse_args()
 
 
@@ -85,10 +103,10 @@ def time_steps(torch, fn, steps, warmup, n_sets):
     return wall_ms, dev_ms, mode
 
 
-def hbm_entry(bytes_per_call, dev_ms):
+def hbm_entry(bytes_per_call, dev_ms, traffic_key=None):
     gbs = bytes_per_call / (dev_ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(traffic_key)}
 
 
 def main():
@@ -110,6 +128,14 @@ def main():
 
     def want(name):
         return args.ops == "all" and (not only or name in only)
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ------------------------------------------------------------ headline: decode
     N, H, Hkv, D, cap = 32, 32, 8, 128, 4096
@@ -141,7 +167,7 @@ def main():
 
     wall_ms, dev_ms, mode = time_steps(torch, decode, args.steps, args.warmup, n_sets)
     value = decode_bytes / (wall_ms * 1e-3) / 1e9
-    roofline = hbm_entry(decode_bytes, dev_ms)
+    roofline = hbm_entry(decode_bytes, dev_ms, "decode")
     roofline["kernel"] = "attn_split (one rg_hip_attention_kvcache call = one launch)"
     roofline["algorithmic_bytes"] = decode_bytes
     roofline["device_ms_per_launch"] = round(dev_ms, 5)
@@ -188,7 +214,7 @@ def main():
         ys = [torch.empty_like(xs[0]) for _ in range(nb)]
         w = torch.rand(4096, device=dev) + 0.5
         wall, dms, mode = time_steps(torch, lambda i: ops.rms_norm(xs[i], w, 1e-5, out=ys[i]), steps, warmup, nb)
-        e = hbm_entry(134234112, dms)
+        e = hbm_entry(134234112, dms, "rms_norm")
         e.update(workload="RmsNormalization f32 [32,128,4096]", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["rms_norm"] = e
         del xs, ys
@@ -198,7 +224,7 @@ def main():
         y = torch.empty_like(x)
         for causal, nbytes, name in ((False, 4294967296, "softmax"), (True, 3221749760, "softmax_causal")):
             wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 4, 5), max(warmup // 8, 3), 1)
-            e = hbm_entry(nbytes, dms)
+            e = hbm_entry(nbytes, dms, name)
             e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_per_launch=round(dms, 5), timing=mode)
             ops_out[name] = e
         del x, y
@@ -209,7 +235,7 @@ def main():
         ys = [torch.empty_like(xs[0]) for _ in range(nb)]
         pos = torch.arange(2048, device=dev, dtype=torch.int64).repeat(16, 1).contiguous()
         wall, dms, mode = time_steps(torch, lambda i: ops.rope(xs[i], pos, 10000.0, out=ys[i]), steps, warmup, nb)
-        e = hbm_entry(537133056, dms)
+        e = hbm_entry(537133056, dms, "rope")
         e.update(workload="RotaryEmbedding fp16 [16,2048,32,128]", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["rope"] = e
         del xs, ys
@@ -220,7 +246,7 @@ def main():
         ys = [torch.empty((4096, 4096), device=dev) for _ in range(nb)]
         sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
         wall, dms, mode = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
-        e = hbm_entry(83902464, dms)
+        e = hbm_entry(83902464, dms, "dequantize_linear")
         e.update(workload="DequantizeLinear i8->f32 [4096,4096] per-axis scale", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["dequantize_linear"] = e
         del xs, ys
@@ -235,7 +261,7 @@ def main():
         tops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
         ops_out["matmul_integer"] = {
             "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-            "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
+            "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC["matmul_integer"],
             "workload": "MatMulInteger u8 x i8 -> i32 4096^3, a_zp=128 b_zp=0",
             "device_ms_per_launch": round(dms, 5), "timing": mode}
         if not args.no_cpu:
