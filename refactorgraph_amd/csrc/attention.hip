@@ -18,6 +18,7 @@
 // form in float.  A segment that ends up in more than one range leaves (max, sum, unnormalised
 // O) partials; the workgroup that finishes such a segment last (a ticket counter per segment)
 // merges them, so one launch does everything.
+#include "attention_prefill.hpp"
 #include "common.hpp"
 
 namespace rg {
@@ -294,7 +295,7 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
         const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
 
         float m[G], l[G], acc[G][8];
-        bool fresh = true;  // no step group consumed yet (wave-uniform)
+        bool empty = true;  // this lane's key rows have not held a valid key yet
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             m[g] = 0.f;
@@ -304,12 +305,14 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
         }
 
         // Online-softmax update with one step group; keys >= limit are masked out.  The running
-        // reference m[g] is only raised (and the accumulators rescaled) when some score exceeds
-        // it by more than kSlack, a wave-uniform and rare event after the first group; otherwise
-        // p = exp2(s - m) <= 2^kSlack is accumulated directly.
+        // reference m[g] is only moved (and the accumulators rescaled) when some score exceeds
+        // it by more than kSlack or a lane meets its first valid key, a rare event after the
+        // first group; otherwise p = exp2(s - m) <= 2^kSlack is accumulated directly.  A lane
+        // that has seen no valid key keeps m = 0 with empty accumulators.
         auto consume = [&](uint32_t step0, uint32_t limit, const Raw16(&kk)[U], const Raw16(&vv)[U]) {
             float t[U][G];  // score - reference, log2 units
             float over = -__builtin_inff();
+            const bool valid0 = step0 + key_in_span < limit;  // keys ascend with u
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const bool valid = step0 + u * KPB + key_in_span < limit;
@@ -323,15 +326,16 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
                     over = fmaxf(over, t[u][g]);
                 }
             }
-            if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
+            if (__builtin_amdgcn_ballot_w64(over > kSlack || (empty && valid0)) != 0) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    // how far the reference moves: to the group maximum the first time (the
-                    // reference starts at 0 with empty accumulators), never down afterwards
-                    float up = fresh ? kMinusBig : 0.f;
+                    // how far the reference moves: to the group maximum at the lane's first valid
+                    // key (the accumulators are still empty), never down afterwards
+                    float up = t[0][g];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) up = fmaxf(up, t[u][g]);
-                    const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
+                    for (int u = 1; u < U; ++u) up = fmaxf(up, t[u][g]);
+                    up = empty ? (valid0 ? up : 0.f) : fmaxf(up, 0.f);
+                    const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f(-up);
                     m[g] += up;
                     l[g] *= alpha;
 #pragma unroll
@@ -339,7 +343,7 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) t[u][g] -= up;
                 }
-                fresh = false;
+                empty = empty && !valid0;
             }
 #pragma unroll
             for (int g = 0; g < G; ++g) {
@@ -423,9 +427,10 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
         }
 
         // ---- merge the four key rows of each wavefront with shuffles, then the four wavefronts
-        // through LDS
+        // through LDS; lanes that never held a valid key drop out of the maxima
 #pragma unroll
         for (int g = 0; g < G; ++g) {
+            if (empty) m[g] = kMinusBig;
             float M = fmaxf(m[g], __shfl_xor(m[g], LPR, kWave));
             if constexpr (KPW >= 4) M = fmaxf(M, __shfl_xor(M, 2 * LPR, kWave));
             if constexpr (KPW >= 8) M = fmaxf(M, __shfl_xor(M, 4 * LPR, kWave));
@@ -543,6 +548,7 @@ uint32_t resident_workgroups() {
 }
 
 constexpr uint32_t kMaxWorkgroups = 4096;  // bound used by the workspace query
+constexpr size_t kPrefillMinSeq = 16;      // query rows per batch row from which the tiled kernel is used
 
 template <class T, int D, int G>
 int launch(AttnParams p, hipStream_t s) {
@@ -615,6 +621,24 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
         (k_cache && (!aligned16(k_cache) || !aligned16(v_cache))))
         return RG_HIP_E_ARGUMENT;
 
+    hipStream_t s = as_stream(stream);
+    // many query rows per batch row: the tiled MFMA kernel (K/V staged once per query tile)
+    if (seq >= kPrefillMinSeq && prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head),
+                                                   static_cast<uint32_t>(D))) {
+        PrefillArgs a{};
+        a.q = q; a.k = k; a.v = v; a.o = o; a.kc = k_cache; a.vc = v_cache;
+        a.past = past_lens;
+        a.past_per_row = past_per_row;
+        a.N = static_cast<uint32_t>(N);
+        a.H = static_cast<uint32_t>(n_head);
+        a.Hkv = static_cast<uint32_t>(n_kv_head);
+        a.seq = static_cast<uint32_t>(seq);
+        a.cap = static_cast<uint32_t>(cap);
+        a.scale = scale;
+        a.dtype = dtype;
+        return launch_prefill(a, s);
+    }
+
     AttnParams p{};
     p.q = q; p.k = k; p.v = v; p.o = o; p.kc = k_cache; p.vc = v_cache;
     p.past = past_lens;
@@ -627,7 +651,6 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
     p.group = p.H / p.Hkv;
     p.scale_log2e = scale * 1.4426950408889634f;
     p.part = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
-    hipStream_t s = as_stream(stream);
     if (sync_state) {
         p.counters = static_cast<uint32_t *>(sync_state);
     } else {

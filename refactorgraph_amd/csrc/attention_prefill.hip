@@ -1,0 +1,326 @@
+// Tiled causal attention for many query rows per batch row (prefill), head dim 128, gfx950.
+//
+// Same contract as the split-KV kernel (layouts of src/08-01llm/README.md:29-63 of the
+// reference: q, o [N, H, seq, D]; k, v [N, Hkv, seq, D]; caches [N, Hkv, cap, D]; query row r
+// attends positions 0 .. past + r; new rows appended at past .. past + seq - 1).
+//
+// A workgroup of four wavefronts works on one kv head: wavefront w owns 32 query rows of one of
+// the query heads that share this kv head (GQA), so a K/V tile staged once in LDS serves up to
+// four query heads.  Keys are walked 64 at a time.  Both products run on the fp16/bf16 MFMA
+// (v_mfma_f32_32x32x16) in transposed form:
+//     S^T[key, q] = K[key, :] . Q[q, :]       A = K rows (LDS, 128-bit reads), B = Q rows (registers)
+//     O^T[d, q]  += V^T[d, key] . P^T[key, q] A = V columns (LDS, 16-bit gathers), B = P (registers)
+// In this form a lane holds one query row of S^T / O^T in its accumulator registers, so the
+// softmax row statistics need no cross-lane reduction beyond one exchange between the two
+// half-wavefronts, and P^T is already in B-operand position.  Softmax is online in float with
+// the lazily raised reference of the split kernel.  O^T is transposed through LDS at the end so
+// that the global stores are 128-bit and row-contiguous.
+#include "attention_prefill.hpp"
+
+namespace rg {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int D = 128;
+constexpr int BN = 64;                 // keys per tile
+constexpr int ROW = 2 * D + 16;        // LDS pitch of a key row, bytes (272: conflict-free fragment reads)
+constexpr int TILE = BN * ROW;         // 17408
+constexpr int LDS_BYTES = 2 * TILE;    // K tile + V tile; reused for the output transposition
+constexpr float kSlack = 6.0f;
+constexpr float kMinusBig = -1e30f;
+
+struct alignas(16) Raw16 {
+    uint32_t w[4];
+};
+
+template <class T> struct Ops;
+template <> struct Ops<__half> {
+    static __device__ __forceinline__ f16v mfma(const Raw16 &a, const Raw16 &b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+};
+template <> struct Ops<__hip_bfloat16> {
+    static __device__ __forceinline__ f16v mfma(const Raw16 &a, const Raw16 &b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        const uint32_t l = __builtin_bit_cast(uint16_t, __float2bfloat16(lo));
+        const uint32_t h = __builtin_bit_cast(uint16_t, __float2bfloat16(hi));
+        return l | (h << 16);
+    }
+};
+
+// HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
+// query sub-tiles of the same heads.
+template <class T, int HW>
+__global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_t group,
+                                                    uint32_t q_tiles, uint32_t head_chunks) {
+    constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
+    constexpr int ROWS = 32 * QS;   // query rows per workgroup
+    __shared__ __align__(16) uint8_t lds[LDS_BYTES];
+    uint8_t *ldsK = lds, *ldsV = lds + TILE;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t half = lane >> 5, l32 = lane & 31;
+
+    // heaviest query tiles (longest key range) first
+    const uint32_t n_rest = a.N * a.Hkv * head_chunks;
+    const uint32_t qt = q_tiles - 1 - blockIdx.x / n_rest;
+    uint32_t rest = blockIdx.x % n_rest;
+    const uint32_t hc = rest % head_chunks;
+    rest /= head_chunks;
+    const uint32_t kvh = rest % a.Hkv, b = rest / a.Hkv;
+
+    // history length of this batch row, clamped so that the new rows fit the cache
+    uint32_t base = 0;
+    if (a.kc && a.past) {
+        int64_t raw = a.past[a.past_per_row ? b : 0];
+        if (raw < 0) raw = 0;
+        const int64_t room = static_cast<int64_t>(a.cap) - static_cast<int64_t>(a.seq);
+        if (raw > room) raw = room < 0 ? 0 : room;
+        base = static_cast<uint32_t>(raw);
+    }
+
+    const T *Q = static_cast<const T *>(a.q);
+    const T *Kn = static_cast<const T *>(a.k);
+    const T *Vn = static_cast<const T *>(a.v);
+    T *Kc = static_cast<T *>(a.kc);
+    T *Vc = static_cast<T *>(a.vc);
+    T *O = static_cast<T *>(a.o);
+    const uint64_t kv_head = static_cast<uint64_t>(b) * a.Hkv + kvh;
+    const T *k_new = Kn + kv_head * a.seq * D;
+    const T *v_new = Vn + kv_head * a.seq * D;
+    const T *k_hist = Kc ? Kc + kv_head * a.cap * D : nullptr;
+    const T *v_hist = Vc ? Vc + kv_head * a.cap * D : nullptr;
+
+    const uint32_t head = kvh * group + hc * HW + wave % HW;
+    const uint32_t r0 = qt * ROWS + 32 * (wave / HW);  // first query row of this wavefront
+    const bool wave_active = r0 < a.seq;
+    const uint32_t wg_rows_end = (qt + 1) * ROWS < a.seq ? (qt + 1) * ROWS : a.seq;
+
+    // append the new rows this workgroup's query rows correspond to (once per kv head)
+    if (Kc && hc == 0) {
+        for (uint32_t idx = tid; idx < (wg_rows_end - qt * ROWS) * 16; idx += 256) {
+            const uint32_t rr = qt * ROWS + idx / 16, c = idx % 16;
+            const uint64_t src = static_cast<uint64_t>(rr) * D + c * 8;
+            const uint64_t dst = (kv_head * a.cap + base + rr) * D + c * 8;
+            *reinterpret_cast<Raw16 *>(Kc + dst) = *reinterpret_cast<const Raw16 *>(k_new + src);
+            *reinterpret_cast<Raw16 *>(Vc + dst) = *reinterpret_cast<const Raw16 *>(v_new + src);
+        }
+    }
+
+    // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
+    Raw16 qf[8];
+    {
+        const uint32_t qrow = r0 + l32 < a.seq ? r0 + l32 : a.seq - 1;
+        const T *qp = Q + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + qrow) * D + 8 * half;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qp + 16 * kk);
+    }
+
+    const uint32_t wg_last_key = base + wg_rows_end - 1;  // inclusive
+    const uint32_t n_tiles = wg_last_key / BN + 1;
+    const uint32_t wave_last_row = r0 + 31 < a.seq ? r0 + 31 : a.seq - 1;
+    const uint32_t wave_tiles = wave_active ? (base + wave_last_row) / BN + 1 : 0;
+    const uint32_t qpos = base + r0 + l32;  // absolute position of this lane's query row
+    const float c_log2e = a.scale * 1.4426950408889634f;
+
+    // staging: thread owns 16-byte chunk tid % 16 of key rows tid / 16 + 16 i
+    const uint32_t st_chunk = tid & 15, st_row = tid >> 4;
+    auto fetch = [&](uint32_t kt, Raw16(&kr)[4], Raw16(&vr)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t pos = kt * BN + st_row + 16 * i;
+            kr[i] = Raw16{{0, 0, 0, 0}};
+            vr[i] = Raw16{{0, 0, 0, 0}};
+            if (pos <= wg_last_key) {
+                if (pos < base) {
+                    const uint64_t off = static_cast<uint64_t>(pos) * D + st_chunk * 8;
+                    kr[i] = *reinterpret_cast<const Raw16 *>(k_hist + off);
+                    vr[i] = *reinterpret_cast<const Raw16 *>(v_hist + off);
+                } else {
+                    const uint64_t off = static_cast<uint64_t>(pos - base) * D + st_chunk * 8;
+                    kr[i] = *reinterpret_cast<const Raw16 *>(k_new + off);
+                    vr[i] = *reinterpret_cast<const Raw16 *>(v_new + off);
+                }
+            }
+        }
+    };
+    auto stage = [&](const Raw16(&kr)[4], const Raw16(&vr)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t off = (st_row + 16 * i) * ROW + st_chunk * 16;
+            *reinterpret_cast<Raw16 *>(ldsK + off) = kr[i];
+            *reinterpret_cast<Raw16 *>(ldsV + off) = vr[i];
+        }
+    };
+
+    f16v o[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+    float m = 0.f, l = 0.f;
+    bool fresh = true;
+
+    Raw16 kr[4], vr[4];
+    fetch(0, kr, vr);
+    stage(kr, vr);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < n_tiles; ++kt) {
+        if (kt + 1 < n_tiles) fetch(kt + 1, kr, vr);
+
+        if (kt < wave_tiles) {
+            // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32
+            f16v s[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) {
+                    const Raw16 kf = *reinterpret_cast<const Raw16 *>(ldsK + (32 * kb + l32) * ROW + (2 * kk + half) * 16);
+                    s[kb] = Ops<T>::mfma(kf, qf[kk], s[kb]);
+                }
+            }
+            // scale, causal mask (only tiles that reach past the wavefront's first query position)
+            const bool need_mask = kt * BN + BN - 1 > base + r0;
+            float over = -__builtin_inff();
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float t = fmaf(s[kb][e], c_log2e, -m);
+                    if (need_mask) {
+                        const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
+                        t = key > qpos ? -__builtin_inff() : t;
+                    }
+                    s[kb][e] = t;
+                    over = fmaxf(over, t);
+                }
+            over = fmaxf(over, __shfl_xor(over, 32, kWave));  // both halves hold the same query row
+            if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
+                const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
+                const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
+                m += up;
+                l *= alpha;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) s[kb][e] -= up;
+                fresh = false;
+            }
+            // P^T in B-operand position: element i of MFMA (kb, jj) is accumulator register 8 jj + i
+            Raw16 pf[2][2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int i2 = 0; i2 < 4; ++i2) {
+                        const float p0 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2]);
+                        const float p1 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2 + 1]);
+                        l += p0 + p1;
+                        pf[kb][jj].w[i2] = Ops<T>::pack2(p0, p1);
+                    }
+            // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
+            // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf
+            const uint16_t *v16 = reinterpret_cast<const uint16_t *>(ldsV);
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+                        Raw16 vf;
+#pragma unroll
+                        for (int i2 = 0; i2 < 4; ++i2) {
+                            const int i = 2 * i2;
+                            const uint32_t key0 = 32 * kb + 16 * jj + (i < 4 ? 4 * half + i : 8 + 4 * half + i - 4);
+                            const uint32_t lo = v16[key0 * (ROW / 2) + 32 * db + l32];
+                            const uint32_t hi = v16[(key0 + 1) * (ROW / 2) + 32 * db + l32];
+                            vf.w[i2] = lo | (hi << 16);
+                        }
+                        o[db] = Ops<T>::mfma(vf, pf[kb][jj], o[db]);
+                    }
+        }
+
+        __syncthreads();  // every wavefront is done with this tile
+        if (kt + 1 < n_tiles) {
+            stage(kr, vr);
+            __syncthreads();
+        }
+    }
+
+    // ---- normalise, transpose O^T -> O through LDS, 128-bit row-contiguous stores
+    l += __shfl_xor(l, 32, kWave);
+    const float inv = 1.f / l;
+    uint8_t *ldsO = lds + wave * (32 * ROW);  // the K/V tiles are no longer needed (barrier above)
+    if (wave_active) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+                const uint32_t d = 32 * db + 8 * (e / 4) + 4 * half + (e % 4);
+                *reinterpret_cast<uint32_t *>(ldsO + l32 * ROW + 2 * d) = Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
+            }
+    }
+    __syncthreads();
+    if (wave_active) {
+        T *op = O + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + r0) * D;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t idx = lane + 64 * i, row = idx / 16, c = idx % 16;
+            if (r0 + row < a.seq)
+                *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
+                    *reinterpret_cast<const Raw16 *>(ldsO + row * ROW + c * 16);
+        }
+    }
+}
+
+template <class T, int HW>
+int launch_hw(const PrefillArgs &a, hipStream_t s) {
+    const uint32_t group = a.H / a.Hkv;
+    const uint32_t head_chunks = group / HW;
+    constexpr uint32_t ROWS = 32 * (4 / HW);
+    const uint32_t q_tiles = (a.seq + ROWS - 1) / ROWS;
+    const uint64_t grid = static_cast<uint64_t>(a.N) * a.Hkv * head_chunks * q_tiles;
+    if (grid > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+    attn_prefill<T, HW><<<static_cast<unsigned>(grid), 256, 0, s>>>(a, group, q_tiles, head_chunks);
+    return launch_status();
+}
+
+template <class T>
+int launch_t(const PrefillArgs &a, hipStream_t s) {
+    const uint32_t group = a.H / a.Hkv;
+    if (group % 4 == 0) return launch_hw<T, 4>(a, s);
+    if (group == 2) return launch_hw<T, 2>(a, s);
+    return launch_hw<T, 1>(a, s);
+}
+
+}  // namespace
+
+bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D_) {
+    const uint32_t group = H / Hkv;
+    return D_ == D && (group % 4 == 0 || group == 2 || group == 1);
+}
+
+int launch_prefill(const PrefillArgs &a, hipStream_t s) {
+    if (a.dtype == RG_FP16) return launch_t<__half>(a, s);
+    return launch_t<__hip_bfloat16>(a, s);
+}
+
+}  // namespace rg

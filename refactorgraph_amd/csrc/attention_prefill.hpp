@@ -1,0 +1,24 @@
+// Interface between the attention entry point and the tiled (MFMA) prefill kernel.
+#pragma once
+
+#include "common.hpp"
+
+namespace rg {
+
+struct PrefillArgs {
+    const void *q, *k, *v;
+    void *o, *kc, *vc;
+    const int64_t *past;
+    int past_per_row;
+    uint32_t N, H, Hkv, seq, cap;
+    float scale;
+    int dtype;  // RG_FP16 or RG_BF16
+};
+
+// True when launch_prefill handles the shape (head dim 128, group size 1, 2 or a multiple of 4).
+bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D);
+
+// Enqueues the kernel; returns a hipError_t as int.
+int launch_prefill(const PrefillArgs &a, hipStream_t s);
+
+}  // namespace rg

@@ -320,6 +320,10 @@ def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_
     (2, 4, 4, 1, 128, 64, [100, 9]),        # MHA
     (2, 8, 2, 5, 64, 128, [0, 20]),         # several new rows with history
     (1, 4, 1, 16, 16, 64, [0]),             # prefill into an exactly fitting cache
+    (1, 6, 2, 8, 64, 128, [7]),             # history shorter than one step: some key rows meet their
+    (1, 2, 1, 48, 64, 64, [7]),             #   first valid key only among the new rows
+    (2, 5, 1, 12, 64, 128, [3, 40]),
+    (1, 1, 1, 9, 32, 64, [1]),
 ])
 def test_attention_decode_and_small_prefill(N, H, Hkv, seq, cap, D, past):
     o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past)
@@ -390,6 +394,32 @@ def test_attention_decode_invariants_full_size():
     vc2[:, :, :1024] = vc[:, :, perm]
     o2 = ops.attention_kvcache(q, k, v, kc2, vc2, past)
     assert float((o1.float() - o2.float()).abs().max()) <= ABS_F16
+
+
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,past,dt", [
+    (2, 8, 2, 40, 128, 128, [0, 20], torch.float16),      # ragged: 40 rows, history on one row
+    (2, 4, 4, 33, 64, 128, [5, 31], torch.float16),       # MHA (one head per workgroup)
+    (1, 4, 2, 64, 200, 128, [100], torch.float16),        # group of 2
+    (2, 16, 2, 96, 96, 128, [0, 0], torch.float16),       # group of 8: two head chunks per kv head
+    (2, 8, 2, 70, 256, 128, [3, 150], torch.bfloat16),
+    (1, 6, 2, 48, 64, 128, [7], torch.float16),           # group of 3: split-KV fallback
+    (1, 8, 2, 129, 512, 128, [300], torch.float16),
+])
+def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt)
+    assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
+def test_attention_prefill_no_cache_tiled():
+    rng = np.random.default_rng(21)
+    mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).half()
+    q, k, v = mk((2, 8, 50, 128)), mk((2, 2, 50, 128)), mk((2, 2, 50, 128))
+    o = host(ops.attention_kvcache(q, k, v, scale=0.1).float())
+    f = lambda t: host(t.float())
+    z = np.zeros((2, 2, 50, 128), np.float32)
+    ref, _, _ = oracle.attention_kvcache(f(q), f(k), f(v), z, z, [0, 0], 0.1)
+    assert np.max(np.abs(o - ref)) <= ABS_F16
 
 
 def test_attention_prefill_config_sample():
