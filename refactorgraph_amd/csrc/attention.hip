@@ -96,6 +96,13 @@ __device__ uint64_t build_partition(const AttnParams &p, Partition part) {
     return part.prefix[p.N];
 }
 
+// Quotient of key counts; almost always both fit 32 bits, where the division is several times
+// cheaper than the emulated 64-bit one.
+__device__ __forceinline__ uint64_t udiv(uint64_t a, uint64_t b) {
+    if (((a | b) >> 32) == 0) return static_cast<uint32_t>(a) / static_cast<uint32_t>(b);
+    return a / b;
+}
+
 struct Segment {
     uint32_t b, r, kvh;
     uint32_t base;       // history length of batch row b
@@ -125,19 +132,20 @@ __device__ Segment locate(const AttnParams &p, const Partition &part, uint64_t f
     s.r = rlo;
     s.len = s.base + s.r + 1;
     const uint64_t u2 = u - keys_before_row(p.Hkv, s.base, s.r);
-    s.kvh = static_cast<uint32_t>(u2 / s.len);
+    s.kvh = static_cast<uint32_t>(udiv(u2, s.len));
     s.start = part.prefix[lo] + keys_before_row(p.Hkv, s.base, s.r) + static_cast<uint64_t>(s.kvh) * s.len;
     return s;
 }
 
 __device__ __forceinline__ uint64_t range_width(uint64_t total, uint32_t n_workgroups) {
-    uint64_t w = (total + n_workgroups - 1) / n_workgroups;
+    uint64_t w = udiv(total + n_workgroups - 1, n_workgroups);
     w = (w + 15) / 16 * 16;
     return w < 64 ? 64 : w;
 }
 
 // ---------------------------------------------------------------- element helpers
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
 
@@ -171,6 +179,13 @@ template <> struct Elem<__hip_bfloat16> {
     }
 };
 
+// 16-byte streaming load from global memory (the address space is stated so that a pointer
+// chosen at run time between two buffers does not fall back to generic addressing)
+typedef const u32x4 __attribute__((address_space(1))) *GlobalVec16;
+__device__ __forceinline__ Raw16 load_stream_global(const void *p) {
+    return __builtin_bit_cast(Raw16, __builtin_nontemporal_load((GlobalVec16)p));
+}
+
 // reduction over the LPR (8 or 16) lanes that share a key row
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {
@@ -187,6 +202,10 @@ __device__ __forceinline__ void store_coherent(float *p, float v) {
     __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void store_coherent2(float *p, float a, float b) {  // p 8-byte aligned
+    const uint64_t v = (static_cast<uint64_t>(__builtin_bit_cast(uint32_t, b)) << 32) | __builtin_bit_cast(uint32_t, a);
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ float load_coherent(const float *p) {
     return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT));
@@ -201,7 +220,7 @@ __device__ void merge_segment(const AttnParams &p, const Segment &sg, uint64_t W
                               uint64_t last) {
     T *O = static_cast<T *>(p.o);
     constexpr int B = 8;
-    for (uint32_t idx = threadIdx.x; idx < G * D; idx += 256) {
+    for (uint32_t idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
         const uint32_t g = idx / D, d = idx % D;
         float M = kMinusBig, o_sum = 0.f, l_sum = 0.f;
         for (uint64_t w0 = first; w0 <= last; w0 += B) {
@@ -241,20 +260,92 @@ __device__ void merge_segment(const AttnParams &p, const Segment &sg, uint64_t W
     }
 }
 
+// Sums (or maxima) over the four 16-lane groups of a wavefront with lane swaps.  The two
+// results of a swap are copied into scalars before they are reinterpreted as floats.
+struct SwapPair {
+    float a, b;
+};
+__device__ __forceinline__ SwapPair swap32(float x, float y) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y),
+                                                    false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return {__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1)};
+}
+__device__ __forceinline__ SwapPair swap16(float x, float y) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y),
+                                                    false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return {__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1)};
+}
+__device__ __forceinline__ float swap32_sum(float lo_keeps, float hi_keeps) {
+    // lanes 0-31 receive lo_keeps summed over both halves, lanes 32-63 hi_keeps
+    const SwapPair r = swap32(lo_keeps, hi_keeps);
+    return r.a + r.b;
+}
+__device__ __forceinline__ float swap16_sum(float even_keeps, float odd_keeps) {
+    // even 16-lane groups receive even_keeps summed over the group pair, odd ones odd_keeps
+    const SwapPair r = swap16(even_keeps, odd_keeps);
+    return r.a + r.b;
+}
+__device__ __forceinline__ float swap_sum(float v) {
+    const float h = swap32_sum(v, v);
+    return swap16_sum(h, h);
+}
+__device__ __forceinline__ float swap_max(float v) {
+    const SwapPair r = swap32(v, v);
+    const float h = fmaxf(r.a, r.b);
+    const SwapPair q = swap16(h, h);
+    return fmaxf(q.a, q.b);
+}
+
+constexpr int kSplitThreads = 512;                   // one workgroup per CU at two wavefronts per SIMD
+constexpr int kSplitWaves = kSplitThreads / kWave;
+constexpr int kMaxPieces = 4;                        // pieces of a range handled per pass
+
+// One piece = the part of a segment that falls into a workgroup's range.
+struct PieceRec {
+    uint64_t start;      // position of key 0 of the segment in the laid-out key space
+    uint64_t hist_row0;  // cache row of key 0 of the kv head
+    int64_t new_row0;    // input row that key 0 would have (key `base` is the first real one)
+    uint32_t b, r, kvh, base, len;  // the segment
+    uint32_t pos0, end;  // keys [pos0, end) of the segment
+    uint32_t blk0;       // first block of the piece within the pass
+    uint32_t flags;      // 1: the whole segment, 2: appends the new rows, 4: starts the range
+    uint32_t pad;
+};
+
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint64_t uni(uint64_t v) {
+    return (static_cast<uint64_t>(uni(static_cast<uint32_t>(v >> 32))) << 32) | uni(static_cast<uint32_t>(v));
+}
+
+// What a wavefront needs of a piece to load and consume its blocks (wave-uniform registers).
+struct PieceView {
+    uint64_t hist_row0;
+    int64_t new_row0;
+    uint32_t base, pos0, end, blk0, flags;
+};
+
 template <class T, int D, int G>
-__global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
+__global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) {
     constexpr int LPR = D / 8;          // lanes per key row
     constexpr int KPW = kWave / LPR;    // key rows per wavefront load
-    constexpr int KPB = KPW * 4;        // key rows per workgroup step
-    constexpr int U = 4;                // steps per register set
-    constexpr uint32_t SPAN = KPB * U;  // keys per step group
+    constexpr int U = 4;                // loads per register set
+    constexpr uint32_t BK = KPW * U;    // keys per block: the unit a wavefront pulls
+    constexpr int NSET = 2;             // blocks a wavefront keeps in flight
+    constexpr int NW = kSplitWaves;
 
     __shared__ uint64_t sh_prefix[kMaxBatch + 1];
     __shared__ uint32_t sh_base[kMaxBatch];
-    __shared__ float sh_o[4][G][D];
-    __shared__ float sh_m[4][G];
-    __shared__ float sh_l[4][G];
-    __shared__ uint32_t sh_last;
+    __shared__ PieceRec sh_pc[kMaxPieces];
+    __shared__ uint64_t sh_f;
+    __shared__ uint32_t sh_np, sh_nblk, sh_next;
+    __shared__ uint32_t sh_has[kMaxPieces];  // wavefronts that hold a state of the piece (bit mask)
+    __shared__ uint32_t sh_last[kMaxPieces];
+    __shared__ alignas(16) uint32_t sh_q[kMaxPieces][G][D / 2];
+    __shared__ alignas(16) float sh_o[kMaxPieces][NW][G][D];
+    __shared__ alignas(16) float sh_m[kMaxPieces][G][NW];
+    __shared__ alignas(16) float sh_l[kMaxPieces][G][NW];
 
     const Partition part{sh_prefix, sh_base};
     const uint64_t total = build_partition(p, part);
@@ -265,7 +356,6 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
 
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t row = lane / LPR, chunk = lane % LPR;  // key row within a wavefront load, 16-byte slice
-    const uint32_t key_in_span = wave * KPW + row;
     const T *Q = static_cast<const T *>(p.q);
     const T *Kn = static_cast<const T *>(p.k);
     const T *Vn = static_cast<const T *>(p.v);
@@ -273,241 +363,370 @@ __global__ __launch_bounds__(256) void attn_split(const AttnParams p) {
     T *Vc = static_cast<T *>(p.vc);
     T *O = static_cast<T *>(p.o);
 
-    uint64_t f = range_begin;
-    while (f < range_end) {
-        const Segment sg = locate(p, part, f);
-        const uint32_t pos0 = static_cast<uint32_t>(f - sg.start);
-        const uint64_t left = range_end - f;
-        const uint32_t len = static_cast<uint32_t>(left < sg.len - pos0 ? left : sg.len - pos0);
-        const bool whole = pos0 == 0 && len == sg.len;
-        const uint32_t end = pos0 + len;
+    uint32_t qv[G][4];  // this lane's slice of the G query rows
+    float m[G], l[G], acc[G][8];
+    bool empty = true;  // this lane's key rows have not held a valid key yet
 
-        // this lane's slice of the G query rows
-        uint32_t qv[G][4];
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const uint32_t h = sg.kvh * p.group + p.head0 + g;
-            const Raw16 raw = *reinterpret_cast<const Raw16 *>(
-                Q + ((static_cast<uint64_t>(sg.b) * p.H + h) * p.seq + sg.r) * D + chunk * 8);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) qv[g][e] = raw.w[e];
-        }
-        const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
-
-        float m[G], l[G], acc[G][8];
-        bool empty = true;  // this lane's key rows have not held a valid key yet
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            m[g] = 0.f;
-            l[g] = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-        }
-
-        // Online-softmax update with one step group; keys >= limit are masked out.  The running
-        // reference m[g] is only moved (and the accumulators rescaled) when some score exceeds
-        // it by more than kSlack or a lane meets its first valid key, a rare event after the
-        // first group; otherwise p = exp2(s - m) <= 2^kSlack is accumulated directly.  A lane
-        // that has seen no valid key keeps m = 0 with empty accumulators.
-        auto consume = [&](uint32_t step0, uint32_t limit, const Raw16(&kk)[U], const Raw16(&vv)[U]) {
-            float t[U][G];  // score - reference, log2 units
-            float over = -__builtin_inff();
-            const bool valid0 = step0 + key_in_span < limit;  // keys ascend with u
+    // Online-softmax update with one block; keys >= the end of the piece are masked out.  The
+    // running reference m[g] is only moved (and the accumulators rescaled) when some score
+    // exceeds it by more than kSlack or a lane meets its first valid key, a rare event after the
+    // first block; otherwise p = exp2(s - m) <= 2^kSlack is accumulated directly.  A lane that
+    // has seen no valid key keeps m = 0 with empty accumulators.
+    auto consume = [&](const PieceView &pc, uint32_t key0, const Raw16(&kk)[U], const Raw16(&vv)[U]) {
+        const uint32_t limit = pc.end;
+        // the segment of the last query row writes the new rows it reads into the caches
+        if ((pc.flags & 2) && key0 + BK > pc.base) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const bool valid = step0 + u * KPB + key_in_span < limit;
-#pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    float d = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) d = Elem<T>::dot2(qv[g][e], kk[u].w[e], d);
-                    d = fmaf(row_sum<LPR>(d), p.scale_log2e, -m[g]);
-                    t[u][g] = valid ? d : -__builtin_inff();
-                    over = fmaxf(over, t[u][g]);
+                const uint32_t key = key0 + u * KPW + row;
+                if (key >= pc.base && key < limit) {
+                    const uint64_t coff = (pc.hist_row0 + key) * D + chunk * 8;
+                    *reinterpret_cast<Raw16 *>(Kc + coff) = kk[u];
+                    *reinterpret_cast<Raw16 *>(Vc + coff) = vv[u];
                 }
             }
-            if (__builtin_amdgcn_ballot_w64(over > kSlack || (empty && valid0)) != 0) {
+        }
+        float t[U][G];  // score - reference, log2 units
+        float over = -__builtin_inff();
+        const bool valid0 = key0 + row < limit;  // keys ascend with u
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    // how far the reference moves: to the group maximum at the lane's first valid
-                    // key (the accumulators are still empty), never down afterwards
-                    float up = t[0][g];
-#pragma unroll
-                    for (int u = 1; u < U; ++u) up = fmaxf(up, t[u][g]);
-                    up = empty ? (valid0 ? up : 0.f) : fmaxf(up, 0.f);
-                    const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f(-up);
-                    m[g] += up;
-                    l[g] *= alpha;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
-#pragma unroll
-                    for (int u = 0; u < U; ++u) t[u][g] -= up;
-                }
-                empty = empty && !valid0;
-            }
+        for (int u = 0; u < U; ++u) {
+            const bool valid = key0 + u * KPW + row < limit;
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                float pr[U];
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) d = Elem<T>::dot2(qv[g][e], kk[u].w[e], d);
+                d = fmaf(row_sum<LPR>(d), p.scale_log2e, -m[g]);
+                t[u][g] = valid ? d : -__builtin_inff();
+                over = fmaxf(over, t[u][g]);
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(over > kSlack || (empty && valid0)) != 0) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                // how far the reference moves: to the block maximum at the lane's first valid
+                // key (the accumulators are still empty), never down afterwards
+                float up = t[0][g];
+#pragma unroll
+                for (int u = 1; u < U; ++u) up = fmaxf(up, t[u][g]);
+                up = empty ? (valid0 ? up : 0.f) : fmaxf(up, 0.f);
+                const float alpha = empty ? 1.f : __builtin_amdgcn_exp2f(-up);
+                m[g] += up;
+                l[g] *= alpha;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
+#pragma unroll
+                for (int u = 0; u < U; ++u) t[u][g] -= up;
+            }
+            empty = empty && !valid0;
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float pr[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                pr[u] = __builtin_amdgcn_exp2f(t[u][g]);
+                l[g] += pr[u];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float a0 = acc[g][2 * e], a1 = acc[g][2 * e + 1];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    pr[u] = __builtin_amdgcn_exp2f(t[u][g]);
-                    l[g] += pr[u];
+                    a0 = fmaf(pr[u], Elem<T>::lo(vv[u].w[e]), a0);
+                    a1 = fmaf(pr[u], Elem<T>::hi(vv[u].w[e]), a1);
                 }
+                acc[g][2 * e] = a0;
+                acc[g][2 * e + 1] = a1;
+            }
+        }
+    };
+
+    // Leaves this wavefront's state of piece j in shared memory.  The key rows of the wavefront
+    // are summed with lane swaps that halve the number of values per step (a lane group keeps
+    // the sums it will store and hands the rest over), ending with two output columns per lane.
+    auto flush = [&](uint32_t j) {
+        const uint32_t quarter = lane >> 4;  // 16-lane group
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float a0 = acc[g][2 * e], a1 = acc[g][2 * e + 1];
+        for (int g = 0; g < G; ++g) {
+            float mg = empty ? kMinusBig : m[g];  // lanes without a valid key drop out of the maxima
+            float M = mg;
+            if constexpr (LPR == 8) M = fmaxf(M, dpp_f32<0x128>(M));
+            M = swap_max(M);
+            const float w = __builtin_amdgcn_exp2f(mg - M);
+            float lv = l[g] * w;
+            if constexpr (LPR == 8) lv += dpp_f32<0x128>(lv);
+            lv = swap_sum(lv);
+            float a[8];
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        a0 = fmaf(pr[u], Elem<T>::lo(vv[u].w[e]), a0);
-                        a1 = fmaf(pr[u], Elem<T>::hi(vv[u].w[e]), a1);
+            for (int e = 0; e < 8; ++e) {
+                a[e] = acc[g][e] * w;
+                if constexpr (LPR == 8) a[e] += dpp_f32<0x128>(a[e]);
+            }
+            float s4[4], s2[2];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s4[e] = swap32_sum(a[e], a[e + 4]);  // lanes 32-63 keep columns 4-7
+#pragma unroll
+            for (int e = 0; e < 2; ++e) s2[e] = swap16_sum(s4[e], s4[e + 2]);  // odd 16-lane groups keep +2
+            // this lane now holds columns chunk*8 + 2*quarter + {0, 1} of the wavefront's sum
+            if (LPR == 16 || (lane & 8) == 0) {
+                float *dst = &sh_o[j][wave][g][(lane & (LPR - 1)) * 8 + 2 * quarter];
+                dst[0] = s2[0];
+                dst[1] = s2[1];
+            }
+            if (lane == 0) {
+                sh_m[j][g][wave] = M;
+                sh_l[j][g][wave] = lv;
+            }
+        }
+        if (lane == 0) atomicOr(&sh_has[j], 1u << wave);
+    };
+
+    Segment sg{};  // walked by thread 0 only
+    uint64_t pass_begin = range_begin;
+    while (pass_begin < range_end) {
+        // ---- one thread lays out the next pieces of the range and numbers their blocks
+        if (threadIdx.x == 0) {
+            uint64_t f = pass_begin;
+            uint32_t np = 0, nblk = 0;
+            while (np < kMaxPieces && f < range_end) {
+                if (f == range_begin) {
+                    sg = locate(p, part, f);
+                } else {  // the previous piece ended with its segment: step to the next one
+                    sg.start += sg.len;
+                    if (++sg.kvh == p.Hkv) {
+                        sg.kvh = 0;
+                        if (++sg.r == p.seq) {
+                            sg.r = 0;
+                            sg.base = sh_base[++sg.b];
+                        }
+                        sg.len = sg.base + sg.r + 1;
                     }
-                    acc[g][2 * e] = a0;
-                    acc[g][2 * e + 1] = a1;
+                }
+                PieceRec rc;
+                rc.start = sg.start;
+                rc.b = sg.b; rc.r = sg.r; rc.kvh = sg.kvh; rc.base = sg.base; rc.len = sg.len;
+                rc.pos0 = static_cast<uint32_t>(f - sg.start);
+                const uint64_t left = range_end - f;
+                const uint32_t len = static_cast<uint32_t>(left < sg.len - rc.pos0 ? left : sg.len - rc.pos0);
+                rc.end = rc.pos0 + len;
+                const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
+                rc.hist_row0 = kv_head * p.cap;
+                rc.new_row0 = static_cast<int64_t>(kv_head * p.seq) - static_cast<int64_t>(sg.base);
+                rc.blk0 = nblk;
+                rc.flags = ((rc.pos0 == 0 && len == sg.len) ? 1u : 0u) |
+                           ((p.append && Kc && sg.r + 1 == p.seq) ? 2u : 0u) | (f == range_begin ? 4u : 0u);
+                rc.pad = 0;
+                sh_pc[np] = rc;
+                nblk += (len + BK - 1) / BK;
+                ++np;
+                f += len;
+            }
+            sh_np = np;
+            sh_nblk = nblk;
+            sh_next = 0;
+            sh_f = f;
+        }
+        if (threadIdx.x < kMaxPieces) sh_has[threadIdx.x] = 0;
+        __syncthreads();
+        const uint32_t np = uni(sh_np), nblk = uni(sh_nblk);
+        const uint64_t next_begin = uni(sh_f);
+        const uint32_t c1 = np > 1 ? uni(sh_pc[1].blk0) : 0xffffffffu;
+        const uint32_t c2 = np > 2 ? uni(sh_pc[2].blk0) : 0xffffffffu;
+        const uint32_t c3 = np > 3 ? uni(sh_pc[3].blk0) : 0xffffffffu;
+        auto piece_of = [&](uint32_t blk) -> uint32_t { return (blk >= c1) + (blk >= c2) + (blk >= c3); };
+        auto view = [&](uint32_t j) {
+            PieceView v;
+            const PieceRec &rc = sh_pc[j];
+            v.hist_row0 = uni(rc.hist_row0);
+            v.new_row0 = static_cast<int64_t>(uni(static_cast<uint64_t>(rc.new_row0)));
+            v.base = uni(rc.base);
+            v.pos0 = uni(rc.pos0);
+            v.end = uni(rc.end);
+            v.blk0 = uni(rc.blk0);
+            v.flags = uni(rc.flags);
+            return v;
+        };
+        // Blocks are handed out through a shared counter, so a wavefront that is served faster
+        // simply takes more of them.
+        auto grab = [&]() -> uint32_t {
+            uint32_t v = 0;
+            if (lane == 0) v = atomicAdd(&sh_next, 1u);
+            return uni(v);
+        };
+
+        // Loads one block: keys below the history length come from the caches, later ones from
+        // the k/v inputs.  Unconditional (a block beyond the last re-reads the last one and is
+        // never consumed), clamped to the last key of the piece, streaming.
+        PieceView iss{};
+        uint32_t iss_j = 0xffffffffu;
+        auto issue = [&](uint32_t blk, Raw16(&kk)[U], Raw16(&vv)[U]) {
+            blk = blk < nblk ? blk : nblk - 1;
+            const uint32_t j = piece_of(blk);
+            if (j != iss_j) {
+                iss = view(j);
+                iss_j = j;
+            }
+            const uint32_t key0 = iss.pos0 + (blk - iss.blk0) * BK;
+            if (key0 + BK <= iss.base) {  // history only (wave-uniform): one base address
+                const T *kb = Kc + iss.hist_row0 * D + chunk * 8;
+                const T *vb = Vc + iss.hist_row0 * D + chunk * 8;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t key = key0 + u * KPW + row;
+                    key = key < iss.end ? key : iss.end - 1;
+                    const uint64_t off = static_cast<uint64_t>(key) * D;
+                    kk[u] = load_stream_global(kb + off);
+                    vv[u] = load_stream_global(vb + off);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t key = key0 + u * KPW + row;
+                    key = key < iss.end ? key : iss.end - 1;
+                    const bool hist = key < iss.base;
+                    const int64_t krow = (hist ? static_cast<int64_t>(iss.hist_row0) : iss.new_row0) + key;
+                    const int64_t off = krow * D + chunk * 8;
+                    kk[u] = load_stream_global((hist ? Kc : Kn) + off);
+                    vv[u] = load_stream_global((hist ? Vc : Vn) + off);
                 }
             }
         };
 
-        // ---- history rows [pos0, hist_end): unconditional, clamped, streaming loads from the
-        // caches; two register sets keep the next step group in flight while one is consumed
-        const uint32_t hist_end = end < sg.base ? end : sg.base;
-        if (pos0 < hist_end) {
-            const T *k_hist = Kc + kv_head * p.cap * D + chunk * 8;
-            const T *v_hist = Vc + kv_head * p.cap * D + chunk * 8;
-            auto issue = [&](uint32_t step0, Raw16(&kk)[U], Raw16(&vv)[U]) {
+        Raw16 kbuf[NSET][U], vbuf[NSET][U];
+        uint32_t blk[NSET];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    uint32_t key = step0 + u * KPB + key_in_span;
-                    key = key < hist_end ? key : hist_end - 1;
-                    const uint64_t off = static_cast<uint64_t>(key) * D;
-                    kk[u] = __builtin_bit_cast(
-                        Raw16, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(k_hist + off)));
-                    vv[u] = __builtin_bit_cast(
-                        Raw16, __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(v_hist + off)));
-                }
-            };
-            Raw16 kA[U], vA[U], kB[U], vB[U];
-            issue(pos0, kA, vA);
-            for (uint32_t step0 = pos0; step0 < hist_end; step0 += 2 * SPAN) {
-                if (step0 + SPAN < hist_end) issue(step0 + SPAN, kB, vB);
-                consume(step0, hist_end, kA, vA);
-                if (step0 + SPAN < hist_end) {
-                    if (step0 + 2 * SPAN < hist_end) issue(step0 + 2 * SPAN, kA, vA);
-                    consume(step0 + SPAN, hist_end, kB, vB);
-                }
-            }
+        for (int s = 0; s < NSET; ++s) {
+            blk[s] = grab();
+            issue(blk[s], kbuf[s], vbuf[s]);
         }
-
-        // ---- new rows [max(pos0, base), end): read from the k/v inputs; the segment of the last
-        // query row also writes them into the caches
-        if (end > sg.base) {
-            const T *k_new = Kn + kv_head * p.seq * D + chunk * 8;
-            const T *v_new = Vn + kv_head * p.seq * D + chunk * 8;
-            const bool do_append = p.append && Kc && sg.r + 1 == p.seq;
-            const uint32_t new0 = pos0 > sg.base ? pos0 : sg.base;
-            for (uint32_t step0 = new0; step0 < end; step0 += SPAN) {
-                Raw16 kk[U], vv[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const uint32_t key = step0 + u * KPB + key_in_span;
-                    kk[u] = Raw16{{0, 0, 0, 0}};
-                    vv[u] = Raw16{{0, 0, 0, 0}};
-                    if (key < end) {
-                        const uint64_t off = static_cast<uint64_t>(key - sg.base) * D;
-                        kk[u] = *reinterpret_cast<const Raw16 *>(k_new + off);
-                        vv[u] = *reinterpret_cast<const Raw16 *>(v_new + off);
-                        if (do_append) {
-                            const uint64_t coff = (kv_head * p.cap + key) * D + chunk * 8;
-                            *reinterpret_cast<Raw16 *>(Kc + coff) = kk[u];
-                            *reinterpret_cast<Raw16 *>(Vc + coff) = vv[u];
-                        }
-                    }
-                }
-                consume(step0, end, kk, vv);
-            }
-        }
-
-        // ---- merge the four key rows of each wavefront with shuffles, then the four wavefronts
-        // through LDS; lanes that never held a valid key drop out of the maxima
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            if (empty) m[g] = kMinusBig;
-            float M = fmaxf(m[g], __shfl_xor(m[g], LPR, kWave));
-            if constexpr (KPW >= 4) M = fmaxf(M, __shfl_xor(M, 2 * LPR, kWave));
-            if constexpr (KPW >= 8) M = fmaxf(M, __shfl_xor(M, 4 * LPR, kWave));
-            const float w = __builtin_amdgcn_exp2f(m[g] - M);
-            m[g] = M;
-            float lv = l[g] * w;
-            lv += __shfl_xor(lv, LPR, kWave);
-            if constexpr (KPW >= 4) lv += __shfl_xor(lv, 2 * LPR, kWave);
-            if constexpr (KPW >= 8) lv += __shfl_xor(lv, 4 * LPR, kWave);
-            l[g] = lv;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float a = acc[g][e] * w;
-                a += __shfl_xor(a, LPR, kWave);
-                if constexpr (KPW >= 4) a += __shfl_xor(a, 2 * LPR, kWave);
-                if constexpr (KPW >= 8) a += __shfl_xor(a, 4 * LPR, kWave);
-                acc[g][e] = a;
-            }
-        }
-        __syncthreads();  // the previous piece has finished reading the shared state
-        if (row == 0) {
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sh_o[wave][g][chunk * 8 + e] = acc[g][e];
-                if (chunk == 0) {
-                    sh_m[wave][g] = m[g];
-                    sh_l[wave][g] = l[g];
-                }
-            }
+        // ---- the query rows of the pieces go to shared memory while the first blocks arrive
+        for (uint32_t idx = threadIdx.x; idx < np * G * LPR; idx += kSplitThreads) {
+            const uint32_t j = idx / (G * LPR), g = (idx / LPR) % G, c = idx % LPR;
+            const PieceRec &rc = sh_pc[j];
+            const uint32_t h = rc.kvh * p.group + p.head0 + g;
+            const Raw16 raw = *reinterpret_cast<const Raw16 *>(
+                Q + ((static_cast<uint64_t>(rc.b) * p.H + h) * p.seq + rc.r) * D + c * 8);
+            *reinterpret_cast<Raw16 *>(&sh_q[j][g][c * 4]) = raw;
         }
         __syncthreads();
-        const uint64_t slot = static_cast<uint64_t>(blockIdx.x) * 2 + (f == range_begin ? 0 : 1);
-        float *pslot = p.part + slot * (G * (D + 2));
-        for (uint32_t idx = threadIdx.x; idx < G * D; idx += 256) {
-            const uint32_t g = idx / D, d = idx % D;
-            float M = kMinusBig;
+
+        // ---- each wavefront consumes the blocks it pulled
+        PieceView cur{};
+        uint32_t cur_j = 0xffffffffu;
+        bool live = true;
+        while (live) {
 #pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2) M = fmaxf(M, sh_m[s2][g]);
-            float o_sum = 0.f, l_sum = 0.f;
-#pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2) {
-                const float w = __builtin_amdgcn_exp2f(sh_m[s2][g] - M);
-                o_sum = fmaf(w, sh_o[s2][g][d], o_sum);
-                l_sum = fmaf(w, sh_l[s2][g], l_sum);
-            }
-            if (whole) {
-                const uint32_t h = sg.kvh * p.group + p.head0 + g;
-                T *dst = O + ((static_cast<uint64_t>(sg.b) * p.H + h) * p.seq + sg.r) * D + d;
-                *reinterpret_cast<uint16_t *>(dst) = Elem<T>::pack(o_sum / l_sum);
-            } else {
-                store_coherent(pslot + g * (D + 2) + d, o_sum);
-                if (d == 0) {
-                    store_coherent(pslot + g * (D + 2) + D, M);
-                    store_coherent(pslot + g * (D + 2) + D + 1, l_sum);
+            for (int s = 0; s < NSET; ++s) {
+                if (!live) break;
+                if (blk[s] >= nblk) {
+                    live = false;
+                    break;
                 }
+                const uint32_t j = piece_of(blk[s]);
+                if (j != cur_j) {
+                    if (cur_j != 0xffffffffu) flush(cur_j);
+                    cur = view(j);
+                    cur_j = j;
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const Raw16 raw = *reinterpret_cast<const Raw16 *>(&sh_q[j][g][chunk * 4]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) qv[g][e] = raw.w[e];
+                        m[g] = 0.f;
+                        l[g] = 0.f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+                    }
+                    empty = true;
+                }
+                consume(cur, cur.pos0 + (blk[s] - cur.blk0) * BK, kbuf[s], vbuf[s]);
+                blk[s] = grab();
+                issue(blk[s], kbuf[s], vbuf[s]);
             }
         }
-        if (!whole) {
+        if (cur_j != 0xffffffffu) flush(cur_j);
+        __syncthreads();
+
+        // ---- merge the wavefronts' states of all pieces at once, four output columns per
+        // thread; whole segments give output rows, cut ones leave a partial
+        bool any_cut = false;
+        for (uint32_t j = 0; j < np; ++j) any_cut = any_cut || !(sh_pc[j].flags & 1);
+        for (uint32_t idx = threadIdx.x; idx < np * G * (D / 4); idx += kSplitThreads) {
+            const uint32_t j = idx / (G * (D / 4)), g = (idx / (D / 4)) % G, d = (idx % (D / 4)) * 4;
+            const PieceRec &rc = sh_pc[j];
+            const uint32_t has = sh_has[j];
+            float mw[NW], lw[NW];
+#pragma unroll
+            for (int w4 = 0; w4 < NW; w4 += 4) {
+                const f32x4 mv = *reinterpret_cast<const f32x4 *>(&sh_m[j][g][w4]);
+                const f32x4 lv = *reinterpret_cast<const f32x4 *>(&sh_l[j][g][w4]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool on = (has >> (w4 + i)) & 1;
+                    mw[w4 + i] = on ? mv[i] : kMinusBig;
+                    lw[w4 + i] = on ? lv[i] : 0.f;
+                }
+            }
+            float M = kMinusBig;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) M = fmaxf(M, mw[w]);
+            float o_sum[4] = {0.f, 0.f, 0.f, 0.f}, l_sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const bool on = (has >> w) & 1;
+                const float wgt = on ? __builtin_amdgcn_exp2f(mw[w] - M) : 0.f;
+                const f32x4 ov = *reinterpret_cast<const f32x4 *>(&sh_o[j][w][g][d]);
+                l_sum = fmaf(wgt, lw[w], l_sum);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o_sum[i] = fmaf(wgt, on ? ov[i] : 0.f, o_sum[i]);
+            }
+            if (rc.flags & 1) {
+                const uint32_t h = rc.kvh * p.group + p.head0 + g;
+                T *dst = O + ((static_cast<uint64_t>(rc.b) * p.H + h) * p.seq + rc.r) * D + d;
+                const float inv = 1.f / l_sum;
+                const uint32_t lo = Elem<T>::pack(o_sum[0] * inv) | (static_cast<uint32_t>(Elem<T>::pack(o_sum[1] * inv)) << 16);
+                const uint32_t hi = Elem<T>::pack(o_sum[2] * inv) | (static_cast<uint32_t>(Elem<T>::pack(o_sum[3] * inv)) << 16);
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(lo, hi);
+            } else {
+                const uint64_t slot = static_cast<uint64_t>(blockIdx.x) * 2 + ((rc.flags & 4) ? 0 : 1);
+                float *ps = p.part + slot * (G * (D + 2)) + g * (D + 2);
+                store_coherent2(ps + d, o_sum[0], o_sum[1]);
+                store_coherent2(ps + d + 2, o_sum[2], o_sum[3]);
+                if (d == 0) store_coherent2(ps + D, M, l_sum);
+            }
+        }
+        if (any_cut) {
             // The workgroup that completes a cut segment last merges its partials.  The partials
             // are written through to device-coherent memory and read back past the per-XCD L2
             // (device-scope atomic accesses), so only this wavefront's outstanding stores have to
-            // drain before the ticket is taken; no cache-wide write-back or invalidate is issued.
-            const uint64_t first = sg.start / W, last = (sg.start + sg.len - 1) / W;
+            // drain before the tickets are taken; no cache-wide write-back or invalidate is issued.
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __syncthreads();
-            if (threadIdx.x == 0) {
-                const uint32_t ticket = __hip_atomic_fetch_add(p.counters + first, 1u, __ATOMIC_RELAXED,
-                                                               __HIP_MEMORY_SCOPE_AGENT);
-                const uint32_t is_last = ticket == static_cast<uint32_t>(last - first);
-                if (is_last) p.counters[first] = 0;  // leave the counters as they were found
-                sh_last = is_last;
+            if (threadIdx.x < kMaxPieces) {
+                uint32_t is_last = 0;
+                if (threadIdx.x < np && !(sh_pc[threadIdx.x].flags & 1)) {
+                    const PieceRec &rc = sh_pc[threadIdx.x];
+                    const uint64_t first = udiv(rc.start, W), last = udiv(rc.start + rc.len - 1, W);
+                    const uint32_t ticket = __hip_atomic_fetch_add(p.counters + first, 1u, __ATOMIC_RELAXED,
+                                                                   __HIP_MEMORY_SCOPE_AGENT);
+                    is_last = ticket == static_cast<uint32_t>(last - first);
+                    if (is_last) p.counters[first] = 0;  // leave the counters as they were found
+                }
+                sh_last[threadIdx.x] = is_last;
             }
             __syncthreads();
-            if (sh_last) merge_segment<T, D, G>(p, sg, W, first, last);
+            for (uint32_t j = 0; j < np; ++j) {
+                if (!sh_last[j]) continue;
+                const PieceRec &rc = sh_pc[j];
+                Segment sg;
+                sg.b = rc.b; sg.r = rc.r; sg.kvh = rc.kvh; sg.base = rc.base; sg.len = rc.len; sg.start = rc.start;
+                merge_segment<T, D, G>(p, sg, W, udiv(sg.start, W), udiv(sg.start + sg.len - 1, W));
+            }
         }
-        f += len;
+        pass_begin = next_begin;
+        __syncthreads();  // the tables are rewritten by the next pass
     }
 }
 
@@ -539,9 +758,9 @@ template <class T, int D, int G>
 uint32_t resident_workgroups() {
     static uint32_t cached = [] {
         int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_split<T, D, G>, 256, 0) != hipSuccess ||
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_split<T, D, G>, kSplitThreads, 0) != hipSuccess ||
             per_cu <= 0)
-            per_cu = 2;
+            per_cu = 1;
         return static_cast<uint32_t>(per_cu) * static_cast<uint32_t>(device_info().cus);
     }();
     return cached;
@@ -555,7 +774,7 @@ int launch(AttnParams p, hipStream_t s) {
     uint32_t wgs = resident_workgroups<T, D, G>();
     if (wgs > kMaxWorkgroups) wgs = kMaxWorkgroups;
     p.n_workgroups = wgs;
-    attn_split<T, D, G><<<wgs, 256, 0, s>>>(p);
+    attn_split<T, D, G><<<wgs, kSplitThreads, 0, s>>>(p);
     return launch_status();
 }
 
