@@ -103,6 +103,37 @@ __device__ __forceinline__ uint64_t udiv(uint64_t a, uint64_t b) {
     return a / b;
 }
 
+// The same partition for at most 64 batch rows, built by one wavefront without barriers: a later
+// read of `part` or `*total_out` by this wavefront sees the values (shared memory accesses of a
+// wavefront complete in program order); other wavefronts need a barrier first.
+__device__ void build_partition_wave(const AttnParams &p, Partition part, uint32_t lane, uint64_t *total_out) {
+    uint32_t base = 0;
+    uint64_t mine = 0;
+    if (lane < p.N) {
+        int64_t raw = 0;
+        if (p.kc && p.past) raw = p.past[p.past_per_row ? lane : 0];
+        if (raw < 0) raw = 0;
+        const int64_t room = static_cast<int64_t>(p.cap) - static_cast<int64_t>(p.seq);
+        if (p.kc && raw > room) raw = room < 0 ? 0 : room;
+        base = static_cast<uint32_t>(raw);
+        mine = keys_before_row(p.Hkv, base, p.seq);
+    }
+    uint64_t incl = mine;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const uint64_t up = __shfl_up(incl, d, kWave);
+        if (lane >= static_cast<uint32_t>(d)) incl += up;
+    }
+    if (lane < p.N) {
+        part.base[lane] = base;
+        part.prefix[lane] = incl - mine;
+    }
+    if (lane == kWave - 1) {
+        part.prefix[p.N] = incl;
+        *total_out = incl;
+    }
+}
+
 struct Segment {
     uint32_t b, r, kvh;
     uint32_t base;       // history length of batch row b
@@ -332,14 +363,16 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
     constexpr int KPW = kWave / LPR;    // key rows per wavefront load
     constexpr int U = 4;                // loads per register set
     constexpr uint32_t BK = KPW * U;    // keys per block: the unit a wavefront pulls
-    constexpr int NSET = 2;             // blocks a wavefront keeps in flight
+    constexpr int NSET = 1;             // blocks a wavefront keeps in flight (more did not pay: the
+                                        // other wavefront of the SIMD covers the wait)
     constexpr int NW = kSplitWaves;
 
     __shared__ uint64_t sh_prefix[kMaxBatch + 1];
     __shared__ uint32_t sh_base[kMaxBatch];
     __shared__ PieceRec sh_pc[kMaxPieces];
     __shared__ uint64_t sh_f;
-    __shared__ uint32_t sh_np, sh_nblk, sh_next;
+    __shared__ uint32_t sh_np, sh_nblk;
+    __shared__ unsigned long long sh_taken;  // blocks handed out: from the front (low word), from the back (high word)
     __shared__ uint32_t sh_has[kMaxPieces];  // wavefronts that hold a state of the piece (bit mask)
     __shared__ uint32_t sh_last[kMaxPieces];
     __shared__ alignas(16) uint32_t sh_q[kMaxPieces][G][D / 2];
@@ -347,14 +380,16 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
     __shared__ alignas(16) float sh_m[kMaxPieces][G][NW];
     __shared__ alignas(16) float sh_l[kMaxPieces][G][NW];
 
-    const Partition part{sh_prefix, sh_base};
-    const uint64_t total = build_partition(p, part);
-    const uint64_t W = range_width(total, p.n_workgroups);
-    const uint64_t range_begin = static_cast<uint64_t>(blockIdx.x) * W;
-    if (range_begin >= total) return;
-    const uint64_t range_end = range_begin + W < total ? range_begin + W : total;
+    __shared__ uint64_t sh_total;
 
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const Partition part{sh_prefix, sh_base};
+    if (p.N <= kWave) {
+        if (wave == 0) build_partition_wave(p, part, lane, &sh_total);
+    } else {
+        const uint64_t t = build_partition(p, part);
+        if (threadIdx.x == 0) sh_total = t;
+    }
     const uint32_t row = lane / LPR, chunk = lane % LPR;  // key row within a wavefront load, 16-byte slice
     const T *Q = static_cast<const T *>(p.q);
     const T *Kn = static_cast<const T *>(p.k);
@@ -483,53 +518,66 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
         if (lane == 0) atomicOr(&sh_has[j], 1u << wave);
     };
 
+    // ---- one thread lays out the next pieces of the range and numbers their blocks
     Segment sg{};  // walked by thread 0 only
-    uint64_t pass_begin = range_begin;
-    while (pass_begin < range_end) {
-        // ---- one thread lays out the next pieces of the range and numbers their blocks
-        if (threadIdx.x == 0) {
-            uint64_t f = pass_begin;
-            uint32_t np = 0, nblk = 0;
-            while (np < kMaxPieces && f < range_end) {
-                if (f == range_begin) {
-                    sg = locate(p, part, f);
-                } else {  // the previous piece ended with its segment: step to the next one
-                    sg.start += sg.len;
-                    if (++sg.kvh == p.Hkv) {
-                        sg.kvh = 0;
-                        if (++sg.r == p.seq) {
-                            sg.r = 0;
-                            sg.base = sh_base[++sg.b];
-                        }
-                        sg.len = sg.base + sg.r + 1;
+    auto build_tables = [&](uint64_t pass_begin, uint64_t range_begin, uint64_t range_end) {
+        uint64_t f = pass_begin;
+        uint32_t np = 0, nblk = 0;
+        while (np < kMaxPieces && f < range_end) {
+            if (f == range_begin) {
+                sg = locate(p, part, f);
+            } else {  // the previous piece ended with its segment: step to the next one
+                sg.start += sg.len;
+                if (++sg.kvh == p.Hkv) {
+                    sg.kvh = 0;
+                    if (++sg.r == p.seq) {
+                        sg.r = 0;
+                        sg.base = sh_base[++sg.b];
                     }
+                    sg.len = sg.base + sg.r + 1;
                 }
-                PieceRec rc;
-                rc.start = sg.start;
-                rc.b = sg.b; rc.r = sg.r; rc.kvh = sg.kvh; rc.base = sg.base; rc.len = sg.len;
-                rc.pos0 = static_cast<uint32_t>(f - sg.start);
-                const uint64_t left = range_end - f;
-                const uint32_t len = static_cast<uint32_t>(left < sg.len - rc.pos0 ? left : sg.len - rc.pos0);
-                rc.end = rc.pos0 + len;
-                const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
-                rc.hist_row0 = kv_head * p.cap;
-                rc.new_row0 = static_cast<int64_t>(kv_head * p.seq) - static_cast<int64_t>(sg.base);
-                rc.blk0 = nblk;
-                rc.flags = ((rc.pos0 == 0 && len == sg.len) ? 1u : 0u) |
-                           ((p.append && Kc && sg.r + 1 == p.seq) ? 2u : 0u) | (f == range_begin ? 4u : 0u);
-                rc.pad = 0;
-                sh_pc[np] = rc;
-                nblk += (len + BK - 1) / BK;
-                ++np;
-                f += len;
             }
-            sh_np = np;
-            sh_nblk = nblk;
-            sh_next = 0;
-            sh_f = f;
+            PieceRec rc;
+            rc.start = sg.start;
+            rc.b = sg.b; rc.r = sg.r; rc.kvh = sg.kvh; rc.base = sg.base; rc.len = sg.len;
+            rc.pos0 = static_cast<uint32_t>(f - sg.start);
+            const uint64_t left = range_end - f;
+            const uint32_t len = static_cast<uint32_t>(left < sg.len - rc.pos0 ? left : sg.len - rc.pos0);
+            rc.end = rc.pos0 + len;
+            const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
+            rc.hist_row0 = kv_head * p.cap;
+            rc.new_row0 = static_cast<int64_t>(kv_head * p.seq) - static_cast<int64_t>(sg.base);
+            rc.blk0 = nblk;
+            rc.flags = ((rc.pos0 == 0 && len == sg.len) ? 1u : 0u) |
+                       ((p.append && Kc && sg.r + 1 == p.seq) ? 2u : 0u) | (f == range_begin ? 4u : 0u);
+            rc.pad = 0;
+            sh_pc[np] = rc;
+            nblk += (len + BK - 1) / BK;
+            ++np;
+            f += len;
         }
-        if (threadIdx.x < kMaxPieces) sh_has[threadIdx.x] = 0;
-        __syncthreads();
+        sh_np = np;
+        sh_nblk = nblk;
+        sh_taken = 0;
+        sh_f = f;
+    };
+    // The thread that builds the first tables belongs to the wavefront that built the partition
+    // (or comes after the barriers of the many-row path), so one barrier covers both.
+    if (threadIdx.x == 0) {
+        const uint64_t total0 = sh_total;
+        const uint64_t W0 = range_width(total0, p.n_workgroups);
+        const uint64_t begin0 = static_cast<uint64_t>(blockIdx.x) * W0;
+        if (begin0 < total0) build_tables(begin0, begin0, begin0 + W0 < total0 ? begin0 + W0 : total0);
+    }
+    if (threadIdx.x < kMaxPieces) sh_has[threadIdx.x] = 0;
+    __syncthreads();
+    const uint64_t total = uni(sh_total);
+    const uint64_t W = range_width(total, p.n_workgroups);
+    const uint64_t range_begin = static_cast<uint64_t>(blockIdx.x) * W;
+    if (range_begin >= total) return;
+    const uint64_t range_end = range_begin + W < total ? range_begin + W : total;
+
+    for (;;) {
         const uint32_t np = uni(sh_np), nblk = uni(sh_nblk);
         const uint64_t next_begin = uni(sh_f);
         const uint32_t c1 = np > 1 ? uni(sh_pc[1].blk0) : 0xffffffffu;
@@ -549,11 +597,17 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
             return v;
         };
         // Blocks are handed out through a shared counter, so a wavefront that is served faster
-        // simply takes more of them.
+        // simply takes more of them.  Half of the wavefronts take blocks from the front of the
+        // list, the others from its back: most of them then stay inside one piece and never
+        // have to set a state aside to start another.
+        constexpr uint32_t kNoBlock = 0xffffffffu;
         auto grab = [&]() -> uint32_t {
-            uint32_t v = 0;
-            if (lane == 0) v = atomicAdd(&sh_next, 1u);
-            return uni(v);
+            const bool from_back = wave >= NW / 2;
+            unsigned long long old = 0;
+            if (lane == 0) old = atomicAdd(&sh_taken, from_back ? (1ull << 32) : 1ull);
+            const uint32_t front = uni(static_cast<uint32_t>(old)), back = uni(static_cast<uint32_t>(old >> 32));
+            if (front + back >= nblk) return kNoBlock;
+            return from_back ? nblk - 1 - back : front;
         };
 
         // Loads one block: keys below the history length come from the caches, later ones from
@@ -725,8 +779,11 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
                 merge_segment<T, D, G>(p, sg, W, udiv(sg.start, W), udiv(sg.start + sg.len - 1, W));
             }
         }
-        pass_begin = next_begin;
-        __syncthreads();  // the tables are rewritten by the next pass
+        if (next_begin >= range_end) break;
+        __syncthreads();  // the tables are rewritten for the next pass
+        if (threadIdx.x == 0) build_tables(next_begin, range_begin, range_end);
+        if (threadIdx.x < kMaxPieces) sh_has[threadIdx.x] = 0;
+        __syncthreads();
     }
 }
 
