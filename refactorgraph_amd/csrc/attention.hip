@@ -52,9 +52,15 @@ struct Partition {
     uint32_t *base;     // [N] clamped history length of batch row b
 };
 
+// Every segment is laid out with kPiecePad positions that hold no key in front of its keys.  A
+// range of the laid-out space is a share of the work, and starting a segment costs a workgroup
+// about as much as streaming that many keys (query rows, a state to merge, a partial to write).
+constexpr uint32_t kPiecePad = 128;
+
 __device__ __forceinline__ uint64_t keys_before_row(uint32_t Hkv, uint32_t base, uint32_t r) {
-    // Hkv * sum_{i<r} (base + i + 1)
-    return static_cast<uint64_t>(Hkv) * (static_cast<uint64_t>(r) * (base + 1) + static_cast<uint64_t>(r) * (r - 1) / 2);
+    // Hkv * sum_{i<r} (base + i + 1 + kPiecePad)
+    return static_cast<uint64_t>(Hkv) *
+           (static_cast<uint64_t>(r) * (base + 1 + kPiecePad) + static_cast<uint64_t>(r) * (r - 1) / 2);
 }
 
 // Fills `part` (shared memory) and returns the total key count.  Called by every thread.
@@ -138,7 +144,7 @@ struct Segment {
     uint32_t b, r, kvh;
     uint32_t base;       // history length of batch row b
     uint32_t len;        // keys of this segment = base + r + 1
-    uint64_t start;      // position of key 0 of the segment in the laid-out key space
+    uint64_t start;      // position of the segment (its padding first) in the laid-out space
 };
 
 // Segment containing laid-out key f.
@@ -162,9 +168,10 @@ __device__ Segment locate(const AttnParams &p, const Partition &part, uint64_t f
     }
     s.r = rlo;
     s.len = s.base + s.r + 1;
+    const uint32_t span = s.len + kPiecePad;
     const uint64_t u2 = u - keys_before_row(p.Hkv, s.base, s.r);
-    s.kvh = static_cast<uint32_t>(udiv(u2, s.len));
-    s.start = part.prefix[lo] + keys_before_row(p.Hkv, s.base, s.r) + static_cast<uint64_t>(s.kvh) * s.len;
+    s.kvh = static_cast<uint32_t>(udiv(u2, span));
+    s.start = part.prefix[lo] + keys_before_row(p.Hkv, s.base, s.r) + static_cast<uint64_t>(s.kvh) * span;
     return s;
 }
 
@@ -335,13 +342,13 @@ constexpr int kMaxPieces = 4;                        // pieces of a range handle
 
 // One piece = the part of a segment that falls into a workgroup's range.
 struct PieceRec {
-    uint64_t start;      // position of key 0 of the segment in the laid-out key space
+    uint64_t start;      // position of key 0 of the segment in the laid-out space
     uint64_t hist_row0;  // cache row of key 0 of the kv head
     int64_t new_row0;    // input row that key 0 would have (key `base` is the first real one)
     uint32_t b, r, kvh, base, len;  // the segment
     uint32_t pos0, end;  // keys [pos0, end) of the segment
     uint32_t blk0;       // first block of the piece within the pass
-    uint32_t flags;      // 1: the whole segment, 2: appends the new rows, 4: starts the range
+    uint32_t flags;      // 1: the whole segment, 2: appends the new rows, 4: begins where the range does
     uint32_t pad;
 };
 
@@ -527,7 +534,7 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
             if (f == range_begin) {
                 sg = locate(p, part, f);
             } else {  // the previous piece ended with its segment: step to the next one
-                sg.start += sg.len;
+                sg.start += sg.len + kPiecePad;
                 if (++sg.kvh == p.Hkv) {
                     sg.kvh = 0;
                     if (++sg.r == p.seq) {
@@ -537,24 +544,31 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
                     sg.len = sg.base + sg.r + 1;
                 }
             }
-            PieceRec rc;
-            rc.start = sg.start;
-            rc.b = sg.b; rc.r = sg.r; rc.kvh = sg.kvh; rc.base = sg.base; rc.len = sg.len;
-            rc.pos0 = static_cast<uint32_t>(f - sg.start);
+            // positions [at, at + width) of the padded segment are in the range; the keys among them
+            const uint32_t at = static_cast<uint32_t>(f - sg.start);
             const uint64_t left = range_end - f;
-            const uint32_t len = static_cast<uint32_t>(left < sg.len - rc.pos0 ? left : sg.len - rc.pos0);
-            rc.end = rc.pos0 + len;
+            const uint32_t span = sg.len + kPiecePad;
+            const uint32_t width = static_cast<uint32_t>(left < span - at ? left : span - at);
+            const uint32_t pos0 = at > kPiecePad ? at - kPiecePad : 0;
+            const uint32_t end = at + width > kPiecePad ? at + width - kPiecePad : 0;
+            f += width;
+            if (end <= pos0) continue;  // padding only
+            PieceRec rc;
+            rc.start = sg.start + kPiecePad;
+            rc.b = sg.b; rc.r = sg.r; rc.kvh = sg.kvh; rc.base = sg.base; rc.len = sg.len;
+            rc.pos0 = pos0;
+            rc.end = end;
             const uint64_t kv_head = static_cast<uint64_t>(sg.b) * p.Hkv + sg.kvh;
             rc.hist_row0 = kv_head * p.cap;
             rc.new_row0 = static_cast<int64_t>(kv_head * p.seq) - static_cast<int64_t>(sg.base);
             rc.blk0 = nblk;
-            rc.flags = ((rc.pos0 == 0 && len == sg.len) ? 1u : 0u) |
-                       ((p.append && Kc && sg.r + 1 == p.seq) ? 2u : 0u) | (f == range_begin ? 4u : 0u);
+            rc.flags = ((pos0 == 0 && end == sg.len) ? 1u : 0u) |
+                       ((p.append && Kc && sg.r + 1 == p.seq) ? 2u : 0u) |
+                       (rc.start + pos0 == range_begin ? 4u : 0u);
             rc.pad = 0;
             sh_pc[np] = rc;
-            nblk += (len + BK - 1) / BK;
+            nblk += (end - pos0 + BK - 1) / BK;
             ++np;
-            f += len;
         }
         sh_np = np;
         sh_nblk = nblk;
@@ -580,6 +594,8 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
     for (;;) {
         const uint32_t np = uni(sh_np), nblk = uni(sh_nblk);
         const uint64_t next_begin = uni(sh_f);
+        // a range that only holds padding has nothing to stream
+        if (np > 0) [&]() {
         const uint32_t c1 = np > 1 ? uni(sh_pc[1].blk0) : 0xffffffffu;
         const uint32_t c2 = np > 2 ? uni(sh_pc[2].blk0) : 0xffffffffu;
         const uint32_t c3 = np > 3 ? uni(sh_pc[3].blk0) : 0xffffffffu;
@@ -779,6 +795,7 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
                 merge_segment<T, D, G>(p, sg, W, udiv(sg.start, W), udiv(sg.start + sg.len - 1, W));
             }
         }
+        }();
         if (next_begin >= range_end) break;
         __syncthreads();  // the tables are rewritten for the next pass
         if (threadIdx.x == 0) build_tables(next_begin, range_begin, range_end);
