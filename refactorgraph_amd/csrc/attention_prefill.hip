@@ -9,7 +9,7 @@
 // four query heads.  Keys are walked 64 at a time.  Both products run on the fp16/bf16 MFMA
 // (v_mfma_f32_32x32x16) in transposed form:
 //     S^T[key, q] = K[key, :] . Q[q, :]       A = K rows (LDS, 128-bit reads), B = Q rows (registers)
-//     O^T[d, q]  += V^T[d, key] . P^T[key, q] A = V columns (LDS, 16-bit gathers), B = P (registers)
+//     O^T[d, q]  += V^T[d, key] . P^T[key, q] A = V columns (LDS, transposing 64-bit reads), B = P (registers)
 // In this form a lane holds one query row of S^T / O^T in its accumulator registers, so the
 // softmax row statistics need no cross-lane reduction beyond one exchange between the two
 // half-wavefronts, and P^T is already in B-operand position.  Softmax is online in float with
@@ -26,15 +26,29 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int D = 128;
 constexpr int BN = 64;                 // keys per tile
-constexpr int ROW = 2 * D + 16;        // LDS pitch of a key row, bytes (272: conflict-free fragment reads)
+constexpr int ROW = 2 * D + 16;        // LDS pitch of a K row, bytes (272: conflict-free fragment reads)
+constexpr int VROW = 2 * D + 64;       // LDS pitch of a V row: four rows of 64 bytes cover all banks
 constexpr int TILE = BN * ROW;         // 17408
-constexpr int LDS_BYTES = 2 * TILE;    // K tile + V tile; reused for the output transposition
+constexpr int VTILE = BN * VROW;       // 20480
+constexpr int BUF_BYTES = TILE + VTILE;  // K tile + V tile
+constexpr int LDS_BYTES = 2 * BUF_BYTES;  // double buffered; reused for the output transposition
 constexpr float kSlack = 6.0f;
 constexpr float kMinusBig = -1e30f;
 
 struct alignas(16) Raw16 {
     uint32_t w[4];
 };
+
+struct U2 {
+    uint32_t w[2];
+};
+// 64-bit LDS read that transposes 16-bit elements inside each group of 16 lanes: lane i of a group
+// receives element i % 4 of what lanes i / 4, i / 4 + 4, i / 4 + 8 and i / 4 + 12 address.
+typedef short s4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ U2 read_tr16(const uint8_t *p) {
+    const s4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *)(p));
+    return __builtin_bit_cast(U2, v);
+}
 
 template <class T> struct Ops;
 template <> struct Ops<__half> {
@@ -61,12 +75,11 @@ template <> struct Ops<__hip_bfloat16> {
 // HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
 // query sub-tiles of the same heads.
 template <class T, int HW>
-__global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_t group,
+__global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint32_t group,
                                                     uint32_t q_tiles, uint32_t head_chunks) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
     constexpr int ROWS = 32 * QS;   // query rows per workgroup
     __shared__ __align__(16) uint8_t lds[LDS_BYTES];
-    uint8_t *ldsK = lds, *ldsV = lds + TILE;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t half = lane >> 5, l32 = lane & 31;
@@ -154,12 +167,13 @@ __global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_
             }
         }
     };
-    auto stage = [&](const Raw16(&kr)[4], const Raw16(&vr)[4]) {
+    auto stage = [&](uint32_t buf, const Raw16(&kr)[4], const Raw16(&vr)[4]) {
+        uint8_t *ldsK = lds + buf * BUF_BYTES, *ldsV = ldsK + TILE;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t off = (st_row + 16 * i) * ROW + st_chunk * 16;
             *reinterpret_cast<Raw16 *>(ldsK + off) = kr[i];
-            *reinterpret_cast<Raw16 *>(ldsV + off) = vr[i];
+            *reinterpret_cast<Raw16 *>(ldsV + (st_row + 16 * i) * VROW + st_chunk * 16) = vr[i];
         }
     };
 
@@ -173,12 +187,13 @@ __global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_
 
     Raw16 kr[4], vr[4];
     fetch(0, kr, vr);
-    stage(kr, vr);
+    stage(0, kr, vr);
     __syncthreads();
 
     for (uint32_t kt = 0; kt < n_tiles; ++kt) {
         if (kt + 1 < n_tiles) fetch(kt + 1, kr, vr);
 
+        const uint8_t *ldsK = lds + (kt & 1) * BUF_BYTES, *ldsV = ldsK + TILE;
         if (kt < wave_tiles) {
             // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32
             f16v s[2];
@@ -195,18 +210,26 @@ __global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_
             // scale, causal mask (only tiles that reach past the wavefront's first query position)
             const bool need_mask = kt * BN + BN - 1 > base + r0;
             float over = -__builtin_inff();
+            if (need_mask) {  // wave-uniform: only the tiles on the diagonal pay for the comparisons
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float t = fmaf(s[kb][e], c_log2e, -m);
-                    if (need_mask) {
+                    for (int e = 0; e < 16; ++e) {
                         const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
-                        t = key > qpos ? -__builtin_inff() : t;
+                        const float t = key > qpos ? -__builtin_inff() : fmaf(s[kb][e], c_log2e, -m);
+                        s[kb][e] = t;
+                        over = fmaxf(over, t);
                     }
-                    s[kb][e] = t;
-                    over = fmaxf(over, t);
-                }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float t = fmaf(s[kb][e], c_log2e, -m);
+                        s[kb][e] = t;
+                        over = fmaxf(over, t);
+                    }
+            }
             over = fmaxf(over, __shfl_xor(over, 32, kWave));  // both halves hold the same query row
             if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
                 const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
@@ -237,32 +260,27 @@ __global__ __launch_bounds__(256) void attn_prefill(const PrefillArgs a, uint32_
                         pf[kb][jj].w[i2] = Ops<T>::pack2(p0, p1);
                     }
             // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
-            // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf
-            const uint16_t *v16 = reinterpret_cast<const uint16_t *>(ldsV);
+            // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
+            // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
+            // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
+            const uint32_t tr_off = (4 * half + (lane & 15) / 4) * VROW + 2 * (16 * ((lane >> 4) & 1) + 4 * (lane & 3));
 #pragma unroll
             for (int db = 0; db < 4; ++db)
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
-                        Raw16 vf;
-#pragma unroll
-                        for (int i2 = 0; i2 < 4; ++i2) {
-                            const int i = 2 * i2;
-                            const uint32_t key0 = 32 * kb + 16 * jj + (i < 4 ? 4 * half + i : 8 + 4 * half + i - 4);
-                            const uint32_t lo = v16[key0 * (ROW / 2) + 32 * db + l32];
-                            const uint32_t hi = v16[(key0 + 1) * (ROW / 2) + 32 * db + l32];
-                            vf.w[i2] = lo | (hi << 16);
-                        }
+                        const uint8_t *vp = ldsV + (32 * kb + 16 * jj) * VROW + 64 * db + tr_off;
+                        const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * VROW);
+                        const Raw16 vf{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
                         o[db] = Ops<T>::mfma(vf, pf[kb][jj], o[db]);
                     }
         }
 
-        __syncthreads();  // every wavefront is done with this tile
-        if (kt + 1 < n_tiles) {
-            stage(kr, vr);
-            __syncthreads();
-        }
+        // the other buffer was last read in the previous iteration, which every wavefront left
+        // through the barrier below
+        if (kt + 1 < n_tiles) stage((kt + 1) & 1, kr, vr);
+        __syncthreads();
     }
 
     // ---- normalise, transpose O^T -> O through LDS, 128-bit row-contiguous stores
