@@ -119,17 +119,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     const bool wave_active = r0 < a.seq;
     const uint32_t wg_rows_end = (qt + 1) * ROWS < a.seq ? (qt + 1) * ROWS : a.seq;
 
-    // append the new rows this workgroup's query rows correspond to (once per kv head)
-    if (Kc && hc == 0) {
-        for (uint32_t idx = tid; idx < (wg_rows_end - qt * ROWS) * 16; idx += 256) {
-            const uint32_t rr = qt * ROWS + idx / 16, c = idx % 16;
-            const uint64_t src = static_cast<uint64_t>(rr) * D + c * 8;
-            const uint64_t dst = (kv_head * a.cap + base + rr) * D + c * 8;
-            *reinterpret_cast<Raw16 *>(Kc + dst) = *reinterpret_cast<const Raw16 *>(k_new + src);
-            *reinterpret_cast<Raw16 *>(Vc + dst) = *reinterpret_cast<const Raw16 *>(v_new + src);
-        }
-    }
-
     // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
     Raw16 qf[8];
     {
@@ -305,6 +294,18 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             if (r0 + row < a.seq)
                 *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
                     *reinterpret_cast<const Raw16 *>(ldsO + row * ROW + c * 16);
+        }
+    }
+
+    // append the new rows this workgroup's query rows correspond to (once per kv head); nothing
+    // in this workgroup waits for the copy
+    if (Kc && hc == 0) {
+        for (uint32_t idx = tid; idx < (wg_rows_end - qt * ROWS) * 16; idx += 256) {
+            const uint32_t rr = qt * ROWS + idx / 16, c = idx % 16;
+            const uint64_t src = static_cast<uint64_t>(rr) * D + c * 8;
+            const uint64_t dst = (kv_head * a.cap + base + rr) * D + c * 8;
+            *reinterpret_cast<Raw16 *>(Kc + dst) = *reinterpret_cast<const Raw16 *>(k_new + src);
+            *reinterpret_cast<Raw16 *>(Vc + dst) = *reinterpret_cast<const Raw16 *>(v_new + src);
         }
     }
 }
