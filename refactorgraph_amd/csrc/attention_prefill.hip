@@ -84,10 +84,20 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t half = lane >> 5, l32 = lane & 31;
 
-    // heaviest query tiles (longest key range) first
+    // Workgroup order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so every
+    // XCD is given whole (batch row, kv head, head chunk) streams, one after the other and the
+    // heaviest query tile (longest key range) of each first.  The query tiles of a stream then
+    // run close together on one XCD and find the K/V rows they share in its L2.
     const uint32_t n_rest = a.N * a.Hkv * head_chunks;
-    const uint32_t qt = q_tiles - 1 - blockIdx.x / n_rest;
-    uint32_t rest = blockIdx.x % n_rest;
+    uint32_t rest, qt;
+    if (n_rest % 8 == 0) {
+        const uint32_t xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+        rest = (slot / q_tiles) * 8 + xcd;
+        qt = q_tiles - 1 - slot % q_tiles;
+    } else {
+        rest = blockIdx.x / q_tiles;
+        qt = q_tiles - 1 - blockIdx.x % q_tiles;
+    }
     const uint32_t hc = rest % head_chunks;
     rest /= head_chunks;
     const uint32_t kvh = rest % a.Hkv, b = rest / a.Hkv;
