@@ -35,13 +35,14 @@ FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 MFMA, published
 # properties of the kernels at these shapes, not of a particular run; the counter summaries are
 # kept in profiles/.
 MEASURED_TRAFFIC = {
-    "decode": (2 * 172652 + 2271) * 1024,
+    "decode": (2 * 172515 + 2309) * 1024,
     "rms_norm": (2 * 32867 + 65619) * 1024,
     "softmax": (2 * 1048617 + 2097156) * 1024,
     "softmax_causal": (2 * 540713 + 2097158) * 1024,
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
     "matmul_integer": (2 * 52558 + 71295) * 1024,
+    "attention_prefill": (2 * 99826 + 196608) * 1024,
 }
 
 
@@ -290,7 +291,7 @@ def main():
             torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp,
                                                    sync_state=state),
             max(steps // 40, 3), max(warmup // 80, 2), 1)
-        e = hbm_entry(402653184, dms)
+        e = hbm_entry(402653184, dms, "attention_prefill")
         flops = 68853694464
         e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=128",
                  device_ms_per_launch=round(dms, 5), timing=mode,
