@@ -331,6 +331,18 @@ def test_attention_decode_and_small_prefill(N, H, Hkv, seq, cap, D, past):
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)  # appended rows, rest untouched
 
 
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,dt", [
+    (16, 8, 8, 8, 32, 64, torch.float16),     # many short segments: several pieces per range, several passes
+    (70, 4, 2, 1, 96, 128, torch.float16),    # more than 64 batch rows: the partition is built by the whole workgroup
+    (24, 12, 4, 3, 40, 128, torch.bfloat16),  # group of 3 heads (two launches), short segments, bf16
+])
+def test_attention_split_many_segments(N, H, Hkv, seq, cap, D, dt):
+    past = np.random.default_rng(21).integers(0, cap - seq + 1, N)
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt, seed=22)
+    assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
 def test_attention_scalar_past_no_cache_and_bf16():
     o, ref_o, kc, ref_kc, _, _ = _attention_case(2, 8, 2, 1, 200, 128, [77])
     assert np.max(np.abs(o - ref_o)) <= ABS_F16 and np.array_equal(kc, ref_kc)
