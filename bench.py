@@ -252,6 +252,30 @@ def main():
         ops_out["dequantize_linear"] = e
         del xs, ys
 
+    if want("dynamic_quantize_linear"):
+        # producer of MatMulInteger's A operand; rotate inputs so that the first pass (min/max)
+        # streams from HBM; the second pass re-reads the 67 MB it has just seen
+        nb = 8
+        xs = [torch.randn((4096, 4096), device=dev) for _ in range(nb)]
+        ys = [torch.empty((4096, 4096), device=dev, dtype=torch.uint8) for _ in range(nb)]
+        wsq = torch.empty(ops.lib().rg_hip_dynamic_quantize_linear_workspace(4096 * 4096), dtype=torch.uint8, device=dev)
+        wall, dms, mode = time_steps(
+            torch, lambda i: ops.dynamic_quantize_linear(xs[i], out=ys[i], workspace=wsq), steps, warmup, nb)
+        e = hbm_entry(4096 * 4096 * 5 + 5, dms, "dynamic_quantize_linear")
+        e.update(workload="DynamicQuantizeLinear f32->u8 [4096,4096] (two launches: min/max, quantize); "
+                          "algorithmic bytes count x once",
+                 device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn = xs[0].cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.dynamic_quantize_linear(xn)
+            dt = time.perf_counter() - t0
+            e["cpu_baseline"] = {"value": round(4096 * 4096 * 5 / dt / 1e9, 3), "unit": "GB/s", "cores": 1,
+                                 "kind": "port", "sample": f"the whole [4096,4096] tensor once ({dt:.2f} s)"}
+        ops_out["dynamic_quantize_linear"] = e
+        del xs, ys
+
     if want("matmul_integer"):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)

@@ -98,6 +98,19 @@ int rg_hip_dequantize_linear(float *y, const void *x, const float *scale, const 
                              size_t outer, size_t axis_len, size_t inner,
                              int in_dtype, int per_axis, void *stream);
 
+/* ---- DynamicQuantizeLinear -------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/dynamic_quantize_linear/cuda_kernel.cu:48-136 (Thrust map +
+ * cub::DeviceReduce + quantize kernel); arithmetic contract
+ * src/04kernel/src/kernels/dynamic_quantize_linear/cpu_kernel.cc:25-70 (float in, uint8 out):
+ * len = max(0, max x) - min(0, min x); scale = len / 255; zp = saturate(0 - min x * 255 / len);
+ * y = saturate(round(x / scale) + zp).  Bit-identical to the CPU kernel, including its running
+ * maximum that starts at FLT_MIN (an all-zero input gives scale FLT_MIN / 255, zp 0, y 0).
+ * Outputs in operator order: y [size] uint8, scale [1] float, zero_point [1] uint8.
+ * workspace: rg_hip_dynamic_quantize_linear_workspace(size) bytes, 4-byte aligned. */
+size_t rg_hip_dynamic_quantize_linear_workspace(size_t size);
+int rg_hip_dynamic_quantize_linear(uint8_t *y, float *scale, uint8_t *zero_point, const float *x,
+                                   size_t size, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- MatMulInteger -----------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust
  * zero-point pre-pass + cublasGemmEx); arithmetic contract

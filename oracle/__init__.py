@@ -48,6 +48,8 @@ def lib() -> C.CDLL:
                                             sz, sz, sz, sz, vp, vp, sz, sz, i32]
         L.oracle_dequantize_linear.argtypes = [vp, vp, vp, vp, sz, sz, sz, i32, sz, i32]
         L.oracle_dequantize_linear.restype = i32
+        L.oracle_dynamic_quantize_linear.argtypes = [vp, vp, vp, vp, sz]
+        L.oracle_dynamic_quantize_linear.restype = None
         L.oracle_matmul_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, f32]
         L.oracle_mul_f32.argtypes = [vp, vp, vp, sz, sz]
         L.oracle_attention_head_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, f32, i32, vp]
@@ -172,6 +174,16 @@ def dequantize_linear(x, scale, zp=None, axis=1, threads=1):
                                         code, scale.size, threads)
     assert rc == 0
     return y
+
+
+def dynamic_quantize_linear(x):
+    """float32 tensor -> (uint8 tensor, float32 scale, uint8 zero point)."""
+    x = _c(x, np.float32)
+    y = np.empty(x.shape, dtype=np.uint8)
+    scale = np.empty(1, dtype=np.float32)
+    zp = np.empty(1, dtype=np.uint8)
+    lib().oracle_dynamic_quantize_linear(_p(y), _p(scale), _p(zp), _p(x), x.size)
+    return y, scale[0], zp[0]
 
 
 def matmul_f32(a, b, trans_b=False, alpha=1.0):

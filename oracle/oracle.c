@@ -4,6 +4,7 @@
  */
 #include "oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <pthread.h>
 #include <stdlib.h>
@@ -309,6 +310,38 @@ int oracle_dequantize_linear(float *y, const void *x, const float *scale, const 
     struct dq_ctx c = {y, x, zp, scale, axis_len, inner, scale_count, in_dtype};
     for_spans(outer * axis_len * inner, threads, dq_span, &c);
     return 0;
+}
+
+/* ------------------------------------------------------- dynamic quantize linear */
+
+/* saturate<uint8_t>: src/04kernel/src/kernels/dynamic_quantize_linear/cpu_kernel.cc:25-31 */
+static uint8_t dql_saturate(float v) {
+    v = v < 0.0f ? 0.0f : v;       /* std::clamp(x, QMIN, QMAX) */
+    v = 255.0f < v ? 255.0f : v;
+    return (uint8_t) roundf(v);    /* std::round: half away from zero */
+}
+
+void oracle_dynamic_quantize_linear(uint8_t *y, float *scale_out, uint8_t *zp_out,
+                                    const float *x, size_t n) {
+    /* cpu_kernel.cc:38-57: the accumulation starts from {max float, min positive float} */
+    float mn = FLT_MAX, mx = FLT_MIN;
+    for (size_t i = 0; i < n; ++i) {
+        mn = x[i] < mn ? x[i] : mn;   /* std::min(min, it) */
+        mx = mx < x[i] ? x[i] : mx;   /* std::max(max, it) */
+    }
+    /* cpu_kernel.cc:58-60 */
+    const float len = (0.0f < mx ? mx : 0.0f) - (mn < 0.0f ? mn : 0.0f);
+    const float scale = len / 255.0f;
+    *scale_out = scale;
+    if (!(len > 0.0f)) { /* cannot happen for finite input (mx >= FLT_MIN); NaN-only input */
+        *zp_out = 0;
+        memset(y, 0, n);
+        return;
+    }
+    const uint8_t zp = dql_saturate(0.0f - mn * 255.0f / len);
+    *zp_out = zp;
+    /* cpu_kernel.cc:62-66 */
+    for (size_t i = 0; i < n; ++i) y[i] = dql_saturate(roundf(x[i] / scale) + (float) zp);
 }
 
 /* ------------------------------------------------------- float matmul + mul */

@@ -19,6 +19,10 @@
  *   oracle_dequantize_linear   src/04kernel/src/kernels/dequantize_linear/cpu_kernel.cc:40-74
  *                              (scalar scale = the reference path; per-axis scale is this
  *                              build's extension with the same one-subtract-one-multiply form)
+ *   oracle_dynamic_quantize_linear
+ *                              src/04kernel/src/kernels/dynamic_quantize_linear/cpu_kernel.cc:25-70
+ *                              (the running maximum starts at FLT_MIN as in the reference, so an
+ *                              all-zero input gives scale FLT_MIN / 255, zero point 0, y 0)
  *   oracle_matmul_f32          src/04kernel/src/kernels/mat_mul/cpu_kernel.cc:28-68
  *                              + mat_mul_common/cpu_template.hpp:18-30 (beta == 0: y ignored)
  *   oracle_mul_f32             src/04kernel/src/kernels/simple_binary/cpu_kernel.cc:33-48,90
@@ -94,6 +98,11 @@ void oracle_matmul_integer(int32_t *y, const void *a, const void *b,
 int oracle_dequantize_linear(float *y, const void *x, const float *scale, const void *zp,
                              size_t outer, size_t axis_len, size_t inner,
                              int in_dtype, size_t scale_count, int threads);
+
+/* y = saturate(round(x / scale) + zp) with scale = (max(0, max x) - min(0, min x)) / 255 and
+ * zp = saturate(0 - min x * 255 / len), all in float; outputs in operator order. */
+void oracle_dynamic_quantize_linear(uint8_t *y, float *scale_out, uint8_t *zp_out,
+                                    const float *x, size_t n);
 
 /* y[M,N] = alpha * sum_k a[i*sa0 + k*sa1] * b[k*sb0 + j*sb1], serial k order, float accumulate. */
 void oracle_matmul_f32(float *y, const float *a, const float *b,

@@ -36,6 +36,14 @@ namespace refactor::kernel {
         std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
     };
 
+    // inputs: x float; outputs: y uint8 like x, scale float [], zero point uint8 []
+    // (src/04kernel/include/kernel/collectors/dynamic_quantize_linear.h:8-15)
+    struct DynamicQuantizeLinearCollector final : public InfoCollector {
+        constexpr explicit DynamicQuantizeLinearCollector(hardware::Device::Type target) noexcept
+            : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
     // inputs: query, key, value [, past_seq_len [, k_cache, v_cache]]; outputs: output
     // [, k_cache, v_cache] (src/08-01llm/README.md:29-63).
     struct AttentionCollector final : public InfoCollector {

@@ -58,6 +58,19 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // mirrors DynamicQuantizeLinearCuda
+    // (src/04kernel/src/kernels/dynamic_quantize_linear/cuda_kernel.hh:8-21): float -> uint8
+    struct DynamicQuantizeLinearHip final : public Kernel {
+        size_t size;
+
+        explicit DynamicQuantizeLinearHip(decltype(size)) noexcept;
+        static KernelBox build(decltype(size)) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct AttentionHip final : public Kernel {
         // the reference's parameter block (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-14)
         // plus what it leaves to the run time: where past_seq_len comes from

@@ -82,6 +82,28 @@ namespace refactor::kernel {
     }
 
     std::vector<KernelBox>
+    DynamicQuantizeLinearCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
+        // src/04kernel/src/collectors/dynamic_quantize_linear.cc:12-33; the reference's kernels
+        // take float input and produce uint8 only, which is checked here instead of assumed
+        auto const &x = inputs[0].get();
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                if (x.dataType == DataType::F32 && outputs.size() == 3 &&
+                    outputs[0].get().dataType == DataType::U8 && outputs[1].get().dataType == DataType::F32 &&
+                    outputs[2].get().dataType == DataType::U8) {
+                    ADD(DynamicQuantizeLinearHip::build(x.elementsSize()))
+                }
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
     AttentionCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
         auto const &query = inputs[0].get();
         auto const &key = inputs[1].get();

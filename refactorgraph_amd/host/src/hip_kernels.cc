@@ -144,6 +144,29 @@ namespace refactor::kernel {
         };
     }
 
+    // ------------------------------------------------------------------ DynamicQuantizeLinear
+
+    using DQL = DynamicQuantizeLinearHip;
+    DQL::DynamicQuantizeLinearHip(decltype(size) size_) noexcept : Kernel(), size(size_) {}
+    KernelBox DQL::build(decltype(size) size) noexcept {
+        return size > 0 ? std::make_unique<DQL>(size) : nullptr;
+    }
+    size_t DQL::typeId() noexcept { return idOf<DQL>(); }
+    size_t DQL::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view DQL::description() const noexcept { return "Performing dynamic quantize linear on AMD gfx950"; }
+    RoutineWorkspace DQL::lower(Resources &) const {
+        auto const workspace = rg_hip_dynamic_quantize_linear_workspace(size);
+        auto routine = [size = size, workspace](Resources &, void *workspacePtr, void const *const *inputs,
+                                                void *const *outputs) {
+            HIP_CALL(rg_hip_dynamic_quantize_linear(static_cast<uint8_t *>(outputs[0]),
+                                                    static_cast<float *>(outputs[1]),
+                                                    static_cast<uint8_t *>(outputs[2]),
+                                                    static_cast<float const *>(inputs[0]), size, workspacePtr,
+                                                    workspace, nullptr));
+        };
+        return {std::move(routine), workspace};
+    }
+
     // ------------------------------------------------------------------ Attention
 
     HipAttentionState::HipAttentionState() : _counters(nullptr) {

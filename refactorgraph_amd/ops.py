@@ -87,6 +87,22 @@ def dequantize_linear(x, scale, zp=None, axis=1, out=None):
     return y
 
 
+def dynamic_quantize_linear(x, out=None, workspace=None):
+    """x float32 (any shape) -> (y uint8 like x, scale float32 [1], zero_point uint8 [1])."""
+    _need_gpu(x)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    n = x.numel()
+    y = torch.empty(x.shape, dtype=torch.uint8, device=x.device) if out is None else out
+    assert y.dtype == torch.uint8 and y.numel() == n and y.is_contiguous()
+    scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    zp = torch.empty(1, dtype=torch.uint8, device=x.device)
+    nbytes = lib().rg_hip_dynamic_quantize_linear_workspace(n)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if workspace is None else workspace
+    check(lib().rg_hip_dynamic_quantize_linear(_ptr(y), _ptr(scale), _ptr(zp), _ptr(x), n, _ptr(ws), ws.numel(),
+                                               _stream()), "rg_hip_dynamic_quantize_linear")
+    return y, scale, zp
+
+
 def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):
     """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
     (batch, row) of the operand as the reference's CPU kernel reads them."""

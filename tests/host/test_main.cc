@@ -10,6 +10,7 @@
 #include "kernel/attributes/softmax_info.h"
 #include "kernel/collectors/attention.h"
 #include "kernel/collectors/dequantize_linear.h"
+#include "kernel/collectors/dynamic_quantize_linear.h"
 #include "kernel/collectors/mat_mul_integer.h"
 #include "kernel/collectors/rms_normalization.h"
 #include "kernel/collectors/rotary_embedding.h"
@@ -25,6 +26,7 @@
 #include <cstring>
 #include <numeric>
 #include <random>
+#include <tuple>
 
 using namespace refactor;
 using namespace kernel;
@@ -183,6 +185,19 @@ static void collectorsSelectOrDecline() {
     EXPECT(k6.size() == 1 && static_cast<DequantizeLinearHip const &>(*k6[0]).axisLen == 6);
     EXPECT(DequantizeLinearCollector(T::Amd, 0).filter({*x8, *s6}, {*y}).empty());  // axis 0 has 4 entries
     EXPECT(DequantizeLinearCollector(T::Amd, 1).filter({*x8, *s6, *z6u}, {*y}).empty());
+
+    // DynamicQuantizeLinear: float -> (uint8, float scalar, uint8 scalar); the routine asks for a workspace
+    auto xf = Tensor::share(DataType::F32, Shape{4, 6});
+    auto yq = Tensor::share(DataType::U8, Shape{4, 6});
+    auto zq = Tensor::share(DataType::U8, Shape{});
+    auto dq = DynamicQuantizeLinearCollector(T::Amd).filter({*xf}, {*yq, *s1, *zq});
+    EXPECT(dq.size() == 1 && static_cast<DynamicQuantizeLinearHip const &>(*dq[0]).size == 24);
+    {
+        runtime::Resources res_;
+        EXPECT(dq[0]->lower(res_).workspaceOffset > 0);
+    }
+    EXPECT(DynamicQuantizeLinearCollector(T::Amd).filter({*x8}, {*yq, *s1, *zq}).empty());
+    EXPECT(DynamicQuantizeLinearCollector(T::Cpu).filter({*xf}, {*yq, *s1, *zq}).empty());
 
     // Attention: parameter block from the tensors; head-count and dtype rules
     auto q = Tensor::share(DataType::FP16, Shape{2, 8, 1, 128});
@@ -344,6 +359,60 @@ static void matMulIntegerHip() {
         oracle_matmul_integer(ref.data(), a.data(), b.data(), &azv, 0, 1, &bzv, 1, 1, 6, 256, 128, 256, aOff, bOff, 2, 3, 8);
         EXPECT(y == ref);
     }
+}
+
+static void dynamicQuantizeLinearHip() {
+    runtime::Resources res;
+    auto &dev = amd();
+    auto run = [&](std::vector<float> const &x_) {
+        auto const n = x_.size();
+        auto x = Tensor::share(DataType::F32, Shape{static_cast<dim_t>(n)});
+        auto y = Tensor::share(DataType::U8, Shape{static_cast<dim_t>(n)});
+        auto scale = Tensor::share(DataType::F32, Shape{});
+        auto zp = Tensor::share(DataType::U8, Shape{});
+        auto kernels = DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*x}, {*y, *scale, *zp});
+        EXPECT(kernels.size() == 1);
+        auto [routine, workspaceSize] = kernels[0]->lower(res);
+        auto mx = dev.malloc(n * 4), my = dev.malloc(n), ms = dev.malloc(4), mz = dev.malloc(1),
+             ws = dev.malloc(workspaceSize);
+        mx->copyFromHost(x_.data());
+        void const *inputs[]{*mx};
+        void *outputs[]{*my, *ms, *mz};
+        routine(res, *ws, inputs, outputs);
+        std::vector<uint8_t> yData(n), ref(n);
+        float s, sRef;
+        uint8_t z, zRef;
+        my->copyToHost(yData.data());
+        ms->copyToHost(&s);
+        mz->copyToHost(&z);
+        oracle_dynamic_quantize_linear(ref.data(), &sRef, &zRef, x_.data(), n);
+        EXPECT(yData == ref && s == sRef && z == zRef);
+        return std::tuple{yData, s, z};
+    };
+    {// src/04kernel/test/kernels/dynamic_quantize_linear/test_cpu.cpp:8-39
+        auto [y, s, z] = run({0, 2, -3, -2.5, 1.34, 0.5});
+        EXPECT(s == (2 + 3) / 255.f && z == 153);
+        std::vector<float> x{0, 2, -3, -2.5, 1.34, 0.5};
+        for (size_t i = 0; i < x.size(); ++i) EXPECT(y[i] == static_cast<uint8_t>(std::round(x[i] / s) + z));
+    }
+    {// src/04kernel/test/kernels/dynamic_quantize_linear/test_cuda.cpp:14-73 (device result == CPU result)
+        std::vector<float> x(20);
+        for (size_t i = 0; i < x.size(); ++i) x[i] = i * 3 + 15;
+        run(x);
+    }
+    {
+        std::mt19937 rng(11);
+        std::normal_distribution<float> g(0.f, 3.f);
+        std::vector<float> x(100003);
+        for (auto &v : x) v = g(rng);
+        run(x);
+    }
+    // anything but float -> (uint8, float, uint8) is declined
+    auto xh = Tensor::share(DataType::FP16, Shape{8});
+    auto y = Tensor::share(DataType::U8, Shape{8});
+    auto scale = Tensor::share(DataType::F32, Shape{});
+    auto zp = Tensor::share(DataType::U8, Shape{});
+    EXPECT(DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*xh}, {*y, *scale, *zp}).empty());
 }
 
 static void dequantizeLinearHip() {
@@ -515,6 +584,7 @@ int main(int argc, char **argv) {
         RUN(softmaxHip);
         RUN(matMulIntegerHip);
         RUN(dequantizeLinearHip);
+        RUN(dynamicQuantizeLinearHip);
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
     }

@@ -188,6 +188,53 @@ def test_rope_full_config_properties():
     assert np.max(np.abs(host(y[11:12, sl].float()) - ref)) <= ABS_F16
 
 
+# ------------------------------------------------------------------ DynamicQuantizeLinear (bit-exact)
+
+def _dql_check(x):
+    y, scale, zp = ops.dynamic_quantize_linear(dev(x))
+    ry, rs, rz = oracle.dynamic_quantize_linear(x)
+    assert host(scale)[0] == rs and host(zp)[0] == rz
+    assert np.array_equal(host(y), ry)
+    return host(y), host(scale)[0], host(zp)[0]
+
+
+def test_dynamic_quantize_reference_kats():
+    # src/04kernel/test/kernels/dynamic_quantize_linear/test_cpu.cpp:21-38 and test_cuda.cpp:36-39
+    y, scale, zp = _dql_check(np.array([0, 2, -3, -2.5, 1.34, 0.5], np.float32))
+    assert scale == np.float32(5) / np.float32(255) and zp == 153 and y.tolist() == [153, 255, 0, 26, 221, 179]
+    y, scale, zp = _dql_check((3 * np.arange(20) + 15).astype(np.float32))
+    assert zp == 0 and y[-1] == 255
+
+
+@pytest.mark.parametrize("n", [1, 7, 255, 4096, 4097, (1 << 20) + 3, 3 * 5 * 7 * 1024])
+@pytest.mark.parametrize("lo,hi", [(-3.0, 5.0), (0.5, 9.0), (-7.0, -0.25)])
+def test_dynamic_quantize_bit_exact(n, lo, hi):
+    x = np.random.default_rng(n).uniform(lo, hi, n).astype(np.float32)
+    _dql_check(x)
+
+
+def test_dynamic_quantize_ties_zeros_and_unaligned():
+    y, scale, zp = _dql_check(np.array([0.0, 255.0, 2.5, 0.5, 1.5, 254.5], np.float32))
+    assert y.tolist() == [0, 255, 3, 1, 2, 255]           # ties away from zero
+    y, scale, zp = _dql_check(np.zeros(1000, np.float32))
+    assert not y.any() and zp == 0
+    # operands that are not 16-byte aligned take the element-wise path
+    x = np.random.default_rng(5).normal(0, 2, 10001).astype(np.float32)
+    xd = dev(x)
+    out = torch.empty(10003, dtype=torch.uint8, device=DEV)
+    y, scale, zp = ops.dynamic_quantize_linear(xd[1:], out=out[3:3 + 10000])
+    ry, rs, rz = oracle.dynamic_quantize_linear(x[1:])
+    assert np.array_equal(host(y), ry) and host(scale)[0] == rs and host(zp)[0] == rz
+
+
+def test_dynamic_quantize_full_config():
+    # the producer of MatMulInteger's A operand: fp32 [4096, 4096]
+    x = np.random.default_rng(15).normal(0, 1, (4096, 4096)).astype(np.float32)
+    y, scale, zp = _dql_check(x)
+    back = (y.astype(np.float32) - np.float32(zp)) * scale
+    assert np.max(np.abs(back - x)) <= 0.5 * scale * (1 + 1e-5)
+
+
 # ------------------------------------------------------------------ DequantizeLinear (bit-exact)
 
 def test_dequantize_reference_kat():

@@ -243,6 +243,57 @@ def test_dequantize_scalar_and_per_axis_closed_form(dt):
                               x.astype(np.float32) * s.reshape(shape))
 
 
+# ------------------------------------------------------------------ DynamicQuantizeLinear
+
+def test_dynamic_quantize_kats():
+    c = GOLDEN["dynamic_quantize_linear"][0]
+    y, scale, zp = oracle.dynamic_quantize_linear(np.array(c["x"], np.float32))
+    assert scale == np.float32(c["scale_num"]) / np.float32(c["scale_den"])
+    assert zp == c["zp"] and y.tolist() == c["expect_y"]
+    c = GOLDEN["dynamic_quantize_linear"][1]
+    x = (3 * np.arange(20) + 15).astype(np.float32)
+    y, scale, zp = oracle.dynamic_quantize_linear(x)
+    assert scale == np.float32(c["scale_num"]) / np.float32(c["scale_den"]) and zp == c["zp"]
+    q = x / scale
+    assert np.all(np.abs(q - np.round(q)) != 0.5)  # no ties: numpy's rounding rule does not matter here
+    assert np.array_equal(y, np.round(q).astype(np.uint8)) and y[-1] == 255
+
+
+def test_dynamic_quantize_properties():
+    rng = np.random.default_rng(31)
+    for lo, hi in [(-3.0, 5.0), (0.5, 9.0), (-7.0, -0.25), (-1e-3, 2e-3)]:
+        x = rng.uniform(lo, hi, 4097).astype(np.float32)
+        x[17] = 0.0
+        y, scale, zp = oracle.dynamic_quantize_linear(x)
+        mn, mx = min(float(x.min()), 0.0), max(float(x.max()), 0.0)
+        assert scale == np.float32(np.float32(mx) - np.float32(mn)) / np.float32(255)
+        # the zero point is where 0 lands, and the ends of the covered range land on 0 and 255
+        assert y[17] == zp
+        assert zp == int(np.clip(np.floor(-mn / float(scale) + 0.5), 0, 255))
+        assert y.min() == (0 if lo < 0 else y.min()) and y.max() == (255 if hi > 0 else y.max())
+        # float64 recomputation: equal except for values within rounding noise of a tie
+        q64 = np.clip(np.floor(np.abs(x.astype(np.float64) / float(scale)) + 0.5) * np.sign(x) + int(zp), 0, 255)
+        assert np.max(np.abs(y.astype(np.int64) - q64.astype(np.int64))) <= 1
+        assert np.mean(y == q64.astype(np.uint8)) > 0.999
+        # dequantising recovers x to half a step
+        back = (y.astype(np.float64) - int(zp)) * float(scale)
+        inside = (x >= mn) & (x <= mx)
+        assert np.max(np.abs(back - x)[inside]) <= 0.5 * float(scale) * (1 + 1e-5)
+
+
+def test_dynamic_quantize_rounds_half_away_and_saturates():
+    # scale exactly 1, zero point 0: ties must go away from zero (2.5 -> 3, 0.5 -> 1), not to even
+    x = np.array([0.0, 255.0, 2.5, 0.5, 1.5, 254.5], np.float32)
+    y, scale, zp = oracle.dynamic_quantize_linear(x)
+    assert scale == 1.0 and zp == 0 and y.tolist() == [0, 255, 3, 1, 2, 255]
+    # zero point saturates at 255 for an all-negative input; an all-zero input stays all zero
+    y, scale, zp = oracle.dynamic_quantize_linear(np.array([-4.0, -2.0, -1.0], np.float32))
+    assert zp == 255 and y.tolist() == [0, 128, 191] and scale == np.float32(4) / np.float32(255)
+    y, scale, zp = oracle.dynamic_quantize_linear(np.zeros(9, np.float32))
+    # the running maximum starts at the smallest normal float, which keeps the range positive
+    assert scale == np.float32(np.finfo(np.float32).tiny) / np.float32(255) and zp == 0 and not y.any()
+
+
 # ------------------------------------------------------------------ MatMul / Mul (oracle blocks)
 
 def test_matmul_f32_exact_on_integer_operands_and_transb():
