@@ -102,16 +102,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     rest /= head_chunks;
     const uint32_t kvh = rest % a.Hkv, b = rest / a.Hkv;
 
-    // history length of this batch row, clamped so that the new rows fit the cache
-    uint32_t base = 0;
-    if (a.kc && a.past) {
-        int64_t raw = a.past[a.past_per_row ? b : 0];
-        if (raw < 0) raw = 0;
-        const int64_t room = static_cast<int64_t>(a.cap) - static_cast<int64_t>(a.seq);
-        if (raw > room) raw = room < 0 ? 0 : room;
-        base = static_cast<uint32_t>(raw);
-    }
-
     const T *Q = static_cast<const T *>(a.q);
     const T *Kn = static_cast<const T *>(a.k);
     const T *Vn = static_cast<const T *>(a.v);
@@ -136,6 +126,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
         const T *qp = Q + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + qrow) * D + 8 * half;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qp + 16 * kk);
+    }
+
+    // history length of this batch row, clamped so that the new rows fit the cache (read after the
+    // query loads are on their way: they do not depend on it)
+    uint32_t base = 0;
+    if (a.kc && a.past) {
+        int64_t raw = a.past[a.past_per_row ? b : 0];
+        if (raw < 0) raw = 0;
+        const int64_t room = static_cast<int64_t>(a.cap) - static_cast<int64_t>(a.seq);
+        if (raw > room) raw = room < 0 ? 0 : room;
+        base = static_cast<uint32_t>(raw);
     }
 
     const uint32_t wg_last_key = base + wg_rows_end - 1;  // inclusive
@@ -166,13 +167,29 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             }
         }
     };
-    auto stage = [&](uint32_t buf, const Raw16(&kr)[4], const Raw16(&vr)[4]) {
-        uint8_t *ldsK = lds + buf * BUF_BYTES, *ldsV = ldsK + TILE;
+    // The new rows that correspond to this workgroup's query rows are appended to the caches
+    // (once per kv head) from the registers that carry them to LDS: every such row is among the
+    // keys the workgroup needs.
+    const bool do_append = Kc && hc == 0;
+    const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
+    auto stage = [&](uint32_t kt, const Raw16(&kr)[4], const Raw16(&vr)[4]) {
+        uint8_t *ldsK = lds + (kt & 1) * BUF_BYTES, *ldsV = ldsK + TILE;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t off = (st_row + 16 * i) * ROW + st_chunk * 16;
             *reinterpret_cast<Raw16 *>(ldsK + off) = kr[i];
             *reinterpret_cast<Raw16 *>(ldsV + (st_row + 16 * i) * VROW + st_chunk * 16) = vr[i];
+        }
+        if (do_append && kt * BN + BN > own_lo) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t pos = kt * BN + st_row + 16 * i;
+                if (pos >= own_lo && pos < own_hi) {
+                    const uint64_t dst = (kv_head * a.cap + pos) * D + st_chunk * 8;
+                    *reinterpret_cast<Raw16 *>(Kc + dst) = kr[i];
+                    *reinterpret_cast<Raw16 *>(Vc + dst) = vr[i];
+                }
+            }
         }
     };
 
@@ -194,24 +211,32 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
 
         const uint8_t *ldsK = lds + (kt & 1) * BUF_BYTES, *ldsV = ldsK + TILE;
         if (kt < wave_tiles) {
-            // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32
+            // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32.  Both
+            // blocks of the tile are issued first; the softmax of a block then runs on the VALU
+            // while the matrix core still works on the next product (S^T of block 1, or the PV
+            // update of block 0).  A block that lies entirely above the diagonal is skipped.
+            const bool second = kt * BN + 32 <= base + r0 + 31;
             f16v s[2];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+                if (kb == 0 || second) {
 #pragma unroll
-                for (int kk = 0; kk < 8; ++kk) {
-                    const Raw16 kf = *reinterpret_cast<const Raw16 *>(ldsK + (32 * kb + l32) * ROW + (2 * kk + half) * 16);
-                    s[kb] = Ops<T>::mfma(kf, qf[kk], s[kb]);
+                    for (int kk = 0; kk < 8; ++kk) {
+                        const Raw16 kf = *reinterpret_cast<const Raw16 *>(ldsK + (32 * kb + l32) * ROW + (2 * kk + half) * 16);
+                        s[kb] = Ops<T>::mfma(kf, qf[kk], s[kb]);
+                    }
                 }
             }
-            // scale, causal mask (only tiles that reach past the wavefront's first query position)
-            const bool need_mask = kt * BN + BN - 1 > base + r0;
-            float over = -__builtin_inff();
-            if (need_mask) {  // wave-uniform: only the tiles on the diagonal pay for the comparisons
+            const uint32_t tr_off = (4 * half + (lane & 15) / 4) * VROW + 2 * (16 * ((lane >> 4) & 1) + 4 * (lane & 3));
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb) {
+                if (kb == 1 && !second) break;
+                // scale, causal mask (only blocks that reach past the wavefront's first query position)
+                const bool need_mask = kt * BN + 32 * kb + 31 > base + r0;
+                float over = -__builtin_inff();
+                if (need_mask) {  // wave-uniform: only the blocks on the diagonal pay for the comparisons
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
@@ -219,36 +244,30 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                         s[kb][e] = t;
                         over = fmaxf(over, t);
                     }
-            } else {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                } else {
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const float t = fmaf(s[kb][e], c_log2e, -m);
                         s[kb][e] = t;
                         over = fmaxf(over, t);
                     }
-            }
-            over = fmaxf(over, __shfl_xor(over, 32, kWave));  // both halves hold the same query row
-            if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
-                const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
-                const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
-                m += up;
-                l *= alpha;
+                }
+                over = fmaxf(over, __shfl_xor(over, 32, kWave));  // both halves hold the same query row
+                if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
+                    const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
+                    const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
+                    m += up;
+                    l *= alpha;
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                    for (int db = 0; db < 4; ++db)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) s[kb][e] -= up;
-                fresh = false;
-            }
-            // P^T in B-operand position: element i of MFMA (kb, jj) is accumulator register 8 jj + i
-            Raw16 pf[2][2];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                    fresh = false;
+                }
+                // P^T in B-operand position: element i of MFMA (kb, jj) is accumulator register 8 jj + i
+                Raw16 pf[2];
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
@@ -256,29 +275,27 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                         const float p0 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2]);
                         const float p1 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2 + 1]);
                         l += p0 + p1;
-                        pf[kb][jj].w[i2] = Ops<T>::pack2(p0, p1);
+                        pf[jj].w[i2] = Ops<T>::pack2(p0, p1);
                     }
-            // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
-            // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
-            // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
-            // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
-            const uint32_t tr_off = (4 * half + (lane & 15) / 4) * VROW + 2 * (16 * ((lane >> 4) & 1) + 4 * (lane & 3));
+                // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
+                // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
+                // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
+                // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int db = 0; db < 4; ++db)
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
                         const uint8_t *vp = ldsV + (32 * kb + 16 * jj) * VROW + 64 * db + tr_off;
                         const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * VROW);
                         const Raw16 vf{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
-                        o[db] = Ops<T>::mfma(vf, pf[kb][jj], o[db]);
+                        o[db] = Ops<T>::mfma(vf, pf[jj], o[db]);
                     }
+            }
         }
 
         // the other buffer was last read in the previous iteration, which every wavefront left
         // through the barrier below
-        if (kt + 1 < n_tiles) stage((kt + 1) & 1, kr, vr);
+        if (kt + 1 < n_tiles) stage(kt + 1, kr, vr);
         __syncthreads();
     }
 
@@ -307,17 +324,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
         }
     }
 
-    // append the new rows this workgroup's query rows correspond to (once per kv head); nothing
-    // in this workgroup waits for the copy
-    if (Kc && hc == 0) {
-        for (uint32_t idx = tid; idx < (wg_rows_end - qt * ROWS) * 16; idx += 256) {
-            const uint32_t rr = qt * ROWS + idx / 16, c = idx % 16;
-            const uint64_t src = static_cast<uint64_t>(rr) * D + c * 8;
-            const uint64_t dst = (kv_head * a.cap + base + rr) * D + c * 8;
-            *reinterpret_cast<Raw16 *>(Kc + dst) = *reinterpret_cast<const Raw16 *>(k_new + src);
-            *reinterpret_cast<Raw16 *>(Vc + dst) = *reinterpret_cast<const Raw16 *>(v_new + src);
-        }
-    }
 }
 
 template <class T, int HW>
