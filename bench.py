@@ -209,6 +209,20 @@ def main():
     ops_out = {}
     steps, warmup = args.steps, args.warmup
 
+    def cpu_leg(fn, algorithmic_bytes, sample):
+        """Times the oracle on a bounded sample for about a second; the rate is quoted in the algorithmic bytes
+        of that sample so that it compares with `achieved`."""
+        fn()  # page in
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 1.0:
+                break
+        return {"value": round(algorithmic_bytes * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{sample} ({reps} repetitions, {dt / reps * 1e3:.1f} ms each)"}
+
     if want("rms_norm"):
         nb = 5  # 5 x (134 MB in + 134 MB out): beyond the 256 MB MALL
         xs = [torch.randn((32, 128, 4096), device=dev) for _ in range(nb)]
@@ -217,6 +231,10 @@ def main():
         wall, dms, mode = time_steps(torch, lambda i: ops.rms_norm(xs[i], w, 1e-5, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(134234112, dms, "rms_norm")
         e.update(workload="RmsNormalization f32 [32,128,4096]", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn, wn = xs[0][:4].cpu().numpy(), w.cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.rms_norm(xn, wn, 1e-5), 134234112 // 8, "4 of the 32 [128,4096] slabs")
         ops_out["rms_norm"] = e
         del xs, ys
 
@@ -227,6 +245,11 @@ def main():
             wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 4, 5), max(warmup // 8, 3), 1)
             e = hbm_entry(nbytes, dms, name)
             e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_per_launch=round(dms, 5), timing=mode)
+            if not args.no_cpu:
+                import oracle
+                xn = x[0, :2].float().cpu().numpy()
+                fn = (lambda: oracle.softmax_causal(xn)) if causal else (lambda: oracle.softmax(xn))
+                e["cpu_baseline"] = cpu_leg(fn, nbytes // 128, "2 of the 256 [2048,2048] matrices, fp32 on up-cast input")
             ops_out[name] = e
         del x, y
 
@@ -238,6 +261,11 @@ def main():
         wall, dms, mode = time_steps(torch, lambda i: ops.rope(xs[i], pos, 10000.0, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(537133056, dms, "rope")
         e.update(workload="RotaryEmbedding fp16 [16,2048,32,128]", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn, pn = xs[0][:1].float().cpu().numpy(), pos[:1].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.rope(xn, pn, 10000.0), 537133056 // 16,
+                                        "batch row 0 of 16, fp32 on up-cast input")
         ops_out["rope"] = e
         del xs, ys
 
@@ -249,6 +277,10 @@ def main():
         wall, dms, mode = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
         e = hbm_entry(83902464, dms, "dequantize_linear")
         e.update(workload="DequantizeLinear i8->f32 [4096,4096] per-axis scale", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn, sn = xs[0].cpu().numpy(), sc.cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.dequantize_linear(xn, sn, axis=1), 83902464, "the whole tensor once")
         ops_out["dequantize_linear"] = e
         del xs, ys
 
@@ -321,6 +353,15 @@ def main():
                  device_ms_per_launch=round(dms, 5), timing=mode,
                  mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
                  mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
+        if not args.no_cpu:
+            import oracle
+            f32 = lambda t: t.float().cpu().numpy()
+            qn, kn, vn = f32(q[:1]), f32(k[:1]), f32(v[:1])
+            kcn, vcn = f32(kc[:1]), f32(vc[:1])
+            pairs = [(0, h) for h in range(4)]
+            e["cpu_baseline"] = cpu_leg(
+                lambda: oracle.attention_kvcache(qn, kn, vn, kcn, vcn, np.zeros(1, np.int64), scale, heads=pairs),
+                402653184 * 4 // (Np * H), "4 of the 1024 (batch row, head) pairs; composed oracle in fp32")
         ops_out["attention_prefill"] = e
 
     if ops_out:
