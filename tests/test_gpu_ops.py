@@ -382,6 +382,8 @@ def test_attention_decode_and_small_prefill(N, H, Hkv, seq, cap, D, past):
     (16, 8, 8, 8, 32, 64, torch.float16),     # many short segments: several pieces per range, several passes
     (70, 4, 2, 1, 96, 128, torch.float16),    # more than 64 batch rows: the partition is built by the whole workgroup
     (24, 12, 4, 3, 40, 128, torch.bfloat16),  # group of 3 heads (two launches), short segments, bf16
+    (4, 8, 8, 200, 256, 64, torch.float16),   # head dim 64 prefill through the split kernel: ~25 segments per range
+    (200, 2, 1, 1, 48, 64, torch.float16),    # 200 batch rows
 ])
 def test_attention_split_many_segments(N, H, Hkv, seq, cap, D, dt):
     past = np.random.default_rng(21).integers(0, cap - seq + 1, N)
