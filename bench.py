@@ -41,7 +41,7 @@ MEASURED_TRAFFIC = {
     "softmax_causal": (2 * 540713 + 2097158) * 1024,
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
-    "matmul_integer": (2 * 52558 + 71295) * 1024,
+    "matmul_integer": (2 * 49313 + 65638) * 1024,
     "attention_prefill": (2 * 99826 + 196608) * 1024,
 }
 

@@ -7,10 +7,12 @@
 // order is bit-identical to the reference's serial loop.
 //
 // Fast path (m, n multiples of 256, k multiple of 128): one 256x256 output tile per workgroup of
-// four wavefronts, int8 MFMA 32x32x32, LDS double-buffered k-tiles of 128.  B [k,n] is byte-
-// transposed on its way into LDS so that both MFMA operands are k-contiguous.  Zero points are
-// folded into the staging step (XOR / packed byte subtract), so there is no pre-pass over A or
-// B and no workspace.  Everything else goes through a plain tiled kernel.
+// four wavefronts, int8 MFMA 32x32x32, k-tiles of 128 copied from global memory straight into two
+// LDS buffers.  B [k,n] stays as in memory and is byte-transposed by the LDS read, so that both
+// MFMA operands are k-contiguous.  Zero points are applied to the operand fragments, so there is
+// no pre-pass over A or B and no workspace.  Everything else goes through a plain tiled kernel.
+#include <utility>
+
 #include "common.hpp"
 
 namespace rg {
@@ -77,239 +79,158 @@ __global__ __launch_bounds__(256) void mmi_generic(int32_t *__restrict__ y,
 //
 // Workgroup = 256 threads = four wavefronts (one per SIMD), one 256x256 tile of Y; wavefront
 // (wm, wn) owns the 128x128 quadrant as 4x4 blocks of v_mfma_i32_32x32x32_i8 (256 accumulator
-// registers).  k is walked in tiles of 128 (64 MFMAs per wavefront between barriers):
-//   A tile: 256 rows x 128 bytes, k-contiguous as in memory (each row segment is one full
-//           128-byte line), LDS rows padded to 144 bytes so that the 128-bit fragment reads of
-//           consecutive rows fall into different banks;
-//   B tile: 128 k-rows x 256 columns in memory; a thread takes 4 k-rows x 16 columns (four
-//           128-bit loads) and byte-transposes the four 4x4 blocks with v_perm_b32, which leaves
-//           one dword (4 consecutive k) per column.  The four lanes 16 apart hold the four
-//           k-quads of one 16-k group for the same columns; a 4x4 dword transpose across them
-//           (v_permlane32_swap + v_permlane16_swap) gives each lane 16 consecutive k of four
-//           columns, written with 128-bit stores into LDS laid out [k/16][column][16 k-bytes].
-//           The 16-byte slot of a column inside its 256-byte block is XOR-swizzled with the
-//           block index so that both these writes and the 128-bit fragment reads are free of
-//           bank conflicts.
-// Both operands present the same k order to the MFMA, so the contraction is exact.
-// Global loads run ahead in registers (two register stages: a tile is loaded one and a half
-// iterations before it is written to LDS), LDS is double buffered, and the staging work of
-// tile kt+1 (zero-point subtract, transposition, LDS writes) sits in the same basic block as
-// the MFMAs of tile kt, with scheduling-group hints that issue it in their shadow.
+// registers).  k is walked in tiles of 128 (64 MFMAs per wavefront) through two LDS buffers.
+// There is no register staging: both tiles go from global memory into LDS with
+// global_load_lds_dwordx4 (lane L of a wavefront-wide copy fills bytes 16 L .. 16 L + 15 behind a
+// wave-uniform LDS base, from a global address of its own), 16 copies per wavefront and k-tile.
+//   A tile: 256 rows of 128 bytes, unpadded; the 16-byte chunk c of row r sits at chunk position
+//           c ^ (r & 7) ^ ((r >> 3) & 1), which spreads the 128-bit fragment reads of 8 as well
+//           as of 16 consecutive rows over all banks.
+//   B tile: as in memory, 128 k-rows of 256 bytes; chunk c of k-row r sits at chunk position
+//           c ^ swz(r & 7).  The MFMA operand (16 consecutive k of one column per lane) is formed
+//           by ds_read_b64_tr_b8: within 16 lanes, lane i receives byte i % 8 of the 8-byte pieces
+//           addressed by lanes i / 8, i / 8 + 2, ..., so lanes 2 j and 2 j + 1 address the two
+//           halves of the 16 columns in k-row j and every lane gets 8 consecutive k of its column.
+// Both operands present the same k order to the MFMA, so the contraction is exact.  Zero points
+// are applied to the fragments (one XOR mask, or a packed byte subtract), so there is no pre-pass
+// over A or B and no workspace.  One k-tile is 64 MFMAs per wavefront in a fixed order (a
+// scheduling barrier after each with its share of LDS reads and copies); fragments are double
+// buffered by k-step.  The barrier of a tile sits before its last k-step: after it the buffer
+// just multiplied is refilled with tile kt+2 while the last 16 MFMAs run from registers and the
+// first fragments of tile kt+1 arrive.
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 128;
-constexpr int A_ROW = BK + 16;                       // padded LDS row of the A tile, bytes
-constexpr int A_TILE = BM * A_ROW;                   // 36864
-constexpr int KG_BYTES = BN * 16;                    // one 16-k group of the B tile: [column][16 k-bytes]
-constexpr int B_TILE = (BK / 16) * KG_BYTES;         // 32768
-constexpr int STAGE_BYTES = A_TILE + B_TILE;         // one LDS buffer (69632)
-constexpr int LDS_BYTES = 2 * STAGE_BYTES;           // 139264 of the 160 KiB per CU
-constexpr int A_LOADS = BM * BK / (256 * 16);        // 8 128-bit loads per thread per tile
-constexpr int B_LOADS = BK * BN / (256 * 16);        // 8
+constexpr int D_TILE = 32768;            // A 256 x 128 or B 128 x 256
+constexpr int D_STAGE = 2 * D_TILE;      // one LDS buffer
 
+__device__ __forceinline__ uint32_t b_swizzle(uint32_t x) { return ((x & 3) << 1) | ((x >> 2) * 9); }  // x < 8
 
-// 4x4 byte transpose: in[r] holds bytes (r,0..3); out[c] holds bytes (0..3,c).
-__device__ __forceinline__ void transpose4x4(uint32_t i0, uint32_t i1, uint32_t i2, uint32_t i3,
-                                             uint32_t out[4]) {
-    // v_perm_b32(s0, s1, sel): result byte i = byte sel[i] of the 8 bytes {s1 (0-3), s0 (4-7)}
-    const uint32_t t0 = __builtin_amdgcn_perm(i1, i0, 0x05010400u);  // r0b0 r1b0 r0b1 r1b1
-    const uint32_t t1 = __builtin_amdgcn_perm(i1, i0, 0x07030602u);  // r0b2 r1b2 r0b3 r1b3
-    const uint32_t t2 = __builtin_amdgcn_perm(i3, i2, 0x05010400u);  // r2b0 r3b0 r2b1 r3b1
-    const uint32_t t3 = __builtin_amdgcn_perm(i3, i2, 0x07030602u);  // r2b2 r3b2 r2b3 r3b3
-    out[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);  // r0b0 r1b0 r2b0 r3b0
-    out[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
-    out[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
-    out[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
-}
-
-struct alignas(16) U4 {
-    uint32_t v[4];
-};
-
-// Register-staged global loads of one k-tile for one thread.
-struct Stage {
-    U4 a[A_LOADS];  // rows tid/8 + 32*i, bytes (tid%8)*16 .. +15 of the k-tile
-    U4 b[B_LOADS];  // k-rows 64*(i/4) + 4*(tid/16) + i%4, columns 16*(tid%16) .. +15
-};
-
-// A_MODE 0: zero point absent, 0 or 128 (one XOR mask); 1: any scalar / per-row zero point.
 template <int A_MODE, bool B_ZP>
-__device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds, const uint8_t *A,
-                                              const uint8_t *B, uint32_t k, uint32_t n,
-                                              uint32_t a_xor, const uint32_t (&za_w)[A_LOADS],
-                                              ZeroPoint zb, uint64_t zb_row0) {
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t wm = wave >> 1, wn = wave & 1;
-    const uint8_t *a_src = A + static_cast<uint64_t>(tid >> 3) * k + (tid & 7) * 16;
-    const uint8_t *b_src = B + static_cast<uint64_t>(4 * (tid >> 4)) * n + (tid & 15) * 16;
-    const uint32_t a_dst = (tid >> 3) * A_ROW + (tid & 7) * 16;
-    // B staging: this lane ends up with columns 16*nb + 4*r + c (c = 0..3) of 16-k group wave + 4h
-    const uint32_t nb = tid & 15, r_grp = lane >> 4;
-    uint32_t b_dst[4];
+__device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, uint8_t *lds1,
+                                              const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t n,
+                                              uint32_t a_xor, const uint32_t (&za_f)[4], ZeroPoint zb,
+                                              uint64_t zb_row0) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
+    // copy q < 8: A rows 8 (8 wave + q) .. + 7, this lane row + lane / 8, chunk position lane % 8;
+    // copy 8 + p: B k-rows 4 (8 wave + p) .. + 3, this lane k-row + lane / 16, chunk position lane % 16
+    const uint8_t *a_wave = A + static_cast<uint64_t>(wave * 64) * k;
+    const uint32_t a_lane = (lane >> 3) * k + 16 * ((lane & 7) ^ (lane >> 3));
+    const uint8_t *b_wave = B + static_cast<uint64_t>(wave * 32) * n;
+    uint32_t b_lane[2];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) b_dst[c] = A_TILE + wave * KG_BYTES + 256 * nb + 16 * ((4 * r_grp + c) ^ nb);
-    const uint32_t a_frag = (wm * 128 + (lane & 31)) * A_ROW + (lane >> 5) * 16;
-    // B fragment j: column wn*128 + 32*j + lane%32 of 16-k group 2*ks + lane/32
-    uint32_t b_frag[4];
+    for (int p = 0; p < 2; ++p) b_lane[p] = (lane >> 4) * n + 16 * ((lane & 15) ^ b_swizzle(4 * p + (lane >> 4)));
+    auto copy = [&](uint8_t *base, uint32_t k0, int q) {
+        const uint8_t *src;
+        uint8_t *dst;
+        if (q < 8) {
+            src = a_wave + (k0 + 8 * q * k) + (a_lane ^ (16 * (q & 1)));
+            dst = base + (wave * 8 + q) * 1024;
+        } else {
+            src = b_wave + static_cast<uint64_t>(k0 + 4 * (q - 8)) * n + b_lane[q & 1];
+            dst = base + D_TILE + (wave * 8 + (q - 8)) * 1024;
+        }
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                         (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+    };
+    // A fragment i of k-step ks: row wm 128 + 32 i + lane % 32, chunk 2 ks + h
+    const uint32_t a_off = (wm * 128 + (lane & 31)) * 128 + 16 * (h ^ (lane & 7) ^ ((lane >> 3) & 1));
+    auto read_a = [&](const uint8_t *base, int ks, int i) -> v4i {
+        return *reinterpret_cast<const v4i *>(base + (a_off ^ (32 * ks)) + i * 4096);
+    };
+    // B fragment j of k-step ks: column wn 128 + 32 j + lane % 32, k 16 (2 ks + h) .. + 15 in two reads
+    uint32_t b_off[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const uint32_t blk = 8 * wn + 2 * j + ((lane >> 4) & 1);
-        b_frag[j] = A_TILE + (lane >> 5) * KG_BYTES + 256 * blk + 16 * ((lane & 15) ^ (blk & 15));
+        const uint32_t a16 = lane & 15, chunk = wn * 8 + 2 * j + ((lane >> 4) & 1);
+        b_off[j] = D_TILE + (16 * h + (a16 >> 1)) * 256 + 16 * (chunk ^ b_swizzle(a16 >> 1)) + 8 * (a16 & 1);
     }
-
-    auto load_stage = [&](Stage &st, uint32_t k0) {
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i)
-            st.a[i] = *reinterpret_cast<const U4 *>(a_src + static_cast<uint64_t>(32 * i) * k + k0);
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i)
-            st.b[i] = *reinterpret_cast<const U4 *>(
-                b_src + static_cast<uint64_t>(k0 + 64 * (i / 4) + (i % 4)) * n);
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    auto read_b = [&](const uint8_t *base, int ks, int j, int half, v4i &f) {
+        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (__attribute__((address_space(3))) v2i *)(base + b_off[j] + (32 * ks + 8 * half) * 256));
+        f[2 * half] = r[0];
+        f[2 * half + 1] = r[1];
     };
-
-    auto store_stage = [&](const Stage &st, uint32_t buf, uint32_t k0) {
-        uint8_t *base = lds + buf * STAGE_BYTES;
+    auto fix_a = [&](v4i &f, int i) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) {
-            U4 v = st.a[i];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if constexpr (A_MODE == 0) v.v[e] ^= a_xor;
-                else v.v[e] = sub_bytes(v.v[e], za_w[i]);
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (A_MODE == 0) f[e] ^= static_cast<int>(a_xor);
+            else f[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(f[e]), za_f[i]));
+        }
+    };
+    auto fix_b = [&](v4i &f, uint32_t k0, int ks) {
+        if constexpr (B_ZP) {
+            uint32_t z[4];
+            if (zb.per_row) {
+                __builtin_memcpy(z, zb.ptr + zb_row0 + k0 + 16 * (2 * ks + h), 16);
+            } else {
+                z[0] = z[1] = z[2] = z[3] = splat(zb.ptr[0]);
             }
-            *reinterpret_cast<U4 *>(base + a_dst + 32 * i * A_ROW) = v;
-        }
 #pragma unroll
-        for (int h = 0; h < B_LOADS / 4; ++h) {
-            uint32_t r[4][4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint32_t zw = 0;
-                if constexpr (B_ZP) zw = splat(zp_byte(zb, zb_row0 + k0 + 64 * h + 4 * (tid >> 4) + i));
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    r[i][q] = B_ZP ? sub_bytes(st.b[4 * h + i].v[q], zw) : st.b[4 * h + i].v[q];
-            }
-            uint32_t d[4][4];  // d[q][c]: this lane's k-quad of column 4q + c
-#pragma unroll
-            for (int q = 0; q < 4; ++q) transpose4x4(r[0][q], r[1][q], r[2][q], r[3][q], d[q]);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                // 4x4 dword transpose across the lane groups 0-15 / 16-31 / 32-47 / 48-63:
-                // afterwards lane group g holds k-quads 0..3 of column 4g + c in d[0..3][c]
-                auto s02 = __builtin_amdgcn_permlane32_swap(d[0][c], d[2][c], false, false);
-                auto s13 = __builtin_amdgcn_permlane32_swap(d[1][c], d[3][c], false, false);
-                auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
-                auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
-                U4 out;
-                out.v[0] = t01[0];
-                out.v[1] = t01[1];
-                out.v[2] = t23[0];
-                out.v[3] = t23[1];
-                *reinterpret_cast<U4 *>(base + b_dst[c] + 4 * h * KG_BYTES) = out;
-            }
-        }
-    };
-
-    // Fragments: the four B fragments of a k-step stay live through its 16 MFMAs and are double
-    // buffered; an A fragment is dead after its row of four MFMAs and is refilled in place with
-    // the next k-step's fragment.
-    auto read_a = [&](uint32_t buf, int ks, int i) -> v4i {
-        return *reinterpret_cast<const v4i *>(lds + buf * STAGE_BYTES + a_frag + i * 32 * A_ROW + ks * 32);
-    };
-    auto read_b = [&](uint32_t buf, int ks, v4i (&fb)[4]) {
-        const uint8_t *base = lds + buf * STAGE_BYTES;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            fb[j] = *reinterpret_cast<const v4i *>(base + b_frag[j] + ks * 2 * KG_BYTES);
-    };
-    // one k-step: 16 MFMAs; NEXT_KS < 0: no refill (the tile ends)
-    auto kstep = [&](v4i (&fa)[4], const v4i (&fb)[4], uint32_t buf, int next_ks) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-            if (next_ks >= 0) fa[i] = read_a(buf, next_ks, i);
-        }
-    };
-    // Issue order requested from the scheduler for one tile (64 MFMAs): fragment reads, the global
-    // loads of tile kt+2 and the register part of the staging of tile kt+1 (zero point,
-    // transposition) behind the first 48, its LDS writes behind the last 16.  The LDS writes
-    // follow the tile's last fragment read in program order because the compiler cannot prove
-    // that the two LDS buffers do not alias.
-    auto interleave = [&]() {
-#pragma unroll
-        for (int i = 0; i < 48; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+            for (int e = 0; e < 4; ++e) f[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(f[e]), z[e]));
         }
     };
 
     const uint32_t k_tiles = k / BK;
-    Stage s0, s1;
-    v4i fa[4], fb0[4], fb1[4];
-    load_stage(s0, 0);
-    store_stage(s0, 0, 0);
-    if (k_tiles > 1) load_stage(s1, BK);
+    v4i fa[2][4], fb[2][4];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) copy(lds0, 0, q);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) copy(lds1, k_tiles > 1 ? BK : 0, q);  // k_tiles == 1: tile 0 again, never multiplied
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 (the 16 older copies)
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fa[i] = read_a(0, 0, i);
-    read_b(0, 0, fb0);
+    for (int i = 0; i < 4; ++i) fa[0][i] = read_a(lds0, 0, i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        read_b(lds0, 0, j, 0, fb[0][j]);
+        read_b(lds0, 0, j, 1, fb[0][j]);
+    }
 
-    // tile j lives in register stage j % 2 and LDS buffer j % 2; fa / fb0 hold the ks = 0
-    // fragments of the tile about to be multiplied.  S_FREE is the stage whose tile (kt) is
-    // already in LDS.
-#define RG_MMI_STEP(KT, S_FREE, S_NEXT1, HAS2, HAS1)                        \
-    {                                                                       \
-        const uint32_t kt_ = (KT), buf_ = kt_ & 1;                          \
-        if (HAS2) load_stage(S_FREE, (kt_ + 2) * BK);                       \
-        read_b(buf_, 1, fb1);                                               \
-        kstep(fa, fb0, buf_, 1);                                            \
-        read_b(buf_, 2, fb0);                                               \
-        kstep(fa, fb1, buf_, 2);                                            \
-        read_b(buf_, 3, fb1);                                               \
-        kstep(fa, fb0, buf_, 3);                                            \
-        /* every LDS read of this tile is issued: the LDS writes may follow */ \
-        if (HAS1) store_stage(S_NEXT1, buf_ ^ 1, (kt_ + 1) * BK);           \
-        kstep(fa, fb1, buf_, -1);                                           \
-        interleave();                                                       \
-        __syncthreads();                                                    \
-        if (HAS1) {                                                         \
-            _Pragma("unroll") for (int i = 0; i < 4; ++i) fa[i] = read_a(buf_ ^ 1, 0, i); \
-            read_b(buf_ ^ 1, 0, fb0);                                       \
-        }                                                                   \
-    }
+    // Tile kt is in buffer RB, tile kt+1 arrives in WB.
+    auto step = [&](uint32_t kt_, uint8_t *RB, const uint8_t *WB) __attribute__((always_inline)) {
+        const uint32_t k_cp = (kt_ + 2) * BK;
+        const bool more = kt_ + 2 < k_tiles;  // uniform
+        auto slot = [&]<int s>() __attribute__((always_inline)) {
+            constexpr int ks = s / 16, o = s % 16, row = o / 4, col = o % 4, cur = ks & 1, nxt = cur ^ 1;
+            if constexpr (s == 48) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of tile kt+1
+                __syncthreads();                                  // tile kt+1 complete, RB no longer read
+            }
+            if constexpr (col == 0) fix_a(fa[cur][row], row);
+            if constexpr (row == 0) fix_b(fb[cur][col], kt_ * BK, ks);
+            acc[row][col] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[cur][row], fb[cur][col], acc[row][col], 0, 0, 0);
+            const uint8_t *src = ks == 3 ? WB : RB;
+            constexpr int nks = (ks + 1) % 4;
+            if constexpr (o < 4) fa[nxt][o] = read_a(src, nks, o);
+            else if constexpr (o < 12) read_b(src, nks, (o - 4) / 2, (o - 4) % 2, fb[nxt][(o - 4) / 2]);
+            if constexpr (s >= 48) if (more) copy(RB, k_cp, s - 48);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) {
+            (slot.template operator()<I>(), ...);
+        }(std::make_integer_sequence<int, 64>{});
+    };
     uint32_t kt = 0;
-    for (; kt + 4 <= k_tiles; kt += 2) {  // both steps here have two more tiles behind them
-        RG_MMI_STEP(kt, s0, s1, true, true)
-        RG_MMI_STEP(kt + 1, s1, s0, true, true)
+    for (; kt + 2 <= k_tiles; kt += 2) {
+        step(kt, lds0, lds1);
+        step(kt + 1, lds1, lds0);
     }
-    // up to three remaining tiles, register stages continuing the alternation
-    if (kt < k_tiles) { RG_MMI_STEP(kt, s0, s1, kt + 2 < k_tiles, kt + 1 < k_tiles) ++kt; }
-    if (kt < k_tiles) { RG_MMI_STEP(kt, s1, s0, kt + 2 < k_tiles, kt + 1 < k_tiles) ++kt; }
-    if (kt < k_tiles) { RG_MMI_STEP(kt, s0, s1, kt + 2 < k_tiles, kt + 1 < k_tiles) ++kt; }
-#undef RG_MMI_STEP
+    if (kt < k_tiles) step(kt, lds0, lds1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
 }
 
-__global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__ y,
-                                                           const uint8_t *__restrict__ a,
-                                                           const uint8_t *__restrict__ b,
-                                                           ZeroPoint za, ZeroPoint zb, uint32_t m,
-                                                           uint32_t k, uint32_t n,
-                                                           uint32_t a_matrix0, uint32_t b_matrix0,
-                                                           uint32_t y_matrix0) {
-    extern __shared__ __align__(16) uint8_t lds[];
+__global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
+                                                           const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb,
+                                                           uint32_t m, uint32_t k, uint32_t n, uint32_t a_matrix0,
+                                                           uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(1024) uint8_t lds0[D_STAGE];
+    __shared__ __align__(1024) uint8_t lds1[D_STAGE];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t bz = blockIdx.z;
@@ -317,11 +238,10 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
 
     // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
     // give each XCD a contiguous block of tiles (they then share A row-panels / B column-panels
-    // in that XCD's L2).
+    // in that XCD's L2); within it walk tiles in column-major groups of 4 rows to keep panels hot.
     const uint32_t tiles_n = n / BN, tiles_m = m / BM, n_tiles = tiles_m * tiles_n;
     uint32_t t = blockIdx.x;
     if (n_tiles % 8 == 0) t = (t % 8) * (n_tiles / 8) + t / 8;
-    // within the linear order walk tiles in column-major groups of 4 rows to keep panels hot
     const uint32_t group = 4 * tiles_n;
     const uint32_t g = t / group, r = t % group;
     const uint32_t rows_here = tiles_m - g * 4 < 4 ? tiles_m - g * 4 : 4;
@@ -338,16 +258,17 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-    // zero points of this thread's staged A rows; scalar 0 / 128 (or none) reduce to one XOR mask
-    uint32_t za_w[A_LOADS] = {};
+    const uint32_t wm = wave >> 1, wn = wave & 1;
+    // zero points of the rows of this lane's A fragments; scalar 0 / 128 (or none) reduce to one XOR mask
+    uint32_t za_f[4] = {};
     uint32_t a_xor = 0;
     bool a_simple = true;
     if (za.ptr) {
         if (za.per_row) {
             a_simple = false;
 #pragma unroll
-            for (int i = 0; i < A_LOADS; ++i)
-                za_w[i] = splat(za.ptr[am * m + static_cast<uint64_t>(tile_m) * BM + (tid >> 3) + 32 * i]);
+            for (int i = 0; i < 4; ++i)
+                za_f[i] = splat(za.ptr[am * m + static_cast<uint64_t>(tile_m) * BM + wm * 128 + 32 * i + (lane & 31)]);
         } else {
             const uint32_t z = za.ptr[0];
             if (z == 0 || z == 128) {
@@ -355,26 +276,22 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
             } else {
                 a_simple = false;
 #pragma unroll
-                for (int i = 0; i < A_LOADS; ++i) za_w[i] = splat(z);
+                for (int i = 0; i < 4; ++i) za_f[i] = splat(z);
             }
         }
     }
-    // a scalar zero point of 0 on B is the common case: skip the subtract entirely
     bool b_zp = zb.ptr != nullptr;
     if (b_zp && !zb.per_row && zb.ptr[0] == 0) b_zp = false;
     const uint64_t zb_row0 = bm * k;
 
     if (a_simple) {
-        if (!b_zp) mmi_tile_loop<0, false>(acc, lds, A, B, k, n, a_xor, za_w, zb, zb_row0);
-        else mmi_tile_loop<0, true>(acc, lds, A, B, k, n, a_xor, za_w, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<0, false>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
+        else mmi_tile_loop<0, true>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
     } else {
-        if (!b_zp) mmi_tile_loop<1, false>(acc, lds, A, B, k, n, a_xor, za_w, zb, zb_row0);
-        else mmi_tile_loop<1, true>(acc, lds, A, B, k, n, a_xor, za_w, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<1, false>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
+        else mmi_tile_loop<1, true>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
     }
 
-    // 32x32 accumulator layout: lane holds column (lane % 32); register e holds row
-    // 8*(e/4) + 4*(lane/32) + e%4.  Y is written once and not re-read: streaming stores.
-    const uint32_t wm = wave >> 1, wn = wave & 1;
     int32_t *Y = y + (ym * m + static_cast<uint64_t>(tile_m) * BM + wm * 128) * n +
                  static_cast<uint64_t>(tile_n) * BN + wn * 128;
 #pragma unroll
@@ -412,17 +329,8 @@ extern "C" int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b, c
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if (fast) {
-            static bool attr_set = false;
-            constexpr size_t lds_bytes = LDS_BYTES;
-            if (!attr_set) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(mmi_mfma_256x256),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   static_cast<int>(lds_bytes));
-                if (e != hipSuccess) return static_cast<int>(e);
-                attr_set = true;
-            }
             const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
-            mmi_mfma_256x256<<<grid, 256, lds_bytes, s>>>(
+            mmi_mfma_256x256<<<grid, 256, 0, s>>>(
                 y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb,
                 static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), am0, bm0, ym0);
         } else {

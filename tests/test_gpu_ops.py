@@ -290,7 +290,7 @@ def test_matmul_integer_reference_kats():
 
 
 @pytest.mark.parametrize("m,k,n", [(37, 53, 29), (256, 64, 256), (256, 192, 512), (512, 1024, 256), (300, 64, 256),
-                                   (1, 4096, 1), (768, 128, 768)])
+                                   (1, 4096, 1), (768, 128, 768), (256, 256, 256), (512, 640, 256)])
 def test_matmul_integer_bit_exact_config_zero_points(m, k, n):
     a = np.random.default_rng(5).integers(0, 256, (m, k), dtype=np.uint8)
     b = np.random.default_rng(6).integers(-128, 128, (k, n), dtype=np.int8)
@@ -299,7 +299,7 @@ def test_matmul_integer_bit_exact_config_zero_points(m, k, n):
     assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
 
 
-@pytest.mark.parametrize("m,k,n", [(20, 33, 17), (256, 128, 256)])
+@pytest.mark.parametrize("m,k,n", [(20, 33, 17), (256, 128, 256), (256, 384, 512)])
 def test_matmul_integer_zero_point_variants_and_broadcast(m, k, n):
     rng = np.random.default_rng(6)
     a = rng.integers(0, 256, (2, 1, m, k), dtype=np.uint8)
