@@ -197,12 +197,14 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
         const uint32_t k_cp = (kt_ + 2) * BK;
         const bool more = kt_ + 2 < k_tiles;  // uniform
         auto slot = [&]<int s>() __attribute__((always_inline)) {
-            constexpr int ks = s / 16, o = s % 16, row = o / 4, col = o % 4, cur = ks & 1, nxt = cur ^ 1;
+            // rows walk the columns back and forth, so that only one operand changes between MFMAs
+            constexpr int ks = s / 16, o = s % 16, row = o / 4, col = (row & 1) ? 3 - o % 4 : o % 4;
+            constexpr int cur = ks & 1, nxt = cur ^ 1;
             if constexpr (s == 48) {
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of tile kt+1
                 __syncthreads();                                  // tile kt+1 complete, RB no longer read
             }
-            if constexpr (col == 0) fix_a(fa[cur][row], row);
+            if constexpr (o % 4 == 0) fix_a(fa[cur][row], row);
             if constexpr (row == 0) fix_b(fb[cur][col], kt_ * BK, ks);
             acc[row][col] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[cur][row], fb[cur][col], acc[row][col], 0, 0, 0);
             const uint8_t *src = ks == 3 ? WB : RB;
