@@ -6,7 +6,11 @@
 //
 // A workgroup of four wavefronts works on one kv head: wavefront w owns 32 query rows of one of
 // the query heads that share this kv head (GQA), so a K/V tile staged once in LDS serves up to
-// four query heads.  Keys are walked 64 at a time.  Both products run on the fp16/bf16 MFMA
+// four query heads.  Keys are walked 64 at a time; a tile of K and V rows is copied from global
+// memory straight into one of two LDS buffers (global_load_lds_dwordx4: lane L of a wavefront-wide
+// copy fills bytes 16 L .. 16 L + 15 behind a wave-uniform LDS base from an address of its own),
+// one tile ahead of its use, with the 16-byte chunks of a row XOR-swizzled so that the fragment
+// reads below are free of bank conflicts.  Both products run on the fp16/bf16 MFMA
 // (v_mfma_f32_32x32x16) in transposed form:
 //     S^T[key, q] = K[key, :] . Q[q, :]       A = K rows (LDS, 128-bit reads), B = Q rows (registers)
 //     O^T[d, q]  += V^T[d, key] . P^T[key, q] A = V columns (LDS, transposing 64-bit reads), B = P (registers)
@@ -26,14 +30,18 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int D = 128;
 constexpr int BN = 64;                 // keys per tile
-constexpr int ROW = 2 * D + 16;        // LDS pitch of a K row, bytes (272: conflict-free fragment reads)
-constexpr int VROW = 2 * D + 64;       // LDS pitch of a V row: four rows of 64 bytes cover all banks
-constexpr int TILE = BN * ROW;         // 17408
-constexpr int VTILE = BN * VROW;       // 20480
-constexpr int BUF_BYTES = TILE + VTILE;  // K tile + V tile
-constexpr int LDS_BYTES = 2 * BUF_BYTES;  // double buffered; reused for the output transposition
+constexpr int ROWB = 2 * D;            // bytes of a K or V row (unpadded in LDS)
+constexpr int TILE = BN * ROWB;        // 16384: one K or V tile
+constexpr int BUF_BYTES = 2 * TILE;    // K tile + V tile; two such buffers, reused for the output transposition
+constexpr int OROW = 2 * D + 16;       // LDS pitch of an output row during the transposition
 constexpr float kSlack = 6.0f;
 constexpr float kMinusBig = -1e30f;
+
+// LDS layout of a tile: the 16-byte chunk c of K row r sits at chunk position c ^ (r & 15), which
+// puts the 128-bit fragment reads of 8 or 16 consecutive rows on distinct banks; chunk c of V row r
+// sits at c ^ v_swizzle(r & 3), which does the same for the transposing 64-bit reads (4 rows x 32
+// or 64 bytes per group of lanes).
+__device__ __forceinline__ uint32_t v_swizzle(uint32_t r) { return 4 * (r & 1) + 10 * ((r >> 1) & 1); }
 
 struct alignas(16) Raw16 {
     uint32_t w[4];
@@ -79,7 +87,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                                                     uint32_t q_tiles, uint32_t head_chunks) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
     constexpr int ROWS = 32 * QS;   // query rows per workgroup
-    __shared__ __align__(16) uint8_t lds[LDS_BYTES];
+    __shared__ __align__(1024) uint8_t lds0[BUF_BYTES];
+    __shared__ __align__(1024) uint8_t lds1[BUF_BYTES];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t half = lane >> 5, l32 = lane & 31;
@@ -146,49 +155,45 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     const uint32_t qpos = base + r0 + l32;  // absolute position of this lane's query row
     const float c_log2e = a.scale * 1.4426950408889634f;
 
-    // staging: thread owns 16-byte chunk tid % 16 of key rows tid / 16 + 16 i
-    const uint32_t st_chunk = tid & 15, st_row = tid >> 4;
-    auto fetch = [&](uint32_t kt, Raw16(&kr)[4], Raw16(&vr)[4]) {
+    // Tile copies: wavefront w copies key rows 16 w .. 16 w + 15 of K and of V, four rows (1 KiB)
+    // per instruction; this lane brings chunk position lane % 16 of row 16 w + 4 i + lane / 16.
+    // A tile that lies inside the history or inside the new rows is addressed as a uniform base
+    // plus a per-lane byte offset prepared once (rows of the new tensors beyond the workgroup's last
+    // key are read along: they are masked); only a tile that straddles the two tensors or the end
+    // of the new rows computes its addresses row by row.
+    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t cp_row = 16 * wave_u + (lane >> 4);
+    const uint32_t v_lane = cp_row * ROWB + 16 * ((lane & 15) ^ v_swizzle(lane >> 4));
+    uint32_t k_lane[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t pos = kt * BN + st_row + 16 * i;
-            kr[i] = Raw16{{0, 0, 0, 0}};
-            vr[i] = Raw16{{0, 0, 0, 0}};
-            if (pos <= wg_last_key) {
-                if (pos < base) {
-                    const uint64_t off = static_cast<uint64_t>(pos) * D + st_chunk * 8;
-                    kr[i] = *reinterpret_cast<const Raw16 *>(k_hist + off);
-                    vr[i] = *reinterpret_cast<const Raw16 *>(v_hist + off);
-                } else {
-                    const uint64_t off = static_cast<uint64_t>(pos - base) * D + st_chunk * 8;
-                    kr[i] = *reinterpret_cast<const Raw16 *>(k_new + off);
-                    vr[i] = *reinterpret_cast<const Raw16 *>(v_new + off);
-                }
-            }
-        }
-    };
-    // The new rows that correspond to this workgroup's query rows are appended to the caches
-    // (once per kv head) from the registers that carry them to LDS: every such row is among the
-    // keys the workgroup needs.
-    const bool do_append = Kc && hc == 0;
-    const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
-    auto stage = [&](uint32_t kt, const Raw16(&kr)[4], const Raw16(&vr)[4]) {
-        uint8_t *ldsK = lds + (kt & 1) * BUF_BYTES, *ldsV = ldsK + TILE;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t off = (st_row + 16 * i) * ROW + st_chunk * 16;
-            *reinterpret_cast<Raw16 *>(ldsK + off) = kr[i];
-            *reinterpret_cast<Raw16 *>(ldsV + (st_row + 16 * i) * VROW + st_chunk * 16) = vr[i];
-        }
-        if (do_append && kt * BN + BN > own_lo) {
+    for (int i = 0; i < 4; ++i) k_lane[i] = (cp_row + 4 * i) * ROWB + 16 * ((lane & 15) ^ ((4 * i + (lane >> 4)) & 15));
+    const uint32_t total_keys = base + a.seq;
+    typedef const __attribute__((address_space(1))) void *GlobalPtr;
+    typedef __attribute__((address_space(3))) void *LdsPtr;
+    auto copy_tile = [&](uint32_t kt, uint8_t *buf) {
+        const uint32_t first = kt * BN;
+        const bool in_hist = first + BN <= base, in_new = first >= base && first + BN <= total_keys;
+        if (in_hist || in_new) {  // uniform
+            const uint64_t tile_off = static_cast<uint64_t>(in_hist ? first : first - base) * ROWB;
+            const uint8_t *kb_ = reinterpret_cast<const uint8_t *>(in_hist ? k_hist : k_new) + tile_off;
+            const uint8_t *vb_ = reinterpret_cast<const uint8_t *>(in_hist ? v_hist : v_new) + tile_off;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const uint32_t pos = kt * BN + st_row + 16 * i;
-                if (pos >= own_lo && pos < own_hi) {
-                    const uint64_t dst = (kv_head * a.cap + pos) * D + st_chunk * 8;
-                    *reinterpret_cast<Raw16 *>(Kc + dst) = kr[i];
-                    *reinterpret_cast<Raw16 *>(Vc + dst) = vr[i];
-                }
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + k_lane[i]), (LdsPtr)(buf + (4 * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(vb_ + v_lane + 4 * i * ROWB), (LdsPtr)(buf + TILE + (4 * wave_u + i) * 1024), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                uint32_t pos = first + cp_row + 4 * i;
+                pos = pos < total_keys ? pos : total_keys - 1;
+                const bool old = pos < base;
+                const uint64_t row_off = static_cast<uint64_t>(old ? pos : pos - base) * D;
+                const uint32_t kc = (lane & 15) ^ ((4 * i + (lane >> 4)) & 15), vc = (lane & 15) ^ v_swizzle(lane >> 4);
+                const T *ksrc = (old ? k_hist : k_new) + row_off + 8 * kc;
+                const T *vsrc = (old ? v_hist : v_new) + row_off + 8 * vc;
+                __builtin_amdgcn_global_load_lds((GlobalPtr)ksrc, (LdsPtr)(buf + (4 * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)vsrc, (LdsPtr)(buf + TILE + (4 * wave_u + i) * 1024), 16, 0, 0);
             }
         }
     };
@@ -201,15 +206,45 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     float m = 0.f, l = 0.f;
     bool fresh = true;
 
-    Raw16 kr[4], vr[4];
-    fetch(0, kr, vr);
-    stage(0, kr, vr);
-    __syncthreads();
+    copy_tile(0, lds0);
+    // The new rows that correspond to this workgroup's query rows are appended to the caches (once
+    // per kv head): thread owns 16-byte chunk tid % 16 of rows tid / 16 + 16 j.  These loads are in
+    // flight together with the query fragments and the first tiles.
+    if (Kc && hc == 0) {
+        const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
+#pragma unroll
+        for (int j = 0; j < ROWS / 16; ++j) {
+            const uint32_t pos = own_lo + (tid >> 4) + 16 * j;
+            if (pos < own_hi) {
+                const uint64_t off = static_cast<uint64_t>(pos - base) * D + (tid & 15) * 8;
+                const uint64_t dst = (kv_head * a.cap + pos) * D + (tid & 15) * 8;
+                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                const u32x4 k_row = *reinterpret_cast<const u32x4 *>(k_new + off);
+                const u32x4 v_row = *reinterpret_cast<const u32x4 *>(v_new + off);
+                *reinterpret_cast<u32x4 *>(Kc + dst) = k_row;
+                *reinterpret_cast<u32x4 *>(Vc + dst) = v_row;
+            }
+        }
+    }
+    // query fragments and tiles have landed (how many of the guarded stores above were issued is not
+    // known here, so everything is waited for)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
 
-    for (uint32_t kt = 0; kt < n_tiles; ++kt) {
-        if (kt + 1 < n_tiles) fetch(kt + 1, kr, vr);
+    // fragment addresses inside a buffer: K row l32 (+ 32 kb), chunk 2 kk + half; V see below
+    const uint32_t k_off = l32 * ROWB + 16 * (half ^ (l32 & 15));
+    // V piece of block db: row 4 half + r (+ 32 kb + 16 jj, + 8), chunk 4 db + cl; the swizzle leaves
+    // 4 db to bits 6-7 of the byte offset, so a block is reached by XOR with 64 db
+    const uint32_t s16 = lane & 15, v_r = s16 >> 2, v_cl = 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1);
+    const uint32_t v_off = TILE + (4 * half + v_r) * ROWB + 16 * (v_cl ^ v_swizzle(v_r)) + 8 * (s16 & 1);
 
-        const uint8_t *ldsK = lds + (kt & 1) * BUF_BYTES, *ldsV = ldsK + TILE;
+    auto tile = [&]<int P>(uint32_t kt) __attribute__((always_inline)) {
+        uint8_t *const buf = P ? lds1 : lds0, *const other = P ? lds0 : lds1;
+        // The copy of tile kt+1 into the other buffer (free since the barrier that ended tile kt-1)
+        // is issued behind this tile's first fragment reads: the compiler waits for every copy in
+        // flight before the first read of a buffer that a copy has written, and at that point
+        // none is.
+        if (kt >= wave_tiles && kt + 1 < n_tiles) copy_tile(kt + 1, other);
         if (kt < wave_tiles) {
             // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32.  Both
             // blocks of the tile are issued first; the softmax of a block then runs on the VALU
@@ -224,12 +259,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                 if (kb == 0 || second) {
 #pragma unroll
                     for (int kk = 0; kk < 8; ++kk) {
-                        const Raw16 kf = *reinterpret_cast<const Raw16 *>(ldsK + (32 * kb + l32) * ROW + (2 * kk + half) * 16);
+                        const Raw16 kf = *reinterpret_cast<const Raw16 *>(buf + 32 * kb * ROWB + (k_off ^ (32 * kk)));
                         s[kb] = Ops<T>::mfma(kf, qf[kk], s[kb]);
                     }
                 }
             }
-            const uint32_t tr_off = (4 * half + (lane & 15) / 4) * VROW + 2 * (16 * ((lane >> 4) & 1) + 4 * (lane & 3));
+            if (kt + 1 < n_tiles) copy_tile(kt + 1, other);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 if (kb == 1 && !second) break;
@@ -285,31 +320,36 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                 for (int db = 0; db < 4; ++db)
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
-                        const uint8_t *vp = ldsV + (32 * kb + 16 * jj) * VROW + 64 * db + tr_off;
-                        const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * VROW);
+                        const uint8_t *vp = buf + (32 * kb + 16 * jj) * ROWB + (v_off ^ (64 * db));
+                        const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * ROWB);
                         const Raw16 vf{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
                         o[db] = Ops<T>::mfma(vf, pf[jj], o[db]);
                     }
             }
         }
 
-        // the other buffer was last read in the previous iteration, which every wavefront left
-        // through the barrier below
-        if (kt + 1 < n_tiles) stage(kt + 1, kr, vr);
-        __syncthreads();
+        // This wavefront's copies of tile kt+1 have landed and its reads of this buffer are done;
+        // after the barrier that holds for the workgroup.
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    };
+    for (uint32_t kt = 0; kt < n_tiles; kt += 2) {
+        tile.template operator()<0>(kt);
+        if (kt + 1 < n_tiles) tile.template operator()<1>(kt + 1);
     }
 
     // ---- normalise, transpose O^T -> O through LDS, 128-bit row-contiguous stores
     l += __shfl_xor(l, 32, kWave);
     const float inv = 1.f / l;
-    uint8_t *ldsO = lds + wave * (32 * ROW);  // the K/V tiles are no longer needed (barrier above)
+    // the K/V tiles are no longer needed (barrier above, no copy in flight): two wavefronts per buffer
+    uint8_t *ldsO = (wave & 2 ? lds1 : lds0) + (wave & 1) * (32 * OROW);
     if (wave_active) {
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int e = 0; e < 16; e += 2) {
                 const uint32_t d = 32 * db + 8 * (e / 4) + 4 * half + (e % 4);
-                *reinterpret_cast<uint32_t *>(ldsO + l32 * ROW + 2 * d) = Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
+                *reinterpret_cast<uint32_t *>(ldsO + l32 * OROW + 2 * d) = Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
             }
     }
     __syncthreads();
@@ -320,10 +360,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             const uint32_t idx = lane + 64 * i, row = idx / 16, c = idx % 16;
             if (r0 + row < a.seq)
                 *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
-                    *reinterpret_cast<const Raw16 *>(ldsO + row * ROW + c * 16);
+                    *reinterpret_cast<const Raw16 *>(ldsO + row * OROW + c * 16);
         }
     }
-
 }
 
 template <class T, int HW>
