@@ -207,27 +207,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     bool fresh = true;
 
     copy_tile(0, lds0);
-    // The new rows that correspond to this workgroup's query rows are appended to the caches (once
-    // per kv head): thread owns 16-byte chunk tid % 16 of rows tid / 16 + 16 j.  These loads are in
-    // flight together with the query fragments and the first tiles.
-    if (Kc && hc == 0) {
-        const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
-#pragma unroll
-        for (int j = 0; j < ROWS / 16; ++j) {
-            const uint32_t pos = own_lo + (tid >> 4) + 16 * j;
-            if (pos < own_hi) {
-                const uint64_t off = static_cast<uint64_t>(pos - base) * D + (tid & 15) * 8;
-                const uint64_t dst = (kv_head * a.cap + pos) * D + (tid & 15) * 8;
-                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                const u32x4 k_row = *reinterpret_cast<const u32x4 *>(k_new + off);
-                const u32x4 v_row = *reinterpret_cast<const u32x4 *>(v_new + off);
-                *reinterpret_cast<u32x4 *>(Kc + dst) = k_row;
-                *reinterpret_cast<u32x4 *>(Vc + dst) = v_row;
-            }
-        }
-    }
-    // query fragments and tiles have landed (how many of the guarded stores above were issued is not
-    // known here, so everything is waited for)
+    // query fragments and tile 0 have landed
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 
@@ -338,6 +318,24 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
         if (kt + 1 < n_tiles) tile.template operator()<1>(kt + 1);
     }
 
+    // The new rows that correspond to this workgroup's query rows are appended to the caches (once
+    // per kv head): thread owns 16-byte chunk tid % 16 of rows tid / 16 + 16 j.  The loads are
+    // issued here and the stores follow the output write-out, which hides their latency.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const bool do_append = Kc && hc == 0;
+    const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
+    u32x4 ak[ROWS / 16], av[ROWS / 16];
+    if (do_append) {
+#pragma unroll
+        for (int j = 0; j < ROWS / 16; ++j) {
+            uint32_t pos = own_lo + (tid >> 4) + 16 * j;
+            pos = pos < own_hi ? pos : own_hi - 1;  // loads stay unconditional, the stores are guarded
+            const uint64_t off = static_cast<uint64_t>(pos - base) * D + (tid & 15) * 8;
+            ak[j] = *reinterpret_cast<const u32x4 *>(k_new + off);
+            av[j] = *reinterpret_cast<const u32x4 *>(v_new + off);
+        }
+    }
+
     // ---- normalise, transpose O^T -> O through LDS, 128-bit row-contiguous stores
     l += __shfl_xor(l, 32, kWave);
     const float inv = 1.f / l;
@@ -352,7 +350,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
                 *reinterpret_cast<uint32_t *>(ldsO + l32 * OROW + 2 * d) = Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
             }
     }
-    __syncthreads();
+    // (each wavefront reads back only what it wrote itself: no barrier)
     if (wave_active) {
         T *op = O + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + r0) * D;
 #pragma unroll
@@ -361,6 +359,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             if (r0 + row < a.seq)
                 *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
                     *reinterpret_cast<const Raw16 *>(ldsO + row * OROW + c * 16);
+        }
+    }
+    if (do_append) {
+#pragma unroll
+        for (int j = 0; j < ROWS / 16; ++j) {
+            const uint32_t pos = own_lo + (tid >> 4) + 16 * j;
+            if (pos < own_hi) {
+                const uint64_t dst = (kv_head * a.cap + pos) * D + (tid & 15) * 8;
+                *reinterpret_cast<u32x4 *>(Kc + dst) = ak[j];
+                *reinterpret_cast<u32x4 *>(Vc + dst) = av[j];
+            }
         }
     }
 }
