@@ -60,6 +60,10 @@ def lib() -> C.CDLL:
             raise RgHipError(
                 f"{LIB_PATH} is missing: build it with `python -m refactorgraph_amd.build` "
                 "(there is no CPU or PyTorch fallback)")
+        # PyTorch carries its own copy of the HIP runtime and owns the device memory this package is
+        # handed: it has to be in the process first, so that the library binds to that same copy
+        # (loaded the other way round, launches fail with "no ROCm-capable device").
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)  # AttributeError if the library does not export it

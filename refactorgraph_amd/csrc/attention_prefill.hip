@@ -6,7 +6,7 @@
 //
 // A workgroup of four wavefronts works on one kv head: wavefront w owns 32 query rows of one of
 // the query heads that share this kv head (GQA), so a K/V tile staged once in LDS serves up to
-// four query heads.  Keys are walked 64 at a time; a tile of K and V rows is copied from global
+// four query heads.  Keys are walked 32 at a time; a tile of K and V rows is copied from global
 // memory straight into one of two LDS buffers (global_load_lds_dwordx4: lane L of a wavefront-wide
 // copy fills bytes 16 L .. 16 L + 15 behind a wave-uniform LDS base from an address of its own),
 // one tile ahead of its use, with the 16-byte chunks of a row XOR-swizzled so that the fragment
@@ -29,11 +29,13 @@ typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int D = 128;
-constexpr int BN = 64;                 // keys per tile
+constexpr int BN = 32;                 // keys per tile (32 or 64); 32 keeps the kernel within the registers and
+                                       // LDS of three workgroups per CU, which hides more of the memory latency
+constexpr int KB = BN / 32;            // blocks of 32 keys per tile
+constexpr int CPI = BN / 16;           // K (and V) copy instructions per wavefront and tile
 constexpr int ROWB = 2 * D;            // bytes of a K or V row (unpadded in LDS)
 constexpr int TILE = BN * ROWB;        // 16384: one K or V tile
 constexpr int BUF_BYTES = 2 * TILE;    // K tile + V tile; two such buffers, reused for the output transposition
-constexpr int OROW = 2 * D + 16;       // LDS pitch of an output row during the transposition
 constexpr float kSlack = 6.0f;
 constexpr float kMinusBig = -1e30f;
 
@@ -83,7 +85,7 @@ template <> struct Ops<__hip_bfloat16> {
 // HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
 // query sub-tiles of the same heads.
 template <class T, int HW>
-__global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint32_t group,
+__global__ __launch_bounds__(256, 3) void attn_prefill(const PrefillArgs a, uint32_t group,
                                                     uint32_t q_tiles, uint32_t head_chunks) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
     constexpr int ROWS = 32 * QS;   // query rows per workgroup
@@ -162,11 +164,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     // key are read along: they are masked); only a tile that straddles the two tensors or the end
     // of the new rows computes its addresses row by row.
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t cp_row = 16 * wave_u + (lane >> 4);
+    const uint32_t cp_row = (BN / 4) * wave_u + (lane >> 4);
     const uint32_t v_lane = cp_row * ROWB + 16 * ((lane & 15) ^ v_swizzle(lane >> 4));
-    uint32_t k_lane[4];
+    uint32_t k_lane[CPI];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) k_lane[i] = (cp_row + 4 * i) * ROWB + 16 * ((lane & 15) ^ ((4 * i + (lane >> 4)) & 15));
+    for (int i = 0; i < CPI; ++i) k_lane[i] = (cp_row + 4 * i) * ROWB + 16 * ((lane & 15) ^ ((cp_row + 4 * i) & 15));
     const uint32_t total_keys = base + a.seq;
     typedef const __attribute__((address_space(1))) void *GlobalPtr;
     typedef __attribute__((address_space(3))) void *LdsPtr;
@@ -178,22 +180,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             const uint8_t *kb_ = reinterpret_cast<const uint8_t *>(in_hist ? k_hist : k_new) + tile_off;
             const uint8_t *vb_ = reinterpret_cast<const uint8_t *>(in_hist ? v_hist : v_new) + tile_off;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + k_lane[i]), (LdsPtr)(buf + (4 * wave_u + i) * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((GlobalPtr)(vb_ + v_lane + 4 * i * ROWB), (LdsPtr)(buf + TILE + (4 * wave_u + i) * 1024), 16, 0, 0);
+            for (int i = 0; i < CPI; ++i) {
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + k_lane[i]), (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(vb_ + v_lane + 4 * i * ROWB), (LdsPtr)(buf + TILE + (CPI * wave_u + i) * 1024), 16, 0, 0);
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < CPI; ++i) {
                 uint32_t pos = first + cp_row + 4 * i;
                 pos = pos < total_keys ? pos : total_keys - 1;
                 const bool old = pos < base;
                 const uint64_t row_off = static_cast<uint64_t>(old ? pos : pos - base) * D;
-                const uint32_t kc = (lane & 15) ^ ((4 * i + (lane >> 4)) & 15), vc = (lane & 15) ^ v_swizzle(lane >> 4);
+                const uint32_t kc = (lane & 15) ^ ((cp_row + 4 * i) & 15), vc = (lane & 15) ^ v_swizzle(lane >> 4);
                 const T *ksrc = (old ? k_hist : k_new) + row_off + 8 * kc;
                 const T *vsrc = (old ? v_hist : v_new) + row_off + 8 * vc;
-                __builtin_amdgcn_global_load_lds((GlobalPtr)ksrc, (LdsPtr)(buf + (4 * wave_u + i) * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((GlobalPtr)vsrc, (LdsPtr)(buf + TILE + (4 * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)ksrc, (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)vsrc, (LdsPtr)(buf + TILE + (CPI * wave_u + i) * 1024), 16, 0, 0);
             }
         }
     };
@@ -226,14 +228,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
         // none is.
         if (kt >= wave_tiles && kt + 1 < n_tiles) copy_tile(kt + 1, other);
         if (kt < wave_tiles) {
-            // S^T block kb: keys 64 kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32.  Both
-            // blocks of the tile are issued first; the softmax of a block then runs on the VALU
-            // while the matrix core still works on the next product (S^T of block 1, or the PV
-            // update of block 0).  A block that lies entirely above the diagonal is skipped.
-            const bool second = kt * BN + 32 <= base + r0 + 31;
-            f16v s[2];
+            // S^T block kb: keys BN kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32.  With two
+            // blocks per tile (BN = 64) both are issued first; the softmax of a block then runs on
+            // the VALU while the matrix core still works on the next product (S^T of block 1, or
+            // the PV update of block 0), and a block entirely above the diagonal is skipped.
+            const bool second = KB > 1 && kt * BN + 32 <= base + r0 + 31;
+            f16v s[KB];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
                 if (kb == 0 || second) {
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             }
             if (kt + 1 < n_tiles) copy_tile(kt + 1, other);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < KB; ++kb) {
                 if (kb == 1 && !second) break;
                 // scale, causal mask (only blocks that reach past the wavefront's first query position)
                 const bool need_mask = kt * BN + 32 * kb + 31 > base + r0;
@@ -340,14 +342,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
     l += __shfl_xor(l, 32, kWave);
     const float inv = 1.f / l;
     // the K/V tiles are no longer needed (barrier above, no copy in flight): two wavefronts per buffer
-    uint8_t *ldsO = (wave & 2 ? lds1 : lds0) + (wave & 1) * (32 * OROW);
+    uint8_t *ldsO = (wave & 2 ? lds1 : lds0) + (wave & 1) * (32 * ROWB);  // chunk c of row r at chunk position c ^ (r & 15)
     if (wave_active) {
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int e = 0; e < 16; e += 2) {
                 const uint32_t d = 32 * db + 8 * (e / 4) + 4 * half + (e % 4);
-                *reinterpret_cast<uint32_t *>(ldsO + l32 * OROW + 2 * d) = Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
+                *reinterpret_cast<uint32_t *>(ldsO + l32 * ROWB + ((2 * d) ^ (16 * (l32 & 15)))) =
+                    Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
             }
     }
     // (each wavefront reads back only what it wrote itself: no barrier)
@@ -358,7 +361,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, uint
             const uint32_t idx = lane + 64 * i, row = idx / 16, c = idx % 16;
             if (r0 + row < a.seq)
                 *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
-                    *reinterpret_cast<const Raw16 *>(ldsO + row * OROW + c * 16);
+                    *reinterpret_cast<const Raw16 *>(ldsO + row * ROWB + 16 * (c ^ (row & 15)));
         }
     }
     if (do_append) {
