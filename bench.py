@@ -43,6 +43,7 @@ MEASURED_TRAFFIC = {
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
     "matmul_integer": (2 * 49313 + 65638) * 1024,
     "attention_prefill": (2 * 99826 + 196608) * 1024,
+    "cast": (2 * 32784 + 32768) * 1024,
 }
 
 
@@ -358,6 +359,22 @@ def main():
             e["cpu_baseline"] = {"value": round(4096 * 4096 * 5 / dt / 1e9, 3), "unit": "GB/s", "cores": 1,
                                  "kind": "port", "sample": f"the whole [4096,4096] tensor once ({dt:.2f} s)"}
         ops_out["dynamic_quantize_linear"] = e
+        del xs, ys
+
+    if want("cast"):
+        # the Cast either side of the fp16 operators: f32 -> fp16 of an activation tensor (6 B per element)
+        nb = 6  # 6 x 100 MB
+        xs = [torch.randn((32, 128, 4096), device=dev) for _ in range(nb)]
+        ys = [torch.empty((32, 128, 4096), device=dev, dtype=torch.float16) for _ in range(nb)]
+        wall, dms, mode = time_steps(torch, lambda i: ops.cast(xs[i], torch.float16, out=ys[i]), steps, warmup, nb)
+        cast_bytes = 32 * 128 * 4096 * 6
+        e = hbm_entry(cast_bytes, dms, "cast")
+        e.update(workload="Cast f32->fp16 [32,128,4096]", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn = xs[0].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.cast(xn, "f32", "fp16"), cast_bytes, "the whole tensor once")
+        ops_out["cast"] = e
         del xs, ys
 
     if want("matmul_integer"):

@@ -12,7 +12,7 @@
  *   - every pointer named y/x/a/b/... is a DEVICE address unless said otherwise;
  *   - `dtype` is the reference's DataType code
  *     (src/00common/include/common/data_type.h:19-36): F32=1 U8=2 I8=3 U16=4
- *     I16=5 I32=6 I64=7 FP16=10 F64=11 BF16=16;
+ *     I16=5 I32=6 I64=7 Bool=9 FP16=10 F64=11 U32=12 U64=13 BF16=16;
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream, which
  *     is what a Routine uses: src/03runtime/src/stream.cc:60-69);
  *   - launchers only enqueue work: no synchronisation, no allocation, no throw;
@@ -31,7 +31,7 @@ extern "C" {
 
 enum {
     RG_F32 = 1, RG_U8 = 2, RG_I8 = 3, RG_U16 = 4, RG_I16 = 5, RG_I32 = 6, RG_I64 = 7,
-    RG_FP16 = 10, RG_F64 = 11, RG_BF16 = 16,
+    RG_BOOL = 9, RG_FP16 = 10, RG_F64 = 11, RG_U32 = 12, RG_U64 = 13, RG_BF16 = 16,
 };
 
 enum {
@@ -110,6 +110,18 @@ int rg_hip_dequantize_linear(float *y, const void *x, const float *scale, const 
 size_t rg_hip_dynamic_quantize_linear_workspace(size_t size);
 int rg_hip_dynamic_quantize_linear(uint8_t *y, float *scale, uint8_t *zero_point, const float *x,
                                    size_t size, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Cast -------------------------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/cast/cuda_kernel.cc:38-124 (a kernel generated and compiled at
+ * run time per type pair); arithmetic contract: for U8/U16/U32/U64/I8/I16/I32/I64/F32/F64/Bool the
+ * `static_cast<U>(a)` of src/04kernel/src/kernels/cast/cpu_kernel.cc:28-40; for pairs with FP16 or
+ * BF16 the expressions of cuda_kernel.cc:55-96 (to FP16/BF16: floats round to nearest even, a double
+ * through float first, integers are taken as `int` and rounded toward zero; from FP16/BF16 to
+ * integers: truncated as `int`), except that `-> Bool` is `x != 0` for every source type (the
+ * reference's generated code tests `== 0` for floating sources).  Bool is one byte holding 0 or 1.
+ * Out-of-range float -> integer conversions saturate.  from_dtype == to_dtype copies (nothing is
+ * done when y == x).  y, x: `size` elements each. */
+int rg_hip_cast(void *y, const void *x, size_t size, int from_dtype, int to_dtype, void *stream);
 
 /* ---- MatMulInteger -----------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust

@@ -257,3 +257,90 @@ def rope(x, pos, theta=10000.0, threads=1):
     y = np.empty_like(x)
     lib().oracle_rope_f32(_p(y), _p(x), _p(pos), per_batch, batch, seq, heads, D, float(theta), threads)
     return y
+
+
+# ---------------------------------------------------------------------------------------------
+# Cast.  numpy restatement (no C): the conversions are single machine operations.
+#   - types of the reference's CPU kernel (u8 u16 u32 u64 i8 i16 i32 i64 f32 f64 bool):
+#     `static_cast<U>(a)` of src/04kernel/src/kernels/cast/cpu_kernel.cc:28-40 = numpy `astype`
+#     (C conversion rules: integer narrowing wraps, float -> integer truncates, integer -> float
+#     rounds to nearest even), `-> bool` is `a != 0`;
+#   - fp16 / bf16: the expressions the reference's CUDA kernel generates,
+#     src/04kernel/src/kernels/cast/cuda_kernel.cc:55-96: float/double -> fp16|bf16 round to
+#     nearest even (a double through float first); integer -> fp16|bf16 takes the value as `int`
+#     and rounds toward zero; fp16|bf16 -> integer truncates as `int`; fp16 <-> bf16 through float.
+#     `-> bool` from a floating source is written `x == 0` there (true for zeros): NOT followed,
+#     `x != 0` is used for every source (cast_bool_reference_literal keeps the literal form).
+# bf16 tensors are uint16 arrays of bit patterns (numpy has no bfloat16).
+CAST_TYPES = ("u8", "u16", "u32", "u64", "i8", "i16", "i32", "i64", "f32", "f64", "bool", "fp16", "bf16")
+_CAST_NP = {"u8": np.uint8, "u16": np.uint16, "u32": np.uint32, "u64": np.uint64, "i8": np.int8,
+            "i16": np.int16, "i32": np.int32, "i64": np.int64, "f32": np.float32, "f64": np.float64,
+            "bool": np.bool_, "fp16": np.float16, "bf16": np.uint16}
+
+
+def _bf16_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def _f32_to_bf16_rn(f):
+    u = np.ascontiguousarray(f, np.float32).view(np.uint32)
+    rounded = (u + (0x7FFF + ((u >> 16) & 1))) >> 16          # nearest, ties to even
+    nan = np.isnan(f)
+    return np.where(nan, (u >> 16) | 0x40, rounded).astype(np.uint16)
+
+
+def _int_to_f32_rz(v):
+    """int32 values -> float32 rounded toward zero."""
+    f = v.astype(np.float32)                                     # nearest
+    away = np.abs(f.astype(np.float64)) > np.abs(v.astype(np.float64))
+    return np.where(away, np.nextafter(f, np.float32(0)), f).astype(np.float32)
+
+
+def _f32_to_fp16_rz(f):
+    with np.errstate(over="ignore"):
+        h = f.astype(np.float16)                                 # nearest, may overflow to inf
+    away = np.abs(h.astype(np.float64)) > np.abs(f.astype(np.float64))
+    return np.where(away, np.nextafter(h, np.float16(0)), h).astype(np.float16)
+
+
+def cast(x, src, dst):
+    """x: numpy array holding `src` values (CAST_TYPES names); returns the `dst` array."""
+    x = np.ascontiguousarray(x, _CAST_NP[src])
+    narrow = ("fp16", "bf16")
+    if src == dst:
+        return x.copy()
+    if src not in narrow and dst not in narrow:
+        if dst == "bool":
+            return x != 0
+        with np.errstate(invalid="ignore", over="ignore"):
+            return x.astype(_CAST_NP[dst])
+    if src in narrow:
+        f = x.astype(np.float32) if src == "fp16" else _bf16_to_f32(x)
+        if dst == "bool":
+            return f != 0
+        if dst == "fp16":
+            with np.errstate(over="ignore"):
+                return f.astype(np.float16)
+        if dst == "bf16":
+            return _f32_to_bf16_rn(f)
+        if dst in ("f32", "f64"):
+            return f.astype(_CAST_NP[dst])
+        with np.errstate(invalid="ignore"):
+            return np.trunc(f).astype(np.int32).astype(_CAST_NP[dst])   # as int, then the implicit conversion
+    # dst narrow, src one of the CPU types
+    if src in ("f32", "f64"):
+        with np.errstate(over="ignore"):
+            f = x.astype(np.float32)
+            return f.astype(np.float16) if dst == "fp16" else _f32_to_bf16_rn(f)
+    v = x.astype(np.int32)                                        # bool -> 0/1; wider integers wrap, as `int`
+    f = _int_to_f32_rz(v)
+    if dst == "fp16":
+        return _f32_to_fp16_rz(f)
+    return (f.view(np.uint32) >> 16).astype(np.uint16)            # dropping the low half is rounding toward zero
+
+
+def cast_bool_reference_literal(x, src):
+    """The `-> Bool` expression the reference's CUDA kernel generates for floating sources
+    (cuda_kernel.cc:73-88): `x == 0`.  Kept as a named fixture of the defect; not used as oracle."""
+    f = cast(x, src, "f64") if src in ("fp16", "bf16") else np.asarray(x)
+    return f == 0

@@ -12,6 +12,7 @@ HOST_TESTS_PATH = os.path.join(PKG, "lib", "rg_host_tests")
 
 # reference DataType codes (src/00common/include/common/data_type.h:19-36 of the reference)
 F32, U8, I8, U16, I16, I32, I64, FP16, F64, BF16 = 1, 2, 3, 4, 5, 6, 7, 10, 11, 16
+BOOL, U32, U64 = 9, 12, 13
 MMI_A_ZP_SCALAR, MMI_B_ZP_SCALAR = 1, 2
 
 _sz, _vp, _i, _u, _f = C.c_size_t, C.c_void_p, C.c_int, C.c_uint, C.c_float
@@ -36,6 +37,7 @@ SIGNATURES = {
     "rg_hip_dequantize_linear": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _i, _vp]),
     "rg_hip_dynamic_quantize_linear_workspace": (_sz, [_sz]),
     "rg_hip_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp]),
+    "rg_hip_cast": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rg_hip_matmul_integer_workspace": (_sz, [_sz, _sz, _sz, _sz, _u]),
     "rg_hip_matmul_integer": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
     "rg_hip_attention_kvcache_workspace": (_sz, [_sz, _sz, _sz, _sz, _sz, _sz]),

@@ -44,6 +44,14 @@ namespace refactor::kernel {
         std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
     };
 
+    // inputs: x; outputs: y of the requested type, same shape
+    // (src/04kernel/include/kernel/collectors/cast.h:8-14)
+    struct CastCollector final : public InfoCollector {
+        constexpr explicit CastCollector(hardware::Device::Type target) noexcept
+            : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
     // inputs: query, key, value [, past_seq_len [, k_cache, v_cache]]; outputs: output
     // [, k_cache, v_cache] (src/08-01llm/README.md:29-63).
     struct AttentionCollector final : public InfoCollector {

@@ -71,6 +71,20 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // mirrors CastCuda (src/04kernel/src/kernels/cast/cuda_kernel.hh:9-23); no run-time compilation:
+    // every type pair is a precompiled kernel of the device library
+    struct CastHip final : public Kernel {
+        DataType from, to;
+        size_t size;
+
+        CastHip(decltype(from), decltype(to), decltype(size)) noexcept;
+        static KernelBox build(Tensor const &, Tensor const &) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct AttentionHip final : public Kernel {
         // the reference's parameter block (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-14)
         // plus what it leaves to the run time: where past_seq_len comes from

@@ -104,6 +104,24 @@ namespace refactor::kernel {
     }
 
     std::vector<KernelBox>
+    CastCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
+        // src/04kernel/src/collectors/cast.cc:10-33
+        auto const &from = inputs[0].get();
+        auto const &to = outputs[0].get();
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(CastHip::build(from, to))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
     AttentionCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
         auto const &query = inputs[0].get();
         auto const &key = inputs[1].get();

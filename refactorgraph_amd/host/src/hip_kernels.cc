@@ -167,6 +167,28 @@ namespace refactor::kernel {
         return {std::move(routine), workspace};
     }
 
+    // ------------------------------------------------------------------ Cast
+
+    CastHip::CastHip(decltype(from) from_, decltype(to) to_, decltype(size) size_) noexcept
+        : Kernel(), from(from_), to(to_), size(size_) {}
+    KernelBox CastHip::build(Tensor const &from, Tensor const &to) noexcept {
+        auto castable = [](DataType t) {
+            return t.isCpuNumberic() || t == DataType::Bool || t == DataType::FP16 || t == DataType::BF16;
+        };
+        if (!castable(from.dataType) || !castable(to.dataType)) { return nullptr; }
+        if (from.elementsSize() != to.elementsSize()) { return nullptr; }
+        return std::make_unique<CastHip>(from.dataType, to.dataType, from.elementsSize());
+    }
+    size_t CastHip::typeId() noexcept { return idOf<CastHip>(); }
+    size_t CastHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view CastHip::description() const noexcept { return "Performing cast operation on AMD gfx950"; }
+    RoutineWorkspace CastHip::lower(Resources &) const {
+        return [from = from, to = to, size = size](Resources &, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_cast(outputs[0], inputs[0], size, static_cast<int>(from.internal),
+                                 static_cast<int>(to.internal), nullptr));
+        };
+    }
+
     // ------------------------------------------------------------------ Attention
 
     HipAttentionState::HipAttentionState() : _counters(nullptr) {

@@ -19,8 +19,10 @@ _T2CODE = {
     torch.uint8: abi.U8, torch.int8: abi.I8, torch.int16: abi.I16, torch.int32: abi.I32,
     torch.int64: abi.I64,
 }
-if hasattr(torch, "uint16"):
-    _T2CODE[torch.uint16] = abi.U16
+_T2CODE[torch.bool] = abi.BOOL
+for _name, _code in (("uint16", abi.U16), ("uint32", abi.U32), ("uint64", abi.U64)):
+    if hasattr(torch, _name):
+        _T2CODE[getattr(torch, _name)] = _code
 
 
 def _stream():
@@ -101,6 +103,16 @@ def dynamic_quantize_linear(x, out=None, workspace=None):
     check(lib().rg_hip_dynamic_quantize_linear(_ptr(y), _ptr(scale), _ptr(zp), _ptr(x), n, _ptr(ws), ws.numel(),
                                                _stream()), "rg_hip_dynamic_quantize_linear")
     return y, scale, zp
+
+
+def cast(x, dtype, out=None):
+    """Element-wise conversion of x to `dtype` (a torch dtype)."""
+    _need_gpu(x)
+    assert x.is_contiguous()
+    y = torch.empty(x.shape, dtype=dtype, device=x.device) if out is None else out
+    assert y.dtype == dtype and y.numel() == x.numel() and y.is_contiguous()
+    check(lib().rg_hip_cast(_ptr(y), _ptr(x), x.numel(), _T2CODE[x.dtype], _T2CODE[dtype], _stream()), "rg_hip_cast")
+    return y
 
 
 def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):

@@ -199,6 +199,19 @@ static void collectorsSelectOrDecline() {
     EXPECT(DynamicQuantizeLinearCollector(T::Amd).filter({*x8}, {*yq, *s1, *zq}).empty());
     EXPECT(DynamicQuantizeLinearCollector(T::Cpu).filter({*xf}, {*yq, *s1, *zq}).empty());
 
+    // Cast: every pair of numeric types has a kernel; strings and complex numbers do not
+    auto c8 = Tensor::share(DataType::I8, Shape{4, 6});
+    auto ch = Tensor::share(DataType::FP16, Shape{4, 6});
+    auto cb = Tensor::share(DataType::Bool, Shape{4, 6});
+    auto cs = Tensor::share(DataType::String, Shape{4, 6});
+    auto ck = CastCollector(T::Amd).filter({*xf}, {*c8});
+    EXPECT(ck.size() == 1 && static_cast<CastHip const &>(*ck[0]).size == 24 &&
+           static_cast<CastHip const &>(*ck[0]).from == DataType::F32 && static_cast<CastHip const &>(*ck[0]).to == DataType::I8);
+    EXPECT(CastCollector(T::Amd).filter({*ch}, {*cb}).size() == 1);
+    EXPECT(CastCollector(T::Amd).filter({*cs}, {*c8}).empty());
+    EXPECT(CastCollector(T::Amd).filter({*xf}, {*Tensor::share(DataType::I8, Shape{5})}).empty());
+    EXPECT(CastCollector(T::Cpu).filter({*xf}, {*c8}).empty());
+
     // Attention: parameter block from the tensors; head-count and dtype rules
     auto q = Tensor::share(DataType::FP16, Shape{2, 8, 1, 128});
     auto kv = Tensor::share(DataType::FP16, Shape{2, 2, 1, 128});
@@ -415,6 +428,57 @@ static void dynamicQuantizeLinearHip() {
     EXPECT(DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*xh}, {*y, *scale, *zp}).empty());
 }
 
+static void castHip() {
+    runtime::Resources res;
+    auto &dev = amd();
+    {// src/04kernel/test/kernels/cast/test_cpu.cpp:8-33 and test_cuda.cpp: F64 iota [2,3,4,5] -> I8, y[i] == i
+        auto x = Tensor::share(DataType::F64, Shape{2, 3, 4, 5});
+        auto y = Tensor::share(DataType::I8, Shape{2, 3, 4, 5});
+        auto kernels = CastCollector(Device::Type::Amd).filter({*x}, {*y});
+        EXPECT(kernels.size() == 1);
+        auto routine = kernels[0]->lower(res).routine;
+        std::vector<double> x_(x->elementsSize());
+        std::iota(x_.begin(), x_.end(), 0);
+        auto mx = dev.malloc(x_.size() * 8), my = dev.malloc(x_.size());
+        mx->copyFromHost(x_.data());
+        void const *inputs[]{*mx};
+        void *outputs[]{*my};
+        routine(res, nullptr, inputs, outputs);
+        std::vector<int8_t> y_(x_.size());
+        my->copyToHost(y_.data());
+        for (size_t i = 0; i < y_.size(); ++i) EXPECT(y_[i] == static_cast<int8_t>(i));
+    }
+    {// float -> int32 -> float on values the reference's static_cast defines; odd length
+        std::mt19937 rng(5);
+        std::uniform_real_distribution<float> g(-1e6f, 1e6f);
+        std::vector<float> x_(10007);
+        for (auto &v : x_) v = g(rng);
+        auto x = Tensor::share(DataType::F32, Shape{10007});
+        auto y = Tensor::share(DataType::I32, Shape{10007});
+        auto k1 = CastCollector(Device::Type::Amd).filter({*x}, {*y});
+        auto k2 = CastCollector(Device::Type::Amd).filter({*y}, {*x});
+        EXPECT(k1.size() == 1 && k2.size() == 1);
+        auto mx = dev.malloc(x_.size() * 4), my = dev.malloc(x_.size() * 4), mz = dev.malloc(x_.size() * 4);
+        mx->copyFromHost(x_.data());
+        {
+            void const *inputs[]{*mx};
+            void *outputs[]{*my};
+            k1[0]->lower(res).routine(res, nullptr, inputs, outputs);
+        }
+        {
+            void const *inputs[]{*my};
+            void *outputs[]{*mz};
+            k2[0]->lower(res).routine(res, nullptr, inputs, outputs);
+        }
+        std::vector<int32_t> y_(x_.size());
+        std::vector<float> z_(x_.size());
+        my->copyToHost(y_.data());
+        mz->copyToHost(z_.data());
+        for (size_t i = 0; i < x_.size(); ++i)
+            EXPECT(y_[i] == static_cast<int32_t>(x_[i]) && z_[i] == static_cast<float>(y_[i]));
+    }
+}
+
 static void dequantizeLinearHip() {
     runtime::Resources res;
     auto &dev = amd();
@@ -585,6 +649,7 @@ int main(int argc, char **argv) {
         RUN(matMulIntegerHip);
         RUN(dequantizeLinearHip);
         RUN(dynamicQuantizeLinearHip);
+        RUN(castHip);
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
     }

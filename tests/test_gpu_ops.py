@@ -490,3 +490,99 @@ def test_attention_prefill_config_sample():
     for b, h in pairs:
         assert np.max(np.abs(o[b, h] - ref_o[b, h])) <= ABS_F16
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
+# ------------------------------------------------------------------ Cast
+_CAST_TORCH = {"u8": torch.uint8, "i8": torch.int8, "i16": torch.int16, "i32": torch.int32, "i64": torch.int64,
+               "f32": torch.float32, "f64": torch.float64, "bool": torch.bool, "fp16": torch.float16,
+               "bf16": torch.bfloat16, "u16": torch.uint16, "u32": torch.uint32, "u64": torch.uint64}
+_CAST_BITS = {"u8": 8, "i8": 8, "u16": 16, "i16": 16, "u32": 32, "i32": 32, "u64": 64, "i64": 64}
+
+
+def _cast_input(src, dst, n, rng):
+    """Values of type `src` whose conversion to `dst` is defined (float -> integer stays inside
+    the target's range; everything else is unrestricted)."""
+    np_t = oracle._CAST_NP[src]
+    if src == "bool":
+        return rng.integers(0, 2, n).astype(np.bool_)
+    if src in _CAST_BITS:
+        info = np.iinfo(np_t)
+        x = rng.integers(info.min, info.max, n, dtype=np_t, endpoint=True)
+        x[:4] = [info.min, info.max, 0, 1]
+        return x
+    # floating sources
+    if dst in _CAST_BITS:
+        bits = _CAST_BITS[dst]
+        hi = float(2 ** (bits - (0 if dst[0] == "u" else 1)))
+        hi = min(hi, 60000.0 if src == "fp16" else hi, 2.0 ** 62)
+        lo = 0.0 if dst[0] == "u" else -hi
+        f = rng.uniform(lo * 0.999, hi * 0.999, n)
+        if src in ("fp16", "bf16"):
+            hi, lo = min(hi, 2.0 ** 31) * 0.99, max(lo, -2.0 ** 31) * 0.99   # these go through `int`
+            f = rng.uniform(lo, hi, n)
+    else:
+        f = rng.standard_normal(n) * np.exp(rng.uniform(-20, 12, n))
+        f[:6] = [0.0, -0.0, 2049.0, 2051.0, 65519.9, 65520.0]
+    if src == "f64":
+        return f.astype(np.float64)
+    f32 = f.astype(np.float32)
+    if src == "f32":
+        return f32
+    with np.errstate(over="ignore"):
+        return f32.astype(np.float16) if src == "fp16" else oracle.cast(f32, "f32", "bf16")
+
+
+def _cast_to_torch(x, name):
+    if name == "bf16":
+        return dev(x).view(torch.bfloat16)
+    return dev(x)
+
+
+def _cast_bits(t, name):
+    """Result tensor -> numpy array comparable bit for bit."""
+    if name == "bf16":
+        return host(t.view(torch.uint16))
+    a = host(t)
+    return a.view(np.uint16) if name == "fp16" else a
+
+
+@pytest.mark.parametrize("src", oracle.CAST_TYPES)
+def test_cast_all_pairs_bit_exact(src):
+    rng = np.random.default_rng(hash(src) % 1000)
+    for dst in oracle.CAST_TYPES:
+        n = 10007                                     # odd: vector body and scalar tail
+        x = _cast_input(src, dst, n, rng)
+        want = oracle.cast(x, src, dst)
+        got = _cast_bits(ops.cast(_cast_to_torch(x, src), _CAST_TORCH[dst]), dst)
+        want = want.view(np.uint16) if dst == "fp16" else want
+        assert got.shape == want.shape and np.array_equal(got, want), (src, dst)
+
+
+def test_cast_reference_kat_and_edges():
+    x = np.arange(120, dtype=np.float64).reshape(2, 3, 4, 5)      # cast/test_cpu.cpp
+    assert np.array_equal(host(ops.cast(dev(x), torch.int8)).reshape(-1), np.arange(120))
+    # misaligned views (scalar path), same-type copy, in-place no-op
+    base = dev(np.arange(1, 4098, dtype=np.float32))
+    view = base[1:]
+    assert np.array_equal(host(ops.cast(view, torch.float16)).view(np.uint16),
+                          oracle.cast(host(view), "f32", "fp16").view(np.uint16))
+    out = torch.empty(4099, dtype=torch.int32, device="cuda")[3:]
+    ops.cast(view, torch.int32, out=out)
+    assert np.array_equal(host(out), host(view).astype(np.int32))
+    assert np.array_equal(host(ops.cast(view, torch.float32)), host(view))
+    same = ops.cast(view, torch.float32, out=view)
+    assert same.data_ptr() == view.data_ptr() and np.array_equal(host(view), np.arange(2, 4098, dtype=np.float32))
+    # double -> half goes through float (two roundings, like the reference's expression)
+    assert host(ops.cast(dev(np.array([1 + 2.0 ** -11 + 2.0 ** -26])), torch.float16)).view(np.uint16).tolist() == [0x3C00]
+    # integers are taken as `int` and rounded toward zero
+    assert host(ops.cast(dev(np.array([2049, 2051, -2049, 70000, 16777217], np.int32)), torch.float16)).tolist() == \
+        [2048.0, 2050.0, -2048.0, 65504.0, 65504.0]
+    assert host(ops.cast(dev(np.array([3000000000], np.uint32)), torch.float16)).tolist() == [-65504.0]
+
+
+def test_cast_full_config_f32_to_fp16_and_back():
+    x = np.random.default_rng(8).standard_normal(32 * 128 * 4096).astype(np.float32)
+    h = ops.cast(dev(x), torch.float16)
+    assert np.array_equal(host(h).view(np.uint16), x.astype(np.float16).view(np.uint16))
+    back = host(ops.cast(h, torch.float32))
+    assert np.array_equal(back, x.astype(np.float16).astype(np.float32))     # widening is exact

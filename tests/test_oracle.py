@@ -413,3 +413,92 @@ def test_rope_vs_independent_float64_and_invariants():
     big = np.full((B, S), 2047, np.int64)
     assert np.allclose(oracle.rope(x, big), _rope_hf_f64(x, big, 10000.0), atol=1e-3)
     assert np.array_equal(oracle.rope(x, p1, threads=4), oracle.rope(x, p1))
+
+
+# ------------------------------------------------------------------ Cast
+def test_cast_reference_kat():
+    # src/04kernel/test/kernels/cast/test_cpu.cpp: F64 iota [2,3,4,5] -> I8, y[i] == i
+    c = GOLDEN["cast"][0]
+    x = np.arange(120, dtype=np.float64).reshape(c["shape"])
+    y = oracle.cast(x, c["from"], c["to"])
+    assert y.dtype == np.int8 and np.array_equal(y.reshape(-1), np.arange(120))
+
+
+def test_cast_integer_and_bool_rules_against_python_arithmetic():
+    rng = np.random.default_rng(3)
+    v = rng.integers(-2 ** 63, 2 ** 63, 500, dtype=np.int64)
+    for name, bits, signed in (("u8", 8, False), ("i8", 8, True), ("u16", 16, False), ("i16", 16, True),
+                               ("u32", 32, False), ("i32", 32, True), ("u64", 64, False)):
+        want = [(int(t) % (1 << bits)) - ((1 << bits) if signed and (int(t) % (1 << bits)) >= (1 << (bits - 1)) else 0)
+                for t in v]
+        assert oracle.cast(v, "i64", name).tolist() == want                      # narrowing wraps modulo 2^bits
+    f = np.array([-2.9, -0.5, 0.0, 0.5, 2.9, 126.99], np.float64)
+    assert oracle.cast(f, "f64", "i8").tolist() == [int(t) for t in f]           # truncation toward zero
+    assert oracle.cast(f, "f64", "bool").tolist() == [t != 0 for t in f]
+    assert oracle.cast(np.array([0, 1, 1, 0], np.bool_), "bool", "f32").tolist() == [0.0, 1.0, 1.0, 0.0]
+    big = np.array([2 ** 24 + 1, 2 ** 24 + 3, -(2 ** 24 + 1), 2 ** 53 + 1], np.int64)
+    import struct
+    want = [struct.unpack("f", struct.pack("f", float(int(t))))[0] for t in big[:3]]   # struct rounds to nearest even
+    assert oracle.cast(big[:3], "i64", "f32").tolist() == want
+    assert oracle.cast(big[3:], "i64", "f64").tolist() == [float(2 ** 53)]
+
+
+def _nearest_narrow(value, mant_bits, emin, emax):
+    """value (Fraction) rounded to nearest-even in a binary format with `mant_bits` explicit
+    mantissa bits and exponent range [emin, emax]; returns a Fraction or inf."""
+    from fractions import Fraction
+    if value == 0:
+        return Fraction(0)
+    sign = -1 if value < 0 else 1
+    a = abs(value)
+    e = 0
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1
+    while Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, emin)
+    ulp = Fraction(2) ** (e - mant_bits)
+    q, r = divmod(a, ulp)
+    if r * 2 > ulp or (r * 2 == ulp and q % 2 == 1):
+        q += 1
+    out = q * ulp
+    if out >= Fraction(2) ** (emax + 1):
+        return sign * float("inf")
+    return sign * out
+
+
+def test_cast_to_fp16_and_bf16_round_to_nearest_even_against_exact_arithmetic():
+    from fractions import Fraction
+    rng = np.random.default_rng(4)
+    x = np.concatenate([rng.standard_normal(300).astype(np.float32) * 100,
+                        np.array([2049., 2051., 65519.9, 65520., 1e-7, 6e-8, -3e-8, 0.0], np.float32),
+                        np.array([0x3F808000, 0x3F818000, 0x3F808001], np.uint32).view(np.float32)])
+    h = oracle.cast(x, "f32", "fp16")
+    b = oracle.cast(x, "f32", "bf16")
+    for i, t in enumerate(x):
+        want_h = _nearest_narrow(Fraction(float(t)), 10, -14, 15)
+        assert float(h[i]) == float(want_h), (t, h[i], want_h)
+        want_b = _nearest_narrow(Fraction(float(t)), 7, -126, 127)
+        got_b = float((np.uint32(b[i]) << 16).view(np.float32))
+        assert got_b == float(want_b), (t, got_b, want_b)
+    # a double goes through float first (reference: __float2half(double argument)): 1 + 2^-11 + 2^-26
+    # rounds to the tie 1 + 2^-11 in float and then to 1.0, where a single rounding would give 1 + 2^-10
+    assert oracle.cast(np.array([1 + 2.0 ** -11 + 2.0 ** -26]), "f64", "fp16").view(np.uint16).tolist() == [0x3C00]
+
+
+def test_cast_integers_to_fp16_bf16_go_through_int_and_round_toward_zero():
+    assert oracle.cast(np.array([2049, 2051, -2049, 70000, -70000, 16777217], np.int32), "i32", "fp16").tolist() == \
+        [2048.0, 2050.0, -2048.0, 65504.0, -65504.0, 65504.0]
+    assert oracle.cast(np.array([257, -257, 16777217, 2 ** 31 - 1], np.int32), "i32", "bf16").tolist() == \
+        [0x4380, 0xC380, 0x4B80, 0x4EFF]
+    # the value is taken as `int`: 3e9 as uint32 is negative as int
+    assert oracle.cast(np.array([3000000000], np.uint32), "u32", "fp16").tolist() == [-65504.0]
+    # and back: truncated as int, then converted to the target like any int (wraps)
+    assert oracle.cast(np.array([-1.5, 2.9, 300.7], np.float16), "fp16", "u8").tolist() == [255, 2, 44]
+    assert oracle.cast(np.array([0x4380, 0xC3A0], np.uint16), "bf16", "i16").tolist() == [256, -320]
+
+
+def test_cast_bool_from_floating_sources_reference_defect_fixture():
+    x = np.array([0.0, 1.5, -0.0], np.float32)
+    assert oracle.cast(x, "f32", "bool").tolist() == [False, True, False]
+    assert oracle.cast_bool_reference_literal(x, "f32").tolist() == [True, False, True]   # not reproduced
