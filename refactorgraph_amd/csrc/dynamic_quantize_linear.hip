@@ -100,7 +100,14 @@ __global__ __launch_bounds__(256) void dql_quantize(uint8_t *__restrict__ y, flo
         *scale_out = scale;
         *zp_out = static_cast<uint8_t>(zp_f);
     }
-    auto quant = [&](float v) -> uint32_t { return degenerate ? 0u : saturate_u8(roundf(v / scale) + zp_f); };
+    // round(x / scale) + zp is integer-valued (or infinite), so is its clamp to [0, 255]: the second
+    // rounding of the reference's saturate() changes nothing and is left out
+    auto quant = [&](float v) -> uint32_t {
+        float t = roundf(v / scale) + zp_f;
+        t = t < 0.f ? 0.f : t;
+        t = 255.f < t ? 255.f : t;
+        return degenerate ? 0u : static_cast<uint32_t>(t);
+    };
 
     const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256;
     const uint64_t t = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
