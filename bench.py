@@ -42,7 +42,7 @@ MEASURED_TRAFFIC = {
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
     "matmul_integer": (2 * 49313 + 65638) * 1024,
-    "attention_prefill": (2 * 99826 + 196608) * 1024,
+    "attention_prefill": (2 * 100058 + 200612) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
 }
 

@@ -166,9 +166,9 @@ __global__ __launch_bounds__(256, 3) void attn_prefill(const PrefillArgs a, uint
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t cp_row = (BN / 4) * wave_u + (lane >> 4);
     const uint32_t v_lane = cp_row * ROWB + 16 * ((lane & 15) ^ v_swizzle(lane >> 4));
-    uint32_t k_lane[CPI];
-#pragma unroll
-    for (int i = 0; i < CPI; ++i) k_lane[i] = (cp_row + 4 * i) * ROWB + 16 * ((lane & 15) ^ ((cp_row + 4 * i) & 15));
+    // K: chunk position lane % 16 of row r holds chunk (lane % 16) ^ (r & 15); rows 4 i further on flip
+    // bits 2-3 of the chunk index, i.e. bits 6-7 of the byte offset
+    const uint32_t k_lane = cp_row * ROWB + 16 * ((lane & 15) ^ (cp_row & 15));
     const uint32_t total_keys = base + a.seq;
     typedef const __attribute__((address_space(1))) void *GlobalPtr;
     typedef __attribute__((address_space(3))) void *LdsPtr;
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256, 3) void attn_prefill(const PrefillArgs a, uint
             const uint8_t *vb_ = reinterpret_cast<const uint8_t *>(in_hist ? v_hist : v_new) + tile_off;
 #pragma unroll
             for (int i = 0; i < CPI; ++i) {
-                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + k_lane[i]), (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + ((k_lane ^ (64 * i)) + 4 * i * ROWB)), (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
                 __builtin_amdgcn_global_load_lds((GlobalPtr)(vb_ + v_lane + 4 * i * ROWB), (LdsPtr)(buf + TILE + (CPI * wave_u + i) * 1024), 16, 0, 0);
             }
         } else {
@@ -355,7 +355,12 @@ __global__ __launch_bounds__(256, 3) void attn_prefill(const PrefillArgs a, uint
     }
     // (each wavefront reads back only what it wrote itself: no barrier)
     if (wave_active) {
-        T *op = O + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + r0) * D;
+        // computed afresh from an opaque copy of the wavefront index: otherwise the address is built in the
+        // prologue, next to the query pointer it resembles, and kept in scratch memory across the tile loop
+        uint32_t wave_e = wave;
+        asm volatile("" : "+v"(wave_e));
+        const uint32_t head_e = kvh * group + hc * HW + wave_e % HW, r0_e = qt * ROWS + 32 * (wave_e / HW);
+        T *op = O + ((static_cast<uint64_t>(b) * a.H + head_e) * a.seq + r0_e) * D;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t idx = lane + 64 * i, row = idx / 16, c = idx % 16;
