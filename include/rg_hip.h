@@ -123,6 +123,24 @@ int rg_hip_dynamic_quantize_linear(uint8_t *y, float *scale, uint8_t *zero_point
  * done when y == x).  y, x: `size` elements each. */
 int rg_hip_cast(void *y, const void *x, size_t size, int from_dtype, int to_dtype, void *stream);
 
+/* ---- MatMul -----------------------------------------------------------------------------
+ * replaces src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:9-108 (cublasGemmEx /
+ * cublasGemmStridedBatchedEx after an Expand of the bias into Y); arithmetic contract
+ * src/04kernel/src/kernels/mat_mul_common/cpu_template.hpp:19-31:
+ * Y = alpha * op(A) @ op(B) + beta * C.  dtype F32, F64, FP16 or BF16 for all operands; a is
+ * [a_batch, m, k] ([a_batch, k, m] when trans_a), b [b_batch, k, n] ([b_batch, n, k] when trans_b),
+ * y [batch, m, n], row-major.  alpha and beta are converted to dtype first, like the reference;
+ * sums are accumulated in float (double for F64).
+ * a_index / b_index: as for rg_hip_matmul_integer (HOST arrays of `batch` matrix indices, or NULL
+ * for matrix i).  c may be NULL (then beta is ignored); otherwise the bias element of
+ * Y[batch b, row i, column j] is c[b * c_stride_batch + i * c_stride_m + j * c_stride_n] (strides
+ * in elements, 0 broadcasts), which covers every bias the reference expands when its batch
+ * dimensions are all 1 or equal to the output's. */
+int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtype, int trans_a, int trans_b,
+                  float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
+                  const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
+                  size_t c_stride_m, size_t c_stride_n, void *stream);
+
 /* ---- MatMulInteger -----------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust
  * zero-point pre-pass + cublasGemmEx); arithmetic contract

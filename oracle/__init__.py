@@ -52,6 +52,9 @@ def lib() -> C.CDLL:
         L.oracle_dynamic_quantize_linear.restype = None
         L.oracle_matmul_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, f32]
         L.oracle_mul_f32.argtypes = [vp, vp, vp, sz, sz]
+        L.oracle_matmul_bias_f32.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, f32, f32]
+        L.oracle_matmul_bias_f64.argtypes = [vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, C.c_double, C.c_double]
+        L.oracle_matmul_bias_f32.restype = L.oracle_matmul_bias_f64.restype = None
         L.oracle_attention_head_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, f32, i32, vp]
         L.oracle_rope_f32.argtypes = [vp, vp, vp, i32, sz, sz, sz, sz, f32, i32]
         for name in ("oracle_rms_norm_f32", "oracle_rms_norm_f64", "oracle_softmax_f32",
@@ -344,3 +347,53 @@ def cast_bool_reference_literal(x, src):
     (cuda_kernel.cc:73-88): `x == 0`.  Kept as a named fixture of the defect; not used as oracle."""
     f = cast(x, src, "f64") if src in ("fp16", "bf16") else np.asarray(x)
     return f == 0
+
+
+# ---------------------------------------------------------------------------------------------
+# MatMul: Y = alpha * op(A) @ op(B) + beta * C (src/04kernel/src/kernels/mat_mul/cpu_kernel.cc:27-66,
+# mat_mul_common/cpu_template.hpp:19-31; shapes and broadcasting of
+# src/04kernel/src/attributes/mat_mul_info.cc:27-43).  `dtype` names the element type: "f32", "f64"
+# computed as the CPU kernel does; "fp16" / "bf16" (no CPU kernel in the reference: the cuBLAS
+# kernel takes them) computed in float on the up-cast values with alpha / beta rounded to the type
+# first and one rounding of the result.  bf16 tensors are uint16 bit patterns.
+def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, dtype="f32"):
+    def widen(t):
+        if dtype == "bf16":
+            return _bf16_to_f32(np.ascontiguousarray(t, np.uint16))
+        return np.ascontiguousarray(t, np.float64 if dtype == "f64" else np.float32)
+
+    def through(v):  # alpha, beta converted to the data type (cpu_kernel.cc:46-47)
+        if dtype == "fp16":
+            return float(np.float16(v))
+        if dtype == "bf16":
+            return float(_bf16_to_f32(_f32_to_bf16_rn(np.array([v], np.float32)))[0])
+        return float(np.float32(v)) if dtype == "f32" else float(v)
+
+    a, b = widen(a), widen(b)
+    wide = np.float64 if dtype == "f64" else np.float32
+    m, k = (a.shape[-1], a.shape[-2]) if trans_a else (a.shape[-2], a.shape[-1])
+    n = b.shape[-2] if trans_b else b.shape[-1]
+    assert k == (b.shape[-1] if trans_b else b.shape[-2])
+    batch_shape = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    out_shape = tuple(batch_shape) + (m, n)
+    if c is None:
+        y, beta = np.zeros(out_shape, wide), 0.0
+    else:
+        y = np.ascontiguousarray(np.broadcast_to(widen(c), out_shape)).copy()   # the Expand of the bias
+    a_b = np.broadcast_to(a, tuple(batch_shape) + a.shape[-2:]).reshape((-1,) + a.shape[-2:])
+    b_b = np.broadcast_to(b, tuple(batch_shape) + b.shape[-2:]).reshape((-1,) + b.shape[-2:])
+    y2 = y.reshape(-1, m, n)
+    fn = lib().oracle_matmul_bias_f64 if dtype == "f64" else lib().oracle_matmul_bias_f32
+    sa = (1, m) if trans_a else (k, 1)
+    sb = (1, k) if trans_b else (n, 1)
+    for i in range(y2.shape[0]):
+        ai, bi, yi = np.ascontiguousarray(a_b[i]), np.ascontiguousarray(b_b[i]), np.ascontiguousarray(y2[i])
+        fn(_p(yi), _p(ai), _p(bi), m, k, n, sa[0], sa[1], sb[0], sb[1], through(alpha), through(beta))
+        y2[i] = yi
+    y = y2.reshape(out_shape)
+    if dtype == "fp16":
+        with np.errstate(over="ignore"):
+            return y.astype(np.float16)
+    if dtype == "bf16":
+        return _f32_to_bf16_rn(y)
+    return y

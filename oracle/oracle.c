@@ -357,6 +357,31 @@ void oracle_matmul_f32(float *y, const float *a, const float *b,
         }
 }
 
+/* MatMul with bias: src/04kernel/src/kernels/mat_mul_common/cpu_template.hpp:19-31, T = float or
+ * double.  y holds the expanded bias on entry (mat_mul/cpu_kernel.cc:36-37 expands C into Y first);
+ * beta must be 0 when there is no bias (cpu_kernel.cc:48). */
+void oracle_matmul_bias_f32(float *y, const float *a, const float *b,
+                            size_t M, size_t K, size_t N,
+                            size_t sa0, size_t sa1, size_t sb0, size_t sb1, float alpha, float beta) {
+    for (size_t i = 0; i < M; ++i)
+        for (size_t j = 0; j < N; ++j) {
+            float sum = 0.0f;
+            for (size_t q = 0; q < K; ++q) sum += a[i * sa0 + q * sa1] * b[q * sb0 + j * sb1];
+            y[i * N + j] = beta * y[i * N + j] + alpha * sum;
+        }
+}
+
+void oracle_matmul_bias_f64(double *y, const double *a, const double *b,
+                            size_t M, size_t K, size_t N,
+                            size_t sa0, size_t sa1, size_t sb0, size_t sb1, double alpha, double beta) {
+    for (size_t i = 0; i < M; ++i)
+        for (size_t j = 0; j < N; ++j) {
+            double sum = 0.0;
+            for (size_t q = 0; q < K; ++q) sum += a[i * sa0 + q * sa1] * b[q * sb0 + j * sb1];
+            y[i * N + j] = beta * y[i * N + j] + alpha * sum;
+        }
+}
+
 void oracle_mul_f32(float *y, const float *a, const float *b, size_t n_a, size_t n_b) {
     size_t n = n_a > n_b ? n_a : n_b;
     for (size_t i = 0; i < n; ++i) y[i] = a[n_a == 1 ? 0 : i] * b[n_b == 1 ? 0 : i];

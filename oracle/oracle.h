@@ -108,6 +108,11 @@ void oracle_dynamic_quantize_linear(uint8_t *y, float *scale_out, uint8_t *zp_ou
 void oracle_matmul_f32(float *y, const float *a, const float *b,
                        size_t M, size_t K, size_t N,
                        size_t sa0, size_t sa1, size_t sb0, size_t sb1, float alpha);
+/* mat_mul_common/cpu_template.hpp:19-31 with the bias already expanded into y (mat_mul/cpu_kernel.cc:36-37) */
+void oracle_matmul_bias_f32(float *y, const float *a, const float *b, size_t M, size_t K, size_t N,
+                            size_t sa0, size_t sa1, size_t sb0, size_t sb1, float alpha, float beta);
+void oracle_matmul_bias_f64(double *y, const double *a, const double *b, size_t M, size_t K, size_t N,
+                            size_t sa0, size_t sa1, size_t sb0, size_t sb1, double alpha, double beta);
 void oracle_mul_f32(float *y, const float *a, const float *b, size_t n_a, size_t n_b);
 
 /* One (batch row, query head) of causal attention over a KV history.

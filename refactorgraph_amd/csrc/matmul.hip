@@ -1,0 +1,358 @@
+// MatMul (GEMM) for gfx950: Y = alpha * op(A) @ op(B) + beta * C, C broadcast over Y.
+//
+// Contract: src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:9-108 of the reference (row-major
+// A [m,k] or [k,m] when transposed, B [k,n] or [n,k], batches strided or broadcast, alpha / beta
+// converted to the data type, bias expanded into Y before the product is added) and, for the
+// arithmetic, src/04kernel/src/kernels/mat_mul_common/cpu_template.hpp:19-31
+// (y = beta * c + alpha * sum_k a*b).  Floating-point sums are accumulated in float (double for
+// F64) in an order that differs from the CPU loop, so results agree to rounding, not bit for bit.
+// The bias is read through strides inside the epilogue instead of being expanded into Y first.
+//
+// Fast path (FP16 / BF16, A not transposed, m and n multiples of 256, k multiple of 64): one
+// 256x256 tile of Y per workgroup of four wavefronts (128x128 each, 4x4 blocks of
+// v_mfma_f32_32x32x16), k-tiles of 64 copied from global memory straight into two LDS buffers
+// with global_load_lds_dwordx4, fragments double buffered by k-step, one MFMA per scheduling slot:
+// the structure of the MatMulInteger kernel with 16-bit operands.
+//   A tile (and B given as [n,k]): rows of 128 bytes, chunk c of row r at chunk position
+//           c ^ (r & 7) ^ ((r >> 3) & 1); fragments by 128-bit reads.
+//   B given as [k,n]: 64 k-rows of 512 bytes, chunk c of k-row r at c ^ swz(r & 3); the operand
+//           (8 consecutive k of one column per lane) is formed by two ds_read_b64_tr_b16, which
+//           transpose 16-bit elements inside 16 lanes (lane i receives element i % 4 of the 8-byte
+//           pieces addressed by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12).
+// Everything else (F32, F64, transposed A, other shapes) goes through a plain tiled kernel.
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include <utility>
+
+#include "common.hpp"
+
+namespace rg {
+namespace {
+
+// Where the bias element of Y[batch b, row i, column j] lives: c + b*sb + i*sm + j*sn (elements);
+// a stride of 0 broadcasts.  c == nullptr: no bias.
+struct Bias {
+    const void *ptr;
+    uint64_t sb, sm, sn;
+};
+
+template <class T> struct Acc { typedef float type; };
+template <> struct Acc<double> { typedef double type; };
+
+template <class T> __device__ __forceinline__ typename Acc<T>::type up(T v) { return static_cast<typename Acc<T>::type>(v); }
+template <> __device__ __forceinline__ float up<__half>(__half v) { return __half2float(v); }
+template <> __device__ __forceinline__ float up<__hip_bfloat16>(__hip_bfloat16 v) { return __bfloat162float(v); }
+template <class T> __device__ __forceinline__ T down(typename Acc<T>::type v) { return static_cast<T>(v); }
+template <> __device__ __forceinline__ __half down<__half>(float v) { return __float2half(v); }
+template <> __device__ __forceinline__ __hip_bfloat16 down<__hip_bfloat16>(float v) { return __float2bfloat16(v); }
+
+// alpha and beta are converted to the data type first, as the reference does
+template <class T> typename Acc<T>::type through(float v) { return static_cast<typename Acc<T>::type>(static_cast<T>(v)); }
+template <> float through<__half>(float v) { return __half2float(__float2half(v)); }
+template <> float through<__hip_bfloat16>(float v) { return __bfloat162float(__float2bfloat16(v)); }
+
+// ---------------------------------------------------------------- generic kernel
+// 16x16 outputs per workgroup, one per thread; k walked in LDS tiles of 16; element (i, kk) of
+// op(A) is a[i*sa0 + kk*sa1], element (kk, j) of op(B) is b[kk*sb0 + j*sb1].
+template <class T>
+__global__ __launch_bounds__(256) void mm_generic(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b,
+                                                  Bias bias, uint32_t m, uint32_t k, uint32_t n, uint64_t sa0,
+                                                  uint64_t sa1, uint64_t sb0, uint64_t sb1,
+                                                  typename Acc<T>::type alpha, typename Acc<T>::type beta,
+                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    typedef typename Acc<T>::type A_t;
+    __shared__ A_t ta[16][17];
+    __shared__ A_t tb[16][17];
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const T *A = a + am * m * k;
+    const T *B = b + bm * static_cast<uint64_t>(k) * n;
+    const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const uint32_t row = blockIdx.y * 16 + ty, col = blockIdx.x * 16 + tx;
+    A_t acc = 0;
+    for (uint32_t k0 = 0; k0 < k; k0 += 16) {
+        A_t va = 0, vb = 0;
+        if (row < m && k0 + tx < k) va = up(A[row * sa0 + (k0 + tx) * sa1]);
+        if (k0 + ty < k && col < n) vb = up(B[(k0 + ty) * sb0 + col * sb1]);
+        ta[ty][tx] = va;
+        tb[ty][tx] = vb;
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc += ta[ty][q] * tb[q][tx];
+        __syncthreads();
+    }
+    if (row < m && col < n) {
+        A_t r = alpha * acc;
+        if (bias.ptr) r += beta * up(static_cast<const T *>(bias.ptr)[ym * bias.sb + row * bias.sm + col * bias.sn]);
+        y[(ym * m + row) * n + col] = down<T>(r);
+    }
+}
+
+// ---------------------------------------------------------------- MFMA kernel (FP16 / BF16)
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short s4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <class T> struct Mfma;
+template <> struct Mfma<__half> {
+    static __device__ __forceinline__ f16v run(u32x4 a, u32x4 b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma<__hip_bfloat16> {
+    static __device__ __forceinline__ f16v run(u32x4 a, u32x4 b, f16v c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8, a), __builtin_bit_cast(b8, b), c, 0, 0, 0);
+    }
+};
+
+constexpr int BM = 256, BN = 256, BK = 64;   // BK in elements: 128 bytes
+constexpr int M_TILE = 32768;                // one A or B tile in LDS
+constexpr int M_STAGE = 2 * M_TILE;
+
+__device__ __forceinline__ uint32_t n_swizzle(uint32_t r) { return 4 * (r & 1) + 10 * ((r >> 1) & 1); }  // r < 4
+
+// A, B: byte pointers to this workgroup's first row / first column; pitches in bytes.
+template <class T, bool TRANS_B>
+__device__ __forceinline__ void mm_tile_loop(f16v (&acc)[4][4], uint8_t *lds0, uint8_t *lds1, const uint8_t *A,
+                                             const uint8_t *B, uint32_t k, uint32_t pitch_a, uint32_t pitch_b) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
+    // copy q < 8: A rows 8 (8 wave + q) .. + 7, this lane row + lane / 8, chunk position lane % 8.
+    // copy 8 + p, B as [n,k]: the same for B's rows (columns of Y); B as [k,n]: k-rows
+    // 2 (8 wave + p) and the next, this lane k-row + lane / 32, chunk position lane % 32.
+    const uint8_t *a_wave = A + static_cast<uint64_t>(wave * 64) * pitch_a;
+    const uint32_t a_lane = (lane >> 3) * pitch_a + 16 * ((lane & 7) ^ (lane >> 3));
+    const uint8_t *b_wave = B + static_cast<uint64_t>(wave * (TRANS_B ? 64 : 16)) * pitch_b;
+    uint32_t b_lane[2];
+    if constexpr (TRANS_B) {
+        b_lane[0] = b_lane[1] = (lane >> 3) * pitch_b + 16 * ((lane & 7) ^ (lane >> 3));
+    } else {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) b_lane[p] = (lane >> 5) * pitch_b + 16 * ((lane & 31) ^ n_swizzle(2 * p + (lane >> 5)));
+    }
+    auto copy = [&](uint8_t *base, uint32_t kt, int q) {
+        const uint8_t *src;
+        uint8_t *dst;
+        if (q < 8) {
+            src = a_wave + (kt * 128 + 8 * q * pitch_a) + (a_lane ^ (16 * (q & 1)));
+            dst = base + (wave * 8 + q) * 1024;
+        } else if constexpr (TRANS_B) {
+            src = b_wave + (kt * 128 + 8 * (q - 8) * pitch_b) + (b_lane[0] ^ (16 * (q & 1)));
+            dst = base + M_TILE + (wave * 8 + (q - 8)) * 1024;
+        } else {
+            src = b_wave + static_cast<uint64_t>(kt * BK + 2 * (q - 8)) * pitch_b + b_lane[q & 1];
+            dst = base + M_TILE + (wave * 8 + (q - 8)) * 1024;
+        }
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                         (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+    };
+    // A fragment i of k-step ks: row wm 128 + 32 i + lane % 32, chunk 2 ks + h
+    const uint32_t a_off = (wm * 128 + (lane & 31)) * 128 + 16 * (h ^ (lane & 7) ^ ((lane >> 3) & 1));
+    auto read_a = [&](const uint8_t *base, int ks, int i) -> u32x4 {
+        return *reinterpret_cast<const u32x4 *>(base + (a_off ^ (32 * ks)) + i * 4096);
+    };
+    // B fragment j of k-step ks, B as [n,k]: like A with row wn 128 + 32 j + lane % 32.
+    // B as [k,n]: column wn 128 + 32 j + lane % 32, k 16 ks + 8 h .. + 7 in two transposing reads:
+    // lane a of a group of 16 addresses k-row + a / 4, columns 4 (a % 4) .. + 3 of the group's 16.
+    uint32_t b_off;
+    if constexpr (TRANS_B) {
+        b_off = M_TILE + (wn * 128 + (lane & 31)) * 128 + 16 * (h ^ (lane & 7) ^ ((lane >> 3) & 1));
+    } else {
+        const uint32_t a16 = lane & 15, r = a16 >> 2;
+        const uint32_t chunk = wn * 16 + 2 * ((lane >> 4) & 1) + ((a16 & 3) >> 1);  // + 4 j: bits 6-7 of the byte offset
+        b_off = M_TILE + (8 * h + r) * 512 + 16 * (chunk ^ n_swizzle(r)) + 8 * (a16 & 1);
+    }
+    auto read_b = [&](const uint8_t *base, int ks, int j, int half, u32x4 &f) {
+        if constexpr (TRANS_B) {
+            if (half == 0) f = *reinterpret_cast<const u32x4 *>(base + (b_off ^ (32 * ks)) + j * 4096);
+        } else {
+            const s4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (s4 __attribute__((address_space(3))) *)(base + (b_off ^ (64 * j)) + (16 * ks + 4 * half) * 512));
+            const u32x2 w = __builtin_bit_cast(u32x2, v);
+            f[2 * half] = w[0];
+            f[2 * half + 1] = w[1];
+        }
+    };
+
+    const uint32_t k_tiles = k / BK;
+    u32x4 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) copy(lds0, 0, q);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) copy(lds1, k_tiles > 1 ? 1 : 0, q);  // k_tiles == 1: tile 0 again, never multiplied
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 (the 16 older copies)
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[0][i] = read_a(lds0, 0, i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        read_b(lds0, 0, j, 0, fb[0][j]);
+        read_b(lds0, 0, j, 1, fb[0][j]);
+    }
+
+    // Tile kt is in buffer RB, tile kt+1 arrives in WB.
+    auto step = [&](uint32_t kt_, uint8_t *RB, const uint8_t *WB) __attribute__((always_inline)) {
+        const bool more = kt_ + 2 < k_tiles;  // uniform
+        auto slot = [&]<int s>() __attribute__((always_inline)) {
+            // rows walk the columns back and forth, so that only one operand changes between MFMAs
+            constexpr int ks = s / 16, o = s % 16, row = o / 4, col = (row & 1) ? 3 - o % 4 : o % 4;
+            constexpr int cur = ks & 1, nxt = cur ^ 1;
+            if constexpr (s == 48) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of tile kt+1
+                __syncthreads();                                  // tile kt+1 complete, RB no longer read
+            }
+            acc[row][col] = Mfma<T>::run(fa[cur][row], fb[cur][col], acc[row][col]);
+            const uint8_t *src = ks == 3 ? WB : RB;
+            constexpr int nks = (ks + 1) % 4;
+            if constexpr (o < 4) fa[nxt][o] = read_a(src, nks, o);
+            else if constexpr (o < 12) read_b(src, nks, (o - 4) / 2, (o - 4) % 2, fb[nxt][(o - 4) / 2]);
+            if constexpr (s >= 48) if (more) copy(RB, kt_ + 2, s - 48);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) {
+            (slot.template operator()<I>(), ...);
+        }(std::make_integer_sequence<int, 64>{});
+    };
+    uint32_t kt = 0;
+    for (; kt + 2 <= k_tiles; kt += 2) {
+        step(kt, lds0, lds1);
+        step(kt + 1, lds1, lds0);
+    }
+    if (kt < k_tiles) step(kt, lds0, lds1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
+}
+
+template <class T, bool TRANS_B>
+__global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, const T *__restrict__ a,
+                                                          const T *__restrict__ b, Bias bias, uint32_t m, uint32_t k,
+                                                          uint32_t n, float alpha, float beta, uint32_t a_matrix0,
+                                                          uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(1024) uint8_t lds0[M_STAGE];
+    __shared__ __align__(1024) uint8_t lds1[M_STAGE];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+
+    // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
+    // give each XCD a contiguous block of tiles (they then share A row-panels / B column-panels
+    // in that XCD's L2); within it walk tiles in column-major groups of 4 rows to keep panels hot.
+    const uint32_t tiles_n = n / BN, tiles_m = m / BM, n_tiles = tiles_m * tiles_n;
+    uint32_t t = blockIdx.x;
+    if (n_tiles % 8 == 0) t = (t % 8) * (n_tiles / 8) + t / 8;
+    const uint32_t group = 4 * tiles_n;
+    const uint32_t g = t / group, r = t % group;
+    const uint32_t rows_here = tiles_m - g * 4 < 4 ? tiles_m - g * 4 : 4;
+    const uint32_t tile_m = g * 4 + r % rows_here, tile_n = r / rows_here;
+
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m + static_cast<uint64_t>(tile_m) * BM) * k);
+    const T *b_matrix = b + bm * static_cast<uint64_t>(k) * n;
+    const uint8_t *B = reinterpret_cast<const uint8_t *>(
+        TRANS_B ? b_matrix + static_cast<uint64_t>(tile_n) * BN * k : b_matrix + static_cast<uint64_t>(tile_n) * BN);
+
+    f16v acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    mm_tile_loop<T, TRANS_B>(acc, lds0, lds1, A, B, k, 2 * k, TRANS_B ? 2 * k : 2 * n);
+
+    // 32x32 accumulator layout: lane holds column (lane % 32); register e holds row
+    // 8*(e/4) + 4*(lane/32) + e%4.
+    const uint32_t wm = wave >> 1, wn = wave & 1;
+    const uint32_t row0 = tile_m * BM + wm * 128, col0 = tile_n * BN + wn * 128;
+    T *Y = y + (ym * m + row0) * n + col0;
+    const T *C = static_cast<const T *>(bias.ptr);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+                const uint32_t col = j * 32 + (lane & 31);
+                float v = alpha * acc[i][j][e];
+                if (C) v += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
+                Y[static_cast<uint64_t>(row) * n + col] = down<T>(v);
+            }
+}
+
+template <class T>
+int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_a, int trans_b, float alpha, float beta,
+                 size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
+                 hipStream_t s) {
+    auto *y = static_cast<T *>(y_);
+    auto *a = static_cast<const T *>(a_);
+    auto *b = static_cast<const T *>(b_);
+    typedef typename Acc<T>::type A_t;
+    const A_t al = through<T>(alpha), be = bias.ptr ? through<T>(beta) : A_t(0);
+    constexpr bool narrow = sizeof(T) == 2;
+    const bool fast = narrow && !trans_a && m % BM == 0 && n % BN == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
+
+    auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if constexpr (narrow) {
+            if (fast) {
+                const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
+                if (trans_b)
+                    mm_mfma_256x256<T, true><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                                  static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                else
+                    mm_mfma_256x256<T, false><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                                   static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                return launch_status();
+            }
+        }
+        const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
+        mm_generic<T><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                           static_cast<uint32_t>(n), trans_a ? 1 : k, trans_a ? m : 1, trans_b ? 1 : n,
+                                           trans_b ? k : 1, al, be, am0, bm0, ym0);
+        return launch_status();
+    };
+
+    if (!a_index && !b_index) {
+        for (size_t i = 0; i < batch; i += 65535) {  // grid.z is limited to 65535
+            const uint32_t count = static_cast<uint32_t>(batch - i < 65535 ? batch - i : 65535);
+            const int rc = launch(static_cast<uint32_t>(i), static_cast<uint32_t>(i), static_cast<uint32_t>(i), count);
+            if (rc) return rc;
+        }
+        return 0;
+    }
+    for (size_t i = 0; i < batch; ++i) {
+        const int rc = launch(a_index ? a_index[i] : static_cast<uint32_t>(i),
+                              b_index ? b_index[i] : static_cast<uint32_t>(i), static_cast<uint32_t>(i), 1);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+}  // namespace
+}  // namespace rg
+
+extern "C" int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtype, int trans_a, int trans_b,
+                             float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
+                             const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
+                             size_t c_stride_m, size_t c_stride_n, void *stream) {
+    using namespace rg;
+    if (!y || !a || !b) return RG_HIP_E_ARGUMENT;
+    if (batch == 0 || m == 0 || n == 0) return 0;
+    if (m > 0x7fffffffu || n > 0x7fffffffu || k > 0x7fffffffu || batch > 0xffffffffu) return RG_HIP_E_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    const Bias bias{c, c_stride_batch, c_stride_m, c_stride_n};
+    switch (dtype) {
+        case RG_F32: return launch_typed<float>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+        case RG_F64: return launch_typed<double>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+        case RG_FP16: return launch_typed<__half>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+        case RG_BF16:
+            return launch_typed<__hip_bfloat16>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+        default: return RG_HIP_E_UNSUPPORTED;
+    }
+}

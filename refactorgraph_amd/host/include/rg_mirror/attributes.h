@@ -1,7 +1,9 @@
 // Shape pre-digestion used by the hot-path collectors.  Semantics follow
 // src/04kernel/src/attributes/{softmax_info.cc:6-13, broadcaster.cc:17-105,
-// mat_mul_integer_info.cc:5-40}.
+// mat_mul_integer_info.cc:5-40, mat_mul_info.cc:5-43}.
 #pragma once
+
+#include <optional>
 
 #include "rg_mirror/kernel.h"
 
@@ -26,6 +28,25 @@ namespace refactor::kernel {
         explicit Broadcaster(TensorRefs const &inputs);
         void locate(dim_t k, dim_t ans[]) const noexcept;
         bool needBroadcast() const noexcept { return !strides.empty(); }
+    };
+
+    // Mirrors src/04kernel/include/kernel/attributes/mat_mul_info.h:9-24.  The reference keeps an
+    // ExpandInfo for the bias and expands it into Y before the product; here the bias is read through
+    // strides inside the product's epilogue, so the info carries the three strides instead
+    // (elements; 0 broadcasts).  `biasSupported` is false for a bias whose batch dimensions are
+    // neither all 1 nor the output's (such a bias needs the Expand kernel, which is not built).
+    struct MatMulInfo {
+        DataType dataType;
+        float alpha, beta;
+        bool transA, transB;
+        dim_t m, k, n;
+        bool hasBias, biasSupported;
+        size_t biasStrideBatch, biasStrideM, biasStrideN;
+        Broadcaster broadcaster;
+
+        MatMulInfo(Tensor const &, Tensor const &, std::optional<std::reference_wrapper<Tensor const>>,
+                   bool, bool, float, float);
+        dim_t batch() const noexcept { return broadcaster.outputsCount; }
     };
 
     struct MatMulIntegerInfo {

@@ -44,6 +44,16 @@ namespace refactor::kernel {
         std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
     };
 
+    // inputs: A, B [, C]; outputs: Y (src/04kernel/include/kernel/collectors/mat_mul.h:8-18)
+    struct MatMulCollector final : public InfoCollector {
+        float alpha, beta;
+        bool transA, transB;
+        constexpr MatMulCollector(hardware::Device::Type target, float alpha_, float beta_, bool transA_,
+                                  bool transB_) noexcept
+            : InfoCollector(target), alpha(alpha_), beta(beta_), transA(transA_), transB(transB_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
     // inputs: x; outputs: y of the requested type, same shape
     // (src/04kernel/include/kernel/collectors/cast.h:8-14)
     struct CastCollector final : public InfoCollector {

@@ -71,6 +71,19 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // mirrors MatMulCublas (src/04kernel/src/kernels/mat_mul/cublas_kernel.hh): F32, F64, FP16 and,
+    // beyond the reference, BF16; no library handle in the resources, the kernels are this library's
+    struct MatMulHip final : public Kernel {
+        MatMulInfo info;
+
+        explicit MatMulHip(decltype(info)) noexcept;
+        static KernelBox build(decltype(info)) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     // mirrors CastCuda (src/04kernel/src/kernels/cast/cuda_kernel.hh:9-23); no run-time compilation:
     // every type pair is a precompiled kernel of the device library
     struct CastHip final : public Kernel {

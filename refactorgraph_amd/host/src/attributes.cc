@@ -97,6 +97,53 @@ namespace refactor::kernel {
         return std::vector<dim_t>(t.shape.begin(), t.shape.end() - 2);
     }
 
+    MatMulInfo::MatMulInfo(Tensor const &a, Tensor const &b, std::optional<std::reference_wrapper<Tensor const>> c,
+                           bool transA_, bool transB_, float alpha_, float beta_)
+        // src/04kernel/src/attributes/mat_mul_info.cc:27-43
+        : dataType(a.dataType),
+          alpha(alpha_), beta(beta_),
+          transA(transA_), transB(transB_),
+          m(transA ? a.shape.rbegin()[0] : a.shape.rbegin()[1]),
+          k(transA ? a.shape.rbegin()[1] : a.shape.rbegin()[0]),
+          n(transB ? b.shape.rbegin()[1] : b.shape.rbegin()[0]),
+          hasBias(c.has_value()), biasSupported(true),
+          biasStrideBatch(0), biasStrideM(0), biasStrideN(0),
+          broadcaster({batchDims(a), batchDims(b)}) {
+        auto kB = transB ? b.shape.rbegin()[0] : b.shape.rbegin()[1];
+        ASSERT(k == kB, "MatMul: input shape not matched.");
+        if (!c) { return; }
+        // the bias broadcasts unidirectionally to [batch dims..., m, n] (mat_mul_info.cc:5-25)
+        std::vector<dim_t> out(std::max(a.shape.size(), b.shape.size()) - 2);
+        {
+            auto const da = a.shape.size() - 2, db = b.shape.size() - 2;
+            for (size_t i = 0; i < out.size(); ++i) {
+                auto const a_ = i < da ? a.shape[da - i - 1] : 1, b_ = i < db ? b.shape[db - i - 1] : 1;
+                out[out.size() - 1 - i] = std::max(a_, b_);
+            }
+        }
+        auto const &cs = c->get().shape;
+        auto at = [&](size_t fromEnd) -> dim_t { return fromEnd < cs.size() ? cs.rbegin()[fromEnd] : 1; };
+        auto const cn = at(0), cm = at(1);
+        if ((cn != 1 && cn != n) || (cm != 1 && cm != m) || cs.size() > out.size() + 2) {
+            biasSupported = false;
+            return;
+        }
+        biasStrideN = cn == n ? 1 : 0;
+        biasStrideM = cm == m ? cn : 0;
+        bool allOne = true, same = cs.size() == out.size() + 2;
+        for (size_t i = 2; i < cs.size(); ++i) {
+            allOne = allOne && at(i) == 1;
+            same = same && at(i) == out[out.size() + 1 - i];
+        }
+        if (allOne) {
+            biasStrideBatch = 0;
+        } else if (same) {
+            biasStrideBatch = static_cast<size_t>(cm) * cn;
+        } else {
+            biasSupported = false;
+        }
+    }
+
     MatMulIntegerInfo::MatMulIntegerInfo(TensorRefs const &inputs) noexcept
         : a(inputs, 0),
           b(inputs, 1),

@@ -104,6 +104,27 @@ namespace refactor::kernel {
     }
 
     std::vector<KernelBox>
+    MatMulCollector::filter(TensorRefs inputs, TensorRefs) const {
+        // src/04kernel/src/collectors/mat_mul.cc:12-35
+        auto const &a = inputs[0].get();
+        auto const &b = inputs[1].get();
+        auto info = inputs.size() == 3
+                        ? MatMulInfo(a, b, std::make_optional(std::cref(inputs[2].get())), transA, transB, alpha, beta)
+                        : MatMulInfo(a, b, std::nullopt, transA, transB, alpha, beta);
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(MatMulHip::build(info))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
     CastCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
         // src/04kernel/src/collectors/cast.cc:10-33
         auto const &from = inputs[0].get();

@@ -167,6 +167,41 @@ namespace refactor::kernel {
         return {std::move(routine), workspace};
     }
 
+    // ------------------------------------------------------------------ MatMul
+
+    MatMulHip::MatMulHip(decltype(info) info_) noexcept : Kernel(), info(std::move(info_)) {}
+    KernelBox MatMulHip::build(decltype(info) info) noexcept {
+        // src/04kernel/src/kernels/mat_mul/cublas_kernel.cc:9-20 accepts F32, F64, FP16
+        auto const dt = info.dataType;
+        if (dt != DataType::F32 && dt != DataType::F64 && dt != DataType::FP16 && dt != DataType::BF16) { return nullptr; }
+        if (info.hasBias && !info.biasSupported) { return nullptr; }
+        return std::make_unique<MatMulHip>(std::move(info));
+    }
+    size_t MatMulHip::typeId() noexcept { return idOf<MatMulHip>(); }
+    size_t MatMulHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view MatMulHip::description() const noexcept { return "Performing MatMul with MFMA on AMD gfx950"; }
+    RoutineWorkspace MatMulHip::lower(Resources &) const {
+        std::vector<uint32_t> aIndex, bIndex;
+        if (info.broadcaster.needBroadcast()) {
+            aIndex.resize(info.batch());
+            bIndex.resize(info.batch());
+            for (dim_t i = 0; i < info.batch(); ++i) {
+                dim_t at[2];
+                info.broadcaster.locate(i, at);
+                aIndex[i] = at[0];
+                bIndex[i] = at[1];
+            }
+        }
+        return [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
+            (Resources &, void *, void const *const *inputs, void *const *outputs) {
+                HIP_CALL(rg_hip_matmul(outputs[0], inputs[0], inputs[1], info.hasBias ? inputs[2] : nullptr,
+                                       static_cast<int>(info.dataType.internal), info.transA, info.transB, info.alpha,
+                                       info.beta, info.batch(), info.m, info.k, info.n,
+                                       aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
+                                       info.biasStrideBatch, info.biasStrideM, info.biasStrideN, nullptr));
+            };
+    }
+
     // ------------------------------------------------------------------ Cast
 
     CastHip::CastHip(decltype(from) from_, decltype(to) to_, decltype(size) size_) noexcept

@@ -115,6 +115,48 @@ def cast(x, dtype, out=None):
     return y
 
 
+def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=None):
+    """Y = alpha * op(A) @ op(B) + beta * C.  a [..., m, k] ([..., k, m] when trans_a), b [..., k, n]
+    ([..., n, k] when trans_b), batch dimensions broadcast; c broadcasts to [m, n] (any leading
+    dimensions of size 1) or has the output's full shape.  float32/float64/float16/bfloat16."""
+    _need_gpu(a, b, c)
+    assert a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous()
+    m, k = (a.shape[-1], a.shape[-2]) if trans_a else (a.shape[-2], a.shape[-1])
+    n = b.shape[-2] if trans_b else b.shape[-1]
+    assert k == (b.shape[-1] if trans_b else b.shape[-2])
+    ab, bb = tuple(a.shape[:-2]), tuple(b.shape[:-2])
+    ob = tuple(np.broadcast_shapes(ab, bb))
+    batch = math.prod(ob)
+    a_idx = b_idx = None
+    if ab != bb:
+        ia = np.arange(math.prod(ab), dtype=np.uint32).reshape(ab)
+        ib = np.arange(math.prod(bb), dtype=np.uint32).reshape(bb)
+        oa, obb = np.broadcast_arrays(ia, ib)
+        a_idx = np.ascontiguousarray(oa.reshape(-1))
+        b_idx = np.ascontiguousarray(obb.reshape(-1))
+    sb = sm = sn = 0
+    if c is not None:
+        assert c.dtype == a.dtype and c.is_contiguous()
+        cs = (1,) * (len(ob) + 2 - c.dim()) + tuple(c.shape)
+        if cs[:-2] == ob and batch > 1:
+            sb = cs[-2] * cs[-1]
+        else:
+            assert all(d == 1 for d in cs[:-2]), "bias batch dimensions must be 1 or the output's"
+        assert cs[-2] in (1, m) and cs[-1] in (1, n)
+        sm = cs[-1] if cs[-2] == m else 0
+        sn = 1 if cs[-1] == n else 0
+        if cs[-2] == 1:
+            sm = 0
+    y = torch.empty(ob + (m, n), dtype=a.dtype, device=a.device) if out is None else out
+    check(lib().rg_hip_matmul(
+        _ptr(y), _ptr(a), _ptr(b), _ptr(c), _T2CODE[a.dtype], int(trans_a), int(trans_b), float(alpha), float(beta),
+        batch, m, k, n,
+        None if a_idx is None else a_idx.ctypes.data_as(C.c_void_p),
+        None if b_idx is None else b_idx.ctypes.data_as(C.c_void_p),
+        sb, sm, sn, _stream()), "rg_hip_matmul")
+    return y
+
+
 def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):
     """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
     (batch, row) of the operand as the reference's CPU kernel reads them."""

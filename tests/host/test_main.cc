@@ -199,6 +199,29 @@ static void collectorsSelectOrDecline() {
     EXPECT(DynamicQuantizeLinearCollector(T::Amd).filter({*x8}, {*yq, *s1, *zq}).empty());
     EXPECT(DynamicQuantizeLinearCollector(T::Cpu).filter({*xf}, {*yq, *s1, *zq}).empty());
 
+    // MatMul: shapes, transposes and bias strides from the tensors; unsupported types are declined
+    {
+        auto a = Tensor::share(DataType::F32, Shape{2, 1, 5, 7});
+        auto bt = Tensor::share(DataType::F32, Shape{1, 3, 4, 7});
+        auto cRow = Tensor::share(DataType::F32, Shape{5, 1});
+        auto cFull = Tensor::share(DataType::F32, Shape{2, 3, 5, 4});
+        auto cOdd = Tensor::share(DataType::F32, Shape{2, 1, 5, 4});
+        MatMulInfo info(*a, *bt, std::cref(*cRow), false, true, 0.5f, 2.f);
+        EXPECT(info.m == 5 && info.k == 7 && info.n == 4 && info.batch() == 6 && info.hasBias && info.biasSupported);
+        EXPECT(info.biasStrideM == 1 && info.biasStrideN == 0 && info.biasStrideBatch == 0);
+        MatMulInfo full(*a, *bt, std::cref(*cFull), false, true, 1.f, 1.f);
+        EXPECT(full.biasStrideBatch == 20 && full.biasStrideM == 4 && full.biasStrideN == 1);
+        EXPECT(!MatMulInfo(*a, *bt, std::cref(*cOdd), false, true, 1.f, 1.f).biasSupported);
+        EXPECT(MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cRow}, {*cFull}).size() == 1);
+        EXPECT(MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cOdd}, {*cFull}).empty());
+        EXPECT(MatMulCollector(T::Cpu, 1, 1, false, true).filter({*a, *bt}, {*cFull}).empty());
+        auto ai = Tensor::share(DataType::I32, Shape{5, 7});
+        auto bi = Tensor::share(DataType::I32, Shape{7, 4});
+        EXPECT(MatMulCollector(T::Amd, 1, 1, false, false).filter({*ai, *bi}, {*cFull}).empty());
+        EXPECT(throws<std::runtime_error>(
+            [&] { MatMulInfo bad(*a, *Tensor::share(DataType::F32, Shape{6, 4}), std::nullopt, false, false, 1.f, 1.f); }));
+    }
+
     // Cast: every pair of numeric types has a kernel; strings and complex numbers do not
     auto c8 = Tensor::share(DataType::I8, Shape{4, 6});
     auto ch = Tensor::share(DataType::FP16, Shape{4, 6});
@@ -428,6 +451,60 @@ static void dynamicQuantizeLinearHip() {
     EXPECT(DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*xh}, {*y, *scale, *zp}).empty());
 }
 
+static void matMulHip() {
+    runtime::Resources res;
+    auto &dev = amd();
+    auto run = [&](Tensor const &A, Tensor const &B, Tensor const *C, Tensor const &Y, std::vector<float> const &a,
+                   std::vector<float> const &b, std::vector<float> const &c) {
+        auto kernels = C ? MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({A, B, *C}, {Y})
+                         : MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({A, B}, {Y});
+        EXPECT(kernels.size() == 1);
+        auto routine = kernels[0]->lower(res).routine;
+        auto ma = dev.malloc(a.size() * 4), mb = dev.malloc(b.size() * 4), mc = dev.malloc(std::max<size_t>(c.size(), 1) * 4),
+             my = dev.malloc(Y.elementsSize() * 4);
+        ma->copyFromHost(a.data());
+        mb->copyFromHost(b.data());
+        if (!c.empty()) mc->copyFromHost(c.data());
+        void const *inputs[]{*ma, *mb, *mc};
+        void *outputs[]{*my};
+        routine(res, nullptr, inputs, outputs);
+        std::vector<float> y(Y.elementsSize());
+        my->copyToHost(y.data());
+        return y;
+    };
+    {// src/04kernel/test/kernels/mat_mul/test_cpu.cpp:24-39 and test_cublas.cpp (same vectors on the device)
+        auto A = Tensor::share(DataType::F32, Shape{1, 2, 2});
+        auto B = Tensor::share(DataType::F32, Shape{2, 2});
+        auto C = Tensor::share(DataType::F32, Shape{});
+        auto Y = Tensor::share(DataType::F32, Shape{2, 2});
+        auto y = run(*A, *B, C.get(), *Y, {1.0, 2.0, 0.0, 0.5}, {1.0, 2.0, 0.0, 0.5}, {1.0});
+        EXPECT((y == std::vector<float>{2, 4, 1, 1.25}));
+    }
+    {// test_cpu.cpp:57-79: both operands broadcast over the batch, bias [2, 1]
+        auto A = Tensor::share(DataType::F32, Shape{2, 1, 2, 2});
+        auto B = Tensor::share(DataType::F32, Shape{1, 2, 2, 2});
+        auto C = Tensor::share(DataType::F32, Shape{2, 1});
+        auto Y = Tensor::share(DataType::F32, Shape{2, 2, 2, 2});
+        auto y = run(*A, *B, C.get(), *Y, {1.0, 2.0, 0.0, 0.5, 1.0, 0.0, 0.0, 1.0}, {1.0, 2.0, 0.0, 0.5, 1.0, 0.0, 0.0, 1.0},
+                     {1.0, 0.0});
+        EXPECT((y == std::vector<float>{2.0, 4.0, 0.0, 0.25, 2.0, 3.0, 0.0, 0.5, 2.0, 3.0, 0.0, 0.5, 2.0, 1.0, 0.0, 1.0}));
+    }
+    {// against the oracle's serial loop, float, odd sizes, no bias
+        std::mt19937 rng(9);
+        std::uniform_int_distribution<int> g(-4, 4);  // integer-valued: every partial sum is exact
+        dim_t const m = 37, k = 53, n = 29;
+        std::vector<float> a(m * k), b(k * n), ref(m * n, 0.f);
+        for (auto &v : a) v = static_cast<float>(g(rng));
+        for (auto &v : b) v = static_cast<float>(g(rng));
+        auto A = Tensor::share(DataType::F32, Shape{m, k});
+        auto B = Tensor::share(DataType::F32, Shape{k, n});
+        auto Y = Tensor::share(DataType::F32, Shape{m, n});
+        auto y = run(*A, *B, nullptr, *Y, a, b, {});
+        oracle_matmul_bias_f32(ref.data(), a.data(), b.data(), m, k, n, k, 1, n, 1, 1.f, 0.f);
+        EXPECT(y == ref);
+    }
+}
+
 static void castHip() {
     runtime::Resources res;
     auto &dev = amd();
@@ -650,6 +727,7 @@ int main(int argc, char **argv) {
         RUN(dequantizeLinearHip);
         RUN(dynamicQuantizeLinearHip);
         RUN(castHip);
+        RUN(matMulHip);
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
     }

@@ -3,7 +3,9 @@
 Bars: bit-exact for MatMulInteger / DequantizeLinear; <= 1e-5 relative for fp32 RmsNormalization
 and fp32 Softmax; <= 2e-3 absolute for fp16 paths (oracle in fp32 on up-cast inputs).
 """
+import json
 import math
+import os
 
 import numpy as np
 import pytest
@@ -17,6 +19,7 @@ pytestmark = pytest.mark.gpu
 REL_F32 = 1e-5
 ABS_F16 = 2e-3
 DEV = "cuda"
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
 
 
 def dev(a):
@@ -586,3 +589,102 @@ def test_cast_full_config_f32_to_fp16_and_back():
     assert np.array_equal(host(h).view(np.uint16), x.astype(np.float16).view(np.uint16))
     back = host(ops.cast(h, torch.float32))
     assert np.array_equal(back, x.astype(np.float16).astype(np.float32))     # widening is exact
+
+
+# ------------------------------------------------------------------ MatMul
+# Tolerances: F32 products are summed in a different order than the CPU loop: |y - ref| <= 1e-5 * sum|a||b|
+# (covers 1e-5 relative on well-conditioned sums).  FP16 / BF16: float accumulation, one rounding of the
+# result: one half-precision ulp of the reference plus the same accumulation term.
+def _matmul_check(got, ref, a_abs_b_abs, rel_out):
+    tol = rel_out * np.abs(ref) + 1e-5 * a_abs_b_abs + 1e-30
+    assert got.shape == ref.shape
+    assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= tol), \
+        float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) / tol))
+
+
+def _absprod(a, b, ta, tb):
+    A = np.abs(np.swapaxes(a, -1, -2) if ta else a).astype(np.float64)
+    B = np.abs(np.swapaxes(b, -1, -2) if tb else b).astype(np.float64)
+    return A @ B
+
+
+def test_matmul_reference_vectors():
+    for c in GOLDEN["mat_mul"]:
+        if "y" not in c:
+            continue
+        a = np.array(c["a"], np.float32).reshape(c["a_shape"])
+        b = np.array(c["b"], np.float32).reshape(c["b_shape"])
+        bias = np.array(c["c"], np.float32).reshape(c["c_shape"] or [1])
+        y = host(ops.matmul(dev(a), dev(b), dev(bias), alpha=c["alpha"], beta=c["beta"]))
+        assert y.reshape(-1).tolist() == c["y"]
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_matmul_generic_transposes_bias_broadcast(dt):
+    rng = np.random.default_rng(13)
+    np_t = np.float32 if dt == "f32" else np.float64
+    for ta in (False, True):
+        for tb in (False, True):
+            m, k, n = 37, 53, 29
+            a = rng.standard_normal((2, 1) + ((k, m) if ta else (m, k))).astype(np_t)
+            b = rng.standard_normal((1, 3) + ((n, k) if tb else (k, n))).astype(np_t)
+            for bias in (None, rng.standard_normal((m, 1)).astype(np_t), rng.standard_normal((n,)).astype(np_t),
+                         rng.standard_normal((2, 3, m, n)).astype(np_t)):
+                ref = oracle.matmul(a, b, bias, ta, tb, 0.5, 2.0, dt)
+                got = host(ops.matmul(dev(a), dev(b), None if bias is None else dev(bias), ta, tb, 0.5, 2.0))
+                _matmul_check(got, ref, _absprod(a, b, ta, tb), 1e-5 if dt == "f32" else 1e-12)
+
+
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 192, 512), (512, 128, 256)])
+def test_matmul_mfma_path_fp16_bf16(m, k, n, dt, tb):
+    rng = np.random.default_rng(14)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    b = rng.standard_normal((2, n, k) if tb else (2, k, n)).astype(np.float32)
+    bias = rng.standard_normal((n,)).astype(np.float32)
+    ad, bd, cd = (dev(t).to(dt) for t in (a, b, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(bd), to_oracle(cd), False, tb, 0.25, 1.0, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    got = f(ops.matmul(ad, bd, cd, False, tb, 0.25, 1.0))
+    _matmul_check(got, ref, 0.25 * _absprod(f(ad), f(bd), False, tb), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    # broadcast B over the batch (per-matrix launches) and no bias
+    got = f(ops.matmul(ad, bd[:1].contiguous(), None, False, tb))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(bd[:1].contiguous()), None, False, tb, dtype=name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    _matmul_check(got, ref, _absprod(f(ad), f(bd[:1]), False, tb), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+
+
+def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
+    # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
+    # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
+    rng = np.random.default_rng(15)
+    a = rng.integers(-2, 3, (768, 320)).astype(np.float32)
+    b = rng.integers(-2, 3, (320, 512)).astype(np.float32)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.max(np.abs(want)) < 2048
+    got = host(ops.matmul(dev(a).half(), dev(b).half()).float())
+    assert np.array_equal(got, want.astype(np.float32))
+    got_t = host(ops.matmul(dev(a).half(), dev(np.ascontiguousarray(b.T)).half(), trans_b=True).float())
+    assert np.array_equal(got_t, want.astype(np.float32))
+    # generic kernel on the same data (transposed A) and odd shapes
+    got_g = host(ops.matmul(dev(np.ascontiguousarray(a.T)).half(), dev(b).half(), trans_a=True).float())
+    assert np.array_equal(got_g, want.astype(np.float32))
+
+
+def test_matmul_full_config_fp16():
+    # 4096 x 4096 x 4096 (a decoder layer's projection at 4096 tokens): float64 BLAS on the fp16
+    # values as the full-size check, a sample of rows against the oracle
+    rng = np.random.default_rng(16)
+    a = (rng.standard_normal((4096, 4096)) * 0.5).astype(np.float16)
+    b = (rng.standard_normal((4096, 4096)) * 0.05).astype(np.float16)
+    got = host(ops.matmul(dev(a), dev(b), trans_b=True).float())
+    ref64 = a.astype(np.float64) @ b.astype(np.float64).T
+    bound = 2.0 ** -10 * np.abs(ref64) + 1e-5 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T)
+    assert np.all(np.abs(got - ref64) <= bound)
+    rows = [0, 255, 256, 4095]
+    ref = oracle.matmul(a[rows], b, None, False, True, dtype="fp16").astype(np.float32)
+    _matmul_check(got[rows], ref, _absprod(a[rows].astype(np.float32), b.astype(np.float32), False, True), 2.0 ** -10)

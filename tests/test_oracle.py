@@ -502,3 +502,47 @@ def test_cast_bool_from_floating_sources_reference_defect_fixture():
     x = np.array([0.0, 1.5, -0.0], np.float32)
     assert oracle.cast(x, "f32", "bool").tolist() == [False, True, False]
     assert oracle.cast_bool_reference_literal(x, "f32").tolist() == [True, False, True]   # not reproduced
+
+
+# ------------------------------------------------------------------ MatMul (with bias, transposes, broadcast)
+def test_matmul_reference_vectors():
+    for c in GOLDEN["mat_mul"]:
+        if "y" not in c:
+            continue
+        a = np.array(c["a"], np.float32).reshape(c["a_shape"])
+        b = np.array(c["b"], np.float32).reshape(c["b_shape"])
+        bias = np.array(c["c"], np.float32).reshape(c["c_shape"])
+        y = oracle.matmul(a, b, bias, alpha=c["alpha"], beta=c["beta"])
+        assert y.reshape(-1).tolist() == c["y"]
+
+
+def test_matmul_against_exact_integer_arithmetic():
+    # integer-valued operands: every product and partial sum is exact in float32, so numpy's int64
+    # product is the exact answer for any transposition, alpha, beta and bias broadcast
+    rng = np.random.default_rng(12)
+    for ta in (False, True):
+        for tb in (False, True):
+            m, k, n = 5, 7, 3
+            a = rng.integers(-8, 9, (2, 1) + ((k, m) if ta else (m, k))).astype(np.float32)
+            b = rng.integers(-8, 9, (1, 3) + ((n, k) if tb else (k, n))).astype(np.float32)
+            bias = rng.integers(-8, 9, (m, 1)).astype(np.float32)
+            A = np.swapaxes(a, -1, -2) if ta else a
+            B = np.swapaxes(b, -1, -2) if tb else b
+            want = 2 * (A.astype(np.int64) @ B.astype(np.int64)) + 3 * bias.astype(np.int64)
+            got = oracle.matmul(a, b, bias, ta, tb, alpha=2.0, beta=3.0)
+            assert got.shape == (2, 3, m, n) and np.array_equal(got, want.astype(np.float32))
+            got64 = oracle.matmul(a.astype(np.float64), b.astype(np.float64), bias.astype(np.float64), ta, tb, 2.0, 3.0, "f64")
+            assert np.array_equal(got64, want.astype(np.float64))
+    # without bias beta does not enter
+    a, b = np.eye(4, dtype=np.float32), np.arange(16, dtype=np.float32).reshape(4, 4)
+    assert np.array_equal(oracle.matmul(a, b, None, beta=5.0), b)
+
+
+def test_matmul_fp16_rounds_alpha_and_the_result_once():
+    a = np.array([[1.0, 2.0 ** -11]], np.float16)
+    b = np.array([[1.0], [1.0]], np.float16)
+    # the sum 1 + 2^-11 is exact in float and a tie in fp16: one rounding to even gives 1.0
+    assert oracle.matmul(a, b, dtype="fp16").view(np.uint16).tolist() == [[0x3C00]]
+    # alpha = 1 + 2^-12 is not an fp16 number: it is 1.0 after the conversion the reference applies
+    assert oracle.matmul(np.array([[3.0]], np.float16), np.array([[1.0]], np.float16), alpha=1 + 2.0 ** -12,
+                         dtype="fp16").tolist() == [[3.0]]
