@@ -44,6 +44,7 @@ MEASURED_TRAFFIC = {
     "matmul_integer": (2 * 49313 + 65638) * 1024,
     "attention_prefill": (2 * 100058 + 200612) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
+    "matmul": (2 * 98778 + 33024) * 1024,
 }
 
 
@@ -405,6 +406,34 @@ def main():
             ops_out["matmul_integer"]["cpu_baseline"] = {
                 "value": round(2 * m * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
                 "sample": f"first {m} rows of A against all of B ({dt:.1f} s)"}
+        del a, b, y
+
+    if want("matmul"):
+        # a decoder layer's projection at 4096 tokens: activations [4096, 4096] x weights [4096, 4096]^T, fp16
+        a = torch.randn((4096, 4096), device=dev).half()
+        b = (torch.randn((4096, 4096), device=dev) * 0.05).half()
+        y = torch.empty((4096, 4096), device=dev, dtype=torch.float16)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, b, trans_b=True, out=y), steps, warmup, 1)
+        tflops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
+        ops_out["matmul"] = {
+            "bound": "mfma", "achieved": round(tflops, 1), "peak": FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tflops / FP16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get("matmul"),
+            "workload": "MatMul fp16 [4096,4096] x [4096,4096]^T (trans_b), alpha 1, no bias",
+            "device_ms_per_launch": round(dms, 5), "timing": mode, "observed_sclk_mhz": LAST_CLOCK[0]}
+        if LAST_CLOCK[0]:
+            at_clock = FP16_PEAK_TFLOPS * LAST_CLOCK[0]["median"] / 2400.0
+            ops_out["matmul"]["peak_at_observed_clock"] = round(at_clock, 1)
+            ops_out["matmul"]["frac_at_observed_clock"] = round(tflops / at_clock, 4)
+        if not args.no_cpu:
+            import oracle
+            rows = 128
+            an, bn = a[:rows].cpu().numpy(), b.cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.matmul(an, bn, None, False, True, dtype="fp16")
+            dt = time.perf_counter() - t0
+            ops_out["matmul"]["cpu_baseline"] = {
+                "value": round(2 * rows * 4096 * 4096 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": f"first {rows} rows of A against all of B ({dt:.1f} s), float on the up-cast values"}
         del a, b, y
 
     if want("attention_prefill"):
