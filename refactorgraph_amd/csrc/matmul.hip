@@ -267,23 +267,53 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     mm_tile_loop<T, TRANS_B>(acc, lds0, lds1, A, B, k, 2 * k, TRANS_B ? 2 * k : 2 * n);
 
     // 32x32 accumulator layout: lane holds column (lane % 32); register e holds row
-    // 8*(e/4) + 4*(lane/32) + e%4.
+    // 8*(e/4) + 4*(lane/32) + e%4.  The 128x128 block of a wavefront is transposed through LDS (its
+    // own 32 KiB of the tile buffers, free now) so that Y is written with 128-bit row-contiguous
+    // stores: neighbouring lanes first exchange two of their four rows, so that every lane writes
+    // two adjacent columns (one dword) of two rows; chunk c of row r sits at chunk position c ^ (r & 15).
     const uint32_t wm = wave >> 1, wn = wave & 1;
     const uint32_t row0 = tile_m * BM + wm * 128, col0 = tile_n * BN + wn * 128;
-    T *Y = y + (ym * m + row0) * n + col0;
     const T *C = static_cast<const T *>(bias.ptr);
+    __syncthreads();  // every wavefront has read its last fragments
+    uint8_t *stage = (wave & 2 ? lds1 : lds0) + (wave & 1) * 32768;
+    const bool odd = lane & 1;
+    const uint32_t col_pair = (lane & 31) & ~1u;  // first of the two columns this lane writes
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const uint32_t row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
-                const uint32_t col = j * 32 + (lane & 31);
-                float v = alpha * acc[i][j][e];
-                if (C) v += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
-                Y[static_cast<uint64_t>(row) * n + col] = down<T>(v);
+            for (int eg = 0; eg < 4; ++eg) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t row = i * 32 + 8 * eg + 4 * (lane >> 5) + e, col = j * 32 + (lane & 31);
+                    v[e] = alpha * acc[i][j][4 * eg + e];
+                    if (C) v[e] += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
+                }
+                // even lanes keep rows 0 and 1, odd lanes rows 2 and 3 of the group of four
+                const float give0 = odd ? v[0] : v[2], give1 = odd ? v[1] : v[3];
+                const float got0 = __shfl_xor(give0, 1, kWave), got1 = __shfl_xor(give1, 1, kWave);
+                const float lo0 = odd ? got0 : v[0], hi0 = odd ? v[2] : got0;
+                const float lo1 = odd ? got1 : v[1], hi1 = odd ? v[3] : got1;
+                const uint32_t r_first = i * 32 + 8 * eg + 4 * (lane >> 5) + (odd ? 2 : 0);
+                const uint32_t byte_col = 2 * (j * 32 + col_pair);
+                auto put = [&](uint32_t row, float lo, float hi) {
+                    const T pair[2] = {down<T>(lo), down<T>(hi)};
+                    *reinterpret_cast<uint32_t *>(stage + row * 256 + (byte_col ^ (16 * (row & 15)))) =
+                        __builtin_bit_cast(uint32_t, pair);
+                };
+                put(r_first, lo0, hi0);
+                put(r_first + 1, lo1, hi1);
             }
+    // (each wavefront reads back only what it wrote itself: no barrier)
+    T *Y = y + (ym * m + row0) * n + col0;
+#pragma unroll
+    for (int it = 0; it < 32; ++it) {
+        const uint32_t idx = lane + 64 * it, row = idx / 16, chunk = idx % 16;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * 256 + 16 * (chunk ^ (row & 15)));
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(Y + static_cast<uint64_t>(row) * n + chunk * 8));
+    }
 }
 
 template <class T>
