@@ -45,6 +45,7 @@ MEASURED_TRAFFIC = {
     "attention_prefill": (2 * 100058 + 200612) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
+    "matmul_few_rows": (2 * 17456 + 256) * 1024,
 }
 
 
@@ -435,6 +436,24 @@ def main():
                 "value": round(2 * rows * 4096 * 4096 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                 "sample": f"first {rows} rows of A against all of B ({dt:.1f} s), float on the up-cast values"}
         del a, b, y
+
+    if want("matmul_few_rows"):
+        # the same projection in a decode step: 32 rows of activations; bound by reading the weights once
+        nb = 10  # 10 x 33.5 MB of weights: beyond the memory-side cache
+        a = torch.randn((32, 4096), device=dev).half()
+        ws = [(torch.randn((4096, 4096), device=dev) * 0.05).half() for _ in range(nb)]
+        y = torch.empty((32, 4096), device=dev, dtype=torch.float16)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, ws[i], trans_b=True, out=y), steps, warmup, nb)
+        few_bytes = (4096 * 4096 + 2 * 32 * 4096) * 2
+        e = hbm_entry(few_bytes, dms, "matmul_few_rows")
+        e.update(workload="MatMul fp16 [32,4096] x [4096,4096]^T (trans_b)", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            an, bn = a.cpu().numpy(), ws[0][:512].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.matmul(an, bn, None, False, True, dtype="fp16"),
+                                        (512 * 4096 + 32 * 4096 + 32 * 512) * 2, "512 of the 4096 rows of W")
+        ops_out["matmul_few_rows"] = e
+        del a, ws, y
 
     if want("attention_prefill"):
         Np, seq = 32, 512

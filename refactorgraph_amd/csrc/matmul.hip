@@ -316,6 +316,125 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     }
 }
 
+// ---------------------------------------------------------------- few rows of A (decode): weight streaming
+//
+// Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 32, FP16 / BF16: bound by reading W once
+// from HBM.  A workgroup owns 32 rows of W (32 columns of Y); its four wavefronts each take a
+// quarter of k.  A wavefront loads a 32 x 128 tile of W and the matching tile of A with coalesced
+// 128-bit loads (4 rows of 256 bytes per instruction: longer runs per row serve the DRAM pages
+// better than 128 bytes did) two tiles ahead into registers, passes a tile through its own
+// 16 KiB of LDS (chunk-swizzled rows) to bring it into MFMA operand layout, and
+// multiplies with v_mfma_f32_32x32x16 (W rows as the first operand, so a lane holds one row of A in
+// the result).  No barrier in the loop: a wavefront only reads what it wrote itself.  The four
+// partial sums meet once at the end.  (Copying the tiles straight into LDS, as the big kernels
+// do, is slower here: that path moves about 24 bytes per clock and CU, a third of what plain
+// loads reach, and this kernel has nothing else to hide behind.)
+constexpr int SK_DEPTH = 2;   // tiles in flight per wavefront
+constexpr int SK_TK = 128;    // k elements per tile (256 bytes per row)
+constexpr int SK_LOADS = 8;   // 128-bit loads per lane and operand tile
+
+template <class T>
+__global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
+                                                 Bias bias, uint32_t m, uint32_t m_total, uint32_t row_first,
+                                                 uint32_t k, uint32_t n, float alpha, float beta, uint32_t a_matrix0,
+                                                 uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(16) uint8_t lds[4 * 16384 + 4 * 32 * 33 * 4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t n0 = blockIdx.x * 32;
+    const uint64_t pitch = 2ull * k;  // bytes of a row of A or W
+    const uint8_t *W = reinterpret_cast<const uint8_t *>(w + (bm * n + n0) * static_cast<uint64_t>(k));
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m_total + row_first) * static_cast<uint64_t>(k));
+
+    // this wavefront's k-tiles (128 elements = 256 bytes each)
+    const uint32_t k_tiles = k / SK_TK;
+    const uint32_t t0 = k_tiles * wave / 4, t1 = k_tiles * (wave + 1) / 4;
+
+    // load i of a tile brings rows 4 i .. 4 i + 3: this lane row + lane / 16, 16-byte chunk lane % 16,
+    // kept in LDS at chunk position (lane % 16) ^ (row & 15); rows of A beyond m repeat its last row
+    // (their results are not stored)
+    const uint32_t ld_row = lane >> 4, ld_chunk = lane & 15;
+    const uint8_t *w_src = W + ld_row * pitch + 16 * ld_chunk;
+    uint32_t a_row[SK_LOADS];
+#pragma unroll
+    for (int i = 0; i < SK_LOADS; ++i) a_row[i] = 4 * i + ld_row < m ? 4 * i + ld_row : m - 1;
+    struct Tile {
+        u32x4 w[SK_LOADS], a[SK_LOADS];
+    };
+    auto load = [&](Tile &t, uint32_t kt) {
+#pragma unroll
+        for (int i = 0; i < SK_LOADS; ++i)
+            t.w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(w_src + 4 * i * pitch + kt * 256));
+#pragma unroll
+        for (int i = 0; i < SK_LOADS; ++i)
+            t.a[i] = *reinterpret_cast<const u32x4 *>(A + a_row[i] * pitch + 16 * ld_chunk + kt * 256);
+    };
+    // fragment of k-step ks: row lane % 32, chunk 2 ks + lane / 32
+    const uint32_t r = lane & 31, h = lane >> 5;
+    const uint32_t f_off = r * 256 + 16 * (h ^ (r & 15));
+    uint8_t *mine = lds + wave * 16384;
+
+    f16v acc0, acc1;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.f;
+    auto multiply = [&](const Tile &t) {
+#pragma unroll
+        for (int i = 0; i < SK_LOADS; ++i) {
+            const uint32_t row = 4 * i + ld_row, off = row * 256 + 16 * (ld_chunk ^ (row & 15));
+            *reinterpret_cast<u32x4 *>(mine + off) = t.w[i];
+            *reinterpret_cast<u32x4 *>(mine + 8192 + off) = t.a[i];
+        }
+#pragma unroll
+        for (int ks = 0; ks < SK_TK / 16; ks += 2) {
+            const u32x4 w0 = *reinterpret_cast<const u32x4 *>(mine + (f_off ^ (32 * ks)));
+            const u32x4 a0 = *reinterpret_cast<const u32x4 *>(mine + 8192 + (f_off ^ (32 * ks)));
+            const u32x4 w1 = *reinterpret_cast<const u32x4 *>(mine + (f_off ^ (32 * (ks + 1))));
+            const u32x4 a1 = *reinterpret_cast<const u32x4 *>(mine + 8192 + (f_off ^ (32 * (ks + 1))));
+            acc0 = Mfma<T>::run(w0, a0, acc0);
+            acc1 = Mfma<T>::run(w1, a1, acc1);
+        }
+    };
+
+    Tile tile[SK_DEPTH];
+#pragma unroll
+    for (int i = 0; i < SK_DEPTH; ++i)
+        if (t0 + i < t1) load(tile[i], t0 + i);
+    for (uint32_t t = t0; t < t1; t += SK_DEPTH) {
+#pragma unroll
+        for (int i = 0; i < SK_DEPTH; ++i) {
+            if (t + i < t1) {
+                multiply(tile[i]);
+                if (t + i + SK_DEPTH < t1) load(tile[i], t + i + SK_DEPTH);
+            }
+        }
+    }
+
+    // partial sums: lane holds row (lane % 32) of A, register e column 8 (e/4) + 4 (lane/32) + e%4 of the block
+    float *part = reinterpret_cast<float *>(lds + 4 * 16384);  // [wave][row of A][column], pitch 33
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const uint32_t col = 8 * (e / 4) + 4 * h + (e % 4);
+        part[(wave * 32 + r) * 33 + col] = acc0[e] + acc1[e];
+    }
+    __syncthreads();
+    const T *C = static_cast<const T *>(bias.ptr);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t idx = tid + 256 * q, row = idx / 32, col = idx % 32;
+        if (row < m) {
+            float v = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < 4; ++wv) v += part[(wv * 32 + row) * 33 + col];
+            v *= alpha;
+            const uint64_t yrow = row_first + row;
+            if (C) v += beta * up(C[ym * bias.sb + yrow * bias.sm + (n0 + col) * bias.sn]);
+            y[(ym * m_total + yrow) * n + n0 + col] = down<T>(v);
+        }
+    }
+}
+
 template <class T>
 int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_a, int trans_b, float alpha, float beta,
                  size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
@@ -328,8 +447,23 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     constexpr bool narrow = sizeof(T) == 2;
     const bool fast = narrow && !trans_a && m % BM == 0 && n % BN == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
 
+    // few rows, weights as [n, k]: stream W once per slab of 32 rows of A
+    const bool skinny = narrow && !fast && !trans_a && trans_b && m <= 128 && n % 32 == 0 && k % SK_TK == 0 &&
+                        aligned16(a) && aligned16(b);
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            if (skinny) {
+                for (size_t r0 = 0; r0 < m; r0 += 32) {
+                    const uint32_t rows = static_cast<uint32_t>(m - r0 < 32 ? m - r0 : 32);
+                    mm_skinny<T><<<dim3(static_cast<unsigned>(n / 32), 1, count), 256, 0, s>>>(
+                        y, a, b, bias, rows, static_cast<uint32_t>(m), static_cast<uint32_t>(r0), static_cast<uint32_t>(k),
+                        static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                    const int rc = launch_status();
+                    if (rc) return rc;
+                }
+                return 0;
+            }
             if (fast) {
                 const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
                 if (trans_b)

@@ -688,3 +688,27 @@ def test_matmul_full_config_fp16():
     rows = [0, 255, 256, 4095]
     ref = oracle.matmul(a[rows], b, None, False, True, dtype="fp16").astype(np.float32)
     _matmul_check(got[rows], ref, _absprod(a[rows].astype(np.float32), b.astype(np.float32), False, True), 2.0 ** -10)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160)])
+def test_matmul_few_rows_weight_streaming(m, k, n, dt):
+    # weights as [n, k] (trans_b), up to 128 rows of A: the kernel that reads W once per 32 rows
+    rng = np.random.default_rng(17)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    w = (rng.standard_normal((2, n, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal((n,)).astype(np.float32)
+    ad, wd, cd = (dev(t).to(dt) for t in (a, w, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(wd), to_oracle(cd), False, True, 0.5, 1.0, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    got = f(ops.matmul(ad, wd, cd, False, True, 0.5, 1.0))
+    _matmul_check(got, ref, 0.5 * _absprod(f(ad), f(wd), False, True), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    # exact on integer-valued operands (every partial sum of every wavefront is exact)
+    ai = rng.integers(-2, 3, (m, k)).astype(np.float32)
+    wi = rng.integers(-2, 3, (n, k)).astype(np.float32)
+    want = ai.astype(np.int64) @ wi.astype(np.int64).T
+    if np.max(np.abs(want)) < (2048 if name == "fp16" else 256):
+        assert np.array_equal(f(ops.matmul(dev(ai).to(dt), dev(wi).to(dt), trans_b=True)), want.astype(np.float32))
