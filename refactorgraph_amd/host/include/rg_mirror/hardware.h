@@ -63,6 +63,27 @@ namespace refactor::hardware {
         void *copyDD(void *dst, void const *src, size_t bytes) const final;
     };
 
+    // smallest multiple of `alignment` that is >= bytes (src/02hardware/include/hardware/functions.h)
+    constexpr size_t alignBytes(size_t bytes, size_t alignment) noexcept {
+        return alignment ? (bytes + alignment - 1) / alignment * alignment : bytes;
+    }
+
+    // Plans offsets inside one range that only grows at its end: alloc() takes the smallest free
+    // block that fits (lowest offset among equals), else lengthens the free block that touches
+    // the end, else appends; free() merges neighbours.  peak() is the range the plan needs.
+    // Behaviour of src/02hardware/src/mem_offset_calculator.cc:28-117 (without its tracing).
+    class OffsetCalculator {
+        size_t _used = 0, _peak = 0, _alignment;
+        std::map<size_t, size_t> _freeByOffset;// offset -> bytes
+
+    public:
+        explicit OffsetCalculator(size_t alignment, bool trace = false);
+        size_t alloc(size_t bytes);
+        void free(size_t offset, size_t bytes);
+        size_t peak() const noexcept { return _peak; }
+        size_t used() const noexcept { return _used; }
+    };
+
     class Device {
     public:
         enum class Type : int32_t {

@@ -1,6 +1,6 @@
 // runtime layer of the host mirror: the Routine signature every kernel lowers to and the
 // per-stream Resources map.  Follows src/03runtime/include/runtime/{stream.h:10-22,
-// resource.h:10-45}; the graph-walking Stream itself is outside this build.
+// resource.h:10-45}; the graph-walking Stream is in rg_mirror/stream.h.
 #pragma once
 
 #include "rg_mirror/common.h"

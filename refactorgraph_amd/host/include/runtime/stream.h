@@ -1,3 +1,3 @@
 // reference include path -> host mirror
 #pragma once
-#include "rg_mirror/runtime.h"
+#include "rg_mirror/stream.h"

@@ -2,6 +2,7 @@
 #include "rg_hip.h"
 #include <cstdlib>
 #include <cstring>
+#include <iterator>
 #include <utility>
 
 #define HIP_ASSERT(CALL)                                                                              \
@@ -39,6 +40,59 @@ namespace refactor::hardware {
     void *AmdMemory::copyDD(void *dst, void const *src, size_t bytes) const {
         HIP_ASSERT(rg_hip_memcpy_d2d(dst, src, bytes));
         return dst;
+    }
+
+    // ------------------------------------------------------------------ offset planning
+
+    OffsetCalculator::OffsetCalculator(size_t alignment, bool) : _alignment(alignment ? alignment : 1) {}
+
+    size_t OffsetCalculator::alloc(size_t bytes) {
+        auto const need = alignBytes(bytes, _alignment);
+        _used += need;
+        auto best = _freeByOffset.end();
+        for (auto it = _freeByOffset.begin(); it != _freeByOffset.end(); ++it)
+            if (it->second >= need && (best == _freeByOffset.end() || it->second < best->second)) best = it;
+        if (best != _freeByOffset.end()) {
+            auto const [offset, size] = *best;
+            _freeByOffset.erase(best);
+            if (size > need) _freeByOffset.emplace(offset + need, size - need);
+            return offset;
+        }
+        if (!_freeByOffset.empty()) {
+            auto last = std::prev(_freeByOffset.end());
+            if (last->first + last->second == _peak) {// too small, but it can grow with the range
+                auto const offset = last->first;
+                _freeByOffset.erase(last);
+                _peak = offset + need;
+                return offset;
+            }
+        }
+        auto const offset = _peak;
+        _peak += need;
+        return offset;
+    }
+
+    void OffsetCalculator::free(size_t offset, size_t bytes) {
+        auto size = alignBytes(bytes, _alignment);
+        _used -= size;
+        auto next = _freeByOffset.lower_bound(offset);
+        if (next != _freeByOffset.begin()) {
+            auto prev = std::prev(next);
+            ASSERT(prev->first + prev->second <= offset, "double free");
+            if (prev->first + prev->second == offset) {
+                offset = prev->first;
+                size += prev->second;
+                _freeByOffset.erase(prev);
+            }
+        }
+        if (next != _freeByOffset.end()) {
+            ASSERT(offset + size <= next->first, "double free");
+            if (offset + size == next->first) {
+                size += next->second;
+                _freeByOffset.erase(next);
+            }
+        }
+        _freeByOffset.emplace(offset, size);
     }
 
     // ------------------------------------------------------------------ pool

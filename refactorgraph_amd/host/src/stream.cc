@@ -1,0 +1,73 @@
+// runtime::Stream of the host mirror (see rg_mirror/stream.h).
+#include "rg_mirror/stream.h"
+
+namespace refactor::runtime {
+
+    Stream::Stream(Resources resources, size_t stackBytes, graph_topo::GraphTopo topology, std::vector<Node> nodes,
+                   std::vector<Edge> edges, Arc<hardware::Device> device)
+        : _device(std::move(device)),
+          _stack(_device->malloc(stackBytes)),
+          _resources(std::move(resources)),
+          _graph{std::move(topology), std::move(nodes), std::move(edges)} {
+        ASSERT(_graph.nodes.size() == _graph.topology.nodeCount(), "one runtime node per topology node");
+        ASSERT(_graph.edges.size() == _graph.topology.edgeCount(), "one runtime edge per topology edge");
+    }
+
+    Arc<hardware::Device::Blob> Stream::setData(count_t edge, size_t bytes) {
+        return _graph.edges.at(edge).blob = _device->malloc(bytes);
+    }
+    void Stream::setData(count_t edge, Arc<hardware::Device::Blob> blob) { _graph.edges.at(edge).blob = std::move(blob); }
+    void Stream::setData(count_t edge, void const *hostData, size_t bytes) {
+        auto blob = _device->malloc(bytes);
+        blob->copyFromHost(hostData, bytes);
+        _graph.edges.at(edge).blob = std::move(blob);
+    }
+    Arc<hardware::Device::Blob> Stream::getData(count_t edge) const { return _graph.edges.at(edge).blob; }
+    bool Stream::copyData(count_t edge, void *hostData, size_t bytes) const {
+        auto const &blob = _graph.edges.at(edge).blob;
+        if (!blob) return false;
+        blob->copyToHost(hostData, bytes);
+        return true;
+    }
+
+    template<class F> void Stream::walk(F &&visit) {
+        auto *stack = _stack->get<uint8_t>();
+        std::vector<void *> addresses;
+        auto address = [&](count_t e) -> void * {
+            auto const &edge = _graph.edges[e];
+            return edge.blob ? edge.blob->get() : stack + edge.stackOffset;
+        };
+        for (auto [idx, inputs, outputs] : _graph.topology) {
+            addresses.clear();
+            for (auto e : inputs) addresses.push_back(address(e));
+            for (auto e : outputs) addresses.push_back(address(e));
+            auto const *in = const_cast<void const *const *>(addresses.data());
+            auto *const *out = addresses.data() + inputs.size();
+            auto const &node = _graph.nodes[idx];
+            _device->setContext();
+            auto const t0 = std::chrono::steady_clock::now();
+            node.routine(_resources, stack + node.workspaceOffset, in, out);
+            visit(idx, in, out, t0);
+        }
+    }
+
+    void Stream::run() {
+        walk([](count_t, void const *const *, void *const *, std::chrono::steady_clock::time_point) {});
+    }
+
+    std::vector<std::chrono::nanoseconds> Stream::bench(void (*sync)()) {
+        std::vector<std::chrono::nanoseconds> ans(_graph.nodes.size());
+        walk([&](count_t idx, void const *const *, void *const *, std::chrono::steady_clock::time_point t0) {
+            if (sync) sync();
+            ans[idx] = std::chrono::steady_clock::now() - t0;
+        });
+        return ans;
+    }
+
+    void Stream::trace(std::function<void(count_t, void const *const *, void const *const *)> record) {
+        walk([&](count_t idx, void const *const *in, void *const *out, std::chrono::steady_clock::time_point) {
+            record(idx, in, const_cast<void const *const *>(out));
+        });
+    }
+
+}// namespace refactor::runtime

@@ -15,7 +15,12 @@
 #include "kernel/collectors/rms_normalization.h"
 #include "kernel/collectors/rotary_embedding.h"
 #include "kernel/collectors/softmax.h"
+#include "graph_topo.h"
 #include "hardware/device_manager.h"
+#include "hardware/mem_offset_calculator.h"
+#include "kernel/allocators.h"
+#include "kernel/graph.h"
+#include "runtime/stream.h"
 #include "hardware/mem_pool.h"
 #include "rg_mirror/hip_kernels.h"
 #include "oracle.h"
@@ -258,6 +263,221 @@ static void collectorsSelectOrDecline() {
 }
 
 // ------------------------------------------------------------------ routines on the AMD device
+
+// ------------------------------------------------------------------ graph -> stream (host logic)
+
+static void graphTopoAndBuilder() {
+    using graph_topo::Builder;
+    // keys chosen so that key order ("a" < "b") is the reverse of the order the nodes can run in
+    Builder<std::string, int, std::string, int> b;
+    b.topology["b"] = {{"x", "w0"}, {"t0"}};
+    b.topology["a"] = {{"t0", "w1", "x"}, {"t1", "t2"}};
+    b.globalInputs = {"x"};
+    b.globalOutputs = {"t2", "t0"};
+    b.nodes = {{"a", 11}, {"b", 22}};
+    b.edges = {{"x", 100}, {"w0", 101}, {"w1", 103}, {"t0", 102}, {"t2", 105}};
+    auto g = b.build();
+    auto const &t = g.topology;
+    EXPECT(t.nodeCount() == 2 && t.edgeCount() == 6 && t.globalInputsCount() == 1 && t.globalOutputsCount() == 2);
+    EXPECT((g.nodes == std::vector<int>{22, 11}));
+    // numbering: x | w0 t0 | w1 t1 t2   (t1 has no value of its own: default-constructed)
+    EXPECT((g.edges == std::vector<int>{100, 101, 102, 103, 0, 105}));
+    std::vector<count_t> conn(t.connections().begin(), t.connections().end());
+    EXPECT((conn == std::vector<count_t>{5, 2, 0, 1, 2, 3, 0}));
+    EXPECT(t.globalOutputs().size() == 2 && t.globalOutputs()[0] == 5 && t.globalOutputs()[1] == 2);
+    size_t seen = 0;
+    for (auto [idx, inputs, outputs] : t) {
+        if (idx == 0) EXPECT(inputs.size() == 2 && inputs[0] == 0 && inputs[1] == 1 && outputs.size() == 1 && outputs[0] == 2);
+        if (idx == 1) EXPECT(inputs.size() == 3 && inputs[0] == 2 && inputs[1] == 3 && inputs[2] == 0 && outputs.size() == 2 && outputs[0] == 4 && outputs[1] == 5);
+        ++seen;
+    }
+    EXPECT(seen == 2);
+    EXPECT(t.node(1).outputs.at(1) == 5 && t.firstEdgeOf(1) == 3 && t.localEdgesOf(1) == 1);
+    EXPECT(throws<std::runtime_error>([&] { t.node(2); }));
+    EXPECT(t.toString().find("node 1: 2 3 0 -> 4 5") != std::string::npos);
+    // two nodes that wait for each other cannot be ordered
+    Builder<int, int, int, int> cyc;
+    cyc.topology[0] = {{1}, {0}};
+    cyc.topology[1] = {{0}, {1}};
+    cyc.nodes = {{0, 0}, {1, 1}};
+    EXPECT(throws<std::runtime_error>([&] { cyc.build(); }));
+    // hand-built topology: an edge numbered after the node's own cannot be read
+    graph_topo::GraphTopo manual(1, 1);
+    EXPECT(manual.pushNode({0}, 0, 1).begin_ == 1);
+    EXPECT(throws<std::runtime_error>([&] { manual.pushNode({3}, 0, 1); }));
+    manual.setGlobalOutput(0, 1);
+    EXPECT(manual.globalOutputs()[0] == 1);
+}
+
+static void offsetCalculatorPlan() {
+    OffsetCalculator c(8);
+    EXPECT(c.alloc(10) == 0 && c.alloc(20) == 16 && c.alloc(8) == 40 && c.peak() == 48);
+    c.free(16, 20);                                  // free: [16, 40)
+    EXPECT(c.alloc(8) == 16);                        // best (only) fit, split: [24, 40) stays free
+    EXPECT(c.alloc(16) == 24 && c.peak() == 48);     // exact fit
+    c.free(40, 8);                                   // the free block now touches the end
+    EXPECT(c.alloc(32) == 40 && c.peak() == 72);     // too small, grows with the range
+    c.free(0, 10);
+    c.free(24, 16);
+    c.free(16, 8);                                   // merges with both neighbours: [0, 40)
+    EXPECT(c.alloc(40) == 0 && c.peak() == 72);
+    // best fit prefers the smaller of two free blocks
+    OffsetCalculator d(1);
+    auto a0 = d.alloc(100), a1 = d.alloc(10), a2 = d.alloc(50), a3 = d.alloc(10);
+    d.free(a0, 100);
+    d.free(a2, 50);
+    EXPECT(d.alloc(40) == a2 && d.alloc(60) == a0 && a1 == 100 && a3 == 160 && d.peak() == 170);
+    EXPECT(throws<std::runtime_error>([&] { d.free(a1, 10); d.free(a1, 10); }));
+    EXPECT(alignBytes(100, 32) == 128 && alignBytes(128, 32) == 128 && alignBytes(0, 32) == 0);
+}
+
+namespace {
+    // y[i] = x[i] + addend over `n` floats; with `viaWorkspace` the sum is formed in the workspace first
+    class AddKernel final : public Kernel {
+        float _addend;
+        size_t _n;
+        bool _viaWorkspace;
+
+    public:
+        AddKernel(float addend, size_t n, bool viaWorkspace) : _addend(addend), _n(n), _viaWorkspace(viaWorkspace) {}
+        static size_t typeId() noexcept {
+            static uint8_t ID = 1;
+            return reinterpret_cast<size_t>(&ID);
+        }
+        size_t kernelTypeId() const final { return typeId(); }
+        std::string_view description() const final { return "test kernel: add a constant on the host"; }
+        RoutineWorkspace lower(Resources &) const final {
+            auto routine = [addend = _addend, n = _n, ws = _viaWorkspace](Resources &, void *workspace, void const *const *inputs, void *const *outputs) {
+                auto x = static_cast<float const *>(inputs[0]);
+                auto y = static_cast<float *>(outputs[0]);
+                auto t = ws ? static_cast<float *>(workspace) : y;
+                for (size_t i = 0; i < n; ++i) t[i] = x[i] + addend;
+                if (ws) std::memcpy(y, t, n * sizeof(float));
+            };
+            return {std::move(routine), _viaWorkspace ? _n * sizeof(float) : 0};
+        }
+    };
+    // y = a + b
+    class SumKernel final : public Kernel {
+        size_t _n;
+
+    public:
+        explicit SumKernel(size_t n) : _n(n) {}
+        static size_t typeId() noexcept {
+            static uint8_t ID = 1;
+            return reinterpret_cast<size_t>(&ID);
+        }
+        size_t kernelTypeId() const final { return typeId(); }
+        std::string_view description() const final { return "test kernel: add two tensors on the host"; }
+        RoutineWorkspace lower(Resources &) const final {
+            return [n = _n](Resources &, void *, void const *const *inputs, void *const *outputs) {
+                auto a = static_cast<float const *>(inputs[0]), b = static_cast<float const *>(inputs[1]);
+                auto y = static_cast<float *>(outputs[0]);
+                for (size_t i = 0; i < n; ++i) y[i] = a[i] + b[i];
+            };
+        }
+    };
+}// namespace
+
+// x -> (+1) -> t0 -> (+2, workspace) -> t1 -> (+ c) -> t2 -> (+4) -> y, with c a constant edge and an
+// unused second output nobody reads
+static kernel::Graph chainGraph(size_t n, Arc<kernel::Blob> constant) {
+    graph_topo::GraphTopo topo(1, 1);
+    topo.pushNode({0}, 0, 1);       // edge 1 = t0
+    topo.pushNode({1}, 0, 1);       // edge 2 = t1
+    topo.pushNode({2, 3}, 1, 1);    // edge 3 = c (local), edge 4 = t2
+    topo.pushNode({4}, 0, 1);       // edge 5 = y
+    topo.setGlobalOutput(0, 5);
+    std::vector<kernel::Node> nodes;
+    nodes.push_back({std::make_unique<AddKernel>(1.f, n, false), "n0"});
+    nodes.push_back({std::make_unique<AddKernel>(2.f, n, true), "n1"});
+    nodes.push_back({std::make_unique<SumKernel>(n), "n2"});
+    nodes.push_back({std::make_unique<AddKernel>(4.f, n, false), "n3"});
+    auto const bytes = n * sizeof(float);
+    std::vector<kernel::Edge> edges{{nullptr, bytes, "x"}, {nullptr, bytes, "t0"}, {nullptr, bytes, "t1"},
+                                    {std::move(constant), bytes, "c"}, {nullptr, bytes, "t2"}, {nullptr, bytes, "y"}};
+    return kernel::Graph(std::move(topo), std::move(nodes), std::move(edges));
+}
+
+static void allocatorsAndStreamOnCpu() {
+    constexpr size_t n = 25;// 100 bytes: 128 once aligned to 32
+    auto [constant, cPtr] = kernel::Blob::share(n * sizeof(float));
+    for (size_t i = 0; i < n; ++i) static_cast<float *>(cPtr)[i] = 10.f * i;
+    auto graph = chainGraph(n, constant);
+    auto const &topo = graph._internal.topology;
+
+    auto lowerNodes = [&] {
+        runtime::Resources res;
+        std::vector<runtime::Node> nodes;
+        for (auto const &node : graph._internal.nodes) nodes.emplace_back(node.kernel->lower(res));
+        return nodes;
+    };
+    {// flat: t0 | t1, workspace of n1 | t2, nothing is reused
+        auto [stack, nodes, edges] = flatAllocate(topo, lowerNodes(), graph._internal.edges, 32);
+        EXPECT(stack == 4 * 128);
+        EXPECT(edges[0].stackOffset == SIZE_MAX && edges[3].stackOffset == SIZE_MAX && edges[5].stackOffset == SIZE_MAX - 1);
+        EXPECT(edges[1].stackOffset == 0 && edges[2].stackOffset == 128 && nodes[1].workspaceOffset == 256 && edges[4].stackOffset == 384);
+        EXPECT(nodes[0].workspaceOffset == 0 && nodes[2].workspaceOffset == 0);
+    }
+    {// reusable: t2 takes the range t0 has given back; the workspace of n1 is free again after n1
+        auto [stack, nodes, edges] = reusableAllocate(topo, lowerNodes(), graph._internal.edges, 32);
+        EXPECT(stack == 3 * 128);
+        EXPECT(edges[1].stackOffset == 0 && edges[2].stackOffset == 128 && nodes[1].workspaceOffset == 256);
+        EXPECT(edges[4].stackOffset == 0);
+        EXPECT(edges[5].stackOffset == SIZE_MAX - 1 && edges[0].stackOffset == SIZE_MAX);
+    }
+
+    for (auto allocator : {flatAllocate, reusableAllocate}) {
+        auto stream = graph.lower(device::fetch(Device::Type::Cpu), allocator);
+        EXPECT(stream.graph().edges[3].blob && stream.graph().edges[3].name == "c");// the constant was uploaded
+        EXPECT(stream.getData(5) && !stream.getData(0) && !stream.getData(1));      // global output has a blob, the input not yet
+        std::vector<float> x(n), y(n, -1.f);
+        std::iota(x.begin(), x.end(), 0.f);
+        stream.setData(0, x.data(), n * sizeof(float));
+        stream.run();
+        EXPECT(stream.copyData(5, y.data(), n * sizeof(float)));
+        bool ok = true;
+        for (size_t i = 0; i < n; ++i) ok &= y[i] == x[i] + 7.f + 10.f * i;
+        EXPECT(ok);
+        EXPECT(!stream.copyData(1, y.data(), n * sizeof(float)));// a stack edge cannot be read back
+
+        // a second run on new data in a caller-provided blob; trace sees every node once, in order,
+        // with the addresses the routines were given
+        auto blob = stream.setData(0, n * sizeof(float));
+        for (auto &v : x) v = -v;
+        blob->copyFromHost(x.data(), n * sizeof(float));
+        std::vector<count_t> order;
+        bool addressesOk = true;
+        stream.trace([&](count_t idx, void const *const *inputs, void const *const *outputs) {
+            order.push_back(idx);
+            if (idx == 0) addressesOk &= inputs[0] == blob->get();
+            if (idx == 2) addressesOk &= inputs[1] == stream.getData(3)->get();
+            if (idx == 3) addressesOk &= outputs[0] == stream.getData(5)->get();
+        });
+        EXPECT((order == std::vector<count_t>{0, 1, 2, 3}) && addressesOk);
+        stream.copyData(5, y.data(), n * sizeof(float));
+        ok = true;
+        for (size_t i = 0; i < n; ++i) ok &= y[i] == x[i] + 7.f + 10.f * i;
+        EXPECT(ok);
+        auto times = stream.bench(nullptr);
+        EXPECT(times.size() == 4);
+    }
+    // the same constant on the same device is uploaded once and shared by the streams that are alive
+    auto s1 = graph.lower(device::fetch(Device::Type::Cpu), flatAllocate);
+    auto s2 = graph.lower(device::fetch(Device::Type::Cpu), reusableAllocate);
+    EXPECT(s1.getData(3) == s2.getData(3));
+    // a node without kernel lowers to the empty routine
+    graph_topo::GraphTopo topo1(1, 1);
+    topo1.pushNode({0}, 0, 1);
+    topo1.setGlobalOutput(0, 1);
+    std::vector<kernel::Node> nodes1;
+    nodes1.push_back({nullptr, "nothing"});
+    kernel::Graph empty(std::move(topo1), std::move(nodes1), {{nullptr, 4, "in"}, {nullptr, 4, "out"}});
+    auto s3 = empty.lower(device::fetch(Device::Type::Cpu), flatAllocate);
+    s3.setData(0, size_t(4));
+    s3.run();
+    EXPECT(s3.getData(1) && s3.getData(1)->size() == 4);
+}
 
 static Device &amd() { return *device::init(Device::Type::Amd, 0, "pool=4294967296"); }
 
@@ -694,6 +914,85 @@ static void rotaryEmbeddingHip() {
     EXPECT(ok);
 }
 
+// DynamicQuantizeLinear -> MatMulInteger -> DequantizeLinear lowered as one graph on the AMD device:
+// the quantised linear layer y = (q(x) - zp) @ W * scale, every kernel picked by its collector,
+// intermediate tensors and workspaces on the stream's stack, W a constant uploaded by lower().
+static void quantisedLinearStream() {
+    constexpr dim_t M = 96, K = 512, N = 256;
+    auto x = Tensor::share(DataType::F32, Shape{M, K});
+    auto xq = Tensor::share(DataType::U8, Shape{M, K});
+    auto scale = Tensor::share(DataType::F32, Shape{});
+    auto zp = Tensor::share(DataType::U8, Shape{});
+    auto [wBlob, wPtr] = kernel::Blob::share(K * N);
+    auto w = Tensor::share(DataType::I8, Shape{K, N}, LayoutType::Others, wBlob);
+    auto acc = Tensor::share(DataType::I32, Shape{M, N});
+    auto y = Tensor::share(DataType::F32, Shape{M, N});
+    std::mt19937 rng(21);
+    std::vector<int8_t> w_(K * N);
+    for (auto &v : w_) v = static_cast<int8_t>(rng());
+    std::memcpy(wPtr, w_.data(), w_.size());
+    std::vector<float> x_(M * K);
+    std::normal_distribution<float> g(0.3f, 2.f);
+    for (auto &v : x_) v = g(rng);
+
+    auto first = [](std::vector<KernelBox> v) {
+        EXPECT(!v.empty());
+        return std::move(v.at(0));
+    };
+    // edges: 0 x | 1 xq 2 scale 3 zp | 4 W (local) 5 acc | 6 y
+    graph_topo::GraphTopo topo(1, 1);
+    topo.pushNode({0}, 0, 3);
+    topo.pushNode({1, 4, 3}, 1, 1);
+    topo.pushNode({5, 2}, 0, 1);
+    topo.setGlobalOutput(0, 6);
+    std::vector<kernel::Node> nodes;
+    nodes.push_back({first(DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*x}, {*xq, *scale, *zp})), "quantise"});
+    nodes.push_back({first(MatMulIntegerCollector(Device::Type::Amd).filter({*xq, *w, *zp}, {*acc})), "matmul"});
+    nodes.push_back({first(DequantizeLinearCollector(Device::Type::Amd).filter({*acc, *scale}, {*y})), "dequantise"});
+    std::vector<kernel::Edge> edges{{nullptr, x->bytesSize(), "x"}, {nullptr, xq->bytesSize(), "xq"},
+                                    {nullptr, 4, "scale"}, {nullptr, 1, "zp"}, {wBlob, w->bytesSize(), "W"},
+                                    {nullptr, acc->bytesSize(), "acc"}, {nullptr, y->bytesSize(), "y"}};
+    kernel::Graph graph(std::move(topo), std::move(nodes), std::move(edges));
+
+    // oracle chain
+    std::vector<uint8_t> q(M * K);
+    float s;
+    uint8_t z;
+    oracle_dynamic_quantize_linear(q.data(), &s, &z, x_.data(), x_.size());
+    std::vector<int32_t> accRef(M * N);
+    oracle_matmul_integer(accRef.data(), q.data(), w_.data(), &z, 0, 1, nullptr, 1, 1, 1, M, K, N, nullptr, nullptr, 1, 1, 8);
+    std::vector<float> ref(M * N), out(M * N);
+    oracle_dequantize_linear(ref.data(), accRef.data(), &s, nullptr, 1, 1, M * N, ORACLE_I32, 1, 1);
+
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    for (auto allocator : {flatAllocate, reusableAllocate}) {
+        auto stream = graph.lower(dev, allocator);
+        // every stack offset is 256-byte aligned on this device
+        bool aligned = true;
+        for (auto const &e : stream.graph().edges)
+            if (!e.blob && e.stackOffset < SIZE_MAX - 1) aligned &= e.stackOffset % 256 == 0;
+        for (auto const &n : stream.graph().nodes) aligned &= n.workspaceOffset % 256 == 0;
+        EXPECT(aligned);
+        stream.setData(0, x_.data(), x->bytesSize());
+        stream.run();
+        device::sync(Device::Type::Amd);
+        EXPECT(stream.copyData(6, out.data(), y->bytesSize()));
+        EXPECT(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0);
+        // bench: one duration per node, each including the wait for the device
+        auto times = stream.bench([] { device::sync(Device::Type::Amd); });
+        EXPECT(times.size() == 3 && times[0].count() > 0 && times[1].count() > 0 && times[2].count() > 0);
+        // trace: copy the intermediate results out node by node (what Executor::trace is for)
+        std::vector<uint8_t> qGpu(M * K);
+        std::vector<int32_t> accGpu(M * N);
+        stream.trace([&](count_t idx, void const *const *, void const *const *outputs) {
+            device::sync(Device::Type::Amd);
+            if (idx == 0) AmdMemory().copyDH(qGpu.data(), outputs[0], qGpu.size());
+            if (idx == 1) AmdMemory().copyDH(accGpu.data(), outputs[0], accGpu.size() * 4);
+        });
+        EXPECT(qGpu == q && accGpu == accRef);
+    }
+}
+
 static void amdDeviceAndPool() {
     auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
     EXPECT(dev && dev->type() == Device::Type::Amd && device::fetch(Device::Type::Amd) == dev);
@@ -719,6 +1018,9 @@ int main(int argc, char **argv) {
     RUN(memPoolBestFit);
     RUN(resourcesAndErrors);
     RUN(collectorsSelectOrDecline);
+    RUN(graphTopoAndBuilder);
+    RUN(offsetCalculatorPlan);
+    RUN(allocatorsAndStreamOnCpu);
     if (mode == "gpu") {
         RUN(amdDeviceAndPool);
         RUN(rmsNormalizationHip);
@@ -730,6 +1032,7 @@ int main(int argc, char **argv) {
         RUN(matMulHip);
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
+        RUN(quantisedLinearStream);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;
