@@ -14,6 +14,7 @@
 #include <algorithm>
 #include <map>
 #include <set>
+#include <unordered_map>
 
 namespace refactor {
 
@@ -94,6 +95,10 @@ namespace refactor::graph_topo {
         // how many edges it writes.  Returns the range of its outputs.
         range_t<count_t> pushNode(std::vector<count_t> const &inputs, count_t localEdges, count_t outputs);
         void setGlobalOutput(count_t i, count_t edge);
+        // Every reader (node input or global output) of an edge that is a key of `map` reads the mapped
+        // edge instead; returns how many connections changed
+        // (src/01graph_topo/src/inplace_modifier.cc:92-101, there a separate InplaceModifier).
+        size_t reconnect(std::unordered_map<count_t, count_t> const &map);
 
         NodeRef node(count_t idx) const;
         Iterator begin() const noexcept { return Iterator(*this, 0); }

@@ -1,0 +1,125 @@
+// computation layer of the host mirror (see rg_mirror/computation.h).
+#include "rg_mirror/computation.h"
+#include <unordered_map>
+
+namespace refactor::computation {
+
+    kernel::CollectorBox Operator::candidateKernels(Target) const {
+        TODO(detail::cat("Operator \"", name(), "\" lower to kernel not implemented"));
+    }
+
+#define RG_OPERATOR_IDS(T, NAME)                                          \
+    size_t T::typeId() noexcept {                                         \
+        static uint8_t ID = 1;                                            \
+        return reinterpret_cast<size_t>(&ID);                             \
+    }                                                                     \
+    size_t T::opTypeId() const noexcept { return typeId(); }              \
+    std::string_view T::name() const noexcept { return NAME; }
+
+    RG_OPERATOR_IDS(RmsNormalization, "RmsNormalization")
+    RG_OPERATOR_IDS(Softmax, "Softmax")
+    RG_OPERATOR_IDS(MatMulInteger, "MatMulInteger")
+    RG_OPERATOR_IDS(DequantizeLinear, "DequantizeLinear")
+    RG_OPERATOR_IDS(DynamicQuantizeLinear, "DynamicQuantizeLinear")
+    RG_OPERATOR_IDS(Cast, "Cast")
+    RG_OPERATOR_IDS(MatMul, "MatMul")
+    RG_OPERATOR_IDS(Attention, "Attention")
+    RG_OPERATOR_IDS(RotaryEmbedding, "RotaryEmbedding")
+    RG_OPERATOR_IDS(Identity, "Identity")
+    RG_OPERATOR_IDS(Reshape, "Reshape")
+#undef RG_OPERATOR_IDS
+
+    kernel::CollectorBox RmsNormalization::candidateKernels(Target target) const {
+        return std::make_unique<kernel::RmsNormalizationCollector>(target, epsilon);
+    }
+    std::string RmsNormalization::serialize() const { return detail::cat(name(), '(', epsilon, ')'); }
+
+    kernel::CollectorBox Softmax::candidateKernels(Target target) const {
+        return std::make_unique<kernel::SoftmaxCollector>(target, axis, causal);
+    }
+    std::string Softmax::serialize() const {
+        return detail::cat(name(), '(', axis, '/', rank, causal ? ", causal)" : ")");
+    }
+
+    kernel::CollectorBox MatMulInteger::candidateKernels(Target target) const {
+        return std::make_unique<kernel::MatMulIntegerCollector>(target);
+    }
+    kernel::CollectorBox DequantizeLinear::candidateKernels(Target target) const {
+        return std::make_unique<kernel::DequantizeLinearCollector>(target, axis);
+    }
+    kernel::CollectorBox DynamicQuantizeLinear::candidateKernels(Target target) const {
+        return std::make_unique<kernel::DynamicQuantizeLinearCollector>(target);
+    }
+    kernel::CollectorBox Cast::candidateKernels(Target target) const {
+        return std::make_unique<kernel::CastCollector>(target);
+    }
+
+    kernel::CollectorBox MatMul::candidateKernels(Target target) const {
+        return std::make_unique<kernel::MatMulCollector>(target, alpha, beta, transA, transB);
+    }
+    std::string MatMul::serialize() const {
+        return detail::cat(name(), '(', alpha, ", ", beta, ", ", transA ? 'T' : 'N', ", ", transB ? 'T' : 'N', ')');
+    }
+
+    kernel::CollectorBox Attention::candidateKernels(Target target) const {
+        return std::make_unique<kernel::AttentionCollector>(target, maxSeqLen);
+    }
+    std::string Attention::serialize() const { return detail::cat(name(), '(', maxSeqLen, ')'); }
+
+    kernel::CollectorBox RotaryEmbedding::candidateKernels(Target target) const {
+        return std::make_unique<kernel::RotaryEmbeddingCollector>(target, theta);
+    }
+    std::string RotaryEmbedding::serialize() const { return detail::cat(name(), '(', theta, ')'); }
+
+    Graph::Graph(graph_topo::Graph<Node, Edge> internal) noexcept : _internal(std::move(internal)) {}
+    Graph::Graph(graph_topo::GraphTopo topology, std::vector<Node> nodes, std::vector<Edge> edges) noexcept
+        : _internal{std::move(topology), std::move(nodes), std::move(edges)} {}
+
+    kernel::Graph Graph::lower(Target target) const {
+        auto const &graph = _internal;
+        std::vector<kernel::Node> nodes(graph.nodes.size());
+        std::vector<kernel::Edge> edges(graph.edges.size());
+
+        std::unordered_map<count_t, count_t> identities;// output edge -> the edge it stands for
+        std::vector<std::string> noKernel;
+        for (auto [idx, inputs, outputs] : graph.topology) {
+            auto const &[op, name] = graph.nodes[idx];
+            nodes[idx] = {nullptr, name};
+            if (!op) continue;
+            if (op->isIdentity()) {
+                ASSERT(!inputs.empty() && outputs.size() == 1, "an identity has one output that renames its first input");
+                // an input that is itself an identity's output was resolved when that node was visited
+                auto source = inputs[0];
+                if (auto it = identities.find(source); it != identities.end()) source = it->second;
+                identities.emplace(outputs[0], source);
+                continue;
+            }
+            kernel::TensorRefs inputs_, outputs_;
+            for (auto e : inputs) inputs_.emplace_back(*graph.edges[e].tensor);
+            for (auto e : outputs) outputs_.emplace_back(*graph.edges[e].tensor);
+            auto candidates = op->candidateKernels(target)->filter(std::move(inputs_), std::move(outputs_));
+            if (candidates.empty()) {
+                noKernel.push_back(name);
+            } else {
+                nodes[idx].kernel = std::move(candidates.front());
+            }
+        }
+        if (!noKernel.empty()) {
+            std::string msg = "No kernel selected for ";
+            for (auto const &n : noKernel) msg += '"' + n + "\" ";
+            RUNTIME_ERROR(msg);
+        }
+        for (size_t i = 0; i < edges.size(); ++i) {
+            auto const &[tensor, name] = graph.edges[i];
+            if (!tensor || identities.count(static_cast<count_t>(i))) {
+                edges[i] = {nullptr, 0, name};
+            } else {
+                edges[i] = {tensor->data, tensor->bytesSize(), name};
+            }
+        }
+        auto topology = graph.topology;
+        topology.reconnect(identities);
+        return kernel::Graph(std::move(topology), std::move(nodes), std::move(edges));
+    }
+
+}// namespace refactor::computation

@@ -22,6 +22,16 @@ namespace refactor::graph_topo {
         _connections[i] = edge;
     }
 
+    size_t GraphTopo::reconnect(std::unordered_map<count_t, count_t> const &map) {
+        size_t changed = 0;
+        for (auto &c : _connections)
+            if (auto it = map.find(c); it != map.end()) {
+                c = it->second;
+                ++changed;
+            }
+        return changed;
+    }
+
     GraphTopo::NodeRef GraphTopo::node(count_t idx) const {
         ASSERT(idx < nodeCount(), "no such node");
         auto const *c = _connections.data();

@@ -48,6 +48,7 @@ namespace refactor::hardware {
 
     size_t OffsetCalculator::alloc(size_t bytes) {
         auto const need = alignBytes(bytes, _alignment);
+        if (need == 0) return _peak;// nothing to place
         _used += need;
         auto best = _freeByOffset.end();
         for (auto it = _freeByOffset.begin(); it != _freeByOffset.end(); ++it)
@@ -74,6 +75,7 @@ namespace refactor::hardware {
 
     void OffsetCalculator::free(size_t offset, size_t bytes) {
         auto size = alignBytes(bytes, _alignment);
+        if (size == 0) return;
         _used -= size;
         auto next = _freeByOffset.lower_bound(offset);
         if (next != _freeByOffset.begin()) {

@@ -15,6 +15,9 @@
 #include "kernel/collectors/rms_normalization.h"
 #include "kernel/collectors/rotary_embedding.h"
 #include "kernel/collectors/softmax.h"
+#include "computation/graph.h"
+#include "computation/operators/attention.h"
+#include "computation/operators/reshape.h"
 #include "graph_topo.h"
 #include "hardware/device_manager.h"
 #include "hardware/mem_offset_calculator.h"
@@ -479,6 +482,57 @@ static void allocatorsAndStreamOnCpu() {
     EXPECT(s3.getData(1) && s3.getData(1)->size() == 4);
 }
 
+static void computationGraphLowers() {
+    using namespace computation;
+    // x -> Identity -> Reshape -> RmsNormalization -> y, y also renamed to the second global output
+    constexpr dim_t R = 4, C = 64;
+    auto x = Tensor::share(DataType::F32, Shape{R, C});
+    auto w = Tensor::share(DataType::F32, Shape{C});
+    graph_topo::GraphTopo topo(2, 2);
+    topo.pushNode({0}, 0, 1);      // 2 = identity(x)
+    topo.pushNode({2}, 0, 1);      // 3 = reshape(2)
+    topo.pushNode({3, 1}, 0, 1);   // 4 = rms(3, w)
+    topo.pushNode({4}, 0, 1);      // 5 = identity(4)
+    topo.setGlobalOutput(0, 4);
+    topo.setGlobalOutput(1, 5);
+    auto nodes = [] {
+        std::vector<computation::Node> n;
+        n.push_back({std::make_unique<Identity>(), "id0"});
+        n.push_back({std::make_unique<Reshape>(), "reshape"});
+        n.push_back({std::make_unique<RmsNormalization>(1e-5f), "norm"});
+        n.push_back({std::make_unique<Identity>(), "id1"});
+        return n;
+    };
+    std::vector<computation::Edge> edges{{x, "x"}, {w, "w"}, {x, "x1"}, {x, "x2"}, {x, "y"}, {x, "y1"}};
+    computation::Graph g(topo, nodes(), edges);
+    EXPECT(g.internal().nodes[2].op->is<RmsNormalization>() && !g.internal().nodes[2].op->is<Softmax>());
+    EXPECT(g.internal().nodes[2].op->serialize() == "RmsNormalization(1e-05)");
+    EXPECT(MatMul(1, 0, false, true).serialize() == "MatMul(1, 0, N, T)" && Attention(64).serialize() == "Attention(64)");
+    auto k = g.lower(Target::Amd);
+    auto const &kt = k._internal.topology;
+    // the norm reads x itself, both global outputs are the norm's output; renamed edges have no size
+    EXPECT(kt.node(2).inputs[0] == 0 && kt.node(2).inputs[1] == 1);
+    EXPECT(kt.globalOutputs()[0] == 4 && kt.globalOutputs()[1] == 4);
+    EXPECT(k._internal.edges[2].size == 0 && k._internal.edges[3].size == 0 && k._internal.edges[5].size == 0);
+    EXPECT(k._internal.edges[4].size == R * C * 4 && k._internal.edges[4].name == "y");
+    EXPECT(!k._internal.nodes[0].kernel && !k._internal.nodes[1].kernel && k._internal.nodes[2].kernel && !k._internal.nodes[3].kernel);
+    EXPECT(k._internal.nodes[2].name == "norm");
+    // planning the stack works with the renamed (empty) edges in place
+    runtime::Resources res;
+    std::vector<runtime::Node> lowered;
+    for (auto const &n : k._internal.nodes) lowered.emplace_back(n.kernel ? n.kernel->lower(res) : runtime::Node(runtime::emptyRoutine));
+    auto plan = reusableAllocate(kt, std::move(lowered), k._internal.edges, 256);
+    EXPECT(plan.stack == 0 && plan.edges[4].stackOffset == SIZE_MAX - 1);
+    // an operator whose collector finds nothing is reported by node name; the base class has no collector
+    auto xi = Tensor::share(DataType::I64, Shape{R, C});
+    std::vector<computation::Edge> bad{{xi, "x"}, {w, "w"}, {xi, "x1"}, {xi, "x2"}, {xi, "y"}, {xi, "y1"}};
+    computation::Graph gBad(topo, nodes(), bad);
+    bool named = false;
+    try { gBad.lower(Target::Amd); } catch (std::runtime_error const &e) { named = std::string(e.what()).find("No kernel selected for \"norm\"") != std::string::npos; }
+    EXPECT(named);
+    EXPECT(throws<UnimplementError>([] { Identity().candidateKernels(Target::Amd); }));
+}
+
 static Device &amd() { return *device::init(Device::Type::Amd, 0, "pool=4294967296"); }
 
 static void rmsNormalizationHip() {
@@ -935,24 +989,20 @@ static void quantisedLinearStream() {
     std::normal_distribution<float> g(0.3f, 2.f);
     for (auto &v : x_) v = g(rng);
 
-    auto first = [](std::vector<KernelBox> v) {
-        EXPECT(!v.empty());
-        return std::move(v.at(0));
-    };
     // edges: 0 x | 1 xq 2 scale 3 zp | 4 W (local) 5 acc | 6 y
     graph_topo::GraphTopo topo(1, 1);
     topo.pushNode({0}, 0, 3);
     topo.pushNode({1, 4, 3}, 1, 1);
     topo.pushNode({5, 2}, 0, 1);
     topo.setGlobalOutput(0, 6);
-    std::vector<kernel::Node> nodes;
-    nodes.push_back({first(DynamicQuantizeLinearCollector(Device::Type::Amd).filter({*x}, {*xq, *scale, *zp})), "quantise"});
-    nodes.push_back({first(MatMulIntegerCollector(Device::Type::Amd).filter({*xq, *w, *zp}, {*acc})), "matmul"});
-    nodes.push_back({first(DequantizeLinearCollector(Device::Type::Amd).filter({*acc, *scale}, {*y})), "dequantise"});
-    std::vector<kernel::Edge> edges{{nullptr, x->bytesSize(), "x"}, {nullptr, xq->bytesSize(), "xq"},
-                                    {nullptr, 4, "scale"}, {nullptr, 1, "zp"}, {wBlob, w->bytesSize(), "W"},
-                                    {nullptr, acc->bytesSize(), "acc"}, {nullptr, y->bytesSize(), "y"}};
-    kernel::Graph graph(std::move(topo), std::move(nodes), std::move(edges));
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
+    ops.push_back({std::make_unique<computation::MatMulInteger>(), "matmul"});
+    ops.push_back({std::make_unique<computation::DequantizeLinear>(), "dequantise"});
+    auto graph = computation::Graph(std::move(topo), std::move(ops),
+                                    {{x, "x"}, {xq, "xq"}, {scale, "scale"}, {zp, "zp"}, {w, "W"}, {acc, "acc"}, {y, "y"}})
+                     .lower(computation::Target::Amd);
+    EXPECT(graph._internal.edges[4].data == wBlob && graph._internal.edges[5].size == acc->bytesSize());
 
     // oracle chain
     std::vector<uint8_t> q(M * K);
@@ -993,6 +1043,96 @@ static void quantisedLinearStream() {
     }
 }
 
+// One decode step of an attention block as a graph: RotaryEmbedding on q and k ([N, 1, heads, D]),
+// Reshape to the attention layout ([N, heads, 1, D]: the same bytes, no kernel), Attention with the
+// caches as persistent global outputs.  Two steps through the same stream.
+static void decodeAttentionStream() {
+    using namespace computation;
+    constexpr dim_t N = 3, H = 8, Hkv = 2, D = 128, S = 64;
+    constexpr float theta = 10000.f;
+    auto q = Tensor::share(DataType::FP16, Shape{N, 1, H, D}), qa = Tensor::share(DataType::FP16, Shape{N, H, 1, D});
+    auto k = Tensor::share(DataType::FP16, Shape{N, 1, Hkv, D}), ka = Tensor::share(DataType::FP16, Shape{N, Hkv, 1, D});
+    auto pos = Tensor::share(DataType::I64, Shape{N, 1}), past = Tensor::share(DataType::I64, Shape{N});
+    auto cache = Tensor::share(DataType::FP16, Shape{N, Hkv, S, D});
+    // edges: 0 q 1 k 2 v 3 pos 4 past | 5 qr | 6 kr | 7 q' | 8 k' | 9 o 10 kcache 11 vcache
+    graph_topo::GraphTopo topo(5, 3);
+    topo.pushNode({0, 3}, 0, 1);
+    topo.pushNode({1, 3}, 0, 1);
+    topo.pushNode({5}, 0, 1);
+    topo.pushNode({6}, 0, 1);
+    topo.pushNode({7, 8, 2, 4}, 0, 3);
+    for (count_t i = 0; i < 3; ++i) topo.setGlobalOutput(i, 9 + i);
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_q"});
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_k"});
+    ops.push_back({std::make_unique<Reshape>(), "q_heads_first"});
+    ops.push_back({std::make_unique<Reshape>(), "k_heads_first"});
+    ops.push_back({std::make_unique<Attention>(S), "attention"});
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    auto stream = computation::Graph(std::move(topo), std::move(ops),
+                                     {{q, "q"}, {k, "k"}, {ka, "v"}, {pos, "pos"}, {past, "past"}, {q, "qr"}, {k, "kr"},
+                                      {qa, "q'"}, {ka, "k'"}, {qa, "o"}, {cache, "k_cache"}, {cache, "v_cache"}})
+                      .lower(Target::Amd)
+                      .lower(dev, reusableAllocate);
+
+    std::mt19937 rng(33);
+    std::normal_distribution<float> n01;
+    auto randomHalf = [&](size_t n) { std::vector<uint16_t> v(n); for (auto &e : v) e = f2h(n01(rng)); return v; };
+    auto kc = randomHalf(cache->elementsSize()), vc = randomHalf(cache->elementsSize());
+    stream.getData(10)->copyFromHost(kc.data());
+    stream.getData(11)->copyFromHost(vc.data());
+    int64_t pastLen[N] = {17, 0, 40};
+    float const scale = 1.0f / std::sqrt(static_cast<float>(D));
+    auto rope = [&](std::vector<uint16_t> const &x, dim_t heads) {// oracle on up-cast values, one rounding back
+        std::vector<float> xf(x.size()), yf(x.size());
+        for (size_t i = 0; i < x.size(); ++i) xf[i] = h2f(x[i]);
+        oracle_rope_f32(yf.data(), xf.data(), pastLen, 1, N, 1, heads, D, theta, 1);
+        std::vector<uint16_t> y(x.size());
+        for (size_t i = 0; i < x.size(); ++i) y[i] = f2h(yf[i]);
+        return y;
+    };
+    for (int step = 0; step < 2; ++step) {
+        auto q_ = randomHalf(q->elementsSize()), k_ = randomHalf(k->elementsSize()), v_ = randomHalf(k->elementsSize());
+        stream.setData(0, q_.data(), q_.size() * 2);
+        stream.setData(1, k_.data(), k_.size() * 2);
+        stream.setData(2, v_.data(), v_.size() * 2);
+        stream.setData(3, pastLen, sizeof pastLen);
+        stream.setData(4, pastLen, sizeof pastLen);
+        stream.run();
+        device::sync(Device::Type::Amd);
+        std::vector<uint16_t> o(q_.size()), kcOut(kc.size()), vcOut(vc.size());
+        EXPECT(stream.copyData(9, o.data(), o.size() * 2) && stream.copyData(10, kcOut.data(), kc.size() * 2) &&
+               stream.copyData(11, vcOut.data(), vc.size() * 2));
+        auto qr = rope(q_, H), kr = rope(k_, Hkv);
+        // caches: V rows appended bit for bit, K rows within the rotary embedding's tolerance, the rest untouched
+        bool rowsOk = true;
+        for (dim_t b = 0; b < N; ++b)
+            for (dim_t h = 0; h < Hkv; ++h) {
+                auto const at = ((b * Hkv + h) * S + pastLen[b]) * D;
+                for (dim_t i = 0; i < D; ++i) rowsOk &= std::fabs(h2f(kcOut[at + i]) - h2f(kr[(b * Hkv + h) * D + i])) <= 2e-3f;
+                std::memcpy(&kc[at], &kcOut[at], D * 2);// continue from what the device wrote
+                std::memcpy(&vc[at], &v_[(b * Hkv + h) * D], D * 2);
+            }
+        EXPECT(rowsOk && kcOut == kc && vcOut == vc);
+        bool ok = true;
+        std::vector<float> scratch(2 * S), ref(D), qf(D);
+        for (dim_t b = 0; b < N; ++b)
+            for (dim_t h = 0; h < H; ++h) {
+                dim_t const len = pastLen[b] + 1, kh = h / (H / Hkv);
+                std::vector<float> kf(len * D), vf(len * D);
+                for (size_t i = 0; i < len * D; ++i) {
+                    kf[i] = h2f(kc[(b * Hkv + kh) * S * D + i]);
+                    vf[i] = h2f(vc[(b * Hkv + kh) * S * D + i]);
+                }
+                for (dim_t i = 0; i < D; ++i) qf[i] = h2f(qr[(b * H + h) * D + i]);
+                oracle_attention_head_f32(ref.data(), qf.data(), kf.data(), vf.data(), 1, pastLen[b], D, scale, 1, scratch.data());
+                for (dim_t i = 0; i < D; ++i) ok &= std::fabs(h2f(o[(b * H + h) * D + i]) - ref[i]) <= 4e-3f;
+            }
+        EXPECT(ok);// 2e-3 of the attention on top of q rotated within 2e-3
+        for (auto &p : pastLen) ++p;
+    }
+}
+
 static void amdDeviceAndPool() {
     auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
     EXPECT(dev && dev->type() == Device::Type::Amd && device::fetch(Device::Type::Amd) == dev);
@@ -1021,6 +1161,7 @@ int main(int argc, char **argv) {
     RUN(graphTopoAndBuilder);
     RUN(offsetCalculatorPlan);
     RUN(allocatorsAndStreamOnCpu);
+    RUN(computationGraphLowers);
     if (mode == "gpu") {
         RUN(amdDeviceAndPool);
         RUN(rmsNormalizationHip);
@@ -1033,6 +1174,7 @@ int main(int argc, char **argv) {
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
         RUN(quantisedLinearStream);
+        RUN(decodeAttentionStream);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;
