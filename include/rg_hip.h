@@ -58,6 +58,21 @@ int rg_hip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stre
 int rg_hip_sync(void);
 const char *rg_hip_error_string(int status);
 
+/* ---- streams and captured graphs ---------------------------------------------------------
+ * No counterpart in the reference, whose routines all use the default stream and are enqueued one
+ * by one on every run (src/03runtime/src/stream.cc:60-69).  A stream created here (default flags
+ * and priority: it stays ordered with the default stream's blocking copies) can be handed to every
+ * launcher above; between rg_hip_graph_begin and rg_hip_graph_end the launches on it are recorded
+ * instead of run, and the executable graph that rg_hip_graph_end returns replays them with one
+ * call.  A replay uses the addresses and scalar arguments of the recording. */
+int rg_hip_stream_create(void **stream);
+int rg_hip_stream_destroy(void *stream);
+int rg_hip_stream_sync(void *stream);
+int rg_hip_graph_begin(void *stream);
+int rg_hip_graph_end(void *stream, void **graph_exec);
+int rg_hip_graph_launch(void *graph_exec, void *stream);
+int rg_hip_graph_destroy(void *graph_exec);
+
 /* ---- RmsNormalization --------------------------------------------------------------------
  * replaces the NVRTC kernel + launch of
  * src/04kernel/src/kernels/rms_normalization/cuda_kernel.cc:53-88,128-130;

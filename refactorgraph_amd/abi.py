@@ -30,6 +30,13 @@ SIGNATURES = {
     "rg_hip_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "rg_hip_memcpy_d2d_async": (_i, [_vp, _vp, _sz, _vp]),
     "rg_hip_sync": (_i, []),
+    "rg_hip_stream_create": (_i, [C.POINTER(_vp)]),
+    "rg_hip_stream_destroy": (_i, [_vp]),
+    "rg_hip_stream_sync": (_i, [_vp]),
+    "rg_hip_graph_begin": (_i, [_vp]),
+    "rg_hip_graph_end": (_i, [_vp, C.POINTER(_vp)]),
+    "rg_hip_graph_launch": (_i, [_vp, _vp]),
+    "rg_hip_graph_destroy": (_i, [_vp]),
     "rg_hip_error_string": (C.c_char_p, [_i]),
     "rg_hip_rms_norm": (_i, [_vp, _vp, _vp, _sz, _sz, _f, _i, _vp]),
     "rg_hip_softmax": (_i, [_vp, _vp, _sz, _sz, _sz, _i, _sz, _vp]),

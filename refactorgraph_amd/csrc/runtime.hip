@@ -57,6 +57,42 @@ int rg_hip_memcpy_d2d_async(void *dst, const void *src, size_t bytes, void *stre
 
 int rg_hip_sync(void) { return static_cast<int>(hipDeviceSynchronize()); }
 
+int rg_hip_stream_create(void **stream) {
+    if (!stream) return RG_HIP_E_ARGUMENT;
+    hipStream_t s = nullptr;
+    const hipError_t rc = hipStreamCreate(&s);
+    *stream = s;
+    return static_cast<int>(rc);
+}
+int rg_hip_stream_destroy(void *stream) { return static_cast<int>(hipStreamDestroy(rg::as_stream(stream))); }
+int rg_hip_stream_sync(void *stream) { return static_cast<int>(hipStreamSynchronize(rg::as_stream(stream))); }
+
+int rg_hip_graph_begin(void *stream) {
+    if (!stream) return RG_HIP_E_ARGUMENT;  // the default stream cannot record
+    return static_cast<int>(hipStreamBeginCapture(rg::as_stream(stream), hipStreamCaptureModeRelaxed));
+}
+int rg_hip_graph_end(void *stream, void **graph_exec) {
+    if (!stream || !graph_exec) return RG_HIP_E_ARGUMENT;
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    hipError_t rc = hipStreamEndCapture(rg::as_stream(stream), &graph);
+    if (rc != hipSuccess) return static_cast<int>(rc);
+    hipGraphExec_t exec = nullptr;
+    rc = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void) hipGraphDestroy(graph);
+    if (rc != hipSuccess) return static_cast<int>(rc);
+    *graph_exec = exec;
+    return 0;
+}
+int rg_hip_graph_launch(void *graph_exec, void *stream) {
+    if (!graph_exec) return RG_HIP_E_ARGUMENT;
+    return static_cast<int>(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), rg::as_stream(stream)));
+}
+int rg_hip_graph_destroy(void *graph_exec) {
+    if (!graph_exec) return 0;
+    return static_cast<int>(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+}
+
 const char *rg_hip_error_string(int status) {
     switch (status) {
         case RG_HIP_E_UNSUPPORTED: return "rg_hip: no kernel for this dtype/shape";

@@ -1,4 +1,5 @@
 #include "rg_mirror/hip_kernels.h"
+#include "rg_mirror/stream.h"
 #include "rg_hip.h"
 #include <cmath>
 
@@ -12,6 +13,13 @@
     }
 
 namespace refactor::kernel {
+
+    // the stream the routines of this Resources enqueue on: the default stream (like the reference's
+    // routines) unless the runtime::Stream has put a HipStream there to record a graph
+    static void *streamOf(Resources &res) noexcept {
+        auto *s = res.fetch<runtime::HipStream>();
+        return s ? s->handle() : nullptr;
+    }
 
     template<class T> static size_t idOf() noexcept {
         static uint8_t ID = 1;
@@ -35,8 +43,8 @@ namespace refactor::kernel {
     std::string_view RN::description() const noexcept { return "Performing rms normalization on AMD gfx950"; }
     RoutineWorkspace RN::lower(Resources &) const {
         return [epsilon = epsilon, code = static_cast<int>(dataType.internal), rows = blockCount, cols = blockSize]//
-            (Resources &, void *, void const *const *inputs, void *const *outputs) {
-                HIP_CALL(rg_hip_rms_norm(outputs[0], inputs[0], inputs[1], rows, cols, epsilon, code, nullptr));
+            (Resources &res, void *, void const *const *inputs, void *const *outputs) {
+                HIP_CALL(rg_hip_rms_norm(outputs[0], inputs[0], inputs[1], rows, cols, epsilon, code, streamOf(res)));
             };
     }
 
@@ -53,9 +61,9 @@ namespace refactor::kernel {
     size_t SM::kernelTypeId() const noexcept { return typeId(); }
     std::string_view SM::description() const noexcept { return "Performing Softmax on AMD gfx950"; }
     RoutineWorkspace SM::lower(Resources &) const {
-        return [info = info, causalRows = causalRows](Resources &, void *, void const *const *inputs, void *const *outputs) {
+        return [info = info, causalRows = causalRows](Resources &res, void *, void const *const *inputs, void *const *outputs) {
             HIP_CALL(rg_hip_softmax(outputs[0], inputs[0], info.pre, info.mid, info.post,
-                                    static_cast<int>(info.type.internal), causalRows, nullptr));
+                                    static_cast<int>(info.type.internal), causalRows, streamOf(res)));
         };
     }
 
@@ -87,7 +95,7 @@ namespace refactor::kernel {
         // needs for adjusted copies (m*k [+ k*n] bytes per batch) is not needed here
         auto const workspace = rg_hip_matmul_integer_workspace(info.batch(), info.m, info.k, info.n, flags);
         auto routine = [info = info, flags, aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
-            (Resources &, void *workspace, void const *const *inputs, void *const *outputs) {
+            (Resources &res, void *workspace, void const *const *inputs, void *const *outputs) {
                 // inputs: A, B [, a_zero_point [, b_zero_point]]; an elided (constant zero) or absent
                 // zero point is passed as null
                 void const *aZp = info.a.withZeroPoint ? inputs[2] : nullptr;
@@ -96,7 +104,7 @@ namespace refactor::kernel {
                     static_cast<int32_t *>(outputs[0]), inputs[0], inputs[1], aZp, bZp, flags,
                     info.batch(), info.m, info.k, info.n,
                     aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
-                    workspace, nullptr));
+                    workspace, streamOf(res)));
             };
         return {std::move(routine), workspace};
     }
@@ -136,11 +144,11 @@ namespace refactor::kernel {
     size_t DQ::kernelTypeId() const noexcept { return typeId(); }
     std::string_view DQ::description() const noexcept { return "Performing dequantize linear on AMD gfx950"; }
     RoutineWorkspace DQ::lower(Resources &) const {
-        return [*this](Resources &, void *, void const *const *inputs, void *const *outputs) {
+        return [*this](Resources &res, void *, void const *const *inputs, void *const *outputs) {
             HIP_CALL(rg_hip_dequantize_linear(static_cast<float *>(outputs[0]), inputs[0],
                                               static_cast<float const *>(inputs[1]),
                                               withZeroPoint ? inputs[2] : nullptr, outer, axisLen, inner,
-                                              static_cast<int>(from.internal), perAxis ? 1 : 0, nullptr));
+                                              static_cast<int>(from.internal), perAxis ? 1 : 0, streamOf(res)));
         };
     }
 
@@ -156,13 +164,13 @@ namespace refactor::kernel {
     std::string_view DQL::description() const noexcept { return "Performing dynamic quantize linear on AMD gfx950"; }
     RoutineWorkspace DQL::lower(Resources &) const {
         auto const workspace = rg_hip_dynamic_quantize_linear_workspace(size);
-        auto routine = [size = size, workspace](Resources &, void *workspacePtr, void const *const *inputs,
+        auto routine = [size = size, workspace](Resources &res, void *workspacePtr, void const *const *inputs,
                                                 void *const *outputs) {
             HIP_CALL(rg_hip_dynamic_quantize_linear(static_cast<uint8_t *>(outputs[0]),
                                                     static_cast<float *>(outputs[1]),
                                                     static_cast<uint8_t *>(outputs[2]),
                                                     static_cast<float const *>(inputs[0]), size, workspacePtr,
-                                                    workspace, nullptr));
+                                                    workspace, streamOf(res)));
         };
         return {std::move(routine), workspace};
     }
@@ -193,12 +201,12 @@ namespace refactor::kernel {
             }
         }
         return [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
-            (Resources &, void *, void const *const *inputs, void *const *outputs) {
+            (Resources &res, void *, void const *const *inputs, void *const *outputs) {
                 HIP_CALL(rg_hip_matmul(outputs[0], inputs[0], inputs[1], info.hasBias ? inputs[2] : nullptr,
                                        static_cast<int>(info.dataType.internal), info.transA, info.transB, info.alpha,
                                        info.beta, info.batch(), info.m, info.k, info.n,
                                        aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
-                                       info.biasStrideBatch, info.biasStrideM, info.biasStrideN, nullptr));
+                                       info.biasStrideBatch, info.biasStrideM, info.biasStrideN, streamOf(res)));
             };
     }
 
@@ -218,9 +226,9 @@ namespace refactor::kernel {
     size_t CastHip::kernelTypeId() const noexcept { return typeId(); }
     std::string_view CastHip::description() const noexcept { return "Performing cast operation on AMD gfx950"; }
     RoutineWorkspace CastHip::lower(Resources &) const {
-        return [from = from, to = to, size = size](Resources &, void *, void const *const *inputs, void *const *outputs) {
+        return [from = from, to = to, size = size](Resources &res, void *, void const *const *inputs, void *const *outputs) {
             HIP_CALL(rg_hip_cast(outputs[0], inputs[0], size, static_cast<int>(from.internal),
-                                 static_cast<int>(to.internal), nullptr));
+                                 static_cast<int>(to.internal), streamOf(res)));
         };
     }
 
@@ -268,15 +276,15 @@ namespace refactor::kernel {
                 if (info.resetCache && kCache) {
                     auto const bytes = static_cast<size_t>(info.batch) * info.nKVHead * info.cacheLen * info.headDim *
                                        info.dataType.size();
-                    if (inputs[4] != kCache) { HIP_CALL(rg_hip_memcpy_d2d_async(kCache, inputs[4], bytes, nullptr)); }
-                    if (inputs[5] != vCache) { HIP_CALL(rg_hip_memcpy_d2d_async(vCache, inputs[5], bytes, nullptr)); }
+                    if (inputs[4] != kCache) { HIP_CALL(rg_hip_memcpy_d2d_async(kCache, inputs[4], bytes, streamOf(res))); }
+                    if (inputs[5] != vCache) { HIP_CALL(rg_hip_memcpy_d2d_async(vCache, inputs[5], bytes, streamOf(res))); }
                 }
                 auto const *past = info.pastFromInput ? static_cast<int64_t const *>(inputs[3]) : nullptr;
                 HIP_CALL(rg_hip_attention_kvcache(
                     outputs[0], inputs[0], inputs[1], inputs[2], kCache, vCache, past,
                     info.pastCount == info.batch && info.batch > 1 ? 1 : 0,
                     info.batch, info.nHead, info.nKVHead, info.seqLen, info.cacheLen, info.headDim, scale,
-                    static_cast<int>(info.dataType.internal), ws, workspace, state->counters(), nullptr));
+                    static_cast<int>(info.dataType.internal), ws, workspace, state->counters(), streamOf(res)));
             };
         return {std::move(routine), workspace};
     }
@@ -302,9 +310,9 @@ namespace refactor::kernel {
     size_t RE::kernelTypeId() const noexcept { return typeId(); }
     std::string_view RE::description() const noexcept { return "Performing rotary embedding on AMD gfx950"; }
     RoutineWorkspace RE::lower(Resources &) const {
-        return [*this](Resources &, void *, void const *const *inputs, void *const *outputs) {
+        return [*this](Resources &res, void *, void const *const *inputs, void *const *outputs) {
             HIP_CALL(rg_hip_rope(outputs[0], inputs[0], static_cast<int64_t const *>(inputs[1]), posPerBatch ? 1 : 0,
-                                 batch, seq, heads, dim, theta, static_cast<int>(dataType.internal), nullptr));
+                                 batch, seq, heads, dim, theta, static_cast<int>(dataType.internal), streamOf(res)));
         };
     }
 

@@ -1045,7 +1045,9 @@ static void quantisedLinearStream() {
 
 // One decode step of an attention block as a graph: RotaryEmbedding on q and k ([N, 1, heads, D]),
 // Reshape to the attention layout ([N, heads, 1, D]: the same bytes, no kernel), Attention with the
-// caches as persistent global outputs.  Two steps through the same stream.
+// caches as persistent global outputs.  Two steps enqueued routine by routine, then the graph is
+// recorded as one HIP graph and three more steps are replays of it with new contents in the same
+// blobs; every step is checked against the oracle in the same way.
 static void decodeAttentionStream() {
     using namespace computation;
     constexpr dim_t N = 3, H = 8, Hkv = 2, D = 128, S = 64;
@@ -1091,14 +1093,28 @@ static void decodeAttentionStream() {
         for (size_t i = 0; i < x.size(); ++i) y[i] = f2h(yf[i]);
         return y;
     };
-    for (int step = 0; step < 2; ++step) {
+    EXPECT(throws<std::runtime_error>([&] { stream.replay(); }));// nothing recorded yet
+    for (int step = 0; step < 5; ++step) {
         auto q_ = randomHalf(q->elementsSize()), k_ = randomHalf(k->elementsSize()), v_ = randomHalf(k->elementsSize());
-        stream.setData(0, q_.data(), q_.size() * 2);
-        stream.setData(1, k_.data(), k_.size() * 2);
-        stream.setData(2, v_.data(), v_.size() * 2);
-        stream.setData(3, pastLen, sizeof pastLen);
-        stream.setData(4, pastLen, sizeof pastLen);
-        stream.run();
+        if (step < 2) {
+            stream.setData(0, q_.data(), q_.size() * 2);
+            stream.setData(1, k_.data(), k_.size() * 2);
+            stream.setData(2, v_.data(), v_.size() * 2);
+            stream.setData(3, pastLen, sizeof pastLen);
+            stream.setData(4, pastLen, sizeof pastLen);
+            stream.run();
+        } else {
+            if (step == 2) {
+                stream.record();// runs the previous step once more (same rows, same values) and records
+                EXPECT(stream.recorded());
+            }
+            stream.getData(0)->copyFromHost(q_.data(), q_.size() * 2);
+            stream.getData(1)->copyFromHost(k_.data(), k_.size() * 2);
+            stream.getData(2)->copyFromHost(v_.data(), v_.size() * 2);
+            stream.getData(3)->copyFromHost(pastLen, sizeof pastLen);
+            stream.getData(4)->copyFromHost(pastLen, sizeof pastLen);
+            stream.replay();
+        }
         device::sync(Device::Type::Amd);
         std::vector<uint16_t> o(q_.size()), kcOut(kc.size()), vcOut(vc.size());
         EXPECT(stream.copyData(9, o.data(), o.size() * 2) && stream.copyData(10, kcOut.data(), kc.size() * 2) &&
@@ -1131,6 +1147,18 @@ static void decodeAttentionStream() {
         EXPECT(ok);// 2e-3 of the attention on top of q rotated within 2e-3
         for (auto &p : pastLen) ++p;
     }
+    // another blob on an edge discards the recording
+    stream.setData(0, q->bytesSize());
+    EXPECT(!stream.recorded() && throws<std::runtime_error>([&] { stream.replay(); }));
+    // a stream on the CPU device has nothing to record
+    graph_topo::GraphTopo topo1(1, 1);
+    topo1.pushNode({0}, 0, 1);
+    topo1.setGlobalOutput(0, 1);
+    std::vector<kernel::Node> nodes1;
+    nodes1.push_back({nullptr, "nothing"});
+    auto onCpu = kernel::Graph(std::move(topo1), std::move(nodes1), {{nullptr, 4, "in"}, {nullptr, 4, "out"}})
+                     .lower(device::fetch(Device::Type::Cpu), flatAllocate);
+    EXPECT(throws<std::runtime_error>([&] { onCpu.record(); }));
 }
 
 static void amdDeviceAndPool() {
