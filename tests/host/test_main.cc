@@ -28,6 +28,7 @@
 #include "rg_mirror/hip_kernels.h"
 #include "oracle.h"
 
+#include <chrono>
 #include <cmath>
 #include <immintrin.h>
 #include <cstdio>
@@ -1147,6 +1148,20 @@ static void decodeAttentionStream() {
         EXPECT(ok);// 2e-3 of the attention on top of q rotated within 2e-3
         for (auto &p : pastLen) ++p;
     }
+    {// what the recording saves per step (printed, not asserted): same work enqueued 200 times each way
+        auto clock = [] { return std::chrono::steady_clock::now(); };
+        device::sync(Device::Type::Amd);
+        auto t0 = clock();
+        for (int i = 0; i < 200; ++i) stream.run();
+        device::sync(Device::Type::Amd);
+        auto t1 = clock();
+        for (int i = 0; i < 200; ++i) stream.replay();
+        device::sync(Device::Type::Amd);
+        auto t2 = clock();
+        std::printf("  decode block (2 x RotaryEmbedding + Attention): %.1f us per step enqueued routine by routine, %.1f us replayed\n",
+                    std::chrono::duration<double, std::micro>(t1 - t0).count() / 200,
+                    std::chrono::duration<double, std::micro>(t2 - t1).count() / 200);
+    }
     // another blob on an edge discards the recording
     stream.setData(0, q->bytesSize());
     EXPECT(!stream.recorded() && throws<std::runtime_error>([&] { stream.replay(); }));
@@ -1159,6 +1174,62 @@ static void decodeAttentionStream() {
     auto onCpu = kernel::Graph(std::move(topo1), std::move(nodes1), {{nullptr, 4, "in"}, {nullptr, 4, "out"}})
                      .lower(device::fetch(Device::Type::Cpu), flatAllocate);
     EXPECT(throws<std::runtime_error>([&] { onCpu.record(); }));
+}
+
+// A chain of 64 small kernels: what a recording is for.  The replayed result must equal the result
+// of the routines enqueued one by one, on every replay, with other work in between.
+static void longChainRecorded() {
+    using namespace computation;
+    constexpr dim_t R = 8, C = 1024, L = 64;
+    auto x = Tensor::share(DataType::F32, Shape{R, C});
+    auto w = Tensor::share(DataType::F32, Shape{C});
+    graph_topo::GraphTopo topo(2, 1);
+    std::vector<computation::Node> ops;
+    std::vector<computation::Edge> edges{{x, "x"}, {w, "w"}};
+    count_t last = 0;
+    for (dim_t i = 0; i < L; ++i) {
+        last = topo.pushNode({last, 1}, 0, 1).begin_;
+        ops.push_back({std::make_unique<RmsNormalization>(1e-5f), "norm" + std::to_string(i)});
+        edges.push_back({x, "t" + std::to_string(i)});
+    }
+    topo.setGlobalOutput(0, last);
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    auto stream = computation::Graph(std::move(topo), std::move(ops), std::move(edges)).lower(Target::Amd).lower(dev, reusableAllocate);
+    // two ranges of the stack are enough for the whole chain
+    EXPECT(stream.graph().edges[2].stackOffset == 0 && stream.graph().edges[3].stackOffset == R * C * 4 && stream.graph().edges[4].stackOffset == 0);
+    std::mt19937 rng(3);
+    std::normal_distribution<float> n01;
+    std::vector<float> x_(R * C), w_(C), eager(R * C), replayed(R * C);
+    for (auto &v : w_) v = 1.f + 0.1f * n01(rng);
+    stream.setData(1, w_.data(), C * 4);
+    stream.setData(0, size_t(R * C * 4));
+    stream.record();
+    bool same = true;
+    for (int round = 0; round < 4; ++round) {
+        for (auto &v : x_) v = n01(rng);
+        stream.getData(0)->copyFromHost(x_.data(), R * C * 4);
+        stream.run();
+        device::sync(Device::Type::Amd);
+        stream.copyData(last, eager.data(), R * C * 4);
+        std::vector<float> zeros(R * C, 0.f);
+        stream.getData(last)->copyFromHost(zeros.data(), R * C * 4);// eager work between the replays
+        stream.replay();
+        device::sync(Device::Type::Amd);
+        stream.copyData(last, replayed.data(), R * C * 4);
+        same &= std::memcmp(eager.data(), replayed.data(), R * C * 4) == 0 && eager[0] != 0.f;
+    }
+    EXPECT(same);
+    auto clock = [] { return std::chrono::steady_clock::now(); };
+    auto t0 = clock();
+    for (int i = 0; i < 50; ++i) stream.run();
+    device::sync(Device::Type::Amd);
+    auto t1 = clock();
+    for (int i = 0; i < 50; ++i) stream.replay();
+    device::sync(Device::Type::Amd);
+    auto t2 = clock();
+    std::printf("  chain of 64 RmsNormalization [8, 1024]: %.1f us per run enqueued routine by routine, %.1f us replayed\n",
+                std::chrono::duration<double, std::micro>(t1 - t0).count() / 50,
+                std::chrono::duration<double, std::micro>(t2 - t1).count() / 50);
 }
 
 static void amdDeviceAndPool() {
@@ -1203,6 +1274,7 @@ int main(int argc, char **argv) {
         RUN(rotaryEmbeddingHip);
         RUN(quantisedLinearStream);
         RUN(decodeAttentionStream);
+        RUN(longChainRecorded);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);
     return g_failed ? 1 : 0;
