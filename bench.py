@@ -379,7 +379,7 @@ def main():
         ops_out["cast"] = e
         del xs, ys
 
-    if want("matmul_integer"):
+    if want("matmul_integer") or want("matmul_integer_dequantize"):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
         az = torch.tensor([128], device=dev, dtype=torch.uint8)
@@ -407,6 +407,23 @@ def main():
             ops_out["matmul_integer"]["cpu_baseline"] = {
                 "value": round(2 * m * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
                 "sample": f"first {m} rows of A against all of B ({dt:.1f} s)"}
+        if want("matmul_integer_dequantize"):
+            # the same product with DequantizeLinear (per-column scale) folded into the epilogue, against
+            # the two operators one after the other
+            sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
+            yf = torch.empty((4096, 4096), device=dev, dtype=torch.float32)
+            wall, dms_f, mode = time_steps(torch, lambda i: ops.matmul_integer(a, b, az, bz, out=yf, dequant_scale=sc),
+                                           steps, warmup, 1)
+            wall, dms_2, mode = time_steps(
+                torch, lambda i: ops.dequantize_linear(ops.matmul_integer(a, b, az, bz, out=y), sc, None, axis=1, out=yf),
+                steps, warmup, 1)
+            tops = 2 * 4096 ** 3 / (dms_f * 1e-3) / 1e12
+            ops_out["matmul_integer_dequantize"] = {
+                "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
+                "workload": "MatMulInteger 4096^3 with DequantizeLinear (scale per column) in its epilogue -> f32",
+                "device_ms_per_launch": round(dms_f, 5), "timing": mode,
+                "two_operators_device_ms": round(dms_2, 5)}
         del a, b, y
 
     if want("matmul"):

@@ -178,6 +178,17 @@ int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b,
                           size_t batch, size_t m, size_t k, size_t n,
                           const uint32_t *a_index, const uint32_t *b_index,
                           void *workspace, void *stream);
+/* MatMulInteger with DequantizeLinear folded into its epilogue: y[b,i,j] = float(sum) * scale[j or 0],
+ * i.e. the result of rg_hip_matmul_integer followed by the reference's DequantizeLinear without zero
+ * point (src/04kernel/src/kernels/dequantize_linear/cpu_kernel.cc:17-28: one int -> float
+ * conversion, one multiplication) on the last axis, bit for bit, without the int32 tensor ever
+ * reaching memory.  No counterpart in the reference, which runs the two operators one after the
+ * other.  scale: device pointer to one float, or to n floats when scale_per_column != 0. */
+int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, const void *a_zp,
+                                     const void *b_zp, unsigned flags, size_t batch, size_t m,
+                                     size_t k, size_t n, const uint32_t *a_index,
+                                     const uint32_t *b_index, const float *scale, int scale_per_column,
+                                     void *workspace, void *stream);
 
 /* ---- Attention with KV cache ---------------------------------------------------------------
  * the reference declares this kernel but never defines it

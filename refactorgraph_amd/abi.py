@@ -48,6 +48,8 @@ SIGNATURES = {
     "rg_hip_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul_integer_workspace": (_sz, [_sz, _sz, _sz, _sz, _u]),
     "rg_hip_matmul_integer": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "rg_hip_matmul_integer_dequantize": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _i,
+                                              _vp, _vp]),
     "rg_hip_attention_kvcache_workspace": (_sz, [_sz, _sz, _sz, _sz, _sz, _sz]),
     "rg_hip_attention_kvcache_state_bytes": (_sz, []),
     "rg_hip_attention_kvcache": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _sz,

@@ -39,13 +39,27 @@ __device__ __forceinline__ uint32_t sub_bytes(uint32_t x, uint32_t z) {
 
 __device__ __forceinline__ uint32_t splat(uint32_t byte) { return byte * 0x01010101u; }
 
+// Optional epilogue: the int32 sum leaves as float(sum) * scale (DequantizeLinear without zero point,
+// src/04kernel/src/kernels/dequantize_linear/cpu_kernel.cc:17-28: one conversion, one multiplication),
+// with one scale for the tensor or one per column of Y.
+struct Dequant {
+    const float *scale;
+    uint32_t per_column;
+};
+template <bool DEQ>
+__device__ __forceinline__ int32_t finish(int32_t sum, float scale) {
+    if constexpr (DEQ) return __builtin_bit_cast(int32_t, static_cast<float>(sum) * scale);
+    else return sum;
+}
+
 // ---------------------------------------------------------------- generic kernel
 // 16x16 outputs per workgroup, one per thread; k walked in LDS tiles of 16.
 
+template <bool DEQ>
 __global__ __launch_bounds__(256) void mmi_generic(int32_t *__restrict__ y,
                                                    const uint8_t *__restrict__ a,
                                                    const uint8_t *__restrict__ b, ZeroPoint za,
-                                                   ZeroPoint zb, uint32_t m, uint32_t k, uint32_t n,
+                                                   ZeroPoint zb, Dequant dq, uint32_t m, uint32_t k, uint32_t n,
                                                    uint32_t a_matrix0, uint32_t b_matrix0,
                                                    uint32_t y_matrix0) {
     __shared__ int8_t ta[16][17];
@@ -72,7 +86,7 @@ __global__ __launch_bounds__(256) void mmi_generic(int32_t *__restrict__ y,
         for (int q = 0; q < 16; ++q) acc += static_cast<int32_t>(ta[ty][q]) * static_cast<int32_t>(tb[q][tx]);
         __syncthreads();
     }
-    if (row < m && col < n) y[(ym * m + row) * n + col] = acc;
+    if (row < m && col < n) y[(ym * m + row) * n + col] = finish<DEQ>(acc, DEQ ? dq.scale[dq.per_column ? col : 0] : 0.f);
 }
 
 // ---------------------------------------------------------------- MFMA kernel
@@ -227,10 +241,11 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
 }
 
+template <bool DEQ>
 __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
                                                            const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb,
-                                                           uint32_t m, uint32_t k, uint32_t n, uint32_t a_matrix0,
-                                                           uint32_t b_matrix0, uint32_t y_matrix0) {
+                                                           Dequant dq, uint32_t m, uint32_t k, uint32_t n,
+                                                           uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
     __shared__ __align__(1024) uint8_t lds0[D_STAGE];
     __shared__ __align__(1024) uint8_t lds1[D_STAGE];
 
@@ -296,6 +311,12 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
 
     int32_t *Y = y + (ym * m + static_cast<uint64_t>(tile_m) * BM + wm * 128) * n +
                  static_cast<uint64_t>(tile_n) * BN + wn * 128;
+    float scale[4] = {};  // of this lane's four columns
+    if constexpr (DEQ) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            scale[j] = dq.scale[dq.per_column ? tile_n * BN + wn * 128 + j * 32 + (lane & 31) : 0];
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -304,7 +325,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
             for (int e = 0; e < 16; ++e) {
                 const uint32_t row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
                 const uint32_t col = j * 32 + (lane & 31);
-                __builtin_nontemporal_store(acc[i][j][e], Y + static_cast<uint64_t>(row) * n + col);
+                __builtin_nontemporal_store(finish<DEQ>(acc[i][j][e], scale[j]), Y + static_cast<uint64_t>(row) * n + col);
             }
 }
 
@@ -315,11 +336,12 @@ extern "C" size_t rg_hip_matmul_integer_workspace(size_t, size_t, size_t, size_t
     return 0;
 }
 
-extern "C" int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b, const void *a_zp,
-                                     const void *b_zp, unsigned flags, size_t batch, size_t m,
-                                     size_t k, size_t n, const uint32_t *a_index,
-                                     const uint32_t *b_index, void * /*workspace*/, void *stream) {
-    using namespace rg;
+namespace rg {
+namespace {
+template <bool DEQ>
+int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const void *b_zp, unsigned flags,
+               size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
+               Dequant dq, void *stream) {
     if (!y || !a || !b) return RG_HIP_E_ARGUMENT;
     if (batch == 0 || m == 0 || n == 0) return 0;
     if (m > 0x7fffffffu || n > 0x7fffffffu || k > 0x7fffffffu || batch > 0xffffffffu)
@@ -332,13 +354,13 @@ extern "C" int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b, c
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if (fast) {
             const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
-            mmi_mfma_256x256<<<grid, 256, 0, s>>>(
-                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb,
+            mmi_mfma_256x256<DEQ><<<grid, 256, 0, s>>>(
+                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
                 static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), am0, bm0, ym0);
         } else {
             const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
-            mmi_generic<<<grid, 256, 0, s>>>(
-                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb,
+            mmi_generic<DEQ><<<grid, 256, 0, s>>>(
+                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
                 static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), am0, bm0, ym0);
         }
         return launch_status();
@@ -359,4 +381,24 @@ extern "C" int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b, c
         if (rc) return rc;
     }
     return 0;
+}
+}  // namespace
+}  // namespace rg
+
+extern "C" int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b, const void *a_zp,
+                                     const void *b_zp, unsigned flags, size_t batch, size_t m,
+                                     size_t k, size_t n, const uint32_t *a_index,
+                                     const uint32_t *b_index, void * /*workspace*/, void *stream) {
+    return rg::mmi_launch<false>(y, a, b, a_zp, b_zp, flags, batch, m, k, n, a_index, b_index, rg::Dequant{nullptr, 0},
+                                 stream);
+}
+
+extern "C" int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, const void *a_zp,
+                                                const void *b_zp, unsigned flags, size_t batch, size_t m,
+                                                size_t k, size_t n, const uint32_t *a_index,
+                                                const uint32_t *b_index, const float *scale, int scale_per_column,
+                                                void * /*workspace*/, void *stream) {
+    if (!scale) return RG_HIP_E_ARGUMENT;
+    return rg::mmi_launch<true>(reinterpret_cast<int32_t *>(y), a, b, a_zp, b_zp, flags, batch, m, k, n, a_index, b_index,
+                                rg::Dequant{scale, scale_per_column ? 1u : 0u}, stream);
 }

@@ -138,7 +138,10 @@ namespace refactor::computation {
         Graph(graph_topo::GraphTopo, std::vector<Node>, std::vector<Edge>) noexcept;
 
         // First candidate of every operator's collector; operators without one are collected and
-        // reported together ("No kernel selected for ...").
+        // reported together ("No kernel selected for ...").  On the AMD target a MatMulInteger whose
+        // result is read by one DequantizeLinear only (no zero point, scale per tensor or per index of
+        // the last axis) and by nothing else becomes one MatMulIntegerDequantizeHip node: the
+        // dequantising node and the int32 edge between the two are gone from the lowered graph.
         kernel::Graph lower(Target) const;
         graph_topo::Graph<Node, Edge> const &internal() const noexcept { return _internal; }
     };

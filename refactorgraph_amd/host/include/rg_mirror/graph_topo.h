@@ -12,6 +12,7 @@
 
 #include "rg_mirror/common.h"
 #include <algorithm>
+#include <iterator>
 #include <map>
 #include <set>
 #include <unordered_map>
@@ -38,9 +39,15 @@ namespace refactor {
     template<class T = size_t> struct range_t {
         T begin_, end_;
         struct Iterator {
+            using iterator_category = std::forward_iterator_tag;
+            using value_type = T;
+            using difference_type = std::ptrdiff_t;
+            using pointer = T const *;
+            using reference = T;
             T v;
             T operator*() const noexcept { return v; }
             Iterator &operator++() noexcept { return ++v, *this; }
+            Iterator operator++(int) noexcept { return Iterator{v++}; }
             bool operator!=(Iterator const &o) const noexcept { return v != o.v; }
             bool operator==(Iterator const &o) const noexcept { return v == o.v; }
         };

@@ -44,6 +44,24 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // MatMulInteger whose result leaves as float(sum) * scale: what MatMulIntegerHip followed by a
+    // DequantizeLinearHip without zero point (scale per tensor, or per index of the last axis)
+    // computes, bit for bit, in one kernel and without the int32 tensor.  No counterpart in the
+    // reference; computation::Graph::lower puts it in place of such a pair.
+    // Inputs: A, B [, a_zero_point [, b_zero_point]], scale.  Output: float [.., m, n].
+    struct MatMulIntegerDequantizeHip final : public Kernel {
+        MatMulIntegerInfo info;
+        dim_t zeroPointInputs;// how many of the optional inputs 2, 3 the operator has
+        bool perColumn;
+
+        MatMulIntegerDequantizeHip(MatMulIntegerInfo, dim_t, bool) noexcept;
+        static KernelBox build(MatMulIntegerInfo, dim_t zeroPointInputs, bool perColumn) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct DequantizeLinearHip final : public Kernel {
         DataType from;
         size_t outer, axisLen, inner;

@@ -1,5 +1,6 @@
 // computation layer of the host mirror (see rg_mirror/computation.h).
 #include "rg_mirror/computation.h"
+#include "rg_mirror/hip_kernels.h"
 #include <unordered_map>
 
 namespace refactor::computation {
@@ -71,6 +72,60 @@ namespace refactor::computation {
     }
     std::string RotaryEmbedding::serialize() const { return detail::cat(name(), '(', theta, ')'); }
 
+    // MatMulIntegerHip -> (int32 edge read once) -> DequantizeLinearHip  ==>  MatMulIntegerDequantizeHip.
+    // The graph is rebuilt from keys (old indices) so that the edge numbering stays what GraphTopo
+    // promises whatever the position of the scale's producer.
+    static kernel::Graph fuseDequantize(graph_topo::GraphTopo topology, std::vector<kernel::Node> nodes,
+                                        std::vector<kernel::Edge> edges) {
+        using kernel::DequantizeLinearHip;
+        using kernel::MatMulIntegerHip;
+        std::vector<size_t> readers(edges.size(), 0);
+        for (auto e : topology.connections()) ++readers[e];
+        std::vector<count_t> producer(edges.size(), count_t(-1));
+        for (auto [idx, inputs, outputs] : topology)
+            for (auto e : outputs) producer[e] = idx;
+
+        std::unordered_map<count_t, count_t> fusedInto;// consumer node -> producer node
+        for (auto [idx, inputs, outputs] : topology) {
+            auto const &k = nodes[idx].kernel;
+            if (!k || !k->is<DequantizeLinearHip>() || inputs.size() != 2 || outputs.size() != 1) continue;
+            auto const &dq = static_cast<DequantizeLinearHip const &>(*k);
+            auto const x = inputs[0];
+            auto const p = producer[x];
+            if (p == count_t(-1) || readers[x] != 1 || !nodes[p].kernel || !nodes[p].kernel->is<MatMulIntegerHip>()) continue;
+            auto const &mm = static_cast<MatMulIntegerHip const &>(*nodes[p].kernel);
+            if (dq.from != DataType::I32 || dq.withZeroPoint) continue;
+            if (dq.perAxis && (dq.inner != 1 || dq.axisLen != mm.info.n)) continue;
+            auto const zeroPointInputs = static_cast<dim_t>(topology.node(p).inputs.size() - 2);
+            auto fused = kernel::MatMulIntegerDequantizeHip::build(mm.info, zeroPointInputs, dq.perAxis);
+            if (!fused) continue;
+            nodes[p].kernel = std::move(fused);
+            nodes[p].name += "+" + nodes[idx].name;
+            fusedInto.emplace(idx, p);
+        }
+        if (fusedInto.empty()) return kernel::Graph(std::move(topology), std::move(nodes), std::move(edges));
+
+        graph_topo::Builder<count_t, kernel::Node, count_t, kernel::Edge> builder;
+        std::unordered_map<count_t, count_t> consumerOf;// producer node -> consumer node
+        for (auto [c, p] : fusedInto) consumerOf.emplace(p, c);
+        for (auto [idx, inputs, outputs] : topology) {
+            if (fusedInto.count(idx)) continue;
+            graph_topo::BuilderNode<count_t> n{{inputs.begin(), inputs.end()}, {outputs.begin(), outputs.end()}};
+            if (auto it = consumerOf.find(idx); it != consumerOf.end()) {
+                auto const consumer = topology.node(it->second);
+                n.inputs.push_back(consumer.inputs[1]);// the scale
+                n.outputs.assign(consumer.outputs.begin(), consumer.outputs.end());
+            }
+            builder.topology.emplace(idx, std::move(n));
+            builder.nodes.emplace(idx, std::move(nodes[idx]));
+        }
+        for (auto e : topology.globalInputs()) builder.globalInputs.push_back(e);
+        for (auto e : topology.globalOutputs()) builder.globalOutputs.push_back(e);
+        for (count_t e = 0; e < edges.size(); ++e) builder.edges.emplace(e, std::move(edges[e]));
+        auto g = builder.build();
+        return kernel::Graph(std::move(g.topology), std::move(g.nodes), std::move(g.edges));
+    }
+
     Graph::Graph(graph_topo::Graph<Node, Edge> internal) noexcept : _internal(std::move(internal)) {}
     Graph::Graph(graph_topo::GraphTopo topology, std::vector<Node> nodes, std::vector<Edge> edges) noexcept
         : _internal{std::move(topology), std::move(nodes), std::move(edges)} {}
@@ -119,6 +174,7 @@ namespace refactor::computation {
         }
         auto topology = graph.topology;
         topology.reconnect(identities);
+        if (target == Target::Amd) return fuseDequantize(std::move(topology), std::move(nodes), std::move(edges));
         return kernel::Graph(std::move(topology), std::move(nodes), std::move(edges));
     }
 

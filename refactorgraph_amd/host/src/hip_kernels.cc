@@ -109,6 +109,49 @@ namespace refactor::kernel {
         return {std::move(routine), workspace};
     }
 
+    // ------------------------------------------------------------------ MatMulInteger + DequantizeLinear
+
+    using MMD = MatMulIntegerDequantizeHip;
+    MMD::MatMulIntegerDequantizeHip(MatMulIntegerInfo info_, dim_t zeroPointInputs_, bool perColumn_) noexcept
+        : Kernel(), info(std::move(info_)), zeroPointInputs(zeroPointInputs_), perColumn(perColumn_) {}
+    KernelBox MMD::build(MatMulIntegerInfo info, dim_t zeroPointInputs, bool perColumn) noexcept {
+        return zeroPointInputs <= 2 ? std::make_unique<MMD>(std::move(info), zeroPointInputs, perColumn) : nullptr;
+    }
+    size_t MMD::typeId() noexcept { return idOf<MMD>(); }
+    size_t MMD::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view MMD::description() const noexcept {
+        return "Performing MatMulInteger with a dequantising epilogue on AMD gfx950";
+    }
+    RoutineWorkspace MMD::lower(Resources &) const {
+        unsigned flags = 0;
+        if (info.a.scalar) { flags |= RG_MMI_A_ZP_SCALAR; }
+        if (info.b.scalar) { flags |= RG_MMI_B_ZP_SCALAR; }
+        std::vector<uint32_t> aIndex, bIndex;
+        if (info.broadcaster.needBroadcast()) {
+            aIndex.resize(info.batch());
+            bIndex.resize(info.batch());
+            for (dim_t i = 0; i < info.batch(); ++i) {
+                dim_t at[2];
+                info.broadcaster.locate(i, at);
+                aIndex[i] = at[0];
+                bIndex[i] = at[1];
+            }
+        }
+        auto const workspace = rg_hip_matmul_integer_workspace(info.batch(), info.m, info.k, info.n, flags);
+        auto routine = [info = info, flags, scaleAt = 2 + zeroPointInputs, perColumn = perColumn,
+                        aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
+            (Resources &res, void *workspacePtr, void const *const *inputs, void *const *outputs) {
+                void const *aZp = info.a.withZeroPoint ? inputs[2] : nullptr;
+                void const *bZp = info.b.withZeroPoint ? inputs[3] : nullptr;
+                HIP_CALL(rg_hip_matmul_integer_dequantize(
+                    static_cast<float *>(outputs[0]), inputs[0], inputs[1], aZp, bZp, flags,
+                    info.batch(), info.m, info.k, info.n,
+                    aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
+                    static_cast<float const *>(inputs[scaleAt]), perColumn ? 1 : 0, workspacePtr, streamOf(res)));
+            };
+        return {std::move(routine), workspace};
+    }
+
     // ------------------------------------------------------------------ DequantizeLinear
 
     using DQ = DequantizeLinearHip;

@@ -157,10 +157,11 @@ def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=
     return y
 
 
-def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):
+def matmul_integer(a, b, a_zp=None, b_zp=None, out=None, dequant_scale=None):
     """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
-    (batch, row) of the operand as the reference's CPU kernel reads them."""
-    _need_gpu(a, b, a_zp, b_zp)
+    (batch, row) of the operand as the reference's CPU kernel reads them.  dequant_scale (float32,
+    one element or n): the result leaves as float32 = float(sum) * scale instead of int32."""
+    _need_gpu(a, b, a_zp, b_zp, dequant_scale)
     m, k = a.shape[-2:]
     k2, n = b.shape[-2:]
     assert k == k2
@@ -180,6 +181,15 @@ def matmul_integer(a, b, a_zp=None, b_zp=None, out=None):
         flags |= abi.MMI_A_ZP_SCALAR
     if b_zp is not None and b_zp.numel() == 1:
         flags |= abi.MMI_B_ZP_SCALAR
+    if dequant_scale is not None:
+        assert dequant_scale.dtype == torch.float32 and dequant_scale.numel() in (1, n)
+        y = torch.empty(ob + (m, n), dtype=torch.float32, device=a.device) if out is None else out
+        check(lib().rg_hip_matmul_integer_dequantize(
+            _ptr(y), _ptr(a), _ptr(b), _ptr(a_zp), _ptr(b_zp), flags, batch, m, k, n,
+            None if a_idx is None else a_idx.ctypes.data_as(C.c_void_p),
+            None if b_idx is None else b_idx.ctypes.data_as(C.c_void_p),
+            _ptr(dequant_scale), int(dequant_scale.numel() != 1), None, _stream()), "rg_hip_matmul_integer_dequantize")
+        return y
     y = torch.empty(ob + (m, n), dtype=torch.int32, device=a.device) if out is None else out
     check(lib().rg_hip_matmul_integer(
         _ptr(y), _ptr(a), _ptr(b), _ptr(a_zp), _ptr(b_zp), flags, batch, m, k, n,

@@ -532,6 +532,30 @@ static void computationGraphLowers() {
     try { gBad.lower(Target::Amd); } catch (std::runtime_error const &e) { named = std::string(e.what()).find("No kernel selected for \"norm\"") != std::string::npos; }
     EXPECT(named);
     EXPECT(throws<UnimplementError>([] { Identity().candidateKernels(Target::Amd); }));
+
+    // MatMulInteger -> DequantizeLinear becomes one node only if the scale runs along the last axis (or is one
+    // value), there is no zero point, and nothing else reads the sums
+    auto quantised = [](int axis, dim_t scales, bool withZeroPoint) {
+        auto a = Tensor::share(DataType::U8, Shape{4, 8}), b = Tensor::share(DataType::I8, Shape{8, 4});
+        auto acc = Tensor::share(DataType::I32, Shape{4, 4}), out = Tensor::share(DataType::F32, Shape{4, 4});
+        auto sc = Tensor::share(DataType::F32, Shape{scales}), zp = Tensor::share(DataType::I32, Shape{scales});
+        graph_topo::GraphTopo t(withZeroPoint ? 4 : 3, 1);
+        auto accEdge = t.pushNode({0, 1}, 0, 1).begin_;
+        std::vector<count_t> in{accEdge, 2};
+        if (withZeroPoint) in.push_back(3);
+        auto outEdge = t.pushNode(in, 0, 1).begin_;
+        t.setGlobalOutput(0, outEdge);
+        std::vector<computation::Node> n;
+        n.push_back({std::make_unique<MatMulInteger>(), "mm"});
+        n.push_back({std::make_unique<DequantizeLinear>(axis), "dq"});
+        std::vector<computation::Edge> e{{a, "a"}, {b, "b"}, {sc, "scale"}};
+        if (withZeroPoint) e.push_back({zp, "zp"});
+        e.push_back({acc, "acc"});
+        e.push_back({out, "out"});
+        return computation::Graph(std::move(t), std::move(n), std::move(e)).lower(Target::Amd)._internal.nodes.size();
+    };
+    EXPECT(quantised(1, 4, false) == 1 && quantised(1, 1, false) == 1 && quantised(-1, 4, false) == 1);
+    EXPECT(quantised(0, 4, false) == 2 && quantised(1, 4, true) == 2);
 }
 
 static Device &amd() { return *device::init(Device::Type::Amd, 0, "pool=4294967296"); }
@@ -991,19 +1015,33 @@ static void quantisedLinearStream() {
     for (auto &v : x_) v = g(rng);
 
     // edges: 0 x | 1 xq 2 scale 3 zp | 4 W (local) 5 acc | 6 y
-    graph_topo::GraphTopo topo(1, 1);
-    topo.pushNode({0}, 0, 3);
-    topo.pushNode({1, 4, 3}, 1, 1);
-    topo.pushNode({5, 2}, 0, 1);
-    topo.setGlobalOutput(0, 6);
-    std::vector<computation::Node> ops;
-    ops.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
-    ops.push_back({std::make_unique<computation::MatMulInteger>(), "matmul"});
-    ops.push_back({std::make_unique<computation::DequantizeLinear>(), "dequantise"});
-    auto graph = computation::Graph(std::move(topo), std::move(ops),
-                                    {{x, "x"}, {xq, "xq"}, {scale, "scale"}, {zp, "zp"}, {w, "W"}, {acc, "acc"}, {y, "y"}})
-                     .lower(computation::Target::Amd);
-    EXPECT(graph._internal.edges[4].data == wBlob && graph._internal.edges[5].size == acc->bytesSize());
+    // With `accIsOutput` the int32 sums are a result of the graph too, which keeps the three operators
+    // apart; otherwise lower() folds the dequantisation into the product.
+    auto build = [&](bool accIsOutput) {
+        graph_topo::GraphTopo topo(1, accIsOutput ? 2 : 1);
+        topo.pushNode({0}, 0, 3);
+        topo.pushNode({1, 4, 3}, 1, 1);
+        topo.pushNode({5, 2}, 0, 1);
+        topo.setGlobalOutput(0, 6);
+        if (accIsOutput) topo.setGlobalOutput(1, 5);
+        std::vector<computation::Node> ops;
+        ops.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
+        ops.push_back({std::make_unique<computation::MatMulInteger>(), "matmul"});
+        ops.push_back({std::make_unique<computation::DequantizeLinear>(), "dequantise"});
+        return computation::Graph(std::move(topo), std::move(ops),
+                                  {{x, "x"}, {xq, "xq"}, {scale, "scale"}, {zp, "zp"}, {w, "W"}, {acc, "acc"}, {y, "y"}})
+            .lower(computation::Target::Amd);
+    };
+    auto apart = build(true), fused = build(false);
+    EXPECT(apart._internal.nodes.size() == 3 && apart._internal.edges[4].data == wBlob && apart._internal.edges[5].size == acc->bytesSize());
+    // fused: x | xq scale zp | W y
+    EXPECT(fused._internal.nodes.size() == 2 && fused._internal.edges.size() == 6);
+    EXPECT(fused._internal.nodes[1].name == "matmul+dequantise" && fused._internal.nodes[1].kernel->is<MatMulIntegerDequantizeHip>());
+    EXPECT(fused._internal.edges[4].data == wBlob && fused._internal.edges[5].name == "y" && fused._internal.topology.globalOutputs()[0] == 5);
+    {
+        auto node = fused._internal.topology.node(1);
+        EXPECT(node.inputs.size() == 4 && node.inputs[0] == 1 && node.inputs[1] == 4 && node.inputs[2] == 3 && node.inputs[3] == 2);
+    }
 
     // oracle chain
     std::vector<uint8_t> q(M * K);
@@ -1016,32 +1054,42 @@ static void quantisedLinearStream() {
     oracle_dequantize_linear(ref.data(), accRef.data(), &s, nullptr, 1, 1, M * N, ORACLE_I32, 1, 1);
 
     auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
-    for (auto allocator : {flatAllocate, reusableAllocate}) {
-        auto stream = graph.lower(dev, allocator);
-        // every stack offset is 256-byte aligned on this device
-        bool aligned = true;
-        for (auto const &e : stream.graph().edges)
-            if (!e.blob && e.stackOffset < SIZE_MAX - 1) aligned &= e.stackOffset % 256 == 0;
-        for (auto const &n : stream.graph().nodes) aligned &= n.workspaceOffset % 256 == 0;
-        EXPECT(aligned);
-        stream.setData(0, x_.data(), x->bytesSize());
-        stream.run();
-        device::sync(Device::Type::Amd);
-        EXPECT(stream.copyData(6, out.data(), y->bytesSize()));
-        EXPECT(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0);
-        // bench: one duration per node, each including the wait for the device
-        auto times = stream.bench([] { device::sync(Device::Type::Amd); });
-        EXPECT(times.size() == 3 && times[0].count() > 0 && times[1].count() > 0 && times[2].count() > 0);
-        // trace: copy the intermediate results out node by node (what Executor::trace is for)
-        std::vector<uint8_t> qGpu(M * K);
-        std::vector<int32_t> accGpu(M * N);
-        stream.trace([&](count_t idx, void const *const *, void const *const *outputs) {
+    for (auto const *graph : {&apart, &fused})
+        for (auto allocator : {flatAllocate, reusableAllocate}) {
+            auto stream = graph->lower(dev, allocator);
+            auto const nodeCount = stream.graph().nodes.size();
+            auto const yEdge = stream.graph().topology.globalOutputs()[0];
+            // every stack offset is 256-byte aligned on this device
+            bool aligned = true;
+            for (auto const &e : stream.graph().edges)
+                if (!e.blob && e.stackOffset < SIZE_MAX - 1) aligned &= e.stackOffset % 256 == 0;
+            for (auto const &n : stream.graph().nodes) aligned &= n.workspaceOffset % 256 == 0;
+            EXPECT(aligned);
+            stream.setData(0, x_.data(), x->bytesSize());
+            stream.run();
             device::sync(Device::Type::Amd);
-            if (idx == 0) AmdMemory().copyDH(qGpu.data(), outputs[0], qGpu.size());
-            if (idx == 1) AmdMemory().copyDH(accGpu.data(), outputs[0], accGpu.size() * 4);
-        });
-        EXPECT(qGpu == q && accGpu == accRef);
-    }
+            std::fill(out.begin(), out.end(), -1.f);
+            EXPECT(stream.copyData(yEdge, out.data(), y->bytesSize()));
+            EXPECT(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0);
+            if (nodeCount == 3) {// the int32 sums are a result as well
+                std::vector<int32_t> accGpu(M * N);
+                EXPECT(stream.copyData(stream.graph().topology.globalOutputs()[1], accGpu.data(), accGpu.size() * 4) && accGpu == accRef);
+            }
+            // bench: one duration per node, each including the wait for the device
+            auto times = stream.bench([] { device::sync(Device::Type::Amd); });
+            bool positive = times.size() == nodeCount;
+            for (auto t : times) positive &= t.count() > 0;
+            EXPECT(positive);
+            // trace: copy results out node by node (what Executor::trace is for)
+            std::vector<uint8_t> qGpu(M * K);
+            std::vector<float> last(M * N);
+            stream.trace([&](count_t idx, void const *const *, void const *const *outputs) {
+                device::sync(Device::Type::Amd);
+                if (idx == 0) AmdMemory().copyDH(qGpu.data(), outputs[0], qGpu.size());
+                if (idx + 1 == nodeCount) AmdMemory().copyDH(last.data(), outputs[0], last.size() * 4);
+            });
+            EXPECT(qGpu == q && std::memcmp(last.data(), ref.data(), last.size() * 4) == 0);
+        }
 }
 
 // One decode step of an attention block as a graph: RotaryEmbedding on q and k ([N, 1, heads, D]),

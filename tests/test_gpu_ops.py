@@ -325,6 +325,39 @@ def test_matmul_integer_zero_point_variants_and_broadcast(m, k, n):
     assert np.array_equal(y, oracle.matmul_integer(a2, b2, az, None, threads=8))
 
 
+@pytest.mark.parametrize("m,k,n", [(37, 53, 29), (256, 128, 256), (512, 640, 768)])
+def test_matmul_integer_with_dequantize_epilogue(m, k, n):
+    # float(sum) * scale in the epilogue == MatMulInteger followed by DequantizeLinear, bit for bit
+    rng = np.random.default_rng(m + n)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    az = rng.integers(0, 256, (1,), dtype=np.uint8)
+    acc = oracle.matmul_integer(a, b, az, None, threads=8)
+    per_column = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    scalar = np.array([3.1e-3], np.float32)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), None, dequant_scale=dev(per_column)))
+    assert y.dtype == np.float32
+    assert np.array_equal(y, oracle.dequantize_linear(acc, per_column, None, axis=2))
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), None, dequant_scale=dev(scalar)))
+    assert np.array_equal(y, oracle.dequantize_linear(acc, scalar, None))
+    # and equal to the two GPU operators run one after the other
+    two = ops.dequantize_linear(ops.matmul_integer(dev(a), dev(b), dev(az), None), dev(per_column), None, axis=2)
+    assert torch.equal(two, ops.matmul_integer(dev(a), dev(b), dev(az), None, dequant_scale=dev(per_column)))
+
+
+def test_matmul_integer_dequantize_large_sums_round_once():
+    # |sum| up to 2^26 > 2^24: the int -> float conversion rounds (to nearest even), then one multiplication
+    rng = np.random.default_rng(2)
+    a = rng.integers(0, 40, (256, 4096), dtype=np.uint8)        # a - 128 in [-128, -89]
+    b = rng.integers(-128, -64, (4096, 256), dtype=np.int8)
+    az = np.array([128], np.uint8)
+    scale = np.array([0.37], np.float32)
+    acc = oracle.matmul_integer(a, b, az, None, threads=8)
+    assert acc.min() > 2 ** 25 and np.any(acc.astype(np.float32).astype(np.int64) != acc)   # not representable
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), None, dequant_scale=dev(scale)))
+    assert np.array_equal(y, acc.astype(np.float32) * scale[0])
+
+
 def test_matmul_integer_extremes():
     a = np.zeros((256, 4096), np.uint8)
     b = np.full((4096, 256), -128, np.int8)
