@@ -379,6 +379,22 @@ def main():
         ops_out["cast"] = e
         del xs, ys
 
+    if want("transpose"):
+        # heads and sequence swap between a projection's output and attention: [32, 512, 32, 128] fp16
+        nb = 3  # 3 x 268 MB
+        xs = [torch.randn((32, 512, 32, 128), device=dev).half() for _ in range(nb)]
+        ys = [torch.empty((32, 32, 512, 128), device=dev, dtype=torch.float16) for _ in range(nb)]
+        wall, dms, mode = time_steps(torch, lambda i: ops.transpose(xs[i], (0, 2, 1, 3), out=ys[i]), steps, warmup, nb)
+        tr_bytes = 2 * 32 * 512 * 32 * 128 * 2
+        e = hbm_entry(tr_bytes, dms, "transpose")
+        e.update(workload="Transpose fp16 [32,512,32,128] perm (0,2,1,3)", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn = xs[0][:4].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.transpose(xn, (0, 2, 1, 3)), tr_bytes // 8, "4 of the 32 batch rows")
+        ops_out["transpose"] = e
+        del xs, ys
+
     if want("matmul_integer") or want("matmul_integer_dequantize"):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)

@@ -156,6 +156,18 @@ int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtyp
                   const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
                   size_t c_stride_m, size_t c_stride_n, void *stream);
 
+/* ---- Transpose ----------------------------------------------------------------------------
+ * replaces src/04kernel/cuda/src/transpose.cu + src/04kernel/src/kernels/transpose/cuda_kernel.cu:8-30;
+ * contract src/04kernel/src/kernels/transpose/cpu_kernel.cc:27-37: the output is block_count blocks
+ * of block_size bytes, output block i is input block locate(i) with
+ * locate (src/04kernel/src/attributes/transpose_info.cc:117-126): for d = 0 .. dims-1:
+ * q = i / stride_o[d]; ans += q * stride_i[d]; i -= q * stride_o[d].
+ * stride_i / stride_o: HOST arrays [dims] (TransposeInfo::dims), dims <= 8; y != x.  Tensors of up
+ * to 2^32 - 1 blocks and words (16 bytes, or the widest power of two that divides block_size and
+ * both addresses). */
+int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o,
+                     size_t dims, size_t block_size, size_t block_count, void *stream);
+
 /* ---- MatMulInteger -----------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust
  * zero-point pre-pass + cublasGemmEx); arithmetic contract

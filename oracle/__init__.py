@@ -57,6 +57,10 @@ def lib() -> C.CDLL:
         L.oracle_matmul_bias_f32.restype = L.oracle_matmul_bias_f64.restype = None
         L.oracle_attention_head_f32.argtypes = [vp, vp, vp, vp, sz, sz, sz, f32, i32, vp]
         L.oracle_rope_f32.argtypes = [vp, vp, vp, i32, sz, sz, sz, sz, f32, i32]
+        L.oracle_transpose_info.argtypes = [vp, vp, vp, vp, vp, vp, i32, C.c_uint32]
+        L.oracle_transpose_info.restype = i32
+        L.oracle_transpose.argtypes = [vp, vp, vp, vp, i32, C.c_uint32]
+        L.oracle_transpose.restype = None
         for name in ("oracle_rms_norm_f32", "oracle_rms_norm_f64", "oracle_softmax_f32",
                      "oracle_softmax_f64", "oracle_softmax_literal_f32", "oracle_softmax_causal_f32",
                      "oracle_matmul_integer", "oracle_matmul_f32", "oracle_mul_f32",
@@ -396,4 +400,24 @@ def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, dtyp
             return y.astype(np.float16)
     if dtype == "bf16":
         return _f32_to_bf16_rn(y)
+    return y
+
+
+def transpose_info(shape, perm, elem_size):
+    """The reference's digest of a transposition: ([(strideI, strideO), ...], block bytes, block count)."""
+    rank = len(shape)
+    assert rank == len(perm) and rank <= 8
+    sh, pm = np.asarray(shape, np.uint32), np.asarray(perm, np.uint32)
+    si, so = np.zeros(8, np.uint32), np.zeros(8, np.uint32)
+    block, count = np.zeros(1, np.uint32), np.zeros(1, np.uint32)
+    dims = lib().oracle_transpose_info(_p(si), _p(so), _p(block), _p(count), _p(sh), _p(pm), rank, elem_size)
+    return [(int(si[i]), int(so[i])) for i in range(dims)], int(block[0]), int(count[0])
+
+
+def transpose(x, perm):
+    """np.transpose(x, perm) made contiguous, computed the reference's way (any dtype, moved as bytes)."""
+    x = np.ascontiguousarray(x)
+    sh, pm = np.asarray(x.shape, np.uint32), np.asarray(perm, np.uint32)
+    y = np.empty(tuple(x.shape[p] for p in perm), dtype=x.dtype)
+    lib().oracle_transpose(_p(y), _p(x), _p(sh), _p(pm), x.ndim, x.dtype.itemsize)
     return y

@@ -446,3 +446,79 @@ void oracle_rope_f32(float *y, const float *x, const int64_t *pos, int pos_per_b
     for_spans(batch * seq, threads, rope_tokens, &c);
     free(inv_freq);
 }
+
+/* ------------------------------------------------------- transpose */
+
+int oracle_transpose_info(uint32_t *stride_i, uint32_t *stride_o, uint32_t *block_size, uint32_t *block_count,
+                          const uint32_t *shape_, const uint32_t *perm_, int rank, uint32_t elem_size) {
+    uint32_t shape[8], perm[8];
+    int map[8];
+    uint32_t count = 1;
+    for (int i = 0; i < rank; ++i) count *= shape_[i];
+    *block_size = elem_size;
+    *block_count = count;
+    /* transpose_info.cc:19-40: dimensions of size 1 go */
+    int r = 0;
+    for (int i = 0; i < rank; ++i) {
+        if (shape_[i] != 1) { map[i] = r; shape[r++] = shape_[i]; } else map[i] = -1;
+    }
+    int p = 0;
+    for (int i = 0; i < rank; ++i)
+        if (map[perm_[i]] >= 0) perm[p++] = (uint32_t) map[perm_[i]];
+    rank = r;
+    if (rank <= 1) goto whole;
+    /* transpose_info.cc:47-79: input dimensions that stay neighbours in the output become one */
+    {
+        int keep[8];
+        for (int i = 0; i < rank; ++i) keep[i] = 1;
+        for (int i = 1; i < rank; ++i)
+            if (perm[i] == perm[i - 1] + 1) keep[perm[i]] = 0;
+        int to[8], j = -1;
+        for (int i = 0; i < rank; ++i) {
+            if (keep[i] || i == 0) { shape[++j] = shape[i]; to[i] = j; keep[i] = 1; }
+            else { shape[j] *= shape[i]; to[i] = -1; }
+        }
+        int q = 0;
+        for (int i = 0; i < rank; ++i)
+            if (to[perm[i]] >= 0 && keep[perm[i]]) perm[q++] = (uint32_t) to[perm[i]];
+        rank = j + 1;
+    }
+    if (rank <= 1) goto whole;
+    /* transpose_info.cc:87-93: a last dimension that stays last is part of the block */
+    if (perm[rank - 1] == (uint32_t) (rank - 1)) {
+        *block_size *= shape[rank - 1];
+        *block_count /= shape[rank - 1];
+        --rank;
+    }
+    /* transpose_info.cc:94-112: strides of the input, taken in output order, and of the output */
+    {
+        uint32_t in_stride[8];
+        in_stride[rank - 1] = 1;
+        for (int i = rank - 1; i > 0; --i) in_stride[i - 1] = in_stride[i] * shape[i];
+        stride_o[rank - 1] = 1;
+        for (int i = rank - 1; i > 0; --i) stride_o[i - 1] = stride_o[i] * shape[perm[i]];
+        for (int i = 0; i < rank; ++i) stride_i[i] = in_stride[perm[i]];
+    }
+    return rank;
+whole:
+    stride_i[0] = stride_o[0] = 1;
+    *block_size *= *block_count;
+    *block_count = 1;
+    return 1;
+}
+
+void oracle_transpose(void *y, const void *x, const uint32_t *shape, const uint32_t *perm, int rank,
+                      uint32_t elem_size) {
+    uint32_t si[8], so[8], block, count;
+    const int dims = oracle_transpose_info(si, so, &block, &count, shape, perm, rank, elem_size);
+    for (uint32_t i = 0; i < count; ++i) {
+        /* transpose_info.cc:117-126 (locate) */
+        uint32_t from = 0, rem = i;
+        for (int d = 0; d < dims; ++d) {
+            from += rem / so[d] * si[d];
+            rem %= so[d];
+        }
+        memcpy((uint8_t *) y + (size_t) i * block, (const uint8_t *) x + (size_t) from * block, block);
+    }
+}
+

@@ -132,6 +132,20 @@ void oracle_attention_head_f32(float *o, const float *q, const float *kc, const 
 void oracle_rope_f32(float *y, const float *x, const int64_t *pos, int pos_per_batch,
                      size_t batch, size_t seq, size_t heads, size_t D, float theta, int threads);
 
+/* Transpose (permutation of dimensions) as the reference computes it:
+ * src/04kernel/src/attributes/transpose_info.cc:7-115 digests (shape, perm) — dimensions of size 1
+ * dropped, dimensions that stay neighbours merged, a last dimension that stays last folded into the
+ * block size — into per-output-dimension (strideI, strideO) pairs; the kernel
+ * (src/04kernel/src/kernels/transpose/cpu_kernel.cc:27-37) copies, for every output block i, the
+ * input block locate(i).  oracle_transpose_info returns the digest (dims <= rank pairs written to
+ * stride_i/stride_o, *block_size in bytes, *block_count) and the number of pairs;
+ * oracle_transpose runs the copy.  rank <= 8.  Pinned by the reference's digest vectors
+ * (src/04kernel/test/attributes/test_transpose_info.cpp:7-43) and by numpy.transpose. */
+int oracle_transpose_info(uint32_t *stride_i, uint32_t *stride_o, uint32_t *block_size, uint32_t *block_count,
+                          const uint32_t *shape, const uint32_t *perm, int rank, uint32_t elem_size);
+void oracle_transpose(void *y, const void *x, const uint32_t *shape, const uint32_t *perm, int rank,
+                      uint32_t elem_size);
+
 #ifdef __cplusplus
 }
 #endif

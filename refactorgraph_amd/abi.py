@@ -45,6 +45,7 @@ SIGNATURES = {
     "rg_hip_dynamic_quantize_linear_workspace": (_sz, [_sz]),
     "rg_hip_dynamic_quantize_linear": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp]),
     "rg_hip_cast": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
+    "rg_hip_transpose": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul_integer_workspace": (_sz, [_sz, _sz, _sz, _sz, _u]),
     "rg_hip_matmul_integer": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),

@@ -1,0 +1,200 @@
+// Transpose (permutation of dimensions) for gfx950: pure data movement, HBM-bound.
+//
+// Contract: src/04kernel/src/kernels/transpose/cpu_kernel.cc:27-37 with the digest of
+// src/04kernel/src/attributes/transpose_info.cc:7-126 — the output is `block_count` blocks of
+// `block_size` bytes; output block i is input block locate(i), where locate() peels the output
+// strides off i from the slowest dimension on and adds up the matching input strides.
+//
+// One kernel for every shape: the tensor is moved in words of W bytes, W the widest of 16, 8, 4, 2, 1
+// that divides the block size and both addresses; word g of the output (consecutive lanes, consecutive
+// words: stores are always contiguous) comes from word g % (block / W) of input block
+// locate(g / (block / W)).  Blocks of 256 bytes and more (a head's row that keeps its place while
+// sequence and head dimensions swap) read whole cache lines too; when it is two neighbouring
+// dimensions that change places in front of such blocks, a workgroup takes 8 x 8 of them so that
+// both sides move in runs of 8 blocks (transpose_tiles).  Small blocks (the innermost dimension
+// itself moves) gather their input word by word: correct, not fast.
+// Divisions by the strides are multiplications by 2^64 / d rounded up (exact for 32-bit dividends).
+#include "common.hpp"
+
+namespace rg {
+namespace {
+
+constexpr int kMaxDims = 8;
+constexpr int UNROLL = 4;  // words a thread has in flight
+constexpr uint32_t TILE_H = 8, TILE_S = 8;   // blocks of a tile along the two dimensions that change places
+
+struct Divisor {
+    uint64_t magic;  // ceil(2^64 / d); 0 stands for d == 1
+    uint32_t d;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const {
+        return magic ? static_cast<uint32_t>(__umul64hi(static_cast<uint64_t>(n), magic)) : n;
+    }
+};
+
+Divisor make_divisor(uint32_t d) {
+    Divisor r;
+    r.d = d;
+    r.magic = d <= 1 ? 0 : ~0ull / d + 1;  // floor((2^64 - 1) / d) + 1 == ceil(2^64 / d) unless d divides 2^64,
+                                           // where it is 2^64 / d as well
+    return r;
+}
+
+struct Plan {
+    Divisor stride_o[kMaxDims];
+    uint32_t stride_i[kMaxDims];
+    Divisor words_per_block;
+    uint32_t dims;
+    uint64_t words;  // of the whole tensor
+};
+
+template <class Word>
+__global__ __launch_bounds__(256) void transpose_words(Word *__restrict__ y, const Word *__restrict__ x, const Plan p) {
+    const uint64_t base = (static_cast<uint64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+    Word v[UNROLL];
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+        const uint64_t g = base + j * 256;
+        if (g < p.words) {
+            const uint32_t g32 = static_cast<uint32_t>(g);
+            const uint32_t block = p.words_per_block.div(g32), word = g32 - block * p.words_per_block.d;
+            uint32_t from = 0, rem = block;
+            for (uint32_t d = 0; d < p.dims; ++d) {
+                const uint32_t q = p.stride_o[d].div(rem);
+                from += q * p.stride_i[d];
+                rem -= q * p.stride_o[d].d;
+            }
+            v[j] = __builtin_nontemporal_load(x + static_cast<uint64_t>(from) * p.words_per_block.d + word);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+        const uint64_t g = base + j * 256;
+        if (g < p.words) __builtin_nontemporal_store(v[j], y + g);
+    }
+}
+
+// The common case of two neighbouring dimensions changing places in front of blocks that stay whole
+// (digest: the last output dimension S has output stride 1, the one before it, H, input stride 1).
+// A workgroup moves a tile of 8 x 8 blocks: it reads 8 runs of 8 neighbouring input blocks and
+// writes 8 runs of 8 neighbouring output blocks, so both sides of the copy work on runs of 2 KiB
+// (for 256-byte blocks) where the word kernel reads single blocks far apart.  (8 x 16 tiles with
+// twice the loads in flight were not faster.)
+struct TilePlan {
+    Plan plan;           // for the dimensions in front of H and S
+    uint32_t extent_h, extent_s, stride_i_s;  // stride_i of H is 1, stride_o of S is 1
+    uint32_t tiles_s;    // extent_s / TILE_S
+    Divisor tiles_per_outer;
+};
+
+template <class Word>
+__global__ __launch_bounds__(256) void transpose_tiles(Word *__restrict__ y, const Word *__restrict__ x, const TilePlan t) {
+    const Plan &p = t.plan;
+    const uint32_t wpb = p.words_per_block.d;
+    // tile -> (outer index, tile row of H, tile column of S); all wave-uniform
+    const uint32_t tile = blockIdx.x;
+    const uint32_t outer = t.tiles_per_outer.div(tile), r = tile - outer * t.tiles_per_outer.d;
+    const uint32_t th = r / t.tiles_s, ts = r - th * t.tiles_s;
+    const uint32_t out0 = outer * t.extent_h * t.extent_s;  // first output block of this outer index
+    uint32_t in0 = 0, rem = out0;
+    for (uint32_t d = 0; d + 2 < p.dims; ++d) {
+        const uint32_t q = p.stride_o[d].div(rem);
+        in0 += q * p.stride_i[d];
+        rem -= q * p.stride_o[d].d;
+    }
+    const uint32_t words = TILE_H * TILE_S * wpb;  // of the tile
+    for (uint32_t w0 = 0; w0 < words; w0 += 256 * UNROLL) {
+        Word v[UNROLL];
+        uint32_t row[UNROLL], col[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const uint32_t w = w0 + j * 256 + threadIdx.x;
+            row[j] = p.words_per_block.div(w);  // TILE_H ss + hh: neighbouring rows are neighbouring input blocks
+            col[j] = w - row[j] * wpb;
+            if (w < words) {
+                const uint32_t hh = row[j] % TILE_H, ss = row[j] / TILE_H;
+                const uint64_t from = in0 + (th * TILE_H + hh) + static_cast<uint64_t>(ts * TILE_S + ss) * t.stride_i_s;
+                v[j] = __builtin_nontemporal_load(x + from * wpb + col[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const uint32_t w = w0 + j * 256 + threadIdx.x;
+            if (w < words) {
+                const uint32_t hh = row[j] % TILE_H, ss = row[j] / TILE_H;
+                const uint64_t to = out0 + static_cast<uint64_t>(th * TILE_H + hh) * t.extent_s + (ts * TILE_S + ss);
+                __builtin_nontemporal_store(v[j], y + to * wpb + col[j]);
+            }
+        }
+    }
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <class Word>
+int launch(void *y, const void *x, const Plan &p, uint64_t block_count, hipStream_t s) {
+    // two neighbouring dimensions change places in front of whole blocks of 64 bytes or more
+    if (p.dims >= 2 && p.stride_i[p.dims - 2] == 1 && p.words_per_block.d * sizeof(Word) >= 64) {
+        const uint32_t extent_s = p.stride_o[p.dims - 2].d;
+        const uint64_t outer_blocks = p.dims >= 3 ? p.stride_o[p.dims - 3].d : block_count;
+        const uint32_t extent_h = static_cast<uint32_t>(outer_blocks / extent_s);
+        if (extent_s % TILE_S == 0 && extent_h % TILE_H == 0 && outer_blocks % extent_s == 0) {
+            TilePlan t{};
+            t.plan = p;
+            t.extent_h = extent_h;
+            t.extent_s = extent_s;
+            t.stride_i_s = p.stride_i[p.dims - 1];
+            t.tiles_s = extent_s / TILE_S;
+            t.tiles_per_outer = make_divisor((extent_h / TILE_H) * (extent_s / TILE_S));
+            const uint64_t tiles = block_count / (TILE_H * TILE_S);
+            if (tiles <= 0x7fffffffull) {
+                transpose_tiles<Word><<<static_cast<unsigned>(tiles), 256, 0, s>>>(static_cast<Word *>(y),
+                                                                                  static_cast<const Word *>(x), t);
+                return launch_status();
+            }
+        }
+    }
+    const uint64_t per_wg = 256ull * UNROLL;
+    const uint64_t grid = (p.words + per_wg - 1) / per_wg;
+    if (grid > 0x7fffffffull) return RG_HIP_E_UNSUPPORTED;
+    transpose_words<Word><<<static_cast<unsigned>(grid), 256, 0, s>>>(static_cast<Word *>(y), static_cast<const Word *>(x), p);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace rg
+
+extern "C" int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o,
+                                size_t dims, size_t block_size, size_t block_count, void *stream) {
+    using namespace rg;
+    if (!y || !x || !stride_i || !stride_o) return RG_HIP_E_ARGUMENT;
+    if (dims == 0 || dims > static_cast<size_t>(kMaxDims)) return RG_HIP_E_UNSUPPORTED;
+    if (block_size == 0 || block_count == 0) return 0;
+    if (y == x) return RG_HIP_E_ARGUMENT;  // not an in-place operation
+    const uint64_t bytes = static_cast<uint64_t>(block_size) * block_count;
+    if (block_count > 0xffffffffull) return RG_HIP_E_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    if (block_count == 1) return static_cast<int>(hipMemcpyAsync(y, x, bytes, hipMemcpyDeviceToDevice, s));
+
+    const uintptr_t misalign = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(x) | block_size;
+    uint32_t w = 16;
+    while (misalign & (w - 1)) w >>= 1;
+    const uint64_t words = bytes / w;
+    if (words > 0xffffffffull) return RG_HIP_E_UNSUPPORTED;  // word indices are 32-bit in the kernel
+
+    Plan p{};
+    p.dims = static_cast<uint32_t>(dims);
+    p.words = words;
+    p.words_per_block = make_divisor(static_cast<uint32_t>(block_size / w));
+    for (size_t d = 0; d < dims; ++d) {
+        if (stride_o[d] == 0) return RG_HIP_E_ARGUMENT;
+        p.stride_o[d] = make_divisor(stride_o[d]);
+        p.stride_i[d] = stride_i[d];
+    }
+    switch (w) {
+        case 16: return launch<u32x4>(y, x, p, block_count, s);
+        case 8: return launch<uint64_t>(y, x, p, block_count, s);
+        case 4: return launch<uint32_t>(y, x, p, block_count, s);
+        case 2: return launch<uint16_t>(y, x, p, block_count, s);
+        default: return launch<uint8_t>(y, x, p, block_count, s);
+    }
+}

@@ -1,0 +1,3 @@
+// reference include path -> host mirror
+#pragma once
+#include "rg_mirror/computation.h"

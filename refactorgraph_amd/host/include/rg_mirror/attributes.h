@@ -1,6 +1,6 @@
 // Shape pre-digestion used by the hot-path collectors.  Semantics follow
 // src/04kernel/src/attributes/{softmax_info.cc:6-13, broadcaster.cc:17-105,
-// mat_mul_integer_info.cc:5-40, mat_mul_info.cc:5-43}.
+// mat_mul_integer_info.cc:5-40, mat_mul_info.cc:5-43, transpose_info.cc:7-126}.
 #pragma once
 
 #include <optional>
@@ -47,6 +47,22 @@ namespace refactor::kernel {
         MatMulInfo(Tensor const &, Tensor const &, std::optional<std::reference_wrapper<Tensor const>>,
                    bool, bool, float, float);
         dim_t batch() const noexcept { return broadcaster.outputsCount; }
+    };
+
+    // Digest of a transposition (src/04kernel/include/kernel/attributes/transpose_info.h:9-29): the
+    // output is blockCount blocks of blockSize bytes; output block i is input block locate(i).
+    // Size-1 dimensions are dropped, dimensions that stay neighbours are merged, a last dimension
+    // that stays last is folded into the block.  dims are in output order, slowest first.
+    using Permutation = std::vector<dim_t>;
+    struct TransposeInfo {
+        struct Dimension {
+            dim_t strideI, strideO;
+        };
+        std::vector<Dimension> dims;
+        dim_t blockSize, blockCount;
+
+        TransposeInfo(DataType, std::vector<dim_t> const &shape, Permutation const &);
+        dim_t locate(dim_t) const noexcept;
     };
 
     struct MatMulIntegerInfo {

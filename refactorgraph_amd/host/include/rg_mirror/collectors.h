@@ -4,6 +4,7 @@
 // dequantize_linear.h, attention.h}; RotaryEmbeddingCollector has no counterpart there.
 #pragma once
 
+#include "rg_mirror/attributes.h"
 #include "rg_mirror/kernel.h"
 
 namespace refactor::kernel {
@@ -59,6 +60,15 @@ namespace refactor::kernel {
     struct CastCollector final : public InfoCollector {
         constexpr explicit CastCollector(hardware::Device::Type target) noexcept
             : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: data; outputs: data with its dimensions permuted
+    // (src/04kernel/include/kernel/collectors/transpose.h, src/04kernel/src/collectors/transpose.cc:7-35)
+    struct TransposeCollector final : public InfoCollector {
+        Permutation perm;
+        TransposeCollector(hardware::Device::Type target, Permutation perm_) noexcept
+            : InfoCollector(target), perm(std::move(perm_)) {}
         std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
     };
 

@@ -4,7 +4,7 @@
 // src/05computation/include/computation/{operator.h:6-47, graph.h:7-35} and
 // src/05computation/src/graph.cc:17-78; operator classes as in
 // src/05computation/include/computation/operators/{rms_normalization,softmax,mat_mul_integer,
-// dequantize_linear,dynamic_quantize_linear,cast,mat_mul,attention,identity,reshape}.h.
+// dequantize_linear,dynamic_quantize_linear,cast,mat_mul,transpose,attention,identity,reshape}.h.
 // Differences: Attention has candidateKernels (the reference declares the operator without one, so
 // a graph that contains it cannot be lowered there); RotaryEmbedding is new; Softmax carries the
 // causal flag and DequantizeLinear the axis that the collectors of this build take; layout
@@ -94,6 +94,14 @@ namespace refactor::computation {
     struct Attention final : public Operator {
         dim_t maxSeqLen;
         constexpr explicit Attention(dim_t maxSeqLen_) noexcept : maxSeqLen(maxSeqLen_) {}
+        RG_OPERATOR_COMMON
+        kernel::CollectorBox candidateKernels(Target) const final;
+        std::string serialize() const final;
+    };
+
+    struct Transpose final : public Operator {
+        kernel::Permutation perm;
+        explicit Transpose(kernel::Permutation perm_) noexcept : perm(std::move(perm_)) {}
         RG_OPERATOR_COMMON
         kernel::CollectorBox candidateKernels(Target) const final;
         std::string serialize() const final;

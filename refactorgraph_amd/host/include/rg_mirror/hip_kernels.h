@@ -116,6 +116,18 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // mirrors TransposeCuda (src/04kernel/src/kernels/transpose/cuda_kernel.hh)
+    struct TransposeHip final : public Kernel {
+        TransposeInfo info;
+
+        explicit TransposeHip(TransposeInfo) noexcept;
+        static KernelBox build(TransposeInfo) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct AttentionHip final : public Kernel {
         // the reference's parameter block (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-14)
         // plus what it leaves to the run time: where past_seq_len comes from

@@ -152,4 +152,73 @@ namespace refactor::kernel {
           n(inputs[1].get().shape.rbegin()[0]),
           broadcaster({batchDims(inputs[0].get()), batchDims(inputs[1].get())}) {}
 
+    // ------------------------------------------------------------------ TransposeInfo
+
+    TransposeInfo::TransposeInfo(DataType dt, std::vector<dim_t> const &shape_, Permutation const &perm_)
+        : dims{}, blockSize(static_cast<dim_t>(dt.size())), blockCount(1) {
+        ASSERT(perm_.size() == shape_.size(), "a permutation names every dimension once");
+        for (auto d : shape_) blockCount *= d;
+        // runs of input dimensions (size 1 left out) that stay neighbours in the output, in output order
+        std::vector<std::vector<dim_t>> runs;
+        for (auto p : perm_) {
+            ASSERT(p < shape_.size(), "a permutation names every dimension once");
+            if (shape_[p] == 1) continue;
+            // the previous kept dimension of the input, skipping size-1 ones
+            bool follows = false;
+            if (!runs.empty()) {
+                auto last = runs.back().back();
+                follows = p > last;
+                for (auto q = last + 1; follows && q < p; ++q) follows = shape_[q] == 1;
+            }
+            if (follows) {
+                runs.back().push_back(p);
+            } else {
+                runs.push_back({p});
+            }
+        }
+        auto whole = [this] {
+            dims = {{1, 1}};
+            blockSize *= blockCount;
+            blockCount = 1;
+        };
+        if (runs.size() <= 1) {
+            whole();
+            return;
+        }
+        auto extent = [&](std::vector<dim_t> const &run) {
+            dim_t n = 1;
+            for (auto d : run) n *= shape_[d];
+            return n;
+        };
+        // input stride of a run, in blocks of the element size: everything behind its last dimension
+        auto strideIn = [&](std::vector<dim_t> const &run) {
+            dim_t n = 1;
+            for (auto d = run.back() + 1; d < shape_.size(); ++d) n *= shape_[d];
+            return n;
+        };
+        // the run that holds the input's last kept dimension, if it is also the output's last: part of the block
+        dim_t inner = 1;
+        if (strideIn(runs.back()) == 1) {
+            inner = extent(runs.back());
+            blockSize *= inner;
+            blockCount /= inner;
+            runs.pop_back();
+        }
+        dims.resize(runs.size());
+        dim_t strideO = 1;
+        for (auto i = runs.size(); i-- > 0;) {
+            dims[i] = {strideIn(runs[i]) / inner, strideO};
+            strideO *= extent(runs[i]);
+        }
+    }
+
+    dim_t TransposeInfo::locate(dim_t i) const noexcept {
+        dim_t ans = 0;
+        for (auto [strideI, strideO] : dims) {
+            ans += i / strideO * strideI;
+            i %= strideO;
+        }
+        return ans;
+    }
+
 }// namespace refactor::kernel

@@ -143,6 +143,22 @@ namespace refactor::kernel {
     }
 
     std::vector<KernelBox>
+    TransposeCollector::filter(TensorRefs inputs, TensorRefs) const {
+        auto const &data = inputs[0].get();
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                if (perm.size() == data.shape.size()) { ADD(TransposeHip::build(TransposeInfo(data.dataType, data.shape, perm))) }
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
     AttentionCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
         auto const &query = inputs[0].get();
         auto const &key = inputs[1].get();

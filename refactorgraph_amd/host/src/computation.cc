@@ -26,6 +26,7 @@ namespace refactor::computation {
     RG_OPERATOR_IDS(MatMul, "MatMul")
     RG_OPERATOR_IDS(Attention, "Attention")
     RG_OPERATOR_IDS(RotaryEmbedding, "RotaryEmbedding")
+    RG_OPERATOR_IDS(Transpose, "Transpose")
     RG_OPERATOR_IDS(Identity, "Identity")
     RG_OPERATOR_IDS(Reshape, "Reshape")
 #undef RG_OPERATOR_IDS
@@ -66,6 +67,16 @@ namespace refactor::computation {
         return std::make_unique<kernel::AttentionCollector>(target, maxSeqLen);
     }
     std::string Attention::serialize() const { return detail::cat(name(), '(', maxSeqLen, ')'); }
+
+    kernel::CollectorBox Transpose::candidateKernels(Target target) const {
+        return std::make_unique<kernel::TransposeCollector>(target, perm);
+    }
+    std::string Transpose::serialize() const {
+        std::string s(name());
+        s += "([";
+        for (auto p : perm) s += ' ' + std::to_string(p);
+        return s + " ])";
+    }
 
     kernel::CollectorBox RotaryEmbedding::candidateKernels(Target target) const {
         return std::make_unique<kernel::RotaryEmbeddingCollector>(target, theta);

@@ -109,6 +109,28 @@ namespace refactor::kernel {
         return {std::move(routine), workspace};
     }
 
+    // ------------------------------------------------------------------ Transpose
+
+    TransposeHip::TransposeHip(TransposeInfo info_) noexcept : Kernel(), info(std::move(info_)) {}
+    KernelBox TransposeHip::build(TransposeInfo info) noexcept {
+        return info.dims.size() <= 8 ? std::make_unique<TransposeHip>(std::move(info)) : nullptr;
+    }
+    size_t TransposeHip::typeId() noexcept { return idOf<TransposeHip>(); }
+    size_t TransposeHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view TransposeHip::description() const noexcept { return "Performing transpose operation on AMD gfx950"; }
+    RoutineWorkspace TransposeHip::lower(Resources &) const {
+        std::vector<uint32_t> strideI, strideO;
+        for (auto [i, o] : info.dims) {
+            strideI.push_back(i);
+            strideO.push_back(o);
+        }
+        return [strideI = std::move(strideI), strideO = std::move(strideO), blockSize = info.blockSize,
+                blockCount = info.blockCount](Resources &res, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_transpose(outputs[0], inputs[0], strideI.data(), strideO.data(), strideI.size(), blockSize,
+                                      blockCount, streamOf(res)));
+        };
+    }
+
     // ------------------------------------------------------------------ MatMulInteger + DequantizeLinear
 
     using MMD = MatMulIntegerDequantizeHip;

@@ -157,6 +157,52 @@ def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=
     return y
 
 
+def transpose_info(shape, perm, itemsize):
+    """(stride_i, stride_o, block bytes, block count): the digest of a transposition that
+    rg_hip_transpose takes (TransposeInfo of the host layer, restated for this driver): size-1
+    dimensions dropped, dimensions that stay neighbours merged, a last dimension that stays last
+    folded into the block."""
+    dims = [(s, p) for p, s in enumerate(shape)]
+    keep = [i for i, s in enumerate(shape) if s != 1]
+    new_of = {old: new for new, old in enumerate(keep)}
+    shape = [shape[i] for i in keep]
+    perm = [new_of[p] for p in perm if p in new_of]
+    # merge runs perm[i], perm[i]+1, ... into one dimension
+    runs = []
+    for p in perm:
+        if runs and p == runs[-1][-1] + 1:
+            runs[-1].append(p)
+        else:
+            runs.append([p])
+    runs_in_input_order = sorted(runs, key=lambda r: r[0])
+    shape = [math.prod(shape[i] for i in r) for r in runs_in_input_order]
+    perm = [runs_in_input_order.index(r) for r in runs]
+    block, count = itemsize, math.prod(shape)
+    if len(shape) <= 1:
+        return [1], [1], block * count, 1
+    if perm[-1] == len(shape) - 1:
+        block *= shape[-1]
+        count //= shape[-1]
+        shape, perm = shape[:-1], perm[:-1]
+    in_stride = [math.prod(shape[i + 1:]) for i in range(len(shape))]
+    out_shape = [shape[p] for p in perm]
+    stride_o = [math.prod(out_shape[i + 1:]) for i in range(len(shape))]
+    stride_i = [in_stride[p] for p in perm]
+    return stride_i, stride_o, block, count
+
+
+def transpose(x, perm, out=None):
+    """Contiguous x with its dimensions permuted (any dtype: bytes are moved)."""
+    _need_gpu(x)
+    assert x.is_contiguous() and sorted(perm) == list(range(x.dim()))
+    si, so, block, count = transpose_info(list(x.shape), list(perm), x.element_size())
+    y = torch.empty([x.shape[p] for p in perm], dtype=x.dtype, device=x.device) if out is None else out
+    si_, so_ = np.asarray(si, np.uint32), np.asarray(so, np.uint32)
+    check(lib().rg_hip_transpose(_ptr(y), _ptr(x), si_.ctypes.data_as(C.c_void_p), so_.ctypes.data_as(C.c_void_p),
+                                 len(si), block, count, _stream()), "rg_hip_transpose")
+    return y
+
+
 def matmul_integer(a, b, a_zp=None, b_zp=None, out=None, dequant_scale=None):
     """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
     (batch, row) of the operand as the reference's CPU kernel reads them.  dequant_scale (float32,

@@ -8,6 +8,9 @@
 #include "kernel/attributes/broadcaster.h"
 #include "kernel/attributes/mat_mul_integer_info.h"
 #include "kernel/attributes/softmax_info.h"
+#include "kernel/attributes/transpose_info.h"
+#include "kernel/collectors/transpose.h"
+#include "computation/operators/transpose.h"
 #include "kernel/collectors/attention.h"
 #include "kernel/collectors/dequantize_linear.h"
 #include "kernel/collectors/dynamic_quantize_linear.h"
@@ -481,6 +484,45 @@ static void allocatorsAndStreamOnCpu() {
     s3.setData(0, size_t(4));
     s3.run();
     EXPECT(s3.getData(1) && s3.getData(1)->size() == 4);
+}
+
+static void transposeInfoDigest() {
+    {// src/04kernel/test/attributes/test_transpose_info.cpp:7-43
+        TransposeInfo a(DataType::F32, {1, 2, 3, 2, 1}, {1, 2, 3, 0, 4});
+        EXPECT(a.blockSize == 48 && a.blockCount == 1 && a.dims.size() == 1);
+        TransposeInfo b(DataType::F32, {1, 1, 2, 1, 1}, {1, 2, 3, 0, 4});
+        EXPECT(b.blockSize == 8 && b.blockCount == 1 && b.dims.size() == 1);
+        TransposeInfo c(DataType::F32, {1, 2, 3, 4, 5}, {2, 3, 1, 0, 4});
+        EXPECT(c.blockSize == 20 && c.blockCount == 24 && c.dims.size() == 2);
+        EXPECT(c.dims[1].strideI == 12 && c.dims[1].strideO == 1 && c.dims[0].strideI == 1 && c.dims[0].strideO == 2);
+    }
+    // random shapes: the digest equals the oracle's, and copying block locate(i) to block i equals its result
+    std::mt19937 rng(4);
+    bool same = true, moved = true;
+    for (int t = 0; t < 500; ++t) {
+        auto const rank = 1 + rng() % 6;
+        std::vector<dim_t> shape(rank), perm(rank);
+        for (auto &d : shape) d = 1 + rng() % 4;
+        std::iota(perm.begin(), perm.end(), 0);
+        std::shuffle(perm.begin(), perm.end(), rng);
+        TransposeInfo info(DataType::I16, shape, perm);
+        uint32_t si[8], so[8], block, count;
+        auto const dims = oracle_transpose_info(si, so, &block, &count, shape.data(), perm.data(), static_cast<int>(rank), 2);
+        same &= static_cast<size_t>(dims) == info.dims.size() && block == info.blockSize && count == info.blockCount;
+        for (size_t i = 0; same && i < info.dims.size(); ++i) same &= info.dims[i].strideI == si[i] && info.dims[i].strideO == so[i];
+        std::vector<int16_t> x(static_cast<size_t>(info.blockSize) * info.blockCount / 2), y(x.size()), ref(x.size());
+        std::iota(x.begin(), x.end(), 0);
+        for (dim_t i = 0; i < info.blockCount; ++i)
+            std::memcpy(reinterpret_cast<uint8_t *>(y.data()) + i * info.blockSize,
+                        reinterpret_cast<uint8_t *>(x.data()) + info.locate(i) * info.blockSize, info.blockSize);
+        oracle_transpose(ref.data(), x.data(), shape.data(), perm.data(), static_cast<int>(rank), 2);
+        moved &= y == ref;
+    }
+    EXPECT(same);
+    EXPECT(moved);
+    EXPECT(throws<std::runtime_error>([] { TransposeInfo(DataType::F32, {2, 3}, {0}); }));
+    EXPECT(TransposeCollector(Device::Type::Amd, {1, 0}).filter({*Tensor::share(DataType::FP16, Shape{4, 6})}, {*Tensor::share(DataType::FP16, Shape{6, 4})}).size() == 1);
+    EXPECT(computation::Transpose({0, 2, 1, 3}).serialize() == "Transpose([ 0 2 1 3 ])");
 }
 
 static void computationGraphLowers() {
@@ -1280,6 +1322,122 @@ static void longChainRecorded() {
                 std::chrono::duration<double, std::micro>(t2 - t1).count() / 50);
 }
 
+static void transposeHip() {
+    runtime::Resources res;
+    auto &dev = amd();
+    auto run = [&](DataType dt, Shape shape, Permutation perm) {
+        auto x = Tensor::share(dt, shape);
+        Shape outShape;
+        for (auto p : perm) outShape.push_back(shape[p]);
+        auto y = Tensor::share(dt, outShape);
+        auto kernels = TransposeCollector(Device::Type::Amd, perm).filter({*x}, {*y});
+        EXPECT(kernels.size() == 1);
+        auto routine = kernels[0]->lower(res).routine;
+        std::vector<uint8_t> x_(x->bytesSize()), y_(x_.size()), ref(x_.size());
+        std::mt19937 rng(8);
+        for (auto &v : x_) v = rng();
+        auto mx = dev.malloc(x_.size()), my = dev.malloc(x_.size());
+        mx->copyFromHost(x_.data());
+        void const *inputs[]{*mx};
+        void *outputs[]{*my};
+        routine(res, nullptr, inputs, outputs);
+        my->copyToHost(y_.data());
+        oracle_transpose(ref.data(), x_.data(), shape.data(), perm.data(), static_cast<int>(shape.size()), static_cast<uint32_t>(dt.size()));
+        EXPECT(y_ == ref);
+    };
+    run(DataType::F32, {1, 3, 2, 5}, {2, 3, 0, 1});// src/04kernel/test/kernels/transpose/test_cuda.cpp
+    run(DataType::FP16, {2, 48, 8, 128}, {0, 2, 1, 3});
+    run(DataType::U8, {5, 7, 3}, {2, 0, 1});
+    run(DataType::F64, {4, 1, 6}, {2, 1, 0});
+}
+
+// Prefill of an attention block with the data in the layout a projection leaves it in
+// ([N, seq, heads, D]): RotaryEmbedding -> Transpose to [N, heads, seq, D] -> Attention (tiled kernel,
+// caches filled from position 0) -> Transpose back.
+static void prefillAttentionStream() {
+    using namespace computation;
+    constexpr dim_t N = 2, H = 4, Hkv = 2, D = 128, S = 32, CAP = 64;
+    constexpr float theta = 10000.f;
+    auto qIn = Tensor::share(DataType::FP16, Shape{N, S, H, D}), qT = Tensor::share(DataType::FP16, Shape{N, H, S, D});
+    auto kIn = Tensor::share(DataType::FP16, Shape{N, S, Hkv, D}), kT = Tensor::share(DataType::FP16, Shape{N, Hkv, S, D});
+    auto pos = Tensor::share(DataType::I64, Shape{N, S}), past = Tensor::share(DataType::I64, Shape{1});
+    auto cache = Tensor::share(DataType::FP16, Shape{N, Hkv, CAP, D});
+    // edges: 0 q 1 k 2 v 3 pos 4 past | 5 qr | 6 kr | 7 qT | 8 kT | 9 vT | 10 oT 11 kc 12 vc | 13 o
+    graph_topo::GraphTopo topo(5, 3);
+    topo.pushNode({0, 3}, 0, 1);
+    topo.pushNode({1, 3}, 0, 1);
+    topo.pushNode({5}, 0, 1);
+    topo.pushNode({6}, 0, 1);
+    topo.pushNode({2}, 0, 1);
+    topo.pushNode({7, 8, 9, 4}, 0, 3);
+    topo.pushNode({10}, 0, 1);
+    topo.setGlobalOutput(0, 13);
+    topo.setGlobalOutput(1, 11);
+    topo.setGlobalOutput(2, 12);
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_q"});
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_k"});
+    for (auto name : {"q_heads_first", "k_heads_first", "v_heads_first"})
+        ops.push_back({std::make_unique<Transpose>(kernel::Permutation{0, 2, 1, 3}), name});
+    ops.push_back({std::make_unique<Attention>(CAP), "attention"});
+    ops.push_back({std::make_unique<Transpose>(kernel::Permutation{0, 2, 1, 3}), "o_tokens_first"});
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    auto stream = computation::Graph(std::move(topo), std::move(ops),
+                                     {{qIn, "q"}, {kIn, "k"}, {kIn, "v"}, {pos, "pos"}, {past, "past"}, {qIn, "qr"}, {kIn, "kr"},
+                                      {qT, "qT"}, {kT, "kT"}, {kT, "vT"}, {qT, "oT"}, {cache, "k_cache"}, {cache, "v_cache"}, {qIn, "o"}})
+                      .lower(Target::Amd)
+                      .lower(dev, reusableAllocate);
+    std::mt19937 rng(12);
+    std::normal_distribution<float> n01;
+    auto randomHalf = [&](size_t n) { std::vector<uint16_t> v(n); for (auto &e : v) e = f2h(n01(rng)); return v; };
+    auto q_ = randomHalf(qIn->elementsSize()), k_ = randomHalf(kIn->elementsSize()), v_ = randomHalf(kIn->elementsSize());
+    std::vector<int64_t> pos_(N * S);
+    for (dim_t b = 0; b < N; ++b)
+        for (dim_t t = 0; t < S; ++t) pos_[b * S + t] = t;
+    int64_t zero = 0;
+    stream.setData(0, q_.data(), q_.size() * 2);
+    stream.setData(1, k_.data(), k_.size() * 2);
+    stream.setData(2, v_.data(), v_.size() * 2);
+    stream.setData(3, pos_.data(), pos_.size() * 8);
+    stream.setData(4, &zero, 8);
+    stream.run();
+    device::sync(Device::Type::Amd);
+    std::vector<uint16_t> o(q_.size()), kc(cache->elementsSize()), vc(kc.size());
+    EXPECT(stream.copyData(13, o.data(), o.size() * 2) && stream.copyData(11, kc.data(), kc.size() * 2) && stream.copyData(12, vc.data(), vc.size() * 2));
+
+    // oracle: rotate (positions 0 .. S-1), then per (batch row, head) causal attention over the new rows
+    auto rope = [&](std::vector<uint16_t> const &x, dim_t heads) {
+        std::vector<float> xf(x.size()), yf(x.size());
+        for (size_t i = 0; i < x.size(); ++i) xf[i] = h2f(x[i]);
+        oracle_rope_f32(yf.data(), xf.data(), pos_.data(), 1, N, S, heads, D, theta, 1);
+        std::vector<uint16_t> y(x.size());
+        for (size_t i = 0; i < x.size(); ++i) y[i] = f2h(yf[i]);
+        return y;
+    };
+    auto qr = rope(q_, H), kr = rope(k_, Hkv);
+    bool cacheOk = true, ok = true;
+    float const scale = 1.0f / std::sqrt(static_cast<float>(D));
+    std::vector<float> scratch(2 * S * S), ref(S * D), qf(S * D), kf(S * D), vf(S * D);
+    for (dim_t b = 0; b < N; ++b)
+        for (dim_t h = 0; h < H; ++h) {
+            dim_t const kh = h / (H / Hkv);
+            for (dim_t t = 0; t < S; ++t)
+                for (dim_t i = 0; i < D; ++i) {
+                    qf[t * D + i] = h2f(qr[((b * S + t) * H + h) * D + i]);
+                    // keys as the device wrote them to the cache (rotated within the rotary embedding's tolerance)
+                    kf[t * D + i] = h2f(kc[((b * Hkv + kh) * CAP + t) * D + i]);
+                    vf[t * D + i] = h2f(vc[((b * Hkv + kh) * CAP + t) * D + i]);
+                    cacheOk &= std::fabs(kf[t * D + i] - h2f(kr[((b * S + t) * Hkv + kh) * D + i])) <= 2e-3f;
+                    cacheOk &= vc[((b * Hkv + kh) * CAP + t) * D + i] == v_[((b * S + t) * Hkv + kh) * D + i];
+                }
+            oracle_attention_head_f32(ref.data(), qf.data(), kf.data(), vf.data(), S, 0, D, scale, 1, scratch.data());
+            for (dim_t t = 0; t < S; ++t)
+                for (dim_t i = 0; i < D; ++i) ok &= std::fabs(h2f(o[((b * S + t) * H + h) * D + i]) - ref[t * D + i]) <= 4e-3f;
+        }
+    EXPECT(cacheOk);
+    EXPECT(ok);
+}
+
 static void amdDeviceAndPool() {
     auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
     EXPECT(dev && dev->type() == Device::Type::Amd && device::fetch(Device::Type::Amd) == dev);
@@ -1308,6 +1466,7 @@ int main(int argc, char **argv) {
     RUN(graphTopoAndBuilder);
     RUN(offsetCalculatorPlan);
     RUN(allocatorsAndStreamOnCpu);
+    RUN(transposeInfoDigest);
     RUN(computationGraphLowers);
     if (mode == "gpu") {
         RUN(amdDeviceAndPool);
@@ -1320,8 +1479,10 @@ int main(int argc, char **argv) {
         RUN(matMulHip);
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
+        RUN(transposeHip);
         RUN(quantisedLinearStream);
         RUN(decodeAttentionStream);
+        RUN(prefillAttentionStream);
         RUN(longChainRecorded);
     }
     std::printf("%d checks, %d failed\n", g_checks, g_failed);

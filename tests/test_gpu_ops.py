@@ -378,6 +378,50 @@ def test_matmul_integer_full_config():
     assert np.array_equal(y[rows], oracle.matmul_integer(a[rows], b, az, bz, threads=8))
 
 
+# ------------------------------------------------------------------ Transpose (bit-exact: data movement)
+
+def test_transpose_driver_digest_equals_the_oracles():
+    rng = np.random.default_rng(1)
+    for _ in range(300):
+        rank = int(rng.integers(1, 7))
+        shape = [int(v) for v in rng.integers(1, 5, rank)]
+        perm = [int(v) for v in rng.permutation(rank)]
+        si, so, block, count = ops.transpose_info(shape, perm, 2)
+        dims, oblock, ocount = oracle.transpose_info(shape, perm, 2)
+        assert (list(zip(si, so)), block, count) == (dims, oblock, ocount), (shape, perm)
+
+
+@pytest.mark.parametrize("shape,perm", [
+    ((1, 3, 2, 5), (2, 3, 0, 1)),            # src/04kernel/test/kernels/transpose/test_cpu.cpp:9-15
+    ((2, 3, 4, 5), (0, 1, 2, 3)), ((7,), (0,)), ((5, 9), (1, 0)), ((3, 5, 7), (2, 1, 0)), ((3, 5, 7), (1, 2, 0)),
+    ((2, 48, 8, 128), (0, 2, 1, 3)), ((4, 6, 33, 17), (0, 2, 1, 3)), ((2, 3, 4, 5, 6), (4, 0, 3, 1, 2)),
+    ((2, 1, 3, 1, 4), (3, 2, 4, 1, 0)), ((64, 40, 24), (1, 0, 2)), ((129, 257), (1, 0))])
+@pytest.mark.parametrize("dt", [np.uint8, np.float16, np.float32, np.float64])
+def test_transpose_bit_exact(shape, perm, dt):
+    x = np.random.default_rng(len(shape)).integers(0, 200, shape).astype(dt)
+    y = ops.transpose(dev(x), perm)
+    ref = oracle.transpose(x, perm)
+    assert tuple(y.shape) == ref.shape and np.array_equal(host(y), ref) and np.array_equal(ref, np.transpose(x, perm))
+
+
+def test_transpose_unaligned_views_and_involution():
+    x = torch.arange(3 * 37 * 11, device=DEV, dtype=torch.int16).reshape(3, 37, 11)
+    buf = torch.empty(3 * 37 * 11 + 1, device=DEV, dtype=torch.int16)
+    y = ops.transpose(x, (1, 0, 2), out=buf[1:].view(37, 3, 11))     # output 2 bytes off a 4-byte boundary
+    assert torch.equal(y, x.permute(1, 0, 2))
+    assert torch.equal(ops.transpose(ops.transpose(x, (2, 0, 1)), (1, 2, 0)), x)
+
+
+def test_transpose_full_config():
+    # heads and sequence swap around attention: [32, 512, 32, 128] fp16 <-> [32, 32, 512, 128]
+    x = torch.randn((32, 512, 32, 128), device=DEV).half()
+    y = ops.transpose(x, (0, 2, 1, 3))
+    assert torch.equal(y, x.permute(0, 2, 1, 3).contiguous())
+    assert torch.equal(ops.transpose(y, (0, 2, 1, 3)), x)
+    sl = np.s_[5:6]
+    assert np.array_equal(host(y[sl]), oracle.transpose(host(x[sl]), (0, 2, 1, 3)))
+
+
 # ------------------------------------------------------------------ AttentionKVCache
 
 def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_row=True, pairs=None,
