@@ -33,6 +33,8 @@
  *                              src/08-01llm/README.md:29-63.  PARITY UNPINNED by the reference.
  *   oracle_rope_f32            no reference item exists; closed-form rotate-half rotary
  *                              embedding.  PARITY UNPINNED by the reference.
+ *   oracle_transpose(_info)    src/04kernel/src/attributes/transpose_info.cc:7-126
+ *                              + src/04kernel/src/kernels/transpose/cpu_kernel.cc:27-37
  *
  * Pinning (see tests/test_oracle_*.py): every function is checked against the
  * known-answer vectors of the reference's own tests where they exist, and

@@ -546,3 +546,33 @@ def test_matmul_fp16_rounds_alpha_and_the_result_once():
     # alpha = 1 + 2^-12 is not an fp16 number: it is 1.0 after the conversion the reference applies
     assert oracle.matmul(np.array([[3.0]], np.float16), np.array([[1.0]], np.float16), alpha=1 + 2.0 ** -12,
                          dtype="fp16").tolist() == [[3.0]]
+
+
+# ------------------------------------------------------------------ Transpose
+
+def test_transpose_digest_reference_vectors():
+    for c in GOLDEN["transpose_info"]["cases"]:
+        dims, block, count = oracle.transpose_info(c["shape"], c["perm"], 4)
+        assert (block, count, len(dims)) == (c["block_size"], c["block_count"], c["dims"])
+        if "strides" in c:
+            assert dims == [tuple(v) for v in c["strides"]]
+
+
+def test_transpose_against_numpy_and_its_invariants():
+    # numpy.transpose is the library routine; identity, involution and composition are what the mathematics fixes
+    rng = np.random.default_rng(3)
+    for t in range(300):
+        rank = int(rng.integers(1, 7))
+        shape = tuple(int(v) for v in rng.integers(1, 6, rank))
+        perm = tuple(int(v) for v in rng.permutation(rank))
+        x = rng.integers(0, 1 << 15, shape).astype([np.uint8, np.int16, np.float32, np.float64][t % 4])
+        y = oracle.transpose(x, perm)
+        assert y.shape == tuple(shape[p] for p in perm) and np.array_equal(y, np.transpose(x, perm))
+        inverse = tuple(int(v) for v in np.argsort(perm))
+        assert np.array_equal(oracle.transpose(y, inverse), x)
+        second = tuple(int(v) for v in rng.permutation(rank))
+        assert np.array_equal(oracle.transpose(y, second), np.transpose(x, [perm[i] for i in second]))
+    x = np.arange(30, dtype=np.float32).reshape(1, 3, 2, 5)          # src/04kernel/test/kernels/transpose/test_cpu.cpp:9-15
+    assert np.array_equal(oracle.transpose(x, (2, 3, 0, 1)), np.transpose(x, (2, 3, 0, 1)))
+    assert np.array_equal(oracle.transpose(x, (0, 1, 2, 3)), x)
+
