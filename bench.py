@@ -46,6 +46,8 @@ MEASURED_TRAFFIC = {
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
     "matmul_few_rows": (2 * 17456 + 256) * 1024,
+    "transpose": (2 * 65552 + 131217) * 1024,
+    "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
 }
 
 
@@ -436,7 +438,7 @@ def main():
             tops = 2 * 4096 ** 3 / (dms_f * 1e-3) / 1e12
             ops_out["matmul_integer_dequantize"] = {
                 "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None,
+                "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC["matmul_integer_dequantize"],
                 "workload": "MatMulInteger 4096^3 with DequantizeLinear (scale per column) in its epilogue -> f32",
                 "device_ms_per_launch": round(dms_f, 5), "timing": mode,
                 "two_operators_device_ms": round(dms_2, 5)}
