@@ -3,6 +3,7 @@
 Bars: bit-exact for MatMulInteger / DequantizeLinear; <= 1e-5 relative for fp32 RmsNormalization
 and fp32 Softmax; <= 2e-3 absolute for fp16 paths (oracle in fp32 on up-cast inputs).
 """
+import ctypes as C
 import json
 import math
 import os
@@ -12,7 +13,7 @@ import pytest
 import torch
 
 import oracle
-from refactorgraph_amd import ops
+from refactorgraph_amd import abi, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -376,6 +377,72 @@ def test_matmul_integer_full_config():
     assert np.array_equal(y.astype(np.float64), ref)
     rows = [0, 1, 255, 256, 2047, 4095]
     assert np.array_equal(y[rows], oracle.matmul_integer(a[rows], b, az, bz, threads=8))
+
+
+# ------------------------------------------------------------------ empty inputs and rejected arguments
+
+def test_empty_inputs_are_no_ops_and_bad_arguments_are_refused():
+    """Through the C ABI itself: every launcher returns 0 for a tensor without elements and leaves the
+    output alone, and refuses (negative code, nothing enqueued) null operands, types it has no kernel
+    for and workspaces that are too small."""
+    L, p = ops.lib(), ops._ptr
+    E_UNSUPPORTED, E_ARGUMENT, E_WORKSPACE = -1, -2, -3
+    buf = torch.full((4096,), 7.0, device=DEV)               # stands in for every operand
+    out = torch.full((4096,), -3.0, device=DEV)
+    i64 = torch.zeros(64, device=DEV, dtype=torch.int64)
+    d, o = p(buf), p(out)
+    calls = {
+        "rms_norm rows=0": L.rg_hip_rms_norm(o, d, d, 0, 64, 1e-5, abi.F32, None),
+        "softmax mid=0": L.rg_hip_softmax(o, d, 4, 0, 1, abi.F32, 0, None),
+        "rope seq=0": L.rg_hip_rope(o, d, p(i64), 0, 2, 0, 4, 64, 1e4, abi.FP16, None),
+        "dequantize inner=0": L.rg_hip_dequantize_linear(o, d, d, None, 1, 4, 0, abi.I8, 1, None),
+        "cast size=0": L.rg_hip_cast(o, d, 0, abi.F32, abi.FP16, None),
+        "matmul batch=0": L.rg_hip_matmul(o, d, d, None, abi.FP16, 0, 0, 1.0, 0.0, 0, 4, 4, 4, None, None, 0, 0, 0, None),
+        "matmul_integer m=0": L.rg_hip_matmul_integer(o, d, d, None, None, 0, 1, 0, 8, 8, None, None, None, None),
+        "transpose no blocks": L.rg_hip_transpose(o, d, p(i64), p(i64), 1, 16, 0, None),
+        "attention N=0": L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 0, 8, 2, 1, 0, 128, 0.1, abi.FP16,
+                                                     None, 0, None, None),
+    }
+    assert all(rc == 0 for rc in calls.values()), calls
+    torch.cuda.synchronize()
+    assert torch.all(out == -3.0)
+
+    one = np.array([1], np.uint32).ctypes.data_as(C.c_void_p)
+    refused = {
+        "rms_norm null": (L.rg_hip_rms_norm(o, None, d, 4, 64, 1e-5, abi.F32, None), E_ARGUMENT),
+        "rms_norm of integers": (L.rg_hip_rms_norm(o, d, d, 4, 64, 1e-5, abi.I32, None), E_UNSUPPORTED),
+        "softmax null": (L.rg_hip_softmax(None, d, 4, 8, 1, abi.F32, 0, None), E_ARGUMENT),
+        "softmax of bytes": (L.rg_hip_softmax(o, d, 4, 8, 1, abi.U8, 0, None), E_UNSUPPORTED),
+        "rope odd dim": (L.rg_hip_rope(o, d, p(i64), 0, 1, 2, 2, 63, 1e4, abi.FP16, None), E_UNSUPPORTED),
+        "dequantize from float": (L.rg_hip_dequantize_linear(o, d, d, None, 1, 1, 8, abi.F32, 0, None), E_UNSUPPORTED),
+        "dequantize null scale": (L.rg_hip_dequantize_linear(o, d, None, None, 1, 1, 8, abi.I8, 0, None), E_ARGUMENT),
+        "dynamic quantize without workspace": (L.rg_hip_dynamic_quantize_linear(o, o, o, d, 64, None, 0, None), E_WORKSPACE),
+        "dynamic quantize size 0": (L.rg_hip_dynamic_quantize_linear(o, o, o, d, 0, d, 1 << 14, None), E_ARGUMENT),
+        "cast from strings": (L.rg_hip_cast(o, d, 8, 8, abi.F32, None), E_UNSUPPORTED),
+        "matmul of bytes": (L.rg_hip_matmul(o, d, d, None, abi.U8, 0, 0, 1.0, 0.0, 1, 4, 4, 4, None, None, 0, 0, 0, None),
+                            E_UNSUPPORTED),
+        "matmul null": (L.rg_hip_matmul(o, None, d, None, abi.FP16, 0, 0, 1.0, 0.0, 1, 4, 4, 4, None, None, 0, 0, 0, None),
+                        E_ARGUMENT),
+        "matmul_integer null": (L.rg_hip_matmul_integer(None, d, d, None, None, 0, 1, 8, 8, 8, None, None, None, None), E_ARGUMENT),
+        "fused dequantize without scale": (L.rg_hip_matmul_integer_dequantize(o, d, d, None, None, 0, 1, 8, 8, 8, None, None,
+                                                                              None, 0, None, None), E_ARGUMENT),
+        "transpose in place": (L.rg_hip_transpose(d, d, one, one, 1, 16, 4, None), E_ARGUMENT),
+        "transpose of nine dimensions": (L.rg_hip_transpose(o, d, p(i64), p(i64), 9, 16, 4, None), E_UNSUPPORTED),
+        "attention head dim 96": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 2, 1, 0, 96, 0.1, abi.FP16,
+                                                              d, 1 << 14, None, None), E_UNSUPPORTED),
+        "attention heads not a multiple": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 3, 1, 0, 128, 0.1,
+                                                                       abi.FP16, d, 1 << 14, None, None), E_ARGUMENT),
+        "attention one cache only": (L.rg_hip_attention_kvcache(o, d, d, d, d, None, None, 0, 1, 8, 2, 1, 16, 128, 0.1, abi.FP16,
+                                                                 d, 1 << 14, None, None), E_ARGUMENT),
+        "attention without workspace": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 2, 1, 0, 128, 0.1,
+                                                                    abi.FP16, None, 0, None, None), E_WORKSPACE),
+    }
+    wrong = {k: v for k, v in refused.items() if v[0] != v[1]}
+    assert not wrong, wrong
+    torch.cuda.synchronize()
+    assert torch.all(out == -3.0) and torch.all(buf == 7.0)
+    for code in (E_UNSUPPORTED, E_ARGUMENT, E_WORKSPACE):
+        assert L.rg_hip_error_string(code).startswith(b"rg_hip:")
 
 
 # ------------------------------------------------------------------ Transpose (bit-exact: data movement)
