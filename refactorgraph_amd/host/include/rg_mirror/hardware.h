@@ -131,6 +131,9 @@ namespace refactor::hardware {
 
         Arc<Blob> malloc(size_t);
         Arc<Blob> absorb(Arc<Blob> &&);
+        // device address -> host memory, blocking (what Executor::trace reads node results with; the
+        // reference has kernel::cuda::copyOut for it, src/04kernel/cuda/src/functions.cu:17-21)
+        void copyOut(void *host, void const *deviceAddress, size_t bytes) const;
     };
 
     class Cpu final : public Device {

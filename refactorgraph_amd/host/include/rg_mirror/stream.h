@@ -53,6 +53,7 @@ namespace refactor::runtime {
         Stream(Resources, size_t stackBytes, graph_topo::GraphTopo, std::vector<Node>, std::vector<Edge>,
                Arc<hardware::Device>);
         Stream(Stream &&) noexcept;
+        Stream &operator=(Stream &&) noexcept;
         Stream(Stream const &) = delete;
         ~Stream();
 

@@ -195,6 +195,10 @@ namespace refactor::hardware {
     Device::Device(int32_t card, Arc<Memory> mem) : _card(card), _mem(std::move(mem)) {}
     void Device::setContext() const {}
     Arc<Device::Blob> Device::malloc(size_t size) { return Arc<Blob>(new Blob(this, size)); }
+    void Device::copyOut(void *host, void const *deviceAddress, size_t bytes) const {
+        setContext();
+        _mem->copyDH(host, deviceAddress, bytes);
+    }
     Arc<Device::Blob> Device::absorb(Arc<Blob> &&blob) {
         if (blob->_device == this) { return std::move(blob); }
         if (blob->_device->_mem == _mem) {

@@ -34,6 +34,18 @@ namespace refactor::runtime {
         : _device(std::move(o._device)), _stack(std::move(o._stack)), _resources(std::move(o._resources)),
           _graph(std::move(o._graph)), _recorded(std::exchange(o._recorded, nullptr)),
           _recordedData(std::move(o._recordedData)) {}
+    Stream &Stream::operator=(Stream &&o) noexcept {
+        if (this != &o) {
+            dropRecording();
+            _device = std::move(o._device);
+            _stack = std::move(o._stack);
+            _resources = std::move(o._resources);
+            _graph = std::move(o._graph);
+            _recorded = std::exchange(o._recorded, nullptr);
+            _recordedData = std::move(o._recordedData);
+        }
+        return *this;
+    }
     Stream::~Stream() { dropRecording(); }
 
     void Stream::dropRecording() noexcept {

@@ -28,6 +28,7 @@
 #include "kernel/graph.h"
 #include "runtime/stream.h"
 #include "hardware/mem_pool.h"
+#include "rg_mirror/executor.h"
 #include "rg_mirror/hip_kernels.h"
 #include "oracle.h"
 
@@ -36,9 +37,12 @@
 #include <immintrin.h>
 #include <cstdio>
 #include <cstring>
+#include <filesystem>
+#include <fstream>
 #include <numeric>
 #include <random>
 #include <tuple>
+#include <unistd.h>
 
 using namespace refactor;
 using namespace kernel;
@@ -484,6 +488,84 @@ static void allocatorsAndStreamOnCpu() {
     s3.setData(0, size_t(4));
     s3.run();
     EXPECT(s3.getData(1) && s3.getData(1)->size() == 4);
+}
+
+namespace {
+    // an operator with a kernel for the CPU target, so that the executor can be driven without a GPU
+    struct AddConstant final : public computation::Operator {
+        float addend;
+        size_t n;
+        AddConstant(float addend_, size_t n_) : addend(addend_), n(n_) {}
+        static size_t typeId() noexcept {
+            static uint8_t ID = 1;
+            return reinterpret_cast<size_t>(&ID);
+        }
+        size_t opTypeId() const noexcept final { return typeId(); }
+        std::string_view name() const noexcept final { return "AddConstant"; }
+        kernel::CollectorBox candidateKernels(computation::Target target) const final {
+            struct Collector final : public InfoCollector {
+                float addend;
+                size_t n;
+                Collector(Device::Type t, float a, size_t n_) : InfoCollector(t), addend(a), n(n_) {}
+                std::vector<KernelBox> filter(TensorRefs, TensorRefs) const final {
+                    std::vector<KernelBox> ans;
+                    if (_target == Device::Type::Cpu) ans.emplace_back(std::make_unique<AddKernel>(addend, n, false));
+                    return ans;
+                }
+            };
+            return std::make_unique<Collector>(target, addend, n);
+        }
+    };
+    std::vector<char> readFile(std::filesystem::path const &p) {
+        std::ifstream is(p, std::ios::binary);
+        return {std::istreambuf_iterator<char>(is), std::istreambuf_iterator<char>()};
+    }
+}// namespace
+
+static void executorOnCpu() {
+    using namespace python_ffi;
+    constexpr dim_t n = 6;
+    auto t = Tensor::share(DataType::F32, Shape{2, 3});
+    auto build = [&] {
+        graph_topo::GraphTopo topo(1, 1);
+        auto mid = topo.pushNode({0}, 0, 1).begin_;
+        auto out = topo.pushNode({mid}, 0, 1).begin_;
+        topo.setGlobalOutput(0, out);
+        std::vector<computation::Node> ops;
+        ops.push_back({std::make_unique<AddConstant>(1.f, n), "plus1"});
+        ops.push_back({std::make_unique<AddConstant>(10.f, n), "plus10"});
+        return computation::Graph(std::move(topo), std::move(ops), {{t, "x"}, {t, "mid"}, {t, "y"}});
+    };
+    EXPECT(findDevice("CPU", 0) == device::fetch(Device::Type::Cpu));
+    EXPECT(throws<UnreachableError>([] { findDevice("tpu", 0); }));
+    EXPECT(throws<UnreachableError>([&] { compile(build(), "cuda", "flat"); }));
+    auto exe = compile(build(), "cpu", "flat");
+    float x[n]{0, 1, 2, 3, 4, 5}, y[n]{};
+    EXPECT(throws<std::runtime_error>([&] { exe->setInput(0, x, 4); }));// size mismatch
+    exe->setInput(0, x, sizeof x);
+    exe->run();
+    exe->getOutput(0, y, sizeof y);
+    EXPECT(y[0] == 11.f && y[5] == 16.f && exe->getOutputBlob(0)->size() == sizeof y);
+    auto times = exe->bench(true);
+    EXPECT(times.size() == 2 && times[0].first == "plus1" && times[1].first == "plus10");
+    // another allocator: the input that was set is carried over
+    exe->dispatch(findDevice("cpu", 0), "reuse");
+    exe->run();
+    std::fill(y, y + n, 0.f);
+    exe->getOutput(0, y, sizeof y);
+    EXPECT(y[0] == 11.f && y[5] == 16.f);
+    // trace: a meta file per node, every tensor as .npy with a parsable header and the right bytes
+    auto dir = std::filesystem::temp_directory_path() / ("rg_host_trace_" + std::to_string(::getpid()));
+    exe->trace(dir.string(), "npy");
+    auto meta = readFile(dir / "node000001.meta");
+    std::string metaText(meta.begin(), meta.end());
+    EXPECT(metaText.find("input\t0\tmid\t") != std::string::npos && metaText.find("output\t0\ty\t") != std::string::npos);
+    auto npy = readFile(dir / "data000003.npy");// node 0: x, mid; node 1: mid, y
+    EXPECT(npy.size() == 128 + sizeof y && std::memcmp(npy.data(), "\x93NUMPY\x01\x00", 8) == 0 && npy[127] == '\n');
+    std::string header(npy.begin() + 10, npy.begin() + 128);
+    EXPECT(header.find("'descr': '<f4'") != std::string::npos && header.find("'shape': (2,3,)") != std::string::npos);
+    EXPECT(std::memcmp(npy.data() + 128, y, sizeof y) == 0);
+    std::filesystem::remove_all(dir);
 }
 
 static void transposeInfoDigest() {
@@ -1322,6 +1404,65 @@ static void longChainRecorded() {
                 std::chrono::duration<double, std::micro>(t2 - t1).count() / 50);
 }
 
+static void executorOnGpu() {
+    using namespace python_ffi;
+    constexpr dim_t M = 64, K = 256, N = 256;
+    auto x = Tensor::share(DataType::F32, Shape{M, K});
+    auto xq = Tensor::share(DataType::U8, Shape{M, K});
+    auto scale = Tensor::share(DataType::F32, Shape{});
+    auto zp = Tensor::share(DataType::U8, Shape{});
+    auto [wBlob, wPtr] = kernel::Blob::share(K * N);
+    auto w = Tensor::share(DataType::I8, Shape{K, N}, LayoutType::Others, wBlob);
+    auto acc = Tensor::share(DataType::I32, Shape{M, N});
+    auto y = Tensor::share(DataType::F32, Shape{M, N});
+    std::mt19937 rng(5);
+    std::vector<int8_t> w_(K * N);
+    for (auto &v : w_) v = static_cast<int8_t>(rng());
+    std::memcpy(wPtr, w_.data(), w_.size());
+    std::vector<float> x_(M * K), out(M * N), ref(M * N);
+    std::normal_distribution<float> g(0.f, 1.f);
+    for (auto &v : x_) v = g(rng);
+    graph_topo::GraphTopo topo(1, 1);
+    topo.pushNode({0}, 0, 3);
+    topo.pushNode({1, 4, 3}, 1, 1);
+    topo.pushNode({5, 2}, 0, 1);
+    topo.setGlobalOutput(0, 6);
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
+    ops.push_back({std::make_unique<computation::MatMulInteger>(), "matmul"});
+    ops.push_back({std::make_unique<computation::DequantizeLinear>(), "dequantise"});
+    EXPECT(findDevice("amd", 0)->type() == Device::Type::Amd);
+    auto exe = compile(computation::Graph(std::move(topo), std::move(ops),
+                                          {{x, "x"}, {xq, "xq"}, {scale, "scale"}, {zp, "zp"}, {w, "W"}, {acc, "acc"}, {y, "y"}}),
+                       "hip", "flat");
+    exe->setInput(0, x_.data(), x_.size() * 4);
+    exe->run();
+    exe->getOutput(0, out.data(), out.size() * 4);// the blocking copy waits for the kernels
+    std::vector<uint8_t> q(M * K);
+    float s;
+    uint8_t z;
+    oracle_dynamic_quantize_linear(q.data(), &s, &z, x_.data(), x_.size());
+    std::vector<int32_t> accRef(M * N);
+    oracle_matmul_integer(accRef.data(), q.data(), w_.data(), &z, 0, 1, nullptr, 1, 1, 1, M, K, N, nullptr, nullptr, 1, 1, 8);
+    oracle_dequantize_linear(ref.data(), accRef.data(), &s, nullptr, 1, 1, M * N, ORACLE_I32, 1, 1);
+    EXPECT(std::memcmp(out.data(), ref.data(), out.size() * 4) == 0);
+    auto times = exe->bench(true);
+    EXPECT(times.size() == 2);// the dequantisation went into the product
+    auto dir = std::filesystem::temp_directory_path() / ("rg_host_trace_gpu_" + std::to_string(::getpid()));
+    exe->trace(dir.string(), "npy");
+    // node 1 reads xq, W, zp, scale and writes y: the fifth file of that node is y
+    auto meta = readFile(dir / "node000001.meta");
+    std::string metaText(meta.begin(), meta.end());
+    auto at = metaText.find("output\t0\ty\t");
+    EXPECT(at != std::string::npos);
+    if (at != std::string::npos) {
+        auto file = metaText.substr(at + 11, metaText.find('\n', at) - at - 11);
+        auto npy = readFile(file);
+        EXPECT(npy.size() == 128 + ref.size() * 4 && std::memcmp(npy.data() + 128, ref.data(), ref.size() * 4) == 0);
+    }
+    std::filesystem::remove_all(dir);
+}
+
 static void transposeHip() {
     runtime::Resources res;
     auto &dev = amd();
@@ -1466,6 +1607,7 @@ int main(int argc, char **argv) {
     RUN(graphTopoAndBuilder);
     RUN(offsetCalculatorPlan);
     RUN(allocatorsAndStreamOnCpu);
+    RUN(executorOnCpu);
     RUN(transposeInfoDigest);
     RUN(computationGraphLowers);
     if (mode == "gpu") {
@@ -1481,6 +1623,7 @@ int main(int argc, char **argv) {
         RUN(rotaryEmbeddingHip);
         RUN(transposeHip);
         RUN(quantisedLinearStream);
+        RUN(executorOnGpu);
         RUN(decodeAttentionStream);
         RUN(prefillAttentionStream);
         RUN(longChainRecorded);
