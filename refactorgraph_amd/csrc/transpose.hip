@@ -11,8 +11,10 @@
 // locate(g / (block / W)).  Blocks of 256 bytes and more (a head's row that keeps its place while
 // sequence and head dimensions swap) read whole cache lines too; when it is two neighbouring
 // dimensions that change places in front of such blocks, a workgroup takes 8 x 8 of them so that
-// both sides move in runs of 8 blocks (transpose_tiles).  Small blocks (the innermost dimension
-// itself moves) gather their input word by word: correct, not fast.
+// both sides move in runs of 8 blocks (transpose_tiles).  When the innermost dimension itself moves
+// and a block is one element, tiles of 64 x 64 (32 x 32 for 8- and 16-byte elements) go through LDS,
+// read in runs along the input's innermost dimension and written in runs along the output's
+// (transpose_tile2d).  Only blocks of several words that are smaller than 64 bytes still gather.
 // Divisions by the strides are multiplications by 2^64 / d rounded up (exact for 32-bit dividends).
 #include "common.hpp"
 
@@ -128,10 +130,97 @@ __global__ __launch_bounds__(256) void transpose_tiles(Word *__restrict__ y, con
     }
 }
 
+// The innermost dimension itself moves (blocks of one element): an LDS tile turns the gather into
+// two coalesced sides.  F is the dimension that is innermost in the input (input stride 1), L the one
+// that is innermost in the output; a workgroup reads a T x T tile in runs along F, writes it in runs
+// along L, and the other dimensions are peeled off the workgroup index.
+constexpr int kMaxOuter = kMaxDims - 2;
+struct Tile2dPlan {
+    uint32_t outer_dims;
+    uint32_t outer_extent[kMaxOuter], outer_si[kMaxOuter], outer_so[kMaxOuter];
+    uint32_t extent_f, extent_l;  // elements along F and L
+    uint32_t si_l, so_f;          // input stride of L, output stride of F (those of F resp. L are 1)
+    uint32_t tiles_f, tiles_l;
+};
+
+template <class Word, int T>
+__global__ __launch_bounds__(256) void transpose_tile2d(Word *__restrict__ y, const Word *__restrict__ x, const Tile2dPlan p) {
+    __shared__ Word tile[T][T + 1];
+    uint32_t b = blockIdx.x;
+    const uint32_t tl = b % p.tiles_l;
+    b /= p.tiles_l;
+    const uint32_t tf = b % p.tiles_f;
+    b /= p.tiles_f;
+    uint64_t in0 = 0, out0 = 0;
+    for (uint32_t d = 0; d < p.outer_dims; ++d) {
+        const uint32_t i = b % p.outer_extent[d];
+        b /= p.outer_extent[d];
+        in0 += static_cast<uint64_t>(i) * p.outer_si[d];
+        out0 += static_cast<uint64_t>(i) * p.outer_so[d];
+    }
+    const uint32_t f0 = tf * T, l0 = tl * T;
+    constexpr int ROWS_PER_PASS = 256 / T;
+    const uint32_t fast = threadIdx.x % T, slow = threadIdx.x / T;
+#pragma unroll
+    for (int j = 0; j < T / ROWS_PER_PASS; ++j) {
+        const uint32_t l = slow + ROWS_PER_PASS * j;
+        if (f0 + fast < p.extent_f && l0 + l < p.extent_l)
+            tile[l][fast] = x[in0 + static_cast<uint64_t>(l0 + l) * p.si_l + f0 + fast];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < T / ROWS_PER_PASS; ++j) {
+        const uint32_t f = slow + ROWS_PER_PASS * j;
+        if (f0 + f < p.extent_f && l0 + fast < p.extent_l)
+            y[out0 + static_cast<uint64_t>(f0 + f) * p.so_f + l0 + fast] = tile[fast][f];
+    }
+}
+
+// Fills the plan if the digest describes single-element blocks with an innermost input dimension that
+// is not the innermost output dimension; returns the grid size or 0.
+uint64_t plan_tile2d(Tile2dPlan &t, const uint32_t *stride_i, const uint32_t *stride_o, size_t dims, uint64_t block_count,
+                     uint32_t tile) {
+    if (dims < 2 || stride_o[dims - 1] != 1) return 0;
+    const size_t l = dims - 1;
+    size_t f = dims;
+    for (size_t d = 0; d + 1 < dims; ++d)
+        if (stride_i[d] == 1) f = d;
+    if (f == dims) return 0;
+    auto extent = [&](size_t d) { return static_cast<uint32_t>((d == 0 ? block_count : stride_o[d - 1]) / stride_o[d]); };
+    t = Tile2dPlan{};
+    t.extent_f = extent(f);
+    t.extent_l = extent(l);
+    t.si_l = stride_i[l];
+    t.so_f = stride_o[f];
+    t.tiles_f = (t.extent_f + tile - 1) / tile;
+    t.tiles_l = (t.extent_l + tile - 1) / tile;
+    uint64_t grid = static_cast<uint64_t>(t.tiles_f) * t.tiles_l;
+    for (size_t d = 0; d < dims; ++d) {
+        if (d == f || d == l) continue;
+        t.outer_extent[t.outer_dims] = extent(d);
+        t.outer_si[t.outer_dims] = stride_i[d];
+        t.outer_so[t.outer_dims] = stride_o[d];
+        grid *= t.outer_extent[t.outer_dims++];
+    }
+    return grid;
+}
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <class Word>
-int launch(void *y, const void *x, const Plan &p, uint64_t block_count, hipStream_t s) {
+int launch(void *y, const void *x, const Plan &p, const uint32_t *stride_i, const uint32_t *stride_o, uint64_t block_count,
+           hipStream_t s) {
+    // blocks of one element: through an LDS tile
+    if (p.words_per_block.d == 1) {
+        constexpr int T = sizeof(Word) <= 4 ? 64 : 32;
+        Tile2dPlan t;
+        const uint64_t grid = plan_tile2d(t, stride_i, stride_o, p.dims, block_count, T);
+        if (grid && grid <= 0x7fffffffull) {
+            transpose_tile2d<Word, T><<<static_cast<unsigned>(grid), 256, 0, s>>>(static_cast<Word *>(y),
+                                                                                 static_cast<const Word *>(x), t);
+            return launch_status();
+        }
+    }
     // two neighbouring dimensions change places in front of whole blocks of 64 bytes or more
     if (p.dims >= 2 && p.stride_i[p.dims - 2] == 1 && p.words_per_block.d * sizeof(Word) >= 64) {
         const uint32_t extent_s = p.stride_o[p.dims - 2].d;
@@ -191,10 +280,10 @@ extern "C" int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i
         p.stride_i[d] = stride_i[d];
     }
     switch (w) {
-        case 16: return launch<u32x4>(y, x, p, block_count, s);
-        case 8: return launch<uint64_t>(y, x, p, block_count, s);
-        case 4: return launch<uint32_t>(y, x, p, block_count, s);
-        case 2: return launch<uint16_t>(y, x, p, block_count, s);
-        default: return launch<uint8_t>(y, x, p, block_count, s);
+        case 16: return launch<u32x4>(y, x, p, stride_i, stride_o, block_count, s);
+        case 8: return launch<uint64_t>(y, x, p, stride_i, stride_o, block_count, s);
+        case 4: return launch<uint32_t>(y, x, p, stride_i, stride_o, block_count, s);
+        case 2: return launch<uint16_t>(y, x, p, stride_i, stride_o, block_count, s);
+        default: return launch<uint8_t>(y, x, p, stride_i, stride_o, block_count, s);
     }
 }

@@ -462,7 +462,8 @@ def test_transpose_driver_digest_equals_the_oracles():
     ((1, 3, 2, 5), (2, 3, 0, 1)),            # src/04kernel/test/kernels/transpose/test_cpu.cpp:9-15
     ((2, 3, 4, 5), (0, 1, 2, 3)), ((7,), (0,)), ((5, 9), (1, 0)), ((3, 5, 7), (2, 1, 0)), ((3, 5, 7), (1, 2, 0)),
     ((2, 48, 8, 128), (0, 2, 1, 3)), ((4, 6, 33, 17), (0, 2, 1, 3)), ((2, 3, 4, 5, 6), (4, 0, 3, 1, 2)),
-    ((2, 1, 3, 1, 4), (3, 2, 4, 1, 0)), ((64, 40, 24), (1, 0, 2)), ((129, 257), (1, 0))])
+    ((2, 1, 3, 1, 4), (3, 2, 4, 1, 0)), ((64, 40, 24), (1, 0, 2)), ((129, 257), (1, 0)),
+    ((3, 130, 70), (2, 0, 1)), ((3, 130, 70), (0, 2, 1)), ((2, 65, 3, 67), (3, 1, 2, 0))])
 @pytest.mark.parametrize("dt", [np.uint8, np.float16, np.float32, np.float64])
 def test_transpose_bit_exact(shape, perm, dt):
     x = np.random.default_rng(len(shape)).integers(0, 200, shape).astype(dt)
