@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
     // give each XCD a contiguous block of tiles (they then share A row-panels / B column-panels
     // in that XCD's L2); within it walk tiles in column-major groups of 4 rows to keep panels hot.
-    const uint32_t tiles_n = n / BN, tiles_m = m / BM, n_tiles = tiles_m * tiles_n;
+    const uint32_t tiles_n = (n + BN - 1) / BN, tiles_m = (m + BM - 1) / BM, n_tiles = tiles_m * tiles_n;
     uint32_t t = blockIdx.x;
     if (n_tiles % 8 == 0) t = (t % 8) * (n_tiles / 8) + t / 8;
     const uint32_t group = 4 * tiles_n;
@@ -251,10 +251,15 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     const uint32_t rows_here = tiles_m - g * 4 < 4 ? tiles_m - g * 4 : 4;
     const uint32_t tile_m = g * 4 + r % rows_here, tile_n = r / rows_here;
 
-    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m + static_cast<uint64_t>(tile_m) * BM) * k);
+    // m and n need not be multiples of the tile: the last tile of a row or column of tiles is moved back
+    // so that it ends with the matrix (m, n >= 256); the outputs it shares with its neighbour are
+    // computed twice, to the same values
+    const uint32_t tile_row0 = tile_m * BM + BM <= m ? tile_m * BM : m - BM;
+    const uint32_t tile_col0 = tile_n * BN + BN <= n ? tile_n * BN : n - BN;
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m + tile_row0) * k);
     const T *b_matrix = b + bm * static_cast<uint64_t>(k) * n;
     const uint8_t *B = reinterpret_cast<const uint8_t *>(
-        TRANS_B ? b_matrix + static_cast<uint64_t>(tile_n) * BN * k : b_matrix + static_cast<uint64_t>(tile_n) * BN);
+        TRANS_B ? b_matrix + static_cast<uint64_t>(tile_col0) * k : b_matrix + tile_col0);
 
     f16v acc[4][4];
 #pragma unroll
@@ -272,7 +277,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     // stores: neighbouring lanes first exchange two of their four rows, so that every lane writes
     // two adjacent columns (one dword) of two rows; chunk c of row r sits at chunk position c ^ (r & 15).
     const uint32_t wm = wave >> 1, wn = wave & 1;
-    const uint32_t row0 = tile_m * BM + wm * 128, col0 = tile_n * BN + wn * 128;
+    const uint32_t row0 = tile_row0 + wm * 128, col0 = tile_col0 + wn * 128;
     const T *C = static_cast<const T *>(bias.ptr);
     __syncthreads();  // every wavefront has read its last fragments
     uint8_t *stage = (wave & 2 ? lds1 : lds0) + (wave & 1) * 32768;
@@ -445,7 +450,11 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     typedef typename Acc<T>::type A_t;
     const A_t al = through<T>(alpha), be = bias.ptr ? through<T>(beta) : A_t(0);
     constexpr bool narrow = sizeof(T) == 2;
-    const bool fast = narrow && !trans_a && m % BM == 0 && n % BN == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
+    // rows of B as [k, n] and of Y start on 16-byte boundaries when n is a multiple of 8; tiles that are moved
+    // back overlap their neighbours, which a bias that is the output itself does not allow
+    const bool ragged = m % BM != 0 || n % BN != 0;
+    const bool fast = narrow && !trans_a && m >= BM && n >= BN && n % 8 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
+                      aligned16(b) && aligned16(y_) && !(ragged && bias.ptr == y_);
 
     // few rows, weights as [n, k]: stream W once per slab of 32 rows of A
     const bool skinny = narrow && !fast && !trans_a && trans_b && m <= 128 && n % 32 == 0 && k % SK_TK == 0 &&
@@ -465,7 +474,7 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
                 return 0;
             }
             if (fast) {
-                const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
+                const dim3 grid(static_cast<unsigned>(((m + BM - 1) / BM) * ((n + BN - 1) / BN)), 1, count);
                 if (trans_b)
                     mm_mfma_256x256<T, true><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
                                                                   static_cast<uint32_t>(n), al, be, am0, bm0, ym0);

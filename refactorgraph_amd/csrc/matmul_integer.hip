@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so
     // give each XCD a contiguous block of tiles (they then share A row-panels / B column-panels
     // in that XCD's L2); within it walk tiles in column-major groups of 4 rows to keep panels hot.
-    const uint32_t tiles_n = n / BN, tiles_m = m / BM, n_tiles = tiles_m * tiles_n;
+    const uint32_t tiles_n = (n + BN - 1) / BN, tiles_m = (m + BM - 1) / BM, n_tiles = tiles_m * tiles_n;
     uint32_t t = blockIdx.x;
     if (n_tiles % 8 == 0) t = (t % 8) * (n_tiles / 8) + t / 8;
     const uint32_t group = 4 * tiles_n;
@@ -264,8 +264,13 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     const uint32_t rows_here = tiles_m - g * 4 < 4 ? tiles_m - g * 4 : 4;
     const uint32_t tile_m = g * 4 + r % rows_here, tile_n = r / rows_here;
 
-    const uint8_t *A = a + (am * m + static_cast<uint64_t>(tile_m) * BM) * k;
-    const uint8_t *B = b + bm * static_cast<uint64_t>(k) * n + static_cast<uint64_t>(tile_n) * BN;
+    // m and n need not be multiples of the tile: the last tile of a row or column of tiles is moved back
+    // so that it ends with the matrix (m, n >= 256); the outputs it shares with its neighbour are
+    // computed twice, to the same values
+    const uint32_t row0 = tile_m * BM + BM <= m ? tile_m * BM : m - BM;
+    const uint32_t col0 = tile_n * BN + BN <= n ? tile_n * BN : n - BN;
+    const uint8_t *A = a + (am * m + row0) * k;
+    const uint8_t *B = b + bm * static_cast<uint64_t>(k) * n + col0;
 
     v16i acc[4][4];
 #pragma unroll
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
             a_simple = false;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                za_f[i] = splat(za.ptr[am * m + static_cast<uint64_t>(tile_m) * BM + wm * 128 + 32 * i + (lane & 31)]);
+                za_f[i] = splat(za.ptr[am * m + row0 + wm * 128 + 32 * i + (lane & 31)]);
         } else {
             const uint32_t z = za.ptr[0];
             if (z == 0 || z == 128) {
@@ -309,13 +314,12 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
         else mmi_tile_loop<1, true>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
     }
 
-    int32_t *Y = y + (ym * m + static_cast<uint64_t>(tile_m) * BM + wm * 128) * n +
-                 static_cast<uint64_t>(tile_n) * BN + wn * 128;
+    int32_t *Y = y + (ym * m + row0 + wm * 128) * n + col0 + wn * 128;
     float scale[4] = {};  // of this lane's four columns
     if constexpr (DEQ) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            scale[j] = dq.scale[dq.per_column ? tile_n * BN + wn * 128 + j * 32 + (lane & 31) : 0];
+            scale[j] = dq.scale[dq.per_column ? col0 + wn * 128 + j * 32 + (lane & 31) : 0];
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -349,11 +353,12 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     hipStream_t s = as_stream(stream);
     const ZeroPoint za{static_cast<const uint8_t *>(a_zp), (flags & RG_MMI_A_ZP_SCALAR) ? 0u : 1u};
     const ZeroPoint zb{static_cast<const uint8_t *>(b_zp), (flags & RG_MMI_B_ZP_SCALAR) ? 0u : 1u};
-    const bool fast = m % BM == 0 && n % BN == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
+    // B rows start on 16-byte boundaries when n is a multiple of 16
+    const bool fast = m >= BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if (fast) {
-            const dim3 grid(static_cast<unsigned>((m / BM) * (n / BN)), 1, count);
+            const dim3 grid(static_cast<unsigned>(((m + BM - 1) / BM) * ((n + BN - 1) / BN)), 1, count);
             mmi_mfma_256x256<DEQ><<<grid, 256, 0, s>>>(
                 y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
                 static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), am0, bm0, ym0);

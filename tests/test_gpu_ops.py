@@ -359,6 +359,22 @@ def test_matmul_integer_dequantize_large_sums_round_once():
     assert np.array_equal(y, acc.astype(np.float32) * scale[0])
 
 
+@pytest.mark.parametrize("m,k,n", [(300, 128, 256), (256, 128, 272), (700, 256, 1008), (513, 384, 528), (257, 128, 257)])
+def test_matmul_integer_ragged_rows_and_columns(m, k, n):
+    # m and n beyond 256 that are no multiples of the MFMA tile: the last tiles are moved back and overlap
+    # their neighbours ((257, 128, 257): n is no multiple of 16, the plain kernel takes it)
+    rng = np.random.default_rng(m * n)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    az = rng.integers(0, 256, (2 * m,), dtype=np.uint8)        # one per (batch, row)
+    bz = rng.integers(-128, 128, (2 * k,), dtype=np.int8)
+    ref = oracle.matmul_integer(a, b, az, bz, threads=8)
+    assert np.array_equal(host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz))), ref)
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale)))
+    assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
+
+
 def test_matmul_integer_extremes():
     a = np.zeros((256, 4096), np.uint8)
     b = np.full((4096, 256), -128, np.int8)
@@ -782,7 +798,9 @@ def test_matmul_generic_transposes_bias_broadcast(dt):
 
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 192, 512), (512, 128, 256)])
+# the last three: m and n that are no multiples of the 256 x 256 tile (last tiles moved back, overlapping)
+@pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 192, 512), (512, 128, 256), (300, 64, 256), (256, 128, 264),
+                                   (513, 192, 520)])
 def test_matmul_mfma_path_fp16_bf16(m, k, n, dt, tb):
     rng = np.random.default_rng(14)
     a = rng.standard_normal((2, m, k)).astype(np.float32)
