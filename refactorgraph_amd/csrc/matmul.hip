@@ -456,8 +456,8 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool fast = narrow && !trans_a && m >= BM && n >= BN && n % 8 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
                       aligned16(b) && aligned16(y_) && !(ragged && bias.ptr == y_);
 
-    // few rows, weights as [n, k]: stream W once per slab of 32 rows of A
-    const bool skinny = narrow && !fast && !trans_a && trans_b && m <= 128 && n % 32 == 0 && k % SK_TK == 0 &&
+    // fewer rows than a tile, weights as [n, k]: stream W once per slab of 32 rows of A
+    const bool skinny = narrow && !fast && !trans_a && trans_b && m < BM && n % 32 == 0 && k % SK_TK == 0 &&
                         aligned16(a) && aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {

@@ -854,9 +854,9 @@ def test_matmul_full_config_fp16():
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160)])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160), (200, 256, 96)])
 def test_matmul_few_rows_weight_streaming(m, k, n, dt):
-    # weights as [n, k] (trans_b), up to 128 rows of A: the kernel that reads W once per 32 rows
+    # weights as [n, k] (trans_b), fewer than 256 rows of A: the kernel that reads W once per 32 rows
     rng = np.random.default_rng(17)
     a = rng.standard_normal((2, m, k)).astype(np.float32)
     w = (rng.standard_normal((2, n, k)) * 0.1).astype(np.float32)
