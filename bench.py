@@ -397,7 +397,7 @@ def main():
         ops_out["transpose"] = e
         del xs, ys
 
-    if want("matmul_integer") or want("matmul_integer_dequantize"):
+    if want("matmul_integer") or want("matmul_integer_dequantize") or want("matmul_integer_few_rows"):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
         az = torch.tensor([128], device=dev, dtype=torch.uint8)
@@ -442,6 +442,15 @@ def main():
                 "workload": "MatMulInteger 4096^3 with DequantizeLinear (scale per column) in its epilogue -> f32",
                 "device_ms_per_launch": round(dms_f, 5), "timing": mode,
                 "two_operators_device_ms": round(dms_2, 5)}
+        if want("matmul_integer_few_rows"):
+            # the same weights against 32 rows of activations (a decode step of the quantised layer): bound by reading B
+            a32 = a[:32].contiguous()
+            y32 = torch.empty((32, 4096), device=dev, dtype=torch.int32)
+            wall, dms_s, mode = time_steps(torch, lambda i: ops.matmul_integer(a32, b, az, bz, out=y32), steps, warmup, 1)
+            e = hbm_entry(4096 * 4096 + 32 * 4096 + 32 * 4096 * 4, dms_s, "matmul_integer_few_rows")
+            e.update(workload="MatMulInteger u8 [32,4096] x i8 [4096,4096] -> i32, a_zp=128 b_zp=0 (zeroing launch included)",
+                     device_ms_per_launch=round(dms_s, 5), timing=mode)
+            ops_out["matmul_integer_few_rows"] = e
         del a, b, y
 
     if want("matmul"):

@@ -342,6 +342,117 @@ extern "C" size_t rg_hip_matmul_integer_workspace(size_t, size_t, size_t, size_t
 
 namespace rg {
 namespace {
+
+// ---------------------------------------------------------------- few rows of A (decode): weight streaming
+//
+// Y[m <= 32, n] for one slab of rows: bound by reading B ([k, n], the weights) once.  A workgroup
+// takes 256 columns and a few k-tiles of 128 (32 KiB of B each, coalesced 256-byte row pieces
+// through registers into LDS, rows padded by 16 bytes, the next tile's loads in flight while one is
+// multiplied), forms the MFMA operand with the transposing 64-bit LDS read as the big kernel
+// does, takes its A fragments (16 consecutive k of a row per lane) straight from global memory,
+// and adds its 32 x 256 partial sums to Y with integer atomics: the k-range of a column block is
+// spread over workgroups, and integer addition gives the same result in any order.  Y is zeroed
+// by a launch of its own before.  Zero points as in the big kernel.
+constexpr int SK_PITCH = 256 + 16;
+constexpr uint64_t kSkinnyWorkgroups = 256;  // per launch: one per CU (512 and 128 were measured: slower)
+
+__global__ __launch_bounds__(256) void mmi_zero(int32_t *__restrict__ y, uint64_t count) {
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<uint64_t>(gridDim.x) * 256)
+        y[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
+                                                  const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb, uint32_t rows,
+                                                  uint32_t m, uint32_t row_first, uint32_t k, uint32_t n, uint32_t tiles,
+                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(16) uint8_t tile[BK * SK_PITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5;
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t col0 = blockIdx.x * 256;
+    const uint32_t t_first = blockIdx.y * tiles, k_tiles = k / BK;
+    const uint32_t t_end = t_first + tiles < k_tiles ? t_first + tiles : k_tiles;
+    const uint8_t *B = b + bm * k * static_cast<uint64_t>(n) + col0;
+
+    // B tile: 128 k-rows of 256 bytes, 16 lanes per row, 16 rows per pass of the workgroup
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 w[8];
+    auto load_b = [&](uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t r = static_cast<uint64_t>(t) * BK + 16 * i + (tid >> 4);
+            w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(B + r * n + 16 * (tid & 15)));
+        }
+    };
+    // A fragments of the four k-steps of a tile: row lane % 32 of the slab (rows beyond it repeat the last one),
+    // k 32 ks + 16 h .. + 15
+    const uint32_t row = (lane & 31) < rows ? (lane & 31) : rows - 1;
+    const uint64_t a_row = am * m + row_first + row;
+    const uint32_t za_splat = za.ptr ? splat(za.per_row ? za.ptr[a_row] : za.ptr[0]) : 0;
+    const bool b_zp = zb.ptr != nullptr;
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    const uint32_t a16 = lane & 15;
+    v16i acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+
+    load_b(t_first);
+    for (uint32_t t = t_first; t < t_end; ++t) {
+        const uint32_t k0 = t * BK;
+        v4i fa[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) fa[ks] = *reinterpret_cast<const v4i *>(a + a_row * k + k0 + 32 * ks + 16 * h);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *reinterpret_cast<u32x4 *>(tile + (16 * i + (tid >> 4)) * SK_PITCH + 16 * (tid & 15)) = w[i];
+        __syncthreads();
+        if (t + 1 < t_end) load_b(t + 1);  // in flight while this tile is multiplied
+        if (za.ptr) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) fa[ks][e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(fa[ks][e]), za_splat));
+        }
+        // B fragment of column block j (32 columns) and k-step ks: column lane % 32, k 32 ks + 16 h .. + 15 in two
+        // transposing reads of 8 k each; lane a of a group of 16 addresses k-row a / 2, columns 8 (a % 2) .. + 7
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            uint32_t z[4] = {0, 0, 0, 0};
+            if (b_zp) {
+                if (zb.per_row) __builtin_memcpy(z, zb.ptr + bm * k + k0 + 32 * ks + 16 * h, 16);
+                else z[0] = z[1] = z[2] = z[3] = splat(zb.ptr[0]);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t cols = 64 * wave + 32 * j + 16 * ((lane >> 4) & 1);
+                const uint8_t *src = tile + (32 * ks + 16 * h + (a16 >> 1)) * SK_PITCH + cols + 8 * (a16 & 1);
+                const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(src));
+                const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(src + 8 * SK_PITCH));
+                v4i fb = {lo[0], lo[1], hi[0], hi[1]};
+                if (b_zp) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fb[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(fb[e]), z[e]));
+                }
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks], fb, acc[j], 0, 0, 0);
+            }
+        }
+        __syncthreads();  // the tile is rewritten
+    }
+    // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 h + e % 4
+    int32_t *Y = y + (ym * m + row_first) * n + col0 + 64 * wave;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t r = 8 * (e / 4) + 4 * h + (e % 4);
+            if (r < rows)
+                __hip_atomic_fetch_add(Y + static_cast<uint64_t>(r) * n + 32 * j + (lane & 31), acc[j][e], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        }
+}
+
 template <bool DEQ>
 int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const void *b_zp, unsigned flags,
                size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
@@ -356,7 +467,35 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     // B rows start on 16-byte boundaries when n is a multiple of 16
     const bool fast = m >= BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
 
+    // fewer rows than a tile: stream B once per slab of 32 rows (int32 output only)
+    const bool skinny = !DEQ && !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
+                        aligned16(b);
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if (skinny) {
+            const uint64_t outputs = static_cast<uint64_t>(count) * m * n;
+            uint64_t zero_grid = (outputs + 1023) / 1024;
+            mmi_zero<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(y + static_cast<uint64_t>(ym0) * m * n,
+                                                                                               outputs);
+            int rc = launch_status();
+            if (rc) return rc;
+            // k-tiles per workgroup: as few as keep about kSkinnyWorkgroups workgroups per launch (fewer atomics per
+            // output the more tiles a workgroup sums itself)
+            const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
+            uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(k_tiles) * (n / 256) * count + kSkinnyWorkgroups - 1) /
+                                                   kSkinnyWorkgroups);
+            tiles = tiles < 1 ? 1 : tiles > k_tiles ? k_tiles : tiles;
+            const unsigned splits = (k_tiles + tiles - 1) / tiles;
+            for (size_t r0 = 0; r0 < m; r0 += 32) {
+                const uint32_t rows = static_cast<uint32_t>(m - r0 < 32 ? m - r0 : 32);
+                mmi_skinny<<<dim3(static_cast<unsigned>(n / 256), splits, count), 256, 0, s>>>(
+                    y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, rows, static_cast<uint32_t>(m),
+                    static_cast<uint32_t>(r0), static_cast<uint32_t>(k), static_cast<uint32_t>(n), tiles, am0, bm0, ym0);
+                rc = launch_status();
+                if (rc) return rc;
+            }
+            return 0;
+        }
         if (fast) {
             const dim3 grid(static_cast<unsigned>(((m + BM - 1) / BM) * ((n + BN - 1) / BN)), 1, count);
             mmi_mfma_256x256<DEQ><<<grid, 256, 0, s>>>(

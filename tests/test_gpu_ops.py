@@ -375,6 +375,24 @@ def test_matmul_integer_ragged_rows_and_columns(m, k, n):
     assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 128, 256), (7, 1024, 512), (32, 4096, 4096), (33, 256, 256), (200, 384, 768)])
+def test_matmul_integer_few_rows_weight_streaming(m, k, n):
+    # fewer than 256 rows of A: B is streamed once per 32 rows, the k-tiles of a column block are added up with
+    # integer atomics (exact in any order); every zero-point form, equal and broadcast batches
+    rng = np.random.default_rng(m + k)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    for az, bz in [(None, None), (np.array([128], np.uint8), np.array([0], np.int8)),
+                   (rng.integers(0, 256, (1,), dtype=np.uint8), rng.integers(-128, 128, (1,), dtype=np.int8)),
+                   (rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (2 * k,), dtype=np.int8))]:
+        y = ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz))
+        assert np.array_equal(host(y), oracle.matmul_integer(a, b, az, bz, threads=8))
+    b1 = b[:1]
+    out = torch.full((2, m, n), 12345, dtype=torch.int32, device=DEV)          # the output is zeroed by the call itself
+    y = ops.matmul_integer(dev(a), dev(np.ascontiguousarray(b1)), out=out)
+    assert np.array_equal(host(y), oracle.matmul_integer(a, b1, None, None, threads=8))
+
+
 def test_matmul_integer_extremes():
     a = np.zeros((256, 4096), np.uint8)
     b = np.full((4096, 256), -128, np.int8)
