@@ -361,6 +361,13 @@ __global__ __launch_bounds__(256) void mmi_zero(int32_t *__restrict__ y, uint64_
         y[i] = 0;
 }
 
+// The dequantising form of the few-rows path: the int32 sums, complete in Y, become float(sum) * scale in place.
+__global__ __launch_bounds__(256) void mmi_dequantize_in_place(int32_t *__restrict__ y, Dequant dq, uint64_t rows, uint32_t n) {
+    const uint64_t count = rows * n;
+    for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<uint64_t>(gridDim.x) * 256)
+        y[i] = finish<true>(y[i], dq.scale[dq.per_column ? static_cast<uint32_t>(i % n) : 0]);
+}
+
 __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
                                                   const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb, uint32_t rows,
                                                   uint32_t m, uint32_t row_first, uint32_t k, uint32_t n, uint32_t tiles,
@@ -467,8 +474,8 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     // B rows start on 16-byte boundaries when n is a multiple of 16
     const bool fast = m >= BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
 
-    // fewer rows than a tile: stream B once per slab of 32 rows (int32 output only)
-    const bool skinny = !DEQ && !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
+    // fewer rows than a tile: stream B once per slab of 32 rows
+    const bool skinny = !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
                         aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
@@ -493,6 +500,11 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
                     static_cast<uint32_t>(r0), static_cast<uint32_t>(k), static_cast<uint32_t>(n), tiles, am0, bm0, ym0);
                 rc = launch_status();
                 if (rc) return rc;
+            }
+            if constexpr (DEQ) {
+                mmi_dequantize_in_place<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(
+                    y + static_cast<uint64_t>(ym0) * m * n, dq, static_cast<uint64_t>(count) * m, static_cast<uint32_t>(n));
+                return launch_status();
             }
             return 0;
         }

@@ -387,6 +387,9 @@ def test_matmul_integer_few_rows_weight_streaming(m, k, n):
                    (rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (2 * k,), dtype=np.int8))]:
         y = ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz))
         assert np.array_equal(host(y), oracle.matmul_integer(a, b, az, bz, threads=8))
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    yd = ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale))
+    assert np.array_equal(host(yd), oracle.dequantize_linear(oracle.matmul_integer(a, b, az, bz, threads=8), scale, None, axis=2))
     b1 = b[:1]
     out = torch.full((2, m, n), 12345, dtype=torch.int32, device=DEV)          # the output is zeroed by the call itself
     y = ops.matmul_integer(dev(a), dev(np.ascontiguousarray(b1)), out=out)
