@@ -48,6 +48,7 @@ MEASURED_TRAFFIC = {
     "matmul_few_rows": (2 * 17456 + 256) * 1024,
     "transpose": (2 * 65552 + 131217) * 1024,
     "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
+    "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
 }
 
 
