@@ -10,7 +10,7 @@ decode call (cache append + attention for the whole batch).  The same line carri
   roofline      the decode call against the 8 TB/s HBM peak,
   cpu_baseline  the CPU oracle (a C restatement of the reference's CPU kernels) timed on a
                 bounded sample of the same workload on this host,
-  ops           the other hot-path kernels at their BASELINE.json configs, each with its own
+  ops           the other hot-path kernels at their full-size configurations, each with its own
                 roofline entry (MatMulInteger against the 5.0 POP/s dense int8 MFMA peak).
 One GPU only: --gpus N with N > 1 exits with a message.
 """

@@ -79,7 +79,7 @@ def test_rms_norm_f64_and_halves():
 
 
 def test_rms_norm_full_config_in_place():
-    # BASELINE config [32,128,4096] fp32, checked on a row sample against the oracle and fully
+    # the full configuration [32,128,4096] fp32, checked on a row sample against the oracle and fully
     # through the invariant sum_j (y_j/w_j)^2 = D*ms/(ms+eps)
     rng = np.random.default_rng(1)
     x = rng.standard_normal((32, 128, 4096), dtype=np.float32)
