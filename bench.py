@@ -500,6 +500,23 @@ def main():
         ops_out["matmul_few_rows"] = e
         del a, ws, y
 
+    if want("matmul_one_row"):
+        # the projection of a single sequence's decode step: one row of activations (matrix-vector product)
+        nb = 10
+        a = torch.randn((1, 4096), device=dev).half()
+        ws = [(torch.randn((4096, 4096), device=dev) * 0.05).half() for _ in range(nb)]
+        y = torch.empty((1, 4096), device=dev, dtype=torch.float16)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, ws[i], trans_b=True, out=y), steps, warmup, nb)
+        e = hbm_entry((4096 * 4096 + 2 * 4096) * 2, dms, "matmul_one_row")
+        e.update(workload="MatMul fp16 [1,4096] x [4096,4096]^T (trans_b)", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            an, bn = a.cpu().numpy(), ws[0].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.matmul(an, bn, None, False, True, dtype="fp16"),
+                                        (4096 * 4096 + 2 * 4096) * 2, "the whole product")
+        ops_out["matmul_one_row"] = e
+        del a, ws, y
+
     if want("attention_prefill"):
         Np, seq = 32, 512
         q = torch.randn((Np, H, seq, D), device=dev).half()

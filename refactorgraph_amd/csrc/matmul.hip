@@ -440,6 +440,149 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
     }
 }
 
+// ---------------------------------------------------------------- one to four rows of A: matrix-vector products
+//
+// Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 4, FP16 / BF16.  A matrix core would spend
+// 32 rows of work on these few, so the products are formed by the vector ALUs instead and the
+// kernel is a plain stream over W: a wavefront owns R rows of W, a lane reads 16 bytes (8
+// elements) of each per step, GV_LOADS / R steps ahead, and multiplies them (two elements per
+// instruction, sums in FP32) with the matching 8 elements of every row of A, which the
+// workgroup keeps in LDS (consecutive lanes read consecutive 16 bytes).  The 64 partial sums
+// of a row meet in a butterfly of lane exchanges at the end.  The first loads of W are issued
+// before A is staged, so the copy of A costs no memory latency of its own.
+constexpr int GV_LOADS = 8;  // 128-bit loads in flight per lane
+
+// acc + w.x * a.x + w.y * a.y on a pair of 16-bit elements held in one register (v_dot2_f32_f16 / v_dot2_f32_bf16)
+template <class T> __device__ __forceinline__ float dot2(uint32_t w, uint32_t a, float acc);
+template <> __device__ __forceinline__ float dot2<__half>(uint32_t w, uint32_t a, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w), __builtin_bit_cast(h2, a), acc, false);
+}
+template <> __device__ __forceinline__ float dot2<__hip_bfloat16>(uint32_t w, uint32_t a, float acc) {
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, w), __builtin_bit_cast(b2, a), acc, false);
+}
+
+template <class T, int M, int R>
+__global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
+                                               Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                                               uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    constexpr int DEPTH = GV_LOADS / R;  // steps of loads in flight
+    extern __shared__ __align__(16) uint8_t gv_lds[];  // M rows of A, k elements each
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t chunks = k / 8;              // 16-byte pieces of a row
+    const uint32_t steps = (chunks + 63) / 64;  // a wavefront covers 64 pieces per step
+    const uint32_t row0 = (blockIdx.x * (blockDim.x / 64) + wave) * R;
+
+    const u32x4 *W[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const uint32_t row = row0 + j < n ? row0 + j : n - 1;  // rows beyond n repeat the last one and are not stored
+        W[j] = reinterpret_cast<const u32x4 *>(w + (bm * n + row) * static_cast<uint64_t>(k));
+    }
+    u32x4 buf[DEPTH][R];
+    auto load = [&](int slot, uint32_t step) {
+        const uint32_t c = step * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (c < chunks) buf[slot][j] = __builtin_nontemporal_load(W[j] + c);
+    };
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < steps) load(d, d);
+
+    // A into LDS while the first pieces of W are on their way; rows beyond m are zero
+    const u32x4 *A = reinterpret_cast<const u32x4 *>(a + am * m * static_cast<uint64_t>(k));
+    u32x4 *sa = reinterpret_cast<u32x4 *>(gv_lds);
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+        for (uint32_t c = tid; c < chunks; c += blockDim.x) {
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (i < m) v = A[static_cast<uint64_t>(i) * chunks + c];
+            sa[i * chunks + c] = v;
+        }
+    __syncthreads();
+
+    float acc[R][M];
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int i = 0; i < M; ++i) acc[j][i] = 0.f;
+
+    for (uint32_t s = 0; s < steps; s += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (s + d < steps) {
+                const uint32_t c = (s + d) * 64 + lane;
+                if (c < chunks) {
+#pragma unroll
+                    for (int i = 0; i < M; ++i) {
+                        const u32x4 av = sa[i * chunks + c];
+#pragma unroll
+                        for (int j = 0; j < R; ++j)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[j][i] = dot2<T>(buf[d][j][e], av[e], acc[j][i]);
+                    }
+                }
+                if (s + d + DEPTH < steps) load(d, s + d + DEPTH);
+            }
+        }
+    }
+
+    // every lane ends with all sums; lane j * M + i keeps and stores the one of (row j of W, row i of A)
+    float mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+#pragma unroll
+        for (int i = 0; i < M; ++i) {
+            float v = acc[j][i];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            if (lane == static_cast<uint32_t>(j * M + i)) mine = v;
+        }
+    if (lane < R * M) {
+        const uint32_t j = lane / M, i = lane % M, col = row0 + j;
+        if (col < n && i < m) {
+            float v = alpha * mine;
+            const T *C = static_cast<const T *>(bias.ptr);
+            if (C) v += beta * up(C[ym * bias.sb + i * bias.sm + col * bias.sn]);
+            y[(ym * m + i) * n + col] = down<T>(v);
+        }
+    }
+}
+
+constexpr size_t GV_LDS_LIMIT = 160 * 1024;
+
+template <class T, int M>
+int launch_gemv(T *y, const T *a, const T *w, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+    constexpr int R = 1;  // rows of W per wavefront: more of them share the reads of A from LDS, and measured slower
+    const size_t lds = static_cast<size_t>(M) * k * 2;
+    if (lds > 64 * 1024) {  // beyond the default limit a kernel has to be told once per device
+        static bool raised[64] = {};
+        int device = 0;
+        if (const hipError_t e = hipGetDevice(&device); e != hipSuccess) return static_cast<int>(e);
+        if (device < 0 || device >= 64) return RG_HIP_E_UNSUPPORTED;
+        if (!raised[device]) {
+            if (const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&mm_gemv<T, M, R>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                         static_cast<int>(GV_LDS_LIMIT));
+                e != hipSuccess)
+                return static_cast<int>(e);
+            raised[device] = true;
+        }
+    }
+    // the wavefronts of a workgroup share one copy of A: as many as still leave a workgroup for every CU
+    uint32_t waves = 16;
+    while (waves > 4 && static_cast<uint64_t>((n + waves * R - 1) / (waves * R)) * count < 256) waves /= 2;
+    const dim3 grid((n + waves * R - 1) / (waves * R), 1, count);
+    mm_gemv<T, M, R><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, alpha, beta, am0, bm0, ym0);
+    return launch_status();
+}
+
 template <class T>
 int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_a, int trans_b, float alpha, float beta,
                  size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
@@ -460,8 +603,22 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool skinny = narrow && !fast && !trans_a && trans_b && m < BM && n % 32 == 0 && k % SK_TK == 0 &&
                         aligned16(a) && aligned16(b);
 
+    // one to four rows: matrix-vector products on the vector ALUs, A (padded to 1, 2 or 4 rows) in LDS; from five
+    // rows on the matrix-core kernel below is as fast
+    const uint32_t gv_m = m <= 1 ? 1 : m <= 2 ? 2 : 4;
+    const bool gemv = narrow && !trans_a && trans_b && m <= 4 && k > 0 && k % 8 == 0 && gv_m * k * 2 <= GV_LDS_LIMIT &&
+                      aligned16(a) && aligned16(b);
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            if (gemv) {
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                switch (gv_m) {
+                    case 1: return launch_gemv<T, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                    case 2: return launch_gemv<T, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                    default: return launch_gemv<T, 4>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                }
+            }
             if (skinny) {
                 for (size_t r0 = 0; r0 < m; r0 += 32) {
                     const uint32_t rows = static_cast<uint32_t>(m - r0 < 32 ? m - r0 : 32);

@@ -896,3 +896,31 @@ def test_matmul_few_rows_weight_streaming(m, k, n, dt):
     want = ai.astype(np.int64) @ wi.astype(np.int64).T
     if np.max(np.abs(want)) < (2048 if name == "fp16" else 256):
         assert np.array_equal(f(ops.matmul(dev(ai).to(dt), dev(wi).to(dt), trans_b=True)), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 8, 1), (1, 4096, 4096), (2, 520, 37), (3, 1000, 250), (4, 4096, 1024), (4, 11008, 72),
+                                   (1, 32768, 16), (4, 20480, 24), (3, 20488, 8), (5, 2048, 33), (7, 1000, 130),
+                                   (8, 4096, 512), (6, 11008, 64)])
+def test_matmul_one_to_four_rows_matrix_vector(m, k, n, dt):
+    # weights as [n, k] (trans_b), at most four rows of A: products on the vector ALUs, W streamed once;
+    # k that is not a multiple of a wavefront's step (512), n that is not a multiple of a workgroup's rows,
+    # rows of A that need more than 64 KiB of LDS; five to eight rows (the matrix-core kernel) for comparison
+    rng = np.random.default_rng(29)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    w = (rng.standard_normal((2, n, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal((m, n)).astype(np.float32)
+    ad, wd, cd = (dev(t).to(dt) for t in (a, w, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(wd), to_oracle(cd), False, True, 0.5, -1.5, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    got = f(ops.matmul(ad, wd, cd, False, True, 0.5, -1.5))
+    _matmul_check(got, ref, 0.5 * _absprod(f(ad), f(wd), False, True), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    # exact on integer-valued operands, and the same answer as the row inside a taller product (another kernel)
+    ai = rng.integers(-2, 3, (m, k)).astype(np.float32)
+    wi = rng.integers(-2, 3, (n, k)).astype(np.float32)
+    want = ai.astype(np.int64) @ wi.astype(np.int64).T
+    if np.max(np.abs(want)) < (2048 if name == "fp16" else 256):
+        assert np.array_equal(f(ops.matmul(dev(ai).to(dt), dev(wi).to(dt), trans_b=True)), want.astype(np.float32))
