@@ -49,6 +49,8 @@ MEASURED_TRAFFIC = {
     "transpose": (2 * 65552 + 131217) * 1024,
     "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
+    "matmul_one_row": (2 * 16444 + 8) * 1024,
+    "matmul_integer_one_row": (2 * 8242 + 512 + 2 * 10 + 16) * 1024,
 }
 
 
@@ -398,7 +400,8 @@ def main():
         ops_out["transpose"] = e
         del xs, ys
 
-    if want("matmul_integer") or want("matmul_integer_dequantize") or want("matmul_integer_few_rows"):
+    if (want("matmul_integer") or want("matmul_integer_dequantize") or want("matmul_integer_few_rows")
+            or want("matmul_integer_one_row")):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
         az = torch.tensor([128], device=dev, dtype=torch.uint8)
@@ -452,6 +455,18 @@ def main():
             e.update(workload="MatMulInteger u8 [32,4096] x i8 [4096,4096] -> i32, a_zp=128 b_zp=0 (zeroing launch included)",
                      device_ms_per_launch=round(dms_s, 5), timing=mode)
             ops_out["matmul_integer_few_rows"] = e
+        if want("matmul_integer_one_row"):
+            # a single sequence's decode step (matrix-vector product); 20 weight matrices in turn: beyond the memory-side cache
+            nb = 20
+            a1 = a[:1].contiguous()
+            bs = [torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8) for _ in range(nb)]
+            y1 = torch.empty((1, 4096), device=dev, dtype=torch.int32)
+            wall, dms_s, mode = time_steps(torch, lambda i: ops.matmul_integer(a1, bs[i], az, bz, out=y1), steps, warmup, nb)
+            e = hbm_entry(4096 * 4096 + 4096 + 4096 * 4, dms_s, "matmul_integer_one_row")
+            e.update(workload="MatMulInteger u8 [1,4096] x i8 [4096,4096] -> i32, a_zp=128 b_zp=0 (zeroing launch included)",
+                     device_ms_per_launch=round(dms_s, 5), timing=mode)
+            ops_out["matmul_integer_one_row"] = e
+            del bs
         del a, b, y
 
     if want("matmul"):

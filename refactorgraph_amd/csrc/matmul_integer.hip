@@ -460,6 +460,166 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
         }
 }
 
+// ---------------------------------------------------------------- one to four rows of A: matrix-vector products
+//
+// Y[m <= 4, n]: the matrix cores would spend 32 rows of work on these few, so the products are
+// formed by v_dot4_i32_i8 on the vector ALUs and the kernel is a plain stream over B ([k, n]).
+// A workgroup takes a strip of 256 columns and a range of k; a lane owns 16 columns (one 128-bit
+// load per k-row) and, per step, four consecutive k-rows (lane / 16 picks which four of the step's
+// 16), GEMV_DEPTH steps of loads in flight.  The four rows are transposed inside the lane with byte
+// permutes, so that a register holds the four k of one column, which is the order of four
+// consecutive bytes of a row of A.  Zero points are subtracted from the bytes before (modulo 256,
+// as everywhere).  The 16 partial sums per column (4 wavefronts x 4 row groups) meet in LDS; the
+// k-ranges of different workgroups meet in Y by integer atomics, as in the few-rows kernel above,
+// unless one workgroup covers all of k: then Y is stored and needs no zeroing.
+constexpr uint64_t kGemvWorkgroups = 512;  // aimed at per launch
+constexpr int GEMV_DEPTH = 2;               // steps of loads in flight per wavefront
+
+template <int M>
+__global__ __launch_bounds__(256) void mmi_gemv(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
+                                                const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb, uint32_t m,
+                                                uint32_t k, uint32_t n, uint32_t steps_per_wave, uint32_t a_matrix0,
+                                                uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(16) int32_t part[16 * M * 256];  // [wavefront * 4 + row group][row of A][column of the strip]
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t tid = threadIdx.x, lane = tid & 63, g = lane >> 4, c = lane & 15;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t col0 = blockIdx.x * 256 + 16 * c;  // this lane's 16 columns
+    const bool live = col0 < n;
+    const uint32_t total_steps = k / 16, step0 = blockIdx.y * 4 * steps_per_wave;
+    const uint8_t *B = b + bm * k * static_cast<uint64_t>(n) + col0;
+    const uint8_t *A[M];
+    uint32_t za_splat[M];
+#pragma unroll
+    for (int i = 0; i < M; ++i) {
+        const uint64_t row = am * m + (static_cast<uint32_t>(i) < m ? i : m - 1);  // rows beyond m repeat the last one
+        A[i] = a + row * k;
+        za_splat[i] = za.ptr ? splat(za.per_row ? za.ptr[row] : za.ptr[0]) : 0;
+    }
+
+    int32_t acc[M][16];
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0;
+
+    // step s of this wavefront: k-rows 16 (step0 + 4 s + wave) .. + 15, this lane 4 g .. 4 g + 3 of them
+    // the four bytes of every row of A and of the zero points of B that go with the k-rows travel with them:
+    // loads return in the order issued, so one issued only when it is needed would wait for everything ahead of it
+    u32x4 buf[GEMV_DEPTH][4];
+    uint32_t a_quad[GEMV_DEPTH][M], z_quad[GEMV_DEPTH];
+    const uint8_t *Z = zb.ptr && zb.per_row ? zb.ptr + bm * k : nullptr;
+    auto load = [&](int slot, uint32_t step) {
+        const uint64_t kk = 16ull * step + 4 * g;
+        if (live) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                buf[slot][r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(B + (kk + r) * n));
+#pragma unroll
+            for (int i = 0; i < M; ++i) a_quad[slot][i] = *reinterpret_cast<const uint32_t *>(A[i] + kk);
+            if (Z) z_quad[slot] = *reinterpret_cast<const uint32_t *>(Z + kk);
+        }
+    };
+    const uint32_t z_all = zb.ptr && !zb.per_row ? splat(zb.ptr[0]) : 0;
+#pragma unroll
+    for (int d = 0; d < GEMV_DEPTH; ++d)
+        if (static_cast<uint32_t>(d) < steps_per_wave && step0 + 4 * d + wave < total_steps) load(d, step0 + 4 * d + wave);
+
+    for (uint32_t s = 0; s < steps_per_wave; s += GEMV_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < GEMV_DEPTH; ++d) {
+            const uint32_t step = step0 + 4 * (s + d) + wave;
+            if (s + d < steps_per_wave && step < total_steps) {
+                if (live) {
+                    uint32_t aq[M];  // bytes: A[i][kk .. kk + 3] minus the zero point
+#pragma unroll
+                    for (int i = 0; i < M; ++i) aq[i] = za.ptr ? sub_bytes(a_quad[d][i], za_splat[i]) : a_quad[d][i];
+                    u32x4 rows[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        rows[r] = buf[d][r];
+                        if (Z || z_all) {  // a zero point of zero changes nothing
+                            const uint32_t z = Z ? splat((z_quad[d] >> (8 * r)) & 0xffu) : z_all;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) rows[r][e] = sub_bytes(rows[r][e], z);
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        // 4 x 4 bytes (k-row r, column 4 e + j) -> register j holds the four k of column 4 e + j;
+                        // v_perm_b32 picks result bytes from {second operand: indices 0-3, first operand: 4-7}
+                        const uint32_t t_lo = __builtin_amdgcn_perm(rows[1][e], rows[0][e], 0x05010400u);
+                        const uint32_t t_hi = __builtin_amdgcn_perm(rows[1][e], rows[0][e], 0x07030602u);
+                        const uint32_t u_lo = __builtin_amdgcn_perm(rows[3][e], rows[2][e], 0x05010400u);
+                        const uint32_t u_hi = __builtin_amdgcn_perm(rows[3][e], rows[2][e], 0x07030602u);
+                        const uint32_t col[4] = {__builtin_amdgcn_perm(u_lo, t_lo, 0x05040100u),
+                                                 __builtin_amdgcn_perm(u_lo, t_lo, 0x07060302u),
+                                                 __builtin_amdgcn_perm(u_hi, t_hi, 0x05040100u),
+                                                 __builtin_amdgcn_perm(u_hi, t_hi, 0x07060302u)};
+#pragma unroll
+                        for (int i = 0; i < M; ++i)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                acc[i][4 * e + j] = __builtin_amdgcn_sdot4(static_cast<int>(aq[i]), static_cast<int>(col[j]),
+                                                                           acc[i][4 * e + j], false);
+                    }
+                }
+                const uint32_t next = step + 4 * GEMV_DEPTH;
+                if (s + d + GEMV_DEPTH < steps_per_wave && next < total_steps) load(d, next);
+            }
+        }
+    }
+
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < M; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const v4i v = {acc[i][4 * e], acc[i][4 * e + 1], acc[i][4 * e + 2], acc[i][4 * e + 3]};
+                *reinterpret_cast<v4i *>(part + ((wave * 4 + g) * M + i) * 256 + 16 * c + 4 * e) = v;
+            }
+    }
+    __syncthreads();
+    const uint32_t col = blockIdx.x * 256 + tid;
+    if (col < n) {
+#pragma unroll
+        for (int i = 0; i < M; ++i) {
+            if (static_cast<uint32_t>(i) < m) {
+                int32_t sum = 0;
+#pragma unroll
+                for (int p = 0; p < 16; ++p) sum += part[(p * M + i) * 256 + tid];
+                int32_t *dst = y + (ym * m + i) * n + col;
+                if (gridDim.y == 1) *dst = sum;
+                else __hip_atomic_fetch_add(dst, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+}
+
+template <int M>
+int launch_gemv(int32_t *y, const uint8_t *a, const uint8_t *b, ZeroPoint za, ZeroPoint zb, uint32_t m, uint32_t k, uint32_t n,
+                uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+    const uint32_t strips = (n + 255) / 256, total_steps = k / 16;
+    // steps per wavefront: as few as keep about kGemvWorkgroups workgroups (the more a workgroup sums itself,
+    // the fewer atomics per output)
+    uint64_t per_wave = static_cast<uint64_t>(total_steps) * strips * count / (4 * kGemvWorkgroups);
+    per_wave = per_wave < 1 ? 1 : per_wave;
+    const uint32_t splits = static_cast<uint32_t>((total_steps + 4 * per_wave - 1) / (4 * per_wave));
+    if (splits > 1) {
+        const uint64_t outputs = static_cast<uint64_t>(count) * m * n;
+        const uint64_t zero_grid = (outputs + 1023) / 1024;
+        mmi_zero<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(y + static_cast<uint64_t>(ym0) * m * n,
+                                                                                           outputs);
+        const int rc = launch_status();
+        if (rc) return rc;
+    }
+    mmi_gemv<M><<<dim3(strips, splits, count), 256, 0, s>>>(y, a, b, za, zb, m, k, n, static_cast<uint32_t>(per_wave), am0, bm0,
+                                                          ym0);
+    return launch_status();
+}
+
 template <bool DEQ>
 int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const void *b_zp, unsigned flags,
                size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
@@ -478,7 +638,27 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     const bool skinny = !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
                         aligned16(b);
 
+    // one to four rows: matrix-vector products on the vector ALUs
+    const bool gemv = m <= 4 && n % 16 == 0 && k % 16 == 0 && k > 0 && aligned16(b) && (reinterpret_cast<uintptr_t>(a) & 3u) == 0 &&
+                      (!zb.ptr || !zb.per_row || (reinterpret_cast<uintptr_t>(zb.ptr) & 3u) == 0);
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if (gemv) {
+            const auto *a8 = static_cast<const uint8_t *>(a);
+            const auto *b8 = static_cast<const uint8_t *>(b);
+            const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+            int rc = m <= 1   ? launch_gemv<1>(y, a8, b8, za, zb, m32, k32, n32, am0, bm0, ym0, count, s)
+                     : m <= 2 ? launch_gemv<2>(y, a8, b8, za, zb, m32, k32, n32, am0, bm0, ym0, count, s)
+                              : launch_gemv<4>(y, a8, b8, za, zb, m32, k32, n32, am0, bm0, ym0, count, s);
+            if (rc) return rc;
+            if constexpr (DEQ) {
+                const uint64_t outputs = static_cast<uint64_t>(count) * m * n, grid = (outputs + 1023) / 1024;
+                mmi_dequantize_in_place<<<static_cast<unsigned>(grid > 4096 ? 4096 : grid), 256, 0, s>>>(
+                    y + static_cast<uint64_t>(ym0) * m * n, dq, static_cast<uint64_t>(count) * m, static_cast<uint32_t>(n));
+                return launch_status();
+            }
+            return 0;
+        }
         if (skinny) {
             const uint64_t outputs = static_cast<uint64_t>(count) * m * n;
             uint64_t zero_grid = (outputs + 1023) / 1024;

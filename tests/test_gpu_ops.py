@@ -396,6 +396,33 @@ def test_matmul_integer_few_rows_weight_streaming(m, k, n):
     assert np.array_equal(host(y), oracle.matmul_integer(a, b1, None, None, threads=8))
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 16, 16), (1, 4096, 4096), (2, 48, 272), (3, 1008, 1040), (4, 4096, 1024), (4, 16384, 64),
+                                   (1, 80, 4112)])
+def test_matmul_integer_one_to_four_rows_matrix_vector(m, k, n):
+    # at most four rows of A: dot products of four bytes on the vector ALUs, B streamed once; k from one step of 16
+    # to many workgroups' ranges (added up with atomics), n that ends inside a strip of 256 columns; every zero-point
+    # form (wrap-around of the byte difference included: all byte values occur), equal and broadcast batches
+    rng = np.random.default_rng(3 * m + k)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    for az, bz in [(None, None), (np.array([128], np.uint8), np.array([0], np.int8)),
+                   (rng.integers(0, 256, (1,), dtype=np.uint8), rng.integers(-128, 128, (1,), dtype=np.int8)),
+                   (rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (2 * k,), dtype=np.int8))]:
+        y = ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz))
+        assert np.array_equal(host(y), oracle.matmul_integer(a, b, az, bz, threads=8))
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    yd = ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale))
+    assert np.array_equal(host(yd), oracle.dequantize_linear(oracle.matmul_integer(a, b, az, bz, threads=8), scale, None, axis=2))
+    b1 = b[:1]
+    out = torch.full((2, m, n), 12345, dtype=torch.int32, device=DEV)          # the output is zeroed by the call itself
+    y = ops.matmul_integer(dev(a), dev(np.ascontiguousarray(b1)), out=out)
+    assert np.array_equal(host(y), oracle.matmul_integer(a, b1, None, None, threads=8))
+    # extremes: every product (-128) * (-128), the largest sum this k can make
+    ae, be = np.zeros((m, k), np.uint8), np.full((k, n), -128, np.int8)
+    ye = host(ops.matmul_integer(dev(ae), dev(be), dev(np.array([128], np.uint8)), None))
+    assert np.all(ye == k * 16384)
+
+
 def test_matmul_integer_extremes():
     a = np.zeros((256, 4096), np.uint8)
     b = np.full((4096, 256), -128, np.int8)
