@@ -345,12 +345,12 @@ namespace {
 
 // ---------------------------------------------------------------- few rows of A (decode): weight streaming
 //
-// Y[m <= 32, n] for one slab of rows: bound by reading B ([k, n], the weights) once.  A workgroup
+// Y[m <= 128, n] for up to four slabs of 32 rows: bound by reading B ([k, n], the weights) once.  A workgroup
 // takes 256 columns and a few k-tiles of 128 (32 KiB of B each, coalesced 256-byte row pieces
 // through registers into LDS, rows padded by 16 bytes, the next tile's loads in flight while one is
 // multiplied), forms the MFMA operand with the transposing 64-bit LDS read as the big kernel
 // does, takes its A fragments (16 consecutive k of a row per lane) straight from global memory,
-// and adds its 32 x 256 partial sums to Y with integer atomics: the k-range of a column block is
+// and adds its partial sums (32 x 256 per slab) to Y with integer atomics: the k-range of a column block is
 // spread over workgroups, and integer addition gives the same result in any order.  Y is zeroed
 // by a launch of its own before.  Zero points as in the big kernel.
 constexpr int SK_PITCH = 256 + 16;
@@ -368,6 +368,7 @@ __global__ __launch_bounds__(256) void mmi_dequantize_in_place(int32_t *__restri
         y[i] = finish<true>(y[i], dq.scale[dq.per_column ? static_cast<uint32_t>(i % n) : 0]);
 }
 
+template <int SLABS>  // slabs of 32 rows of A that share one pass over B
 __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
                                                   const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb, uint32_t rows,
                                                   uint32_t m, uint32_t row_first, uint32_t k, uint32_t n, uint32_t tiles,
@@ -393,24 +394,34 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
     };
     // A fragments of the four k-steps of a tile: row lane % 32 of the slab (rows beyond it repeat the last one),
     // k 32 ks + 16 h .. + 15
-    const uint32_t row = (lane & 31) < rows ? (lane & 31) : rows - 1;
-    const uint64_t a_row = am * m + row_first + row;
-    const uint32_t za_splat = za.ptr ? splat(za.per_row ? za.ptr[a_row] : za.ptr[0]) : 0;
+    uint64_t a_row[SLABS];
+    uint32_t za_splat[SLABS];
+#pragma unroll
+    for (int sl = 0; sl < SLABS; ++sl) {
+        const uint32_t row = 32 * sl + (lane & 31) < rows ? 32 * sl + (lane & 31) : rows - 1;
+        a_row[sl] = am * m + row_first + row;
+        za_splat[sl] = za.ptr ? splat(za.per_row ? za.ptr[a_row[sl]] : za.ptr[0]) : 0;
+    }
     const bool b_zp = zb.ptr != nullptr;
     typedef int v2i __attribute__((ext_vector_type(2)));
     const uint32_t a16 = lane & 15;
-    v16i acc[2];
+    v16i acc[SLABS][2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int sl = 0; sl < SLABS; ++sl)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[sl][j][e] = 0;
 
     load_b(t_first);
     for (uint32_t t = t_first; t < t_end; ++t) {
         const uint32_t k0 = t * BK;
-        v4i fa[4];
+        v4i fa[SLABS][4];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) fa[ks] = *reinterpret_cast<const v4i *>(a + a_row * k + k0 + 32 * ks + 16 * h);
+        for (int sl = 0; sl < SLABS; ++sl)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+                fa[sl][ks] = *reinterpret_cast<const v4i *>(a + a_row[sl] * k + k0 + 32 * ks + 16 * h);
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             *reinterpret_cast<u32x4 *>(tile + (16 * i + (tid >> 4)) * SK_PITCH + 16 * (tid & 15)) = w[i];
@@ -418,9 +429,12 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
         if (t + 1 < t_end) load_b(t + 1);  // in flight while this tile is multiplied
         if (za.ptr) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
+            for (int sl = 0; sl < SLABS; ++sl)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) fa[ks][e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(fa[ks][e]), za_splat));
+                for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        fa[sl][ks][e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(fa[sl][ks][e]), za_splat[sl]));
         }
         // B fragment of column block j (32 columns) and k-step ks: column lane % 32, k 32 ks + 16 h .. + 15 in two
         // transposing reads of 8 k each; lane a of a group of 16 addresses k-row a / 2, columns 8 (a % 2) .. + 7
@@ -442,7 +456,9 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
 #pragma unroll
                     for (int e = 0; e < 4; ++e) fb[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(fb[e]), z[e]));
                 }
-                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks], fb, acc[j], 0, 0, 0);
+#pragma unroll
+                for (int sl = 0; sl < SLABS; ++sl)
+                    acc[sl][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[sl][ks], fb, acc[sl][j], 0, 0, 0);
             }
         }
         __syncthreads();  // the tile is rewritten
@@ -450,14 +466,16 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
     // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 h + e % 4
     int32_t *Y = y + (ym * m + row_first) * n + col0 + 64 * wave;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int sl = 0; sl < SLABS; ++sl)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const uint32_t r = 8 * (e / 4) + 4 * h + (e % 4);
-            if (r < rows)
-                __hip_atomic_fetch_add(Y + static_cast<uint64_t>(r) * n + 32 * j + (lane & 31), acc[j][e], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-        }
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t r = 32 * sl + 8 * (e / 4) + 4 * h + (e % 4);
+                if (r < rows)
+                    __hip_atomic_fetch_add(Y + static_cast<uint64_t>(r) * n + 32 * j + (lane & 31), acc[sl][j][e],
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
 }
 
 // ---------------------------------------------------------------- one to four rows of A: matrix-vector products
@@ -666,18 +684,25 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
                                                                                                outputs);
             int rc = launch_status();
             if (rc) return rc;
-            // k-tiles per workgroup: as few as keep about kSkinnyWorkgroups workgroups per launch (fewer atomics per
-            // output the more tiles a workgroup sums itself)
-            const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
-            uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(k_tiles) * (n / 256) * count + kSkinnyWorkgroups - 1) /
-                                                   kSkinnyWorkgroups);
-            tiles = tiles < 1 ? 1 : tiles > k_tiles ? k_tiles : tiles;
-            const unsigned splits = (k_tiles + tiles - 1) / tiles;
-            for (size_t r0 = 0; r0 < m; r0 += 32) {
-                const uint32_t rows = static_cast<uint32_t>(m - r0 < 32 ? m - r0 : 32);
-                mmi_skinny<<<dim3(static_cast<unsigned>(n / 256), splits, count), 256, 0, s>>>(
-                    y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, rows, static_cast<uint32_t>(m),
-                    static_cast<uint32_t>(r0), static_cast<uint32_t>(k), static_cast<uint32_t>(n), tiles, am0, bm0, ym0);
+            // up to four slabs of 32 rows share one pass over B
+            for (size_t r0 = 0; r0 < m; r0 += 128) {
+                const uint32_t rows = static_cast<uint32_t>(m - r0 < 128 ? m - r0 : 128);
+                // k-tiles per workgroup: as few as keep about kSkinnyWorkgroups workgroups per launch (fewer atomics per
+                // output the more tiles a workgroup sums itself; with two and four slabs half as many workgroups and
+                // twice as many were measured: both slower)
+                const uint64_t target = kSkinnyWorkgroups;
+                const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
+                uint32_t tiles = static_cast<uint32_t>((static_cast<uint64_t>(k_tiles) * (n / 256) * count + target - 1) / target);
+                tiles = tiles < 1 ? 1 : tiles > k_tiles ? k_tiles : tiles;
+                const unsigned splits = (k_tiles + tiles - 1) / tiles;
+                const dim3 grid(static_cast<unsigned>(n / 256), splits, count);
+                const auto *a8 = static_cast<const uint8_t *>(a);
+                const auto *b8 = static_cast<const uint8_t *>(b);
+                const uint32_t m32 = static_cast<uint32_t>(m), r32 = static_cast<uint32_t>(r0), k32 = static_cast<uint32_t>(k),
+                               n32 = static_cast<uint32_t>(n);
+                if (rows <= 32) mmi_skinny<1><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, rows, m32, r32, k32, n32, tiles, am0, bm0, ym0);
+                else if (rows <= 64) mmi_skinny<2><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, rows, m32, r32, k32, n32, tiles, am0, bm0, ym0);
+                else mmi_skinny<4><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, rows, m32, r32, k32, n32, tiles, am0, bm0, ym0);
                 rc = launch_status();
                 if (rc) return rc;
             }

@@ -375,7 +375,8 @@ def test_matmul_integer_ragged_rows_and_columns(m, k, n):
     assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 128, 256), (7, 1024, 512), (32, 4096, 4096), (33, 256, 256), (200, 384, 768)])
+@pytest.mark.parametrize("m,k,n", [(1, 128, 256), (7, 1024, 512), (32, 4096, 4096), (33, 256, 256), (64, 256, 256), (100, 384, 512),
+                                   (200, 384, 768), (255, 128, 256)])
 def test_matmul_integer_few_rows_weight_streaming(m, k, n):
     # fewer than 256 rows of A: B is streamed once per 32 rows, the k-tiles of a column block are added up with
     # integer atomics (exact in any order); every zero-point form, equal and broadcast batches
