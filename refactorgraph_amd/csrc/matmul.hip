@@ -447,7 +447,8 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
 // kernel is a plain stream over W: a wavefront owns R rows of W, a lane reads 16 bytes (8
 // elements) of each per step, GV_LOADS / R steps ahead, and multiplies them (two elements per
 // instruction, sums in FP32) with the matching 8 elements of every row of A, which the
-// workgroup keeps in LDS (consecutive lanes read consecutive 16 bytes).  The 64 partial sums
+// workgroup keeps in LDS (consecutive lanes read consecutive 16 bytes; at most 64 KiB, a longer k
+// is walked in segments).  The 64 partial sums
 // of a row meet in a butterfly of lane exchanges at the end.  The first loads of W are issued
 // before A is staged, so the copy of A costs no memory latency of its own.
 constexpr int GV_LOADS = 8;  // 128-bit loads in flight per lane
@@ -463,18 +464,17 @@ template <> __device__ __forceinline__ float dot2<__hip_bfloat16>(uint32_t w, ui
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, w), __builtin_bit_cast(b2, a), acc, false);
 }
 
-template <class T, int M, int R>
+template <class T, int M, int R, bool LONG>  // LONG: k in more than one segment
 __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
-                                               Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                                               uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+                                               Bias bias, uint32_t m, uint32_t k, uint32_t n, uint32_t segment, float alpha,
+                                               float beta, uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
     constexpr int DEPTH = GV_LOADS / R;  // steps of loads in flight
-    extern __shared__ __align__(16) uint8_t gv_lds[];  // M rows of A, k elements each
+    extern __shared__ __align__(16) uint8_t gv_lds[];  // M rows of A, one segment of k each
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
-    const uint32_t chunks = k / 8;              // 16-byte pieces of a row
-    const uint32_t steps = (chunks + 63) / 64;  // a wavefront covers 64 pieces per step
+    const uint32_t pieces = k / 8;  // 16-byte pieces of a row
     const uint32_t row0 = (blockIdx.x * (blockDim.x / 64) + wave) * R;
 
     const u32x4 *W[R];
@@ -483,54 +483,62 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
         const uint32_t row = row0 + j < n ? row0 + j : n - 1;  // rows beyond n repeat the last one and are not stored
         W[j] = reinterpret_cast<const u32x4 *>(w + (bm * n + row) * static_cast<uint64_t>(k));
     }
-    u32x4 buf[DEPTH][R];
-    auto load = [&](int slot, uint32_t step) {
-        const uint32_t c = step * 64 + lane;
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-            if (c < chunks) buf[slot][j] = __builtin_nontemporal_load(W[j] + c);
-    };
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d)
-        if (d < steps) load(d, d);
-
-    // A into LDS while the first pieces of W are on their way; rows beyond m are zero
     const u32x4 *A = reinterpret_cast<const u32x4 *>(a + am * m * static_cast<uint64_t>(k));
     u32x4 *sa = reinterpret_cast<u32x4 *>(gv_lds);
-#pragma unroll
-    for (int i = 0; i < M; ++i)
-        for (uint32_t c = tid; c < chunks; c += blockDim.x) {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (i < m) v = A[static_cast<uint64_t>(i) * chunks + c];
-            sa[i * chunks + c] = v;
-        }
-    __syncthreads();
-
     float acc[R][M];
 #pragma unroll
     for (int j = 0; j < R; ++j)
 #pragma unroll
         for (int i = 0; i < M; ++i) acc[j][i] = 0.f;
 
-    for (uint32_t s = 0; s < steps; s += DEPTH) {
+    // k in segments of which M rows of A fit into LDS (one segment unless k is very long; that case is compiled
+    // without the loop, which costs a fifth of the speed)
+    uint32_t p0 = 0;
+    do {
+        const uint32_t len = !LONG ? pieces : pieces - p0 < segment ? pieces - p0 : segment;
+        const uint32_t steps = (len + 63) / 64;  // a wavefront covers 64 pieces per step
+        u32x4 buf[DEPTH][R];
+        auto load = [&](int slot, uint32_t step) {
+            const uint32_t c = step * 64 + lane;
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            if (s + d < steps) {
-                const uint32_t c = (s + d) * 64 + lane;
-                if (c < chunks) {
+            for (int j = 0; j < R; ++j)
+                if (c < len) buf[slot][j] = __builtin_nontemporal_load(W[j] + p0 + c);
+        };
 #pragma unroll
-                    for (int i = 0; i < M; ++i) {
-                        const u32x4 av = sa[i * chunks + c];
+        for (int d = 0; d < DEPTH; ++d)
+            if (static_cast<uint32_t>(d) < steps) load(d, d);
+
+        // A into LDS while the first pieces of W are on their way; rows beyond m are zero
+        if (LONG && p0) __syncthreads();  // everybody has finished with the segment before
 #pragma unroll
-                        for (int j = 0; j < R; ++j)
+        for (int i = 0; i < M; ++i)
+            for (uint32_t c = tid; c < len; c += blockDim.x) {
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (static_cast<uint32_t>(i) < m) v = A[static_cast<uint64_t>(i) * pieces + p0 + c];
+                sa[i * len + c] = v;
+            }
+        __syncthreads();
+
+        for (uint32_t s = 0; s < steps; s += DEPTH) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) acc[j][i] = dot2<T>(buf[d][j][e], av[e], acc[j][i]);
+            for (int d = 0; d < DEPTH; ++d) {
+                if (s + d < steps) {
+                    const uint32_t c = (s + d) * 64 + lane;
+                    if (c < len) {
+#pragma unroll
+                        for (int i = 0; i < M; ++i) {
+                            const u32x4 av = sa[i * len + c];
+#pragma unroll
+                            for (int j = 0; j < R; ++j)
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[j][i] = dot2<T>(buf[d][j][e], av[e], acc[j][i]);
+                        }
                     }
+                    if (s + d + DEPTH < steps) load(d, s + d + DEPTH);
                 }
-                if (s + d + DEPTH < steps) load(d, s + d + DEPTH);
             }
         }
-    }
+    } while (LONG && (p0 += segment) < pieces);
 
     // every lane ends with all sums; lane j * M + i keeps and stores the one of (row j of W, row i of A)
     float mine = 0.f;
@@ -554,32 +562,21 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
     }
 }
 
-constexpr size_t GV_LDS_LIMIT = 160 * 1024;
+constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
 
 template <class T, int M>
 int launch_gemv(T *y, const T *a, const T *w, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
                 uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
     constexpr int R = 1;  // rows of W per wavefront: more of them share the reads of A from LDS, and measured slower
-    const size_t lds = static_cast<size_t>(M) * k * 2;
-    if (lds > 64 * 1024) {  // beyond the default limit a kernel has to be told once per device
-        static bool raised[64] = {};
-        int device = 0;
-        if (const hipError_t e = hipGetDevice(&device); e != hipSuccess) return static_cast<int>(e);
-        if (device < 0 || device >= 64) return RG_HIP_E_UNSUPPORTED;
-        if (!raised[device]) {
-            if (const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&mm_gemv<T, M, R>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                         static_cast<int>(GV_LDS_LIMIT));
-                e != hipSuccess)
-                return static_cast<int>(e);
-            raised[device] = true;
-        }
-    }
+    constexpr uint32_t segment_limit = GV_LDS_BYTES / (16 * M);  // 16-byte pieces of a row of A
+    const uint32_t segment = k / 8 < segment_limit ? k / 8 : segment_limit;
+    const size_t lds = static_cast<size_t>(M) * segment * 16;
     // the wavefronts of a workgroup share one copy of A: as many as still leave a workgroup for every CU
     uint32_t waves = 16;
     while (waves > 4 && static_cast<uint64_t>((n + waves * R - 1) / (waves * R)) * count < 256) waves /= 2;
     const dim3 grid((n + waves * R - 1) / (waves * R), 1, count);
-    mm_gemv<T, M, R><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, alpha, beta, am0, bm0, ym0);
+    if (segment == k / 8) mm_gemv<T, M, R, false><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, segment, alpha, beta, am0, bm0, ym0);
+    else mm_gemv<T, M, R, true><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, segment, alpha, beta, am0, bm0, ym0);
     return launch_status();
 }
 
@@ -606,8 +603,7 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     // one to four rows: matrix-vector products on the vector ALUs, A (padded to 1, 2 or 4 rows) in LDS; from five
     // rows on the matrix-core kernel below is as fast
     const uint32_t gv_m = m <= 1 ? 1 : m <= 2 ? 2 : 4;
-    const bool gemv = narrow && !trans_a && trans_b && m <= 4 && k > 0 && k % 8 == 0 && gv_m * k * 2 <= GV_LDS_LIMIT &&
-                      aligned16(a) && aligned16(b);
+    const bool gemv = narrow && !trans_a && trans_b && m <= 4 && k > 0 && k % 8 == 0 && aligned16(a) && aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {

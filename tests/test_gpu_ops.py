@@ -928,12 +928,13 @@ def test_matmul_few_rows_weight_streaming(m, k, n, dt):
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 8, 1), (1, 4096, 4096), (2, 520, 37), (3, 1000, 250), (4, 4096, 1024), (4, 11008, 72),
-                                   (1, 32768, 16), (4, 20480, 24), (3, 20488, 8), (5, 2048, 33), (7, 1000, 130),
+                                   (1, 32768, 16), (4, 20480, 24), (3, 20488, 8), (1, 40000, 8), (2, 33008, 5), (5, 2048, 33), (7, 1000, 130),
                                    (8, 4096, 512), (6, 11008, 64)])
 def test_matmul_one_to_four_rows_matrix_vector(m, k, n, dt):
     # weights as [n, k] (trans_b), at most four rows of A: products on the vector ALUs, W streamed once;
     # k that is not a multiple of a wavefront's step (512), n that is not a multiple of a workgroup's rows,
-    # rows of A that need more than 64 KiB of LDS; five to eight rows (the matrix-core kernel) for comparison
+    # rows of A longer than the 64 KiB of LDS a workgroup uses (k walked in segments, whole and ragged);
+    # five to eight rows (the matrix-core kernel) for comparison
     rng = np.random.default_rng(29)
     a = rng.standard_normal((2, m, k)).astype(np.float32)
     w = (rng.standard_normal((2, n, k)) * 0.1).astype(np.float32)
