@@ -124,16 +124,17 @@ __device__ __forceinline__ uint32_t b_swizzle(uint32_t x) { return ((x & 3) << 1
 
 template <int A_MODE, bool B_ZP>
 __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, uint8_t *lds1,
-                                              const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t n,
+                                              const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t lda, uint32_t n,
                                               uint32_t a_xor, const uint32_t (&za_f)[4], ZeroPoint zb,
                                               uint64_t zb_row0) {
+    // k: length of the range of k walked here (A, B and zb_row0 point at its start); lda: bytes per row of A
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
     // copy q < 8: A rows 8 (8 wave + q) .. + 7, this lane row + lane / 8, chunk position lane % 8;
     // copy 8 + p: B k-rows 4 (8 wave + p) .. + 3, this lane k-row + lane / 16, chunk position lane % 16
-    const uint8_t *a_wave = A + static_cast<uint64_t>(wave * 64) * k;
-    const uint32_t a_lane = (lane >> 3) * k + 16 * ((lane & 7) ^ (lane >> 3));
+    const uint8_t *a_wave = A + static_cast<uint64_t>(wave * 64) * lda;
+    const uint32_t a_lane = (lane >> 3) * lda + 16 * ((lane & 7) ^ (lane >> 3));
     const uint8_t *b_wave = B + static_cast<uint64_t>(wave * 32) * n;
     uint32_t b_lane[2];
 #pragma unroll
@@ -142,7 +143,7 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
         const uint8_t *src;
         uint8_t *dst;
         if (q < 8) {
-            src = a_wave + (k0 + 8 * q * k) + (a_lane ^ (16 * (q & 1)));
+            src = a_wave + (k0 + 8 * q * lda) + (a_lane ^ (16 * (q & 1)));
             dst = base + (wave * 8 + q) * 1024;
         } else {
             src = b_wave + static_cast<uint64_t>(k0 + 4 * (q - 8)) * n + b_lane[q & 1];
@@ -241,11 +242,14 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
 }
 
-template <bool DEQ>
+// SPLIT: blockIdx.y picks a range of `split_tiles` k-tiles and the sums are added to a zeroed Y with integer atomics
+// (exact in any order): for products with too few output tiles to occupy the chip.
+template <bool DEQ, bool SPLIT>
 __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
                                                            const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb,
-                                                           Dequant dq, uint32_t m, uint32_t k, uint32_t n,
+                                                           Dequant dq, uint32_t m, uint32_t k, uint32_t n, uint32_t split_tiles,
                                                            uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    static_assert(!(DEQ && SPLIT), "partial sums cannot be dequantised");
     __shared__ __align__(1024) uint8_t lds0[D_STAGE];
     __shared__ __align__(1024) uint8_t lds1[D_STAGE];
 
@@ -269,8 +273,13 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     // computed twice, to the same values
     const uint32_t row0 = tile_m * BM + BM <= m ? tile_m * BM : m - BM;
     const uint32_t col0 = tile_n * BN + BN <= n ? tile_n * BN : n - BN;
-    const uint8_t *A = a + (am * m + row0) * k;
-    const uint8_t *B = b + bm * static_cast<uint64_t>(k) * n + col0;
+    uint32_t k_begin = 0, k_len = k;
+    if constexpr (SPLIT) {
+        k_begin = blockIdx.y * split_tiles * BK;
+        k_len = k - k_begin < split_tiles * BK ? k - k_begin : split_tiles * BK;
+    }
+    const uint8_t *A = a + (am * m + row0) * k + k_begin;
+    const uint8_t *B = b + (bm * k + k_begin) * static_cast<uint64_t>(n) + col0;
 
     v16i acc[4][4];
 #pragma unroll
@@ -304,14 +313,14 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     }
     bool b_zp = zb.ptr != nullptr;
     if (b_zp && !zb.per_row && zb.ptr[0] == 0) b_zp = false;
-    const uint64_t zb_row0 = bm * k;
+    const uint64_t zb_row0 = bm * k + k_begin;
 
     if (a_simple) {
-        if (!b_zp) mmi_tile_loop<0, false>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
-        else mmi_tile_loop<0, true>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<0, false>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
+        else mmi_tile_loop<0, true>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
     } else {
-        if (!b_zp) mmi_tile_loop<1, false>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
-        else mmi_tile_loop<1, true>(acc, lds0, lds1, A, B, k, n, a_xor, za_f, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<1, false>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
+        else mmi_tile_loop<1, true>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
     }
 
     int32_t *Y = y + (ym * m + row0 + wm * 128) * n + col0 + wn * 128;
@@ -329,7 +338,11 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
             for (int e = 0; e < 16; ++e) {
                 const uint32_t row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
                 const uint32_t col = j * 32 + (lane & 31);
-                __builtin_nontemporal_store(finish<DEQ>(acc[i][j][e], scale[j]), Y + static_cast<uint64_t>(row) * n + col);
+                if constexpr (SPLIT)
+                    __hip_atomic_fetch_add(Y + static_cast<uint64_t>(row) * n + col, acc[i][j][e], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    __builtin_nontemporal_store(finish<DEQ>(acc[i][j][e], scale[j]), Y + static_cast<uint64_t>(row) * n + col);
             }
 }
 
@@ -354,6 +367,12 @@ namespace {
 // spread over workgroups, and integer addition gives the same result in any order.  Y is zeroed
 // by a launch of its own before.  Zero points as in the big kernel.
 constexpr int SK_PITCH = 256 + 16;
+// Splitting k between workgroups when there are few output tiles: up to kSplitMax ranges, as many as bring the
+// launch to about kSplitFill workgroups.  Every range adds one atomic per output, which costs about as much as
+// the idle CUs gain from 64 tiles on ([256,4096] x [4096,4096]: 49.6 us unsplit, 35 / 29 / 27 / 32 us with 2 / 3 /
+// 4 / 8 ranges; 512 rows: 49.6 unsplit, 37.5 / 35.7 / 37.3 / 53; 86 tiles in two ranges 58.6 against 49.3).
+constexpr uint64_t kSplitFill = 128;
+constexpr uint32_t kSplitMax = 4;
 constexpr uint64_t kSkinnyWorkgroups = 256;  // per launch: one per CU (512 and 128 were measured: slower)
 
 __global__ __launch_bounds__(256) void mmi_zero(int32_t *__restrict__ y, uint64_t count) {
@@ -714,10 +733,37 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
             return 0;
         }
         if (fast) {
-            const dim3 grid(static_cast<unsigned>(((m + BM - 1) / BM) * ((n + BN - 1) / BN)), 1, count);
-            mmi_mfma_256x256<DEQ><<<grid, 256, 0, s>>>(
+            const uint64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+            const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
+            // too few tiles for the chip: split k as well, up to kSplitMax ways with at least two k-tiles each
+            uint32_t splits = static_cast<uint32_t>(kSplitFill / (tiles * count));
+            splits = splits > kSplitMax ? kSplitMax : splits;
+            splits = splits > k_tiles / 2 ? k_tiles / 2 : splits;
+            if (m % BM != 0 || n % BN != 0) splits = 1;  // tiles moved back overlap: their outputs would be added twice
+            if (splits > 1) {
+                const uint32_t split_tiles = (k_tiles + splits - 1) / splits;
+                splits = (k_tiles + split_tiles - 1) / split_tiles;
+                const uint64_t outputs = static_cast<uint64_t>(count) * m * n, zero_grid = (outputs + 1023) / 1024;
+                int32_t *y0 = y + static_cast<uint64_t>(ym0) * m * n;
+                mmi_zero<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(y0, outputs);
+                int rc = launch_status();
+                if (rc) return rc;
+                mmi_mfma_256x256<false, true><<<dim3(static_cast<unsigned>(tiles), splits, count), 256, 0, s>>>(
+                    y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
+                    static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), split_tiles, am0, bm0, ym0);
+                rc = launch_status();
+                if (rc) return rc;
+                if constexpr (DEQ) {
+                    mmi_dequantize_in_place<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(
+                        y0, dq, static_cast<uint64_t>(count) * m, static_cast<uint32_t>(n));
+                    return launch_status();
+                }
+                return 0;
+            }
+            const dim3 grid(static_cast<unsigned>(tiles), 1, count);
+            mmi_mfma_256x256<DEQ, false><<<grid, 256, 0, s>>>(
                 y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
-                static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), am0, bm0, ym0);
+                static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), 0, am0, bm0, ym0);
         } else {
             const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
             mmi_generic<DEQ><<<grid, 256, 0, s>>>(

@@ -359,6 +359,26 @@ def test_matmul_integer_dequantize_large_sums_round_once():
     assert np.array_equal(y, acc.astype(np.float32) * scale[0])
 
 
+@pytest.mark.parametrize("m,k,n", [(256, 2048, 256), (1024, 1024, 512), (256, 640, 1024), (512, 4096, 256)])
+def test_matmul_integer_few_tiles_split_k(m, k, n):
+    # too few 256 x 256 tiles for the chip: ranges of k go to different workgroups and meet in a zeroed Y by
+    # integer atomics (exact in any order); every zero-point form, batches, the dequantising form
+    rng = np.random.default_rng(m + k + n)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    for az, bz in [(None, None), (np.array([128], np.uint8), np.array([0], np.int8)),
+                   (rng.integers(0, 256, (1,), dtype=np.uint8), rng.integers(-128, 128, (1,), dtype=np.int8)),
+                   (rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (2 * k,), dtype=np.int8))]:
+        out = torch.full((2, m, n), -7, dtype=torch.int32, device=DEV)         # the output is zeroed by the call itself
+        y = ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz), out=out)
+        assert np.array_equal(host(y), oracle.matmul_integer(a, b, az, bz, threads=8))
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    yd = ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale))
+    assert np.array_equal(host(yd), oracle.dequantize_linear(oracle.matmul_integer(a, b, az, bz, threads=8), scale, None, axis=2))
+    b1 = np.ascontiguousarray(b[:1])                                            # broadcast weights: one launch per matrix
+    assert np.array_equal(host(ops.matmul_integer(dev(a), dev(b1))), oracle.matmul_integer(a, b1, None, None, threads=8))
+
+
 @pytest.mark.parametrize("m,k,n", [(300, 128, 256), (256, 128, 272), (700, 256, 1008), (513, 384, 528), (257, 128, 257)])
 def test_matmul_integer_ragged_rows_and_columns(m, k, n):
     # m and n beyond 256 that are no multiples of the MFMA tile: the last tiles are moved back and overlap
