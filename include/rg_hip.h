@@ -179,7 +179,10 @@ int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i, const uin
  * a_index / b_index: HOST arrays [batch] giving the operand matrix used by each output batch
  * (the Broadcaster's locate(), src/04kernel/src/attributes/broadcaster.cc:87-100); NULL = i.
  * The zero points are fused into the tile loads: no workspace is needed and
- * rg_hip_matmul_integer_workspace() returns 0 (the reference needs m*k [+ k*n] bytes). */
+ * rg_hip_matmul_integer_workspace() returns 0 (the reference needs m*k [+ k*n] bytes).
+ * Integer sums are exact in any order, so every path (matrix cores on 256 x 256 tiles, with k split
+ * between workgroups when the tiles are few; weight streaming for fewer than 256 rows; vector-ALU dot
+ * products for one to four rows) returns the same bits. */
 enum {
     RG_MMI_A_ZP_SCALAR = 1u,
     RG_MMI_B_ZP_SCALAR = 2u,
@@ -194,8 +197,10 @@ int rg_hip_matmul_integer(int32_t *y, const void *a, const void *b,
  * i.e. the result of rg_hip_matmul_integer followed by the reference's DequantizeLinear without zero
  * point (src/04kernel/src/kernels/dequantize_linear/cpu_kernel.cc:17-28: one int -> float
  * conversion, one multiplication) on the last axis, bit for bit, without the int32 tensor ever
- * reaching memory.  No counterpart in the reference, which runs the two operators one after the
- * other.  scale: device pointer to one float, or to n floats when scale_per_column != 0. */
+ * reaching memory (with fewer than 256 rows, or few output tiles, partial sums of ranges of k meet in
+ * y itself as int32 and a finishing launch converts them in place: y is the only memory used).
+ * No counterpart in the reference, which runs the two operators one after the other.
+ * scale: device pointer to one float, or to n floats when scale_per_column != 0. */
 int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, const void *a_zp,
                                      const void *b_zp, unsigned flags, size_t batch, size_t m,
                                      size_t k, size_t n, const uint32_t *a_index,
