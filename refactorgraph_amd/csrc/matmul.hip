@@ -323,7 +323,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 
 // ---------------------------------------------------------------- few rows of A (decode): weight streaming
 //
-// Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 32, FP16 / BF16: bound by reading W once
+// Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 32 SLABS, FP16 / BF16: bound by reading W once
 // from HBM.  A workgroup owns 32 rows of W (32 columns of Y); its four wavefronts each take a
 // quarter of k.  A wavefront loads a 32 x 128 tile of W and the matching tile of A with coalesced
 // 128-bit loads (4 rows of 256 bytes per instruction: longer runs per row serve the DRAM pages
@@ -338,12 +338,13 @@ constexpr int SK_DEPTH = 2;   // tiles in flight per wavefront
 constexpr int SK_TK = 128;    // k elements per tile (256 bytes per row)
 constexpr int SK_LOADS = 8;   // 128-bit loads per lane and operand tile
 
-template <class T>
+template <class T, int SLABS>  // slabs of 32 rows of A that share one pass over W
 __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
                                                  Bias bias, uint32_t m, uint32_t m_total, uint32_t row_first,
                                                  uint32_t k, uint32_t n, float alpha, float beta, uint32_t a_matrix0,
                                                  uint32_t b_matrix0, uint32_t y_matrix0) {
-    __shared__ __align__(16) uint8_t lds[4 * 16384 + 4 * 32 * 33 * 4];
+    constexpr int WAVE_LDS = 8192 * (1 + SLABS);  // the tile of W and one tile of A per slab
+    __shared__ __align__(16) uint8_t lds[4 * WAVE_LDS + 4 * 32 * SLABS * 33 * 4];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bz = blockIdx.z;
@@ -362,43 +363,53 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
     // (their results are not stored)
     const uint32_t ld_row = lane >> 4, ld_chunk = lane & 15;
     const uint8_t *w_src = W + ld_row * pitch + 16 * ld_chunk;
-    uint32_t a_row[SK_LOADS];
+    uint32_t a_row[SLABS][SK_LOADS];
 #pragma unroll
-    for (int i = 0; i < SK_LOADS; ++i) a_row[i] = 4 * i + ld_row < m ? 4 * i + ld_row : m - 1;
+    for (int sl = 0; sl < SLABS; ++sl)
+#pragma unroll
+        for (int i = 0; i < SK_LOADS; ++i) a_row[sl][i] = 32 * sl + 4 * i + ld_row < m ? 32 * sl + 4 * i + ld_row : m - 1;
     struct Tile {
-        u32x4 w[SK_LOADS], a[SK_LOADS];
+        u32x4 w[SK_LOADS], a[SLABS][SK_LOADS];
     };
     auto load = [&](Tile &t, uint32_t kt) {
 #pragma unroll
         for (int i = 0; i < SK_LOADS; ++i)
             t.w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(w_src + 4 * i * pitch + kt * 256));
 #pragma unroll
-        for (int i = 0; i < SK_LOADS; ++i)
-            t.a[i] = *reinterpret_cast<const u32x4 *>(A + a_row[i] * pitch + 16 * ld_chunk + kt * 256);
+        for (int sl = 0; sl < SLABS; ++sl)
+#pragma unroll
+            for (int i = 0; i < SK_LOADS; ++i)
+                t.a[sl][i] = *reinterpret_cast<const u32x4 *>(A + a_row[sl][i] * pitch + 16 * ld_chunk + kt * 256);
     };
     // fragment of k-step ks: row lane % 32, chunk 2 ks + lane / 32
     const uint32_t r = lane & 31, h = lane >> 5;
     const uint32_t f_off = r * 256 + 16 * (h ^ (r & 15));
-    uint8_t *mine = lds + wave * 16384;
+    uint8_t *mine = lds + wave * WAVE_LDS;
 
-    f16v acc0, acc1;
+    f16v acc0[SLABS], acc1[SLABS];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc0[e] = acc1[e] = 0.f;
+    for (int sl = 0; sl < SLABS; ++sl)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc0[sl][e] = acc1[sl][e] = 0.f;
     auto multiply = [&](const Tile &t) {
 #pragma unroll
         for (int i = 0; i < SK_LOADS; ++i) {
             const uint32_t row = 4 * i + ld_row, off = row * 256 + 16 * (ld_chunk ^ (row & 15));
             *reinterpret_cast<u32x4 *>(mine + off) = t.w[i];
-            *reinterpret_cast<u32x4 *>(mine + 8192 + off) = t.a[i];
+#pragma unroll
+            for (int sl = 0; sl < SLABS; ++sl) *reinterpret_cast<u32x4 *>(mine + 8192 * (1 + sl) + off) = t.a[sl][i];
         }
 #pragma unroll
         for (int ks = 0; ks < SK_TK / 16; ks += 2) {
             const u32x4 w0 = *reinterpret_cast<const u32x4 *>(mine + (f_off ^ (32 * ks)));
-            const u32x4 a0 = *reinterpret_cast<const u32x4 *>(mine + 8192 + (f_off ^ (32 * ks)));
             const u32x4 w1 = *reinterpret_cast<const u32x4 *>(mine + (f_off ^ (32 * (ks + 1))));
-            const u32x4 a1 = *reinterpret_cast<const u32x4 *>(mine + 8192 + (f_off ^ (32 * (ks + 1))));
-            acc0 = Mfma<T>::run(w0, a0, acc0);
-            acc1 = Mfma<T>::run(w1, a1, acc1);
+#pragma unroll
+            for (int sl = 0; sl < SLABS; ++sl) {
+                const u32x4 a0 = *reinterpret_cast<const u32x4 *>(mine + 8192 * (1 + sl) + (f_off ^ (32 * ks)));
+                const u32x4 a1 = *reinterpret_cast<const u32x4 *>(mine + 8192 * (1 + sl) + (f_off ^ (32 * (ks + 1))));
+                acc0[sl] = Mfma<T>::run(w0, a0, acc0[sl]);
+                acc1[sl] = Mfma<T>::run(w1, a1, acc1[sl]);
+            }
         }
     };
 
@@ -417,21 +428,23 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
     }
 
     // partial sums: lane holds row (lane % 32) of A, register e column 8 (e/4) + 4 (lane/32) + e%4 of the block
-    float *part = reinterpret_cast<float *>(lds + 4 * 16384);  // [wave][row of A][column], pitch 33
+    float *part = reinterpret_cast<float *>(lds + 4 * WAVE_LDS);  // [wave][row of A][column], pitch 33
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        const uint32_t col = 8 * (e / 4) + 4 * h + (e % 4);
-        part[(wave * 32 + r) * 33 + col] = acc0[e] + acc1[e];
-    }
+    for (int sl = 0; sl < SLABS; ++sl)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t col = 8 * (e / 4) + 4 * h + (e % 4);
+            part[(wave * 32 * SLABS + 32 * sl + r) * 33 + col] = acc0[sl][e] + acc1[sl][e];
+        }
     __syncthreads();
     const T *C = static_cast<const T *>(bias.ptr);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < 4 * SLABS; ++q) {
         const uint32_t idx = tid + 256 * q, row = idx / 32, col = idx % 32;
         if (row < m) {
             float v = 0.f;
 #pragma unroll
-            for (int wv = 0; wv < 4; ++wv) v += part[(wv * 32 + row) * 33 + col];
+            for (int wv = 0; wv < 4; ++wv) v += part[(wv * 32 * SLABS + row) * 33 + col];
             v *= alpha;
             const uint64_t yrow = row_first + row;
             if (C) v += beta * up(C[ym * bias.sb + yrow * bias.sm + (n0 + col) * bias.sn]);
@@ -616,11 +629,16 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
                 }
             }
             if (skinny) {
-                for (size_t r0 = 0; r0 < m; r0 += 32) {
-                    const uint32_t rows = static_cast<uint32_t>(m - r0 < 32 ? m - r0 : 32);
-                    mm_skinny<T><<<dim3(static_cast<unsigned>(n / 32), 1, count), 256, 0, s>>>(
-                        y, a, b, bias, rows, static_cast<uint32_t>(m), static_cast<uint32_t>(r0), static_cast<uint32_t>(k),
-                        static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                // two slabs of 32 rows share one pass over W
+                for (size_t r0 = 0; r0 < m; r0 += 64) {
+                    const uint32_t rows = static_cast<uint32_t>(m - r0 < 64 ? m - r0 : 64);
+                    const dim3 grid(static_cast<unsigned>(n / 32), 1, count);
+                    if (rows <= 32)
+                        mm_skinny<T, 1><<<grid, 256, 0, s>>>(y, a, b, bias, rows, static_cast<uint32_t>(m), static_cast<uint32_t>(r0),
+                                                             static_cast<uint32_t>(k), static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                    else
+                        mm_skinny<T, 2><<<grid, 256, 0, s>>>(y, a, b, bias, rows, static_cast<uint32_t>(m), static_cast<uint32_t>(r0),
+                                                             static_cast<uint32_t>(k), static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
                     const int rc = launch_status();
                     if (rc) return rc;
                 }
