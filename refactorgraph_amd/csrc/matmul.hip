@@ -325,12 +325,12 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 //
 // Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 32 SLABS, FP16 / BF16: bound by reading W once
 // from HBM.  A workgroup owns 32 rows of W (32 columns of Y); its four wavefronts each take a
-// quarter of k.  A wavefront loads a 32 x 128 tile of W and the matching tile of A with coalesced
-// 128-bit loads (4 rows of 256 bytes per instruction: longer runs per row serve the DRAM pages
-// better than 128 bytes did) two tiles ahead into registers, passes a tile through its own
-// 16 KiB of LDS (chunk-swizzled rows) to bring it into MFMA operand layout, and
+// quarter of k.  A wavefront loads a 32 x 128 tile of W and the matching tile of A (one per slab of
+// 32 rows) with coalesced 128-bit loads (4 rows of 256 bytes per instruction: longer runs per row
+// serve the DRAM pages better than 128 bytes did) two tiles ahead into registers, passes a tile
+// through its own 8 KiB of LDS (chunk-swizzled rows) to bring it into MFMA operand layout, and
 // multiplies with v_mfma_f32_32x32x16 (W rows as the first operand, so a lane holds one row of A in
-// the result).  No barrier in the loop: a wavefront only reads what it wrote itself.  The four
+// the result; with two slabs the W fragments are read once for both).  No barrier in the loop: a wavefront only reads what it wrote itself.  The four
 // partial sums meet once at the end.  (Copying the tiles straight into LDS, as the big kernels
 // do, is slower here: that path moves about 24 bytes per clock and CU, a third of what plain
 // loads reach, and this kernel has nothing else to hide behind.)
