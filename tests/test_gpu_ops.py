@@ -947,6 +947,34 @@ def test_matmul_few_rows_weight_streaming(m, k, n, dt):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 8, 8), (1, 4096, 4096), (2, 520, 40), (3, 1000, 248), (4, 4096, 1024), (4, 11008, 72),
+                                   (1, 8200, 16), (2, 12288, 104)])
+def test_matmul_one_to_four_rows_weights_as_k_by_n(m, k, n, dt):
+    # B as [k, n] (not transposed), at most four rows of A: a workgroup walks all of k for a strip of columns
+    # (fixed order of summation, no atomics); k beyond one LDS segment of A (4096), k and n that end inside a
+    # workgroup's step and strip
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    w = (rng.standard_normal((2, k, n)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal((m, n)).astype(np.float32)
+    ad, wd, cd = (dev(t).to(dt) for t in (a, w, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(wd), to_oracle(cd), False, False, 0.5, -1.5, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    got = f(ops.matmul(ad, wd, cd, False, False, 0.5, -1.5))
+    _matmul_check(got, ref, 0.5 * _absprod(f(ad), f(wd), False, False), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    # exact on integer-valued operands; and the same call twice gives the same bits (fixed order of summation)
+    ai = rng.integers(-2, 3, (m, k)).astype(np.float32)
+    wi = rng.integers(-2, 3, (k, n)).astype(np.float32)
+    want = ai.astype(np.int64) @ wi.astype(np.int64)
+    if np.max(np.abs(want)) < (2048 if name == "fp16" else 256):
+        assert np.array_equal(f(ops.matmul(dev(ai).to(dt), dev(wi).to(dt))), want.astype(np.float32))
+    assert torch.equal(ops.matmul(ad, wd, cd, False, False, 0.5, -1.5), ops.matmul(ad, wd, cd, False, False, 0.5, -1.5))
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 8, 1), (1, 4096, 4096), (2, 520, 37), (3, 1000, 250), (4, 4096, 1024), (4, 11008, 72),
                                    (1, 32768, 16), (4, 20480, 24), (3, 20488, 8), (1, 40000, 8), (2, 33008, 5), (5, 2048, 33), (7, 1000, 130),
                                    (8, 4096, 512), (6, 11008, 64)])
