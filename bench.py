@@ -51,6 +51,8 @@ MEASURED_TRAFFIC = {
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
     "matmul_one_row": (2 * 16444 + 8) * 1024,
     "matmul_integer_one_row": (2 * 8242 + 512 + 2 * 10 + 16) * 1024,
+    "matmul_one_row_kn": (2 * 16460 + 8) * 1024,
+    "matmul_four_rows_kn": (2 * 16565 + 32) * 1024,
 }
 
 
@@ -530,6 +532,26 @@ def main():
             e["cpu_baseline"] = cpu_leg(lambda: oracle.matmul(an, bn, None, False, True, dtype="fp16"),
                                         (4096 * 4096 + 2 * 4096) * 2, "the whole product")
         ops_out["matmul_one_row"] = e
+        del a, ws, y
+
+    for name, rows in (("matmul_one_row_kn", 1), ("matmul_four_rows_kn", 4)):
+        if not want(name):
+            continue
+        # the same decode projections with the weights as ONNX MatMul keeps them, [k, n]
+        nb = 10
+        a = torch.randn((rows, 4096), device=dev).half()
+        ws = [(torch.randn((4096, 4096), device=dev) * 0.05).half() for _ in range(nb)]
+        y = torch.empty((rows, 4096), device=dev, dtype=torch.float16)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, ws[i], out=y), steps, warmup, nb)
+        e = hbm_entry((4096 * 4096 + 2 * rows * 4096) * 2, dms, name)
+        e.update(workload=f"MatMul fp16 [{rows},4096] x [4096,4096] (weights as [k,n])", device_ms_per_launch=round(dms, 5),
+                 timing=mode)
+        if not args.no_cpu:
+            import oracle
+            an, bn = a.cpu().numpy(), ws[0].cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.matmul(an, bn, None, False, False, dtype="fp16"),
+                                        (4096 * 4096 + 2 * rows * 4096) * 2, "the whole product")
+        ops_out[name] = e
         del a, ws, y
 
     if want("attention_prefill"):

@@ -582,12 +582,12 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
 // k-row) and L lanes cover a strip of 8 L columns; the 64 / L lane groups of a wavefront and the 16
 // wavefronts of a workgroup take different k-rows, 8 loads per lane in flight.  A workgroup walks
 // all of k for its strip, so the sums need no atomics and no workspace and come out in a fixed
-// order: FP32 FMAs per lane, a butterfly over the lane groups, then the 16 wavefronts' sums added in
-// order through LDS.  A (4096 k at a time) sits in LDS as it is in memory.  With n / (8 L)
-// workgroups this does not fill the chip for n = 4096 (L = 4: 128 workgroups reading 64-byte row
-// pieces), but it is some twenty times faster than the plain tiled kernel these shapes used to take.
+// order: FP32 FMAs per lane, an exchange between the lane groups, then the 16 wavefronts' sums added
+// in order through LDS.  A (4096 k at a time) sits in LDS as it is in memory.  Strips narrower than
+// a 128-byte line (L < 8) share lines with their neighbours: workgroups are dealt to the eight XCDs
+// in turn, so the strips are numbered such that neighbours run on the same XCD at the same time and
+// the second one finds the line in that XCD's L2.
 constexpr int KN_SEG = 4096;  // k per segment of A in LDS
-constexpr int KN_LANES = 4;   // lanes across a strip (8 columns each)
 constexpr int KN_DEPTH = 8;   // loads in flight per lane
 
 template <class T> __device__ __forceinline__ void widen8(const u32x4 &c, float (&f)[8]);
@@ -621,7 +621,9 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
-    const uint32_t col0 = blockIdx.x * SW + 8 * c;  // this lane's 8 columns
+    uint32_t strip = blockIdx.x;
+    if (gridDim.x % 8 == 0) strip = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const uint32_t col0 = strip * SW + 8 * c;  // this lane's 8 columns
     const bool live = col0 < n;
     const T *B = b + bm * k * static_cast<uint64_t>(n) + col0;
     const T *A = a + am * m * static_cast<uint64_t>(k);
@@ -636,6 +638,16 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
         const uint32_t len = k - k0 < KN_SEG ? k - k0 : KN_SEG;
         const uint32_t steps = (len + 16 * G - 1) / (16 * G);  // the workgroup covers 16 G k-rows per step
         // step s: this lane reads k-row k0 + (16 s + wave) G + g
+        // A first (the loads return in order, so the wait for A leaves the loads of B in flight): the two
+        // halves of the workgroup take rows 0, 2 and 1, 3, a thread 16 bytes of each of its rows
+        constexpr int ROWS = (M + 1) / 2;
+        const uint32_t ap = 8 * (tid & 511), ai = tid >> 9;
+        u32x4 av[ROWS];
+#pragma unroll
+        for (int j = 0; j < ROWS; ++j) {
+            av[j] = u32x4{0u, 0u, 0u, 0u};  // rows beyond m are zero
+            if (2 * j + ai < m && ap < len) av[j] = *reinterpret_cast<const u32x4 *>(A + static_cast<uint64_t>(2 * j + ai) * k + k0 + ap);
+        }
         u32x4 buf[KN_DEPTH];
         auto load = [&](int slot, uint32_t step) {
             const uint32_t r = (16 * step + wave) * G + g;
@@ -647,12 +659,8 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
 
         if (k0) __syncthreads();  // everybody has finished with the segment before
 #pragma unroll
-        for (int i = 0; i < M; ++i)
-            for (uint32_t p = tid; p < len / 8; p += 1024) {
-                u32x4 v = {0u, 0u, 0u, 0u};  // rows beyond m are zero
-                if (static_cast<uint32_t>(i) < m) v = *reinterpret_cast<const u32x4 *>(A + static_cast<uint64_t>(i) * k + k0 + 8 * p);
-                *reinterpret_cast<u32x4 *>(&sa[i][8 * p]) = v;
-            }
+        for (int j = 0; j < ROWS; ++j)
+            if (2 * j + ai < M && ap < len) *reinterpret_cast<u32x4 *>(&sa[2 * j + ai][ap]) = av[j];
         __syncthreads();
 
         for (uint32_t s = 0; s < steps; s += KN_DEPTH) {
@@ -676,26 +684,45 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
         }
     }
 
-    // the lane groups of a wavefront (lane bits from L up), then the wavefronts in order
+    // The lane groups of a wavefront (lane bits from L up), then the wavefronts in order.  While a lane
+    // still holds more than one sum, a stage halves them: the lane keeps the lower or the upper half (by its
+    // lane bit) and gets the partner's share of that half, so V sums cost about V exchanges, not V log2 G;
+    // from one sum per lane on, both partners add and hold the same.
+    constexpr int V = M * 8;
+    float *v = &acc[0][0];
+    uint32_t first = 0, twin = 0;  // the lane ends with sums first .. ; twin != 0: another lane writes them
 #pragma unroll
-    for (int i = 0; i < M; ++i)
+    for (int t = 0; (L << t) < 64; ++t) {
+        const int off = L << t;
+        const int nv = (V >> t) > 1 ? (V >> t) : 1;
+        if (nv > 1) {
+            const int half = nv / 2;
+            const bool hi = lane & off;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float v = acc[i][e];
-#pragma unroll
-            for (int off = L; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
-            acc[i][e] = v;
+            for (int j = 0; j < half; ++j) {
+                const float keep = hi ? v[j + half] : v[j];
+                const float send = hi ? v[j] : v[j + half];
+                v[j] = keep + __shfl_xor(send, off, 64);
+            }
+            if (hi) first += half;
+        } else {
+            v[0] += __shfl_xor(v[0], off, 64);
+            twin |= lane & off;
         }
+    }
+    constexpr int STAGES = __builtin_ctz(64 / L);
+    constexpr int LEFT = (V >> STAGES) > 1 ? (V >> STAGES) : 1;  // sums a lane holds at the end
     __syncthreads();  // A is no longer read
-    if (g == 0) {
+    if (!twin) {
 #pragma unroll
-        for (int i = 0; i < M; ++i)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) part[(wave * M + i) * SW + 8 * c + e] = acc[i][e];
+        for (int j = 0; j < LEFT; ++j) {
+            const uint32_t f = first + j;  // sum f: row f / 8 of A, column f % 8 of the lane's eight
+            part[(wave * M + f / 8) * SW + 8 * c + f % 8] = v[j];
+        }
     }
     __syncthreads();
     for (uint32_t t = tid; t < M * SW; t += 1024) {
-        const uint32_t i = t / SW, cc = t % SW, col = blockIdx.x * SW + cc;
+        const uint32_t i = t / SW, cc = t % SW, col = strip * SW + cc;
         if (i < m && col < n) {
             float v = 0.f;
 #pragma unroll
@@ -708,13 +735,24 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
     }
 }
 
-template <class T, int M>
-int launch_gemv_kn(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                   uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
-    constexpr int L = KN_LANES;
+template <class T, int M, int L>
+int launch_gemv_kn_l(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                     uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
     const dim3 grid((n + 8 * L - 1) / (8 * L), 1, count);
     mm_gemv_kn<T, M, L><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0);
     return launch_status();
+}
+
+// The widest strip (8, 4 or 2 lanes of 8 columns) that still gives some 160 workgroups: a wide strip reads
+// whole 128-byte lines and has fewer lane groups to add up, but one workgroup per CU keeps only so many
+// bytes in flight, so the chip has to be covered first.
+template <class T, int M>
+int launch_gemv_kn(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                   uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+    auto groups = [&](uint32_t lanes) { return static_cast<uint64_t>((n + 8 * lanes - 1) / (8 * lanes)) * count; };
+    if (groups(8) >= 160) return launch_gemv_kn_l<T, M, 8>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
+    if (groups(4) >= 160) return launch_gemv_kn_l<T, M, 4>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
+    return launch_gemv_kn_l<T, M, 2>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
 }
 
 constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
