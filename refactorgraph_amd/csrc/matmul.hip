@@ -611,7 +611,9 @@ template <> __device__ __forceinline__ void widen8<__hip_bfloat16>(const u32x4 &
 template <class T, int M, int L>
 __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b,
                                                   Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0, uint32_t row0,
+                                                  uint32_t rows) {
+    // rows row0 .. row0 + rows - 1 (rows <= M) of each m-row matrix
     constexpr int G = 64 / L, SW = 8 * L;  // lane groups per wavefront, columns per strip
     constexpr int A_BYTES = M * KN_SEG * 2, P_BYTES = 16 * M * SW * 4;
     __shared__ __align__(16) uint8_t lds[A_BYTES > P_BYTES ? A_BYTES : P_BYTES];
@@ -626,7 +628,7 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
     const uint32_t col0 = strip * SW + 8 * c;  // this lane's 8 columns
     const bool live = col0 < n;
     const T *B = b + bm * k * static_cast<uint64_t>(n) + col0;
-    const T *A = a + am * m * static_cast<uint64_t>(k);
+    const T *A = a + (am * m + row0) * static_cast<uint64_t>(k);
 
     float acc[M][8];
 #pragma unroll
@@ -645,8 +647,8 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
         u32x4 av[ROWS];
 #pragma unroll
         for (int j = 0; j < ROWS; ++j) {
-            av[j] = u32x4{0u, 0u, 0u, 0u};  // rows beyond m are zero
-            if (2 * j + ai < m && ap < len) av[j] = *reinterpret_cast<const u32x4 *>(A + static_cast<uint64_t>(2 * j + ai) * k + k0 + ap);
+            av[j] = u32x4{0u, 0u, 0u, 0u};  // rows beyond the last are zero
+            if (2 * j + ai < rows && ap < len) av[j] = *reinterpret_cast<const u32x4 *>(A + static_cast<uint64_t>(2 * j + ai) * k + k0 + ap);
         }
         u32x4 buf[KN_DEPTH];
         auto load = [&](int slot, uint32_t step) {
@@ -723,23 +725,23 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
     __syncthreads();
     for (uint32_t t = tid; t < M * SW; t += 1024) {
         const uint32_t i = t / SW, cc = t % SW, col = strip * SW + cc;
-        if (i < m && col < n) {
+        if (i < rows && col < n) {
             float v = 0.f;
 #pragma unroll
             for (int wv = 0; wv < 16; ++wv) v += part[(wv * M + i) * SW + cc];
             v *= alpha;
             const T *C = static_cast<const T *>(bias.ptr);
-            if (C) v += beta * up(C[ym * bias.sb + i * bias.sm + col * bias.sn]);
-            y[(ym * m + i) * n + col] = down<T>(v);
+            if (C) v += beta * up(C[ym * bias.sb + (row0 + i) * bias.sm + col * bias.sn]);
+            y[(ym * m + row0 + i) * n + col] = down<T>(v);
         }
     }
 }
 
 template <class T, int M, int L>
 int launch_gemv_kn_l(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                     uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+                     uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, uint32_t row0, uint32_t rows, hipStream_t s) {
     const dim3 grid((n + 8 * L - 1) / (8 * L), 1, count);
-    mm_gemv_kn<T, M, L><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0);
+    mm_gemv_kn<T, M, L><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, row0, rows);
     return launch_status();
 }
 
@@ -748,11 +750,11 @@ int launch_gemv_kn_l(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32
 // bytes in flight, so the chip has to be covered first.
 template <class T, int M>
 int launch_gemv_kn(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                   uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+                   uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, uint32_t row0, uint32_t rows, hipStream_t s) {
     auto groups = [&](uint32_t lanes) { return static_cast<uint64_t>((n + 8 * lanes - 1) / (8 * lanes)) * count; };
-    if (groups(8) >= 160) return launch_gemv_kn_l<T, M, 8>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
-    if (groups(4) >= 160) return launch_gemv_kn_l<T, M, 4>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
-    return launch_gemv_kn_l<T, M, 2>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, s);
+    if (groups(8) >= 160) return launch_gemv_kn_l<T, M, 8>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, row0, rows, s);
+    if (groups(4) >= 160) return launch_gemv_kn_l<T, M, 4>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, row0, rows, s);
+    return launch_gemv_kn_l<T, M, 2>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, row0, rows, s);
 }
 
 constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
@@ -798,19 +800,27 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const uint32_t gv_m = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const bool gemv = narrow && !trans_a && trans_b && m <= 4 && k > 0 && k % 8 == 0 && aligned16(a) && aligned16(b);
 
-    // the same with B as [k, n]
-    const bool gemv_kn = narrow && !trans_a && !trans_b && m <= 4 && k > 0 && k % 8 == 0 && n % 8 == 0 && aligned16(a) &&
+    // the same with B as [k, n]; up to 32 rows go four at a time, each pass reading B again at the same cost
+    // (20 us per pass at 4096 x 4096: 8 rows in a fifth, 32 rows in six sevenths of the plain kernel's time,
+    // which is what is left for these shapes otherwise)
+    const bool gemv_kn = narrow && !trans_a && !trans_b && m <= 32 && k > 0 && k % 8 == 0 && n % 8 == 0 && aligned16(a) &&
                          aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
             if (gemv_kn) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
-                switch (gv_m) {
-                    case 1: return launch_gemv_kn<T, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
-                    case 2: return launch_gemv_kn<T, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
-                    default: return launch_gemv_kn<T, 4>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                for (uint32_t r0 = 0; r0 < m32; r0 += 4) {
+                    const uint32_t rows = m32 - r0 < 4 ? m32 - r0 : 4;
+                    int e;
+                    switch (rows) {
+                        case 1: e = launch_gemv_kn<T, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, r0, rows, s); break;
+                        case 2: e = launch_gemv_kn<T, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, r0, rows, s); break;
+                        default: e = launch_gemv_kn<T, 4>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, r0, rows, s);
+                    }
+                    if (e) return e;
                 }
+                return 0;
             }
             if (gemv) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);

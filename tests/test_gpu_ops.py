@@ -948,9 +948,11 @@ def test_matmul_few_rows_weight_streaming(m, k, n, dt):
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 8, 8), (1, 4096, 4096), (2, 520, 40), (3, 1000, 248), (4, 4096, 1024), (4, 11008, 72),
-                                   (1, 8200, 16), (2, 12288, 104), (2, 264, 10248), (3, 512, 5120), (4, 136, 2568)])
+                                   (1, 8200, 16), (2, 12288, 104), (2, 264, 10248), (3, 512, 5120), (4, 136, 2568),
+                                   (5, 520, 40), (13, 4096, 264), (32, 1000, 248), (30, 264, 10248)])
 def test_matmul_one_to_four_rows_weights_as_k_by_n(m, k, n, dt):
-    # B as [k, n] (not transposed), at most four rows of A: a workgroup walks all of k for a strip of columns
+    # B as [k, n] (not transposed), at most four rows of A at a time (up to 32 rows as passes of four, the last
+    # one of fewer): a workgroup walks all of k for a strip of columns
     # (fixed order of summation, no atomics); k beyond one LDS segment of A (4096), k and n that end inside a
     # workgroup's step and strip; strips of 16, 32 and 64 columns (the widest that still gives 160 workgroups
     # over the two matrices of the batch: n = 4096 takes 32, 10248 and 5120 take 64), with a number of strips
