@@ -116,19 +116,24 @@ class ClockSampler:
                 "source": "pp_dpm_sclk sampled during the timed region"}
 
 
-LAST_CLOCK = [None]   # shader clock observed during the most recent time_steps() call
+LAST = {"clock": None, "warmup_ms": None, "warmup_steps": None}   # of the most recent time_steps() call
+MIN_WARMUP_S = 0.5    # the GPU leaves its idle clocks only after a few hundred ms of load
+CPU_THREADS = min(os.cpu_count() or 1, 16)   # host cores used by the all-cores CPU rows
 
 
 def time_steps(torch, fn, steps, warmup, n_sets):
-    """Times exactly `steps` calls fn(i % n_sets) after at least `warmup` untimed ones.
+    """Times exactly `steps` calls fn(i % n_sets) after at least `warmup` untimed ones and at least
+    MIN_WARMUP_S seconds of untimed load (whichever is longer; the time spent is reported as warmup_ms).
 
     The calls are captured into a HIP graph of `chunk` steps (chunk divides `steps`; plain kernel
     launches on the capture stream) that is replayed steps/chunk times, so the device sees the
     launches back to back and host launch overhead does not enter.  Warm-up replays the same
     graph: the GPU leaves its idle clocks only after a few hundred milliseconds of load, so a
-    short warm-up would time the clock ramp, not the kernel.  The timed region is bracketed by
-    device synchronisation (wall clock) and by HIP events on the replay stream (device time).
+    short warm-up would time the clock ramp, not the kernel.  Two measurements of exactly `steps`
+    steps each follow: the wall clock between two device synchronisations, and HIP events on the
+    replay stream around replays that follow an untimed one without a gap.
     Returns (wall ms per step, device ms per step, "graph" | "eager")."""
+    steps = max(int(steps), 1)
     chunk = max(d for d in range(1, min(steps, 100) + 1) if steps % d == 0)
     for i in range(min(warmup, 3)):
         fn(i % n_sets)
@@ -148,27 +153,56 @@ def time_steps(torch, fn, steps, warmup, n_sets):
         def run():
             for i in range(chunk):
                 fn(i % n_sets)
-    for _ in range((warmup + chunk - 1) // chunk):
+    # warm-up: at least `warmup` steps AND at least MIN_WARMUP_S of back-to-back replays
+    t_w = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - t_w < MIN_WARMUP_S:
+        for _ in range(4):
+            run()
+        done += 4 * chunk
+        torch.cuda.synchronize()
+    LAST["warmup_ms"] = round((time.perf_counter() - t_w) * 1e3, 1)
+    LAST["warmup_steps"] = done
+    # (a) wall clock around exactly `steps` steps, device idle and synchronised on both sides: this is what
+    #     `value` and `ms_per_step` report; it includes the latency of the first launch into an idle queue
+    t0 = time.perf_counter()
+    for _ in range(steps // chunk):
         run()
     torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # (b) device time of exactly `steps` steps from HIP events on the launch stream.  The timed replays are
+    #     queued directly behind one untimed replay, so the events see the kernels back to back, as a
+    #     profiler's per-kernel durations do, and not the start-up of a queue that had run dry.
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with ClockSampler() as clock:
-        t0 = time.perf_counter()
+        run()
         start.record()
         for _ in range(steps // chunk):
             run()
         stop.record()
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    LAST_CLOCK[0] = clock.result()
+    LAST["clock"] = clock.result()
     dev_ms = start.elapsed_time(stop) / steps
     return wall_ms, dev_ms, mode
+
+
+_POOL = []
+
+
+def pooled(fn_piece, pieces):
+    """Returns a callable that runs fn_piece(piece) for every piece on CPU_THREADS host threads (the oracle's C
+    functions are called through ctypes, which releases the interpreter lock, as numpy's conversions do)."""
+    if not _POOL:
+        from concurrent.futures import ThreadPoolExecutor
+        _POOL.append(ThreadPoolExecutor(CPU_THREADS))
+    return lambda: list(_POOL[0].map(fn_piece, pieces))
 
 
 def hbm_entry(bytes_per_call, dev_ms, traffic_key=None):
     gbs = bytes_per_call / (dev_ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(traffic_key)}
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(traffic_key),
+            "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
 
 
 def main():
@@ -234,7 +268,7 @@ def main():
     roofline["algorithmic_bytes"] = decode_bytes
     roofline["device_ms_per_launch"] = round(dev_ms, 5)
     roofline["timing"] = mode
-    roofline["observed_sclk_mhz"] = LAST_CLOCK[0]
+    roofline["observed_sclk_mhz"] = LAST["clock"]
 
     result = {
         "metric": "AttentionKVCache decode GB/s (% HBM peak); MatMulInteger int8 TOPS (% MFMA)",
@@ -267,9 +301,41 @@ def main():
             "sample": f"batch rows {rows} of the same workload (all 32 heads, {reps} repetitions, "
                       f"{cpu_s * 1e3:.1f} ms each); composed MatMul/scale/softmax/MatMul oracle in fp32"}
 
+        # the same arithmetic with the batch rows dealt to all host cores (one row per thread)
+        rows_all = list(range(min(CPU_THREADS, N)))
+        per_row = [(f(t["q"][r:r + 1]), f(t["k"][r:r + 1]), f(t["v"][r:r + 1]), f(t["kc"][r:r + 1]), f(t["vc"][r:r + 1]),
+                    past_np[r:r + 1]) for r in rows_all]
+        run_all = pooled(lambda a: oracle.attention_kvcache(a[0], a[1], a[2], a[3], a[4], a[5], scale), per_row)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 5.0:
+            run_all()
+            reps += 1
+        all_s = (time.perf_counter() - t0) / reps
+        all_bytes = 4096 * int(past_np[rows_all].sum()) + 786432 * len(rows_all) // N
+        result["cpu_baseline_all_cores"] = {
+            "value": round(all_bytes / all_s / 1e9, 3), "unit": "GB/s", "cores": CPU_THREADS, "kind": "port",
+            "sample": f"batch rows {rows_all[0]}..{rows_all[-1]} of the same workload, one row per thread "
+                      f"({reps} repetitions, {all_s * 1e3:.1f} ms each)"}
+        del per_row
+
     # ------------------------------------------------------------ the other hot-path kernels
     ops_out = {}
     steps, warmup = args.steps, args.warmup
+
+    def cpu_all(fn, algorithmic_bytes, sample, unit="GB/s", per=1e9):
+        """The all-cores row: `fn` runs the same arithmetic as the one-core leg with its rows split over
+        CPU_THREADS host threads (the oracle's own `threads=` argument, or pieces dealt to a thread pool)."""
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 1.0:
+                break
+        return {"value": round(algorithmic_bytes * reps / dt / per, 5), "unit": unit, "cores": CPU_THREADS, "kind": "port",
+                "sample": f"{sample} ({reps} repetitions, {dt / reps * 1e3:.1f} ms each)"}
 
     def cpu_leg(fn, algorithmic_bytes, sample):
         """Times the oracle on a bounded sample for about a second; the rate is quoted in the algorithmic bytes
@@ -297,6 +363,9 @@ def main():
             import oracle
             xn, wn = xs[0][:4].cpu().numpy(), w.cpu().numpy()
             e["cpu_baseline"] = cpu_leg(lambda: oracle.rms_norm(xn, wn, 1e-5), 134234112 // 8, "4 of the 32 [128,4096] slabs")
+            xa = xs[0][:CPU_THREADS].cpu().numpy()
+            e["cpu_baseline_all_cores"] = cpu_all(lambda: oracle.rms_norm(xa, wn, 1e-5, threads=CPU_THREADS),
+                                                  134234112 * len(xa) // 32, f"{len(xa)} of the 32 [128,4096] slabs")
         ops_out["rms_norm"] = e
         del xs, ys
 
@@ -304,7 +373,7 @@ def main():
         x = (3 * torch.randn((8, 32, 2048, 2048), device=dev)).half()
         y = torch.empty_like(x)
         for causal, nbytes, name in ((False, 4294967296, "softmax"), (True, 3221749760, "softmax_causal")):
-            wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 4, 5), max(warmup // 8, 3), 1)
+            wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=causal, out=y), max(steps // 4, 10), max(warmup // 8, 3), 1)
             e = hbm_entry(nbytes, dms, name)
             e.update(workload=f"Softmax fp16 [8,32,2048,2048] causal={causal}", device_ms_per_launch=round(dms, 5), timing=mode)
             if not args.no_cpu:
@@ -312,7 +381,19 @@ def main():
                 xn = x[0, :2].float().cpu().numpy()
                 fn = (lambda: oracle.softmax_causal(xn)) if causal else (lambda: oracle.softmax(xn))
                 e["cpu_baseline"] = cpu_leg(fn, nbytes // 128, "2 of the 256 [2048,2048] matrices, fp32 on up-cast input")
+                n_all = min(CPU_THREADS, 32)
+                xa = x[0, :n_all].float().cpu().numpy()
+                fa = (lambda: oracle.softmax_causal(xa, threads=CPU_THREADS)) if causal else \
+                     (lambda: oracle.softmax(xa, threads=CPU_THREADS))
+                e["cpu_baseline_all_cores"] = cpu_all(fa, nbytes * n_all // 256, f"{n_all} of the 256 [2048,2048] matrices")
             ops_out[name] = e
+        # the causal mask as data (strict upper triangle = -inf) through the plain kernel: full traffic
+        x.masked_fill_(torch.ones((2048, 2048), device=dev, dtype=torch.bool).triu(1), float("-inf"))
+        wall, dms, mode = time_steps(torch, lambda i: ops.softmax(x, causal=False, out=y), max(steps // 4, 10), max(warmup // 8, 3), 1)
+        e = hbm_entry(4294967296, dms, "softmax")
+        e.update(workload="Softmax fp16 [8,32,2048,2048], causal mask in the data (-inf above the diagonal), plain kernel",
+                 device_ms_per_launch=round(dms, 5), timing=mode)
+        ops_out["softmax_causal_data_masked"] = e
         del x, y
 
     if want("rope"):
@@ -328,6 +409,8 @@ def main():
             xn, pn = xs[0][:1].float().cpu().numpy(), pos[:1].cpu().numpy()
             e["cpu_baseline"] = cpu_leg(lambda: oracle.rope(xn, pn, 10000.0), 537133056 // 16,
                                         "batch row 0 of 16, fp32 on up-cast input")
+            e["cpu_baseline_all_cores"] = cpu_all(lambda: oracle.rope(xn, pn, 10000.0, threads=CPU_THREADS), 537133056 // 16,
+                                                  "batch row 0 of 16")
         ops_out["rope"] = e
         del xs, ys
 
@@ -343,6 +426,8 @@ def main():
             import oracle
             xn, sn = xs[0].cpu().numpy(), sc.cpu().numpy()
             e["cpu_baseline"] = cpu_leg(lambda: oracle.dequantize_linear(xn, sn, axis=1), 83902464, "the whole tensor once")
+            e["cpu_baseline_all_cores"] = cpu_all(lambda: oracle.dequantize_linear(xn, sn, axis=1, threads=CPU_THREADS), 83902464,
+                                                  "the whole tensor once")
         ops_out["dequantize_linear"] = e
         del xs, ys
 
@@ -383,6 +468,8 @@ def main():
             import oracle
             xn = xs[0].cpu().numpy()
             e["cpu_baseline"] = cpu_leg(lambda: oracle.cast(xn, "f32", "fp16"), cast_bytes, "the whole tensor once")
+            e["cpu_baseline_all_cores"] = cpu_all(pooled(lambda piece: oracle.cast(piece, "f32", "fp16"), list(xn)), cast_bytes,
+                                                  "the whole tensor once, the 32 slabs dealt to the threads")
         ops_out["cast"] = e
         del xs, ys
 
@@ -399,6 +486,10 @@ def main():
             import oracle
             xn = xs[0][:4].cpu().numpy()
             e["cpu_baseline"] = cpu_leg(lambda: oracle.transpose(xn, (0, 2, 1, 3)), tr_bytes // 8, "4 of the 32 batch rows")
+            xa = xs[0][:CPU_THREADS].cpu().numpy()
+            e["cpu_baseline_all_cores"] = cpu_all(
+                pooled(lambda piece: oracle.transpose(piece, (0, 2, 1, 3)), [xa[i:i + 1] for i in range(len(xa))]),
+                tr_bytes * len(xa) // 32, f"{len(xa)} of the 32 batch rows, one per thread")
         ops_out["transpose"] = e
         del xs, ys
 
@@ -415,10 +506,11 @@ def main():
             "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
             "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC["matmul_integer"],
             "workload": "MatMulInteger u8 x i8 -> i32 4096^3, a_zp=128 b_zp=0 (uniform random bytes)",
-            "device_ms_per_launch": round(dms, 5), "timing": mode, "observed_sclk_mhz": LAST_CLOCK[0]}
-        if LAST_CLOCK[0]:
+            "device_ms_per_launch": round(dms, 5), "timing": mode, "observed_sclk_mhz": LAST["clock"],
+            "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
+        if LAST["clock"]:
             # the published peak is quoted at 2400 MHz: the same pipe at the clock the run held
-            at_clock = INT8_PEAK_TOPS * LAST_CLOCK[0]["median"] / 2400.0
+            at_clock = INT8_PEAK_TOPS * LAST["clock"]["median"] / 2400.0
             ops_out["matmul_integer"]["peak_at_observed_clock"] = round(at_clock, 1)
             ops_out["matmul_integer"]["frac_at_observed_clock"] = round(tops / at_clock, 4)
         if not args.no_cpu:
@@ -431,6 +523,14 @@ def main():
             ops_out["matmul_integer"]["cpu_baseline"] = {
                 "value": round(2 * m * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
                 "sample": f"first {m} rows of A against all of B ({dt:.1f} s)"}
+            ma = m * CPU_THREADS
+            an = a[:ma].cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.matmul_integer(an, bn, np.array([128], np.uint8), np.array([0], np.int8), threads=CPU_THREADS)
+            dt = time.perf_counter() - t0
+            ops_out["matmul_integer"]["cpu_baseline_all_cores"] = {
+                "value": round(2 * ma * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": CPU_THREADS, "kind": "port",
+                "sample": f"first {ma} rows of A against all of B, rows split over the threads ({dt:.1f} s)"}
         if want("matmul_integer_dequantize"):
             # the same product with DequantizeLinear (per-column scale) folded into the epilogue, against
             # the two operators one after the other
@@ -447,7 +547,7 @@ def main():
                 "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC["matmul_integer_dequantize"],
                 "workload": "MatMulInteger 4096^3 with DequantizeLinear (scale per column) in its epilogue -> f32",
                 "device_ms_per_launch": round(dms_f, 5), "timing": mode,
-                "two_operators_device_ms": round(dms_2, 5)}
+                "two_operators_device_ms": round(dms_2, 5), "warmup_ms": LAST["warmup_ms"]}
         if want("matmul_integer_few_rows"):
             # the same weights against 32 rows of activations (a decode step of the quantised layer): bound by reading B
             a32 = a[:32].contiguous()
@@ -482,9 +582,10 @@ def main():
             "bound": "mfma", "achieved": round(tflops, 1), "peak": FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(tflops / FP16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get("matmul"),
             "workload": "MatMul fp16 [4096,4096] x [4096,4096]^T (trans_b), alpha 1, no bias",
-            "device_ms_per_launch": round(dms, 5), "timing": mode, "observed_sclk_mhz": LAST_CLOCK[0]}
-        if LAST_CLOCK[0]:
-            at_clock = FP16_PEAK_TFLOPS * LAST_CLOCK[0]["median"] / 2400.0
+            "device_ms_per_launch": round(dms, 5), "timing": mode, "observed_sclk_mhz": LAST["clock"],
+            "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
+        if LAST["clock"]:
+            at_clock = FP16_PEAK_TFLOPS * LAST["clock"]["median"] / 2400.0
             ops_out["matmul"]["peak_at_observed_clock"] = round(at_clock, 1)
             ops_out["matmul"]["frac_at_observed_clock"] = round(tflops / at_clock, 4)
         if not args.no_cpu:
@@ -497,6 +598,15 @@ def main():
             ops_out["matmul"]["cpu_baseline"] = {
                 "value": round(2 * rows * 4096 * 4096 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
                 "sample": f"first {rows} rows of A against all of B ({dt:.1f} s), float on the up-cast values"}
+            an = a[:rows * CPU_THREADS].cpu().numpy()
+            run_all = pooled(lambda piece: oracle.matmul(piece, bn, None, False, True, dtype="fp16"),
+                             [an[i * rows:(i + 1) * rows] for i in range(CPU_THREADS)])
+            t0 = time.perf_counter()
+            run_all()
+            dt = time.perf_counter() - t0
+            ops_out["matmul"]["cpu_baseline_all_cores"] = {
+                "value": round(2 * rows * CPU_THREADS * 4096 * 4096 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": CPU_THREADS,
+                "kind": "port", "sample": f"first {rows * CPU_THREADS} rows of A, {rows} per thread ({dt:.1f} s)"}
         del a, b, y
 
     if want("matmul_few_rows"):
@@ -567,7 +677,7 @@ def main():
         wall, dms, mode = time_steps(
             torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, scale, out=o, workspace=wsp,
                                                    sync_state=state),
-            max(steps // 40, 3), max(warmup // 80, 2), 1)
+            max(steps // 10, 20), max(warmup // 80, 2), 1)
         e = hbm_entry(402653184, dms, "attention_prefill")
         flops = 68853694464
         e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=128",
@@ -583,6 +693,10 @@ def main():
             e["cpu_baseline"] = cpu_leg(
                 lambda: oracle.attention_kvcache(qn, kn, vn, kcn, vcn, np.zeros(1, np.int64), scale, heads=pairs),
                 402653184 * 4 // (Np * H), "4 of the 1024 (batch row, head) pairs; composed oracle in fp32")
+            pa = [(0, h) for h in range(min(CPU_THREADS, H))]
+            e["cpu_baseline_all_cores"] = cpu_all(
+                pooled(lambda pr: oracle.attention_kvcache(qn, kn, vn, kcn, vcn, np.zeros(1, np.int64), scale, heads=[pr]), pa),
+                402653184 * len(pa) // (Np * H), f"{len(pa)} of the 1024 (batch row, head) pairs, one per thread")
         ops_out["attention_prefill"] = e
 
     if ops_out:

@@ -215,8 +215,10 @@ int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, con
  * For batch row b with past = past_lens[past_per_row ? b : 0] (int64, read on the device):
  *   the new k/v rows are written to cache[b, :, past .. past+seq), then query row r attends
  *   cache positions 0 .. past + r with scores scaled by `scale` (causal decoder mask);
- *   cache rows >= past + seq are left untouched.  past + seq > cap is clamped on the device
- *   (rows that do not fit are dropped), never written out of bounds.
+ *   cache rows >= past + seq are left untouched.  The lengths live on the device, so the host
+ *   cannot refuse them: a negative past counts as 0 and a past above cap - seq is moved back to
+ *   cap - seq (the new rows then replace the last seq rows of the cache and the queries see the
+ *   history shortened accordingly); nothing is ever read or written outside the caches.
  * k_cache == v_cache == NULL: no cache (past = 0, attends k/v directly).  past_lens == NULL: 0.
  * n_head % n_kv_head == 0; D in {64, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
  * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials), contents irrelevant.

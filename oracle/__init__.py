@@ -230,14 +230,17 @@ def attention_kvcache(q, k, v, k_cache, v_cache, past_lens, scale, heads=None):
     """Composed attention with cache append, fp32 math on already up-cast inputs.
 
     q [N,H,seq,D]; k,v [N,Hkv,seq,D]; caches [N,Hkv,S,D] (updated copies are returned);
-    past_lens: int array [N] (or one value).  ``heads``: optional iterable of (b, h) pairs to
-    evaluate (others are left as NaN) so large shapes can be spot-checked.
+    past_lens: int array [N] (or one value); a length outside [0, S - seq] is moved to the nearer
+    end of that interval, the rule the device kernels apply to lengths they cannot refuse.
+    ``heads``: optional iterable of (b, h) pairs to evaluate (others are left as NaN) so large
+    shapes can be spot-checked.
     Returns (o, k_cache_out, v_cache_out)."""
     q = _c(q, np.float32)
     N, H, seq, D = q.shape
     Hkv = k.shape[1]
     g = H // Hkv
     past_lens = np.broadcast_to(np.asarray(past_lens, dtype=np.int64).reshape(-1), (N,))
+    past_lens = np.clip(past_lens, 0, max(k_cache.shape[2] - seq, 0))
     kc = np.array(k_cache, copy=True)
     vc = np.array(v_cache, copy=True)
     for b in range(N):

@@ -768,11 +768,18 @@ __global__ __launch_bounds__(kSplitThreads) void attn_split(const AttnParams p) 
             }
         }
         if (any_cut) {
-            // The workgroup that completes a cut segment last merges its partials.  The partials
-            // are written through to device-coherent memory and read back past the per-XCD L2
-            // (device-scope atomic accesses), so only this wavefront's outstanding stores have to
-            // drain before the tickets are taken; no cache-wide write-back or invalidate is issued.
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            // The workgroup that completes a cut segment last merges its partials.  Ordering of
+            // the hand-off, writer side: the partials are device-scope write-through stores; every
+            // wavefront waits until all of its vector-memory operations have been acknowledged
+            // (vmcnt counts stores on this target and a write-through store is acknowledged once
+            // it has left the XCD's L2), then the barrier collects the wavefronts, and only then
+            // is the ticket taken.  Reader side: the ticket's value decides `sh_last`, which the
+            // merging threads read after another barrier, so their device-scope loads (which
+            // bypass the XCD-local L2) are issued after the ticket add has returned and therefore
+            // after every other piece's stores were acknowledged.  A workgroup-scope fence alone
+            // would not do: it emits no wait for outstanding stores.  No cache-wide write-back or
+            // invalidate is needed (one per workgroup cost 3.5x).
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             if (threadIdx.x < kMaxPieces) {
                 uint32_t is_last = 0;

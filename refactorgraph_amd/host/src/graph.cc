@@ -93,20 +93,33 @@ namespace refactor::kernel {
         auto const align = device->type() == hardware::Device::Type::Amd ? size_t(256) : size_t(32);
         auto [stack, nodes_, edges_] = allocator(_internal.topology, std::move(nodes), _internal.edges, align);
 
-        // a constant is uploaded once per (device, blob) and shared by every stream lowered afterwards;
-        // the entry goes away with the last stream that uses it
-        static std::map<std::pair<hardware::Device *, Blob const *>, std::weak_ptr<hardware::Device::Blob>> uploaded;
+        // A constant is uploaded once per (device, host blob) and shared by every stream lowered
+        // afterwards; the entry goes away with the last stream that uses it.  The map is looked up by
+        // address, so an entry also remembers whose addresses these were: a host blob or device that
+        // was freed and whose address has been reused since does not match, and the constant is
+        // uploaded again (the reference keys by the shared pointers themselves, which keeps every
+        // constant ever lowered alive).  Single-threaded like the rest of the lowering.
+        struct Uploaded {
+            std::weak_ptr<hardware::Device> device;
+            std::weak_ptr<Blob> host;
+            std::weak_ptr<hardware::Device::Blob> copy;
+        };
+        static std::map<std::pair<hardware::Device *, Blob const *>, Uploaded> uploaded;
+        std::erase_if(uploaded, [](auto const &kv) { return kv.second.copy.expired(); });
+        auto const sameOwner = [](auto const &weak, auto const &shared) {
+            return !weak.owner_before(shared) && !shared.owner_before(weak);
+        };
 
         for (size_t i = 0; i < edges_.size(); ++i) {
             auto const &edge = _internal.edges[i];
             edges_[i].name = edge.name;
             if (edge.data) {
                 auto &slot = uploaded[{device.get(), edge.data.get()}];
-                auto blob = slot.lock();
-                if (!blob) {
+                auto blob = slot.copy.lock();
+                if (!blob || !sameOwner(slot.device, device) || !sameOwner(slot.host, edge.data)) {
                     blob = device->malloc(edge.size);
                     blob->copyFromHost(edge.data->get<void>(), edge.size);
-                    slot = blob;
+                    slot = Uploaded{device, edge.data, blob};
                 }
                 edges_[i].blob = std::move(blob);
             } else if (edges_[i].stackOffset == GLOBAL_OUTPUT) {

@@ -57,11 +57,22 @@ static int g_failed = 0, g_checks = 0;
             std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #COND);       \
         }                                                                         \
     } while (0)
-#define RUN(NAME)                                  \
-    do {                                           \
-        std::printf("[ RUN  ] %s\n", #NAME);       \
-        std::fflush(stdout);                       \
-        NAME();                                    \
+// every case prints its name before it starts and its verdict when it returns, so that the
+// output of one run of the driver can be split into one result per case
+#define RUN(NAME)                                                                   \
+    do {                                                                            \
+        if (!only.empty() && only != #NAME) break;                                  \
+        std::printf("[ RUN  ] %s\n", #NAME);                                        \
+        std::fflush(stdout);                                                        \
+        int const failedBefore = g_failed;                                          \
+        try {                                                                       \
+            NAME();                                                                 \
+        } catch (std::exception const &e) {                                         \
+            ++g_failed;                                                             \
+            std::printf("  FAILED %s: exception: %s\n", #NAME, e.what());           \
+        }                                                                           \
+        std::printf("[ %s ] %s\n", g_failed == failedBefore ? " OK " : "FAIL", #NAME); \
+        std::fflush(stdout);                                                        \
     } while (0)
 template<class E, class F> static bool throws(F &&f) {
     try { f(); } catch (E const &) { return true; } catch (...) { return false; }
@@ -477,6 +488,40 @@ static void allocatorsAndStreamOnCpu() {
     auto s1 = graph.lower(device::fetch(Device::Type::Cpu), flatAllocate);
     auto s2 = graph.lower(device::fetch(Device::Type::Cpu), reusableAllocate);
     EXPECT(s1.getData(3) == s2.getData(3));
+    {// A constant that is freed while a stream still holds its device copy, then another constant of the
+        // same size that lands at the same host address: the second graph must see its own values.
+        auto run = [&](runtime::Stream &stream) {
+            std::vector<float> x(n, 0.f), y(n, -1.f);
+            stream.setData(0, x.data(), n * sizeof(float));
+            stream.run();
+            stream.copyData(5, y.data(), n * sizeof(float));
+            return y;
+        };
+        auto [cA, pA] = kernel::Blob::share(n * sizeof(float));
+        for (size_t i = 0; i < n; ++i) static_cast<float *>(pA)[i] = 1.f;
+        auto const addressA = cA.get();
+        auto graphA = std::make_unique<kernel::Graph>(chainGraph(n, std::move(cA)));
+        auto streamA = graphA->lower(device::fetch(Device::Type::Cpu), flatAllocate);
+        graphA.reset();// the host blob of A is gone, its device copy lives on in streamA
+        std::vector<Arc<kernel::Blob>> held;
+        Arc<kernel::Blob> cB;
+        void *pB = nullptr;
+        for (int attempt = 0; attempt < 64 && !cB; ++attempt) {
+            auto [c, ptr] = kernel::Blob::share(n * sizeof(float));
+            if (c.get() == addressA) cB = std::move(c), pB = ptr;
+            else held.push_back(std::move(c));
+        }
+        bool const collided = static_cast<bool>(cB);
+        if (!collided) std::tie(cB, pB) = kernel::Blob::share(n * sizeof(float));
+        std::printf("  constant cache: host address %s\n", collided ? "reused" : "not reused by this allocator");
+        for (size_t i = 0; i < n; ++i) static_cast<float *>(pB)[i] = 100.f;
+        auto graphB = chainGraph(n, cB);
+        auto streamB = graphB.lower(device::fetch(Device::Type::Cpu), flatAllocate);
+        EXPECT(streamB.getData(3) != streamA.getData(3));
+        auto const yA = run(streamA), yB = run(streamB);
+        EXPECT(yA == std::vector<float>(n, 8.f));
+        EXPECT(yB == std::vector<float>(n, 107.f));
+    }
     // a node without kernel lowers to the empty routine
     graph_topo::GraphTopo topo1(1, 1);
     topo1.pushNode({0}, 0, 1);
@@ -1598,7 +1643,9 @@ static void amdDeviceAndPool() {
 }
 
 int main(int argc, char **argv) {
+    // usage: rg_host_tests [cpu|gpu] [case]   (gpu = the cpu cases and those that need the device)
     std::string mode = argc > 1 ? argv[1] : "cpu";
+    std::string only = argc > 2 ? argv[2] : "";
     RUN(broadcasterKnownAnswer);
     RUN(shapeDigests);
     RUN(memPoolBestFit);

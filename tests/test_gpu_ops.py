@@ -725,6 +725,44 @@ def test_attention_prefill_config_sample():
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
 
 
+def test_attention_prefill_full_config():
+    # the whole configuration: N=32, seq 512, past 0, causal, 32/8 heads, D=128, cap 4096 (4096 workgroups,
+    # 256 (batch row, kv head) streams dealt to the XCDs).  Whole-cache append bit-exact, eight (b, h) pairs
+    # spread over the batch against the oracle, every output finite, and rows 0 (which see one key: O = V)
+    g = torch.Generator(device=DEV).manual_seed(31)
+    rnd = lambda shape: torch.randn(shape, generator=g, device=DEV).half()
+    N, H, Hkv, seq, cap, D = 32, 32, 8, 512, 4096, 128
+    q, k, v = rnd((N, H, seq, D)), rnd((N, Hkv, seq, D)), rnd((N, Hkv, seq, D))
+    kc, vc = rnd((N, Hkv, cap, D)), rnd((N, Hkv, cap, D))
+    kc0, vc0 = kc.clone(), vc.clone()
+    past = torch.zeros(N, device=DEV, dtype=torch.int64)
+    scale = 1 / math.sqrt(D)
+    o = ops.attention_kvcache(q, k, v, kc, vc, past, scale)
+    torch.cuda.synchronize()
+    assert torch.equal(kc[:, :, :seq], k) and torch.equal(vc[:, :, :seq], v)
+    assert torch.equal(kc[:, :, seq:], kc0[:, :, seq:]) and torch.equal(vc[:, :, seq:], vc0[:, :, seq:])
+    assert bool(torch.isfinite(o).all())
+    assert torch.equal(o[:, :, 0], v[:, :, 0].repeat_interleave(H // Hkv, 1))
+    f = lambda t: host(t.float())
+    for b, h in [(0, 0), (3, 9), (8, 31), (13, 4), (17, 22), (22, 15), (27, 2), (31, 31)]:
+        kh = h // (H // Hkv)
+        ref = oracle.attention_head(f(q[b, h]), f(k[b, kh]), f(v[b, kh]), 0, scale, True)
+        assert np.max(np.abs(f(o[b, h]) - ref)) <= ABS_F16, (b, h)
+
+
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,past", [
+    (3, 8, 2, 1, 64, 128, [63, 64, 1000]),     # decode: the cache is full (63 fits, the others are moved back)
+    (2, 4, 2, 5, 32, 64, [30, -3]),            # several new rows through the split kernel; a negative length is 0
+    (2, 8, 2, 40, 64, 128, [30, 24]),          # tiled prefill kernel: 30 + 40 > 64 is moved back to 24
+])
+def test_attention_history_length_outside_the_cache(N, H, Hkv, seq, cap, D, past):
+    # the lengths are device data, so the kernels cannot refuse them: they are moved into [0, cap - seq]
+    # and the oracle states the same rule
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past)
+    assert np.max(np.abs(o - ref_o)) <= ABS_F16
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
 # ------------------------------------------------------------------ Cast
 _CAST_TORCH = {"u8": torch.uint8, "i8": torch.int8, "i16": torch.int16, "i32": torch.int32, "i64": torch.int64,
                "f32": torch.float32, "f64": torch.float64, "bool": torch.bool, "fp16": torch.float16,
