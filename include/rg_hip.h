@@ -240,6 +240,28 @@ int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *
                              void *workspace, size_t workspace_bytes, void *sync_state,
                              void *stream);
 
+/* The same operation for callers that cannot allocate device memory or hand over a workspace:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference (every reference kernel gets its workspace from the stack that
+ * kernel::Graph::lower allocates).  The split-KV partials and ticket counters live in a fixed
+ * array of rg_hip_attention_kvcache_static_scratch_bytes() bytes (2 KiB + 2.03 MiB) inside the
+ * library's device image, one copy per GPU, held until the process ends; the call allocates
+ * nothing and frees nothing, and the counters are cleared by a small fill kernel at the start of
+ * every call (not a memset, so the call can be captured).  Limits: those of
+ * rg_hip_attention_kvcache (D in {64, 128}; a larger D is refused with RG_HIP_E_WORKSPACE, the
+ * partial slots being sized for D <= 128); the launch uses at most 512 workgroups, which is what
+ * the array holds partials for.  All calls on one GPU share the array: calls that overlap on one
+ * GPU (two streams, two threads) race and must be serialised by the caller.  Same kernels as
+ * rg_hip_attention_kvcache: the caches come out bit-identical, the output within the rounding of
+ * the summation order (which work a wavefront pulls is decided at run time in either entry). */
+size_t rg_hip_attention_kvcache_static_scratch_bytes(void);
+int rg_hip_attention_kvcache_static(void *o, const void *q, const void *k, const void *v,
+                                    void *k_cache, void *v_cache,
+                                    const int64_t *past_lens, int past_per_row,
+                                    size_t N, size_t n_head, size_t n_kv_head,
+                                    size_t seq, size_t cap, size_t D,
+                                    float scale, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

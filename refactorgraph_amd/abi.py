@@ -55,6 +55,9 @@ SIGNATURES = {
     "rg_hip_attention_kvcache_state_bytes": (_sz, []),
     "rg_hip_attention_kvcache": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _sz,
                                       _f, _i, _vp, _sz, _vp, _vp]),
+    "rg_hip_attention_kvcache_static_scratch_bytes": (_sz, []),
+    "rg_hip_attention_kvcache_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _sz, _sz,
+                                             _f, _i, _vp]),
 }
 
 

@@ -21,6 +21,8 @@
 #include "attention_prefill.hpp"
 #include "common.hpp"
 
+#include <mutex>
+
 namespace rg {
 namespace {
 
@@ -853,7 +855,7 @@ constexpr size_t kPrefillMinSeq = 16;      // query rows per batch row from whic
 template <class T, int D, int G>
 int launch(AttnParams p, hipStream_t s) {
     uint32_t wgs = resident_workgroups<T, D, G>();
-    if (wgs > kMaxWorkgroups) wgs = kMaxWorkgroups;
+    if (wgs > p.n_workgroups) wgs = p.n_workgroups;  // what the partial slots and counters are sized for
     p.n_workgroups = wgs;
     attn_split<T, D, G><<<wgs, kSplitThreads, 0, s>>>(p);
     return launch_status();
@@ -891,22 +893,47 @@ size_t workspace_bytes(size_t D) {
     return kCounterBytes + static_cast<size_t>(kMaxWorkgroups) * 2 * 4 * (D + 2) * sizeof(float);
 }
 
-}  // namespace
-}  // namespace rg
+// ---------------------------------------------------------------- library-owned scratch
+// Split-KV partials and ticket counters for callers that may not allocate: a fixed array in
+// device memory, one copy per GPU the library is loaded on.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; the address it returns for the current device is what
+// kernels and fill launches are given.
+constexpr uint32_t kStaticWorkgroups = 512;                      // the launch is capped at this many
+constexpr size_t kStaticCounterBytes = kStaticWorkgroups * sizeof(uint32_t);
+constexpr size_t kStaticPartBytes = static_cast<size_t>(kStaticWorkgroups) * 2 * 4 * (128 + 2) * sizeof(float);
+constexpr size_t kStaticBytes = kStaticCounterBytes + kStaticPartBytes;  // 2 KiB + 2.03 MiB
 
-extern "C" size_t rg_hip_attention_kvcache_workspace(size_t, size_t, size_t, size_t, size_t, size_t D) {
-    return rg::workspace_bytes(D);
+__device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void *scratch_of_device[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch` (looked up once per device).
+int static_scratch(void **out) {
+    int dev = -1;
+    const hipError_t rc = hipGetDevice(&dev);
+    if (rc != hipSuccess) return static_cast<int>(rc);
+    if (dev < 0 || dev >= kMaxDevices) return RG_HIP_E_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_of_device[dev]) {
+        void *ptr = nullptr;
+        const hipError_t rs = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (rs != hipSuccess) return static_cast<int>(rs);
+        if (!ptr) return RG_HIP_E_WORKSPACE;
+        scratch_of_device[dev] = ptr;
+    }
+    *out = scratch_of_device[dev];
+    return 0;
 }
 
-extern "C" size_t rg_hip_attention_kvcache_state_bytes(void) { return rg::kCounterBytes; }
-
-extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *v,
-                                        void *k_cache, void *v_cache, const int64_t *past_lens,
-                                        int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
-                                        size_t seq, size_t cap, size_t D, float scale, int dtype,
-                                        void *workspace, size_t workspace_bytes, void *sync_state,
-                                        void *stream) {
-    using namespace rg;
+// Argument checks and dispatch shared by the entry points.  `part` holds two partial slots per
+// workgroup for at most `max_workgroups` workgroups; `counters` one ticket counter per workgroup,
+// zero on entry unless `clear_counters` asks for the clearing launch.
+int attention_call(void *o, const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
+                   const int64_t *past_lens, int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
+                   size_t seq, size_t cap, size_t D, float scale, int dtype, float *part, uint32_t *counters,
+                   uint32_t max_workgroups, bool clear_counters, hipStream_t s) {
     if (!o || !q || !k || !v) return RG_HIP_E_ARGUMENT;
     if ((k_cache == nullptr) != (v_cache == nullptr)) return RG_HIP_E_ARGUMENT;
     if (N == 0 || n_head == 0 || seq == 0) return 0;
@@ -916,12 +943,11 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
     if (N > kMaxBatch || seq > 0xffffu || cap > 0x3fffffffu || n_head > 0xffffu) return RG_HIP_E_UNSUPPORTED;
     if (k_cache && cap < seq) return RG_HIP_E_ARGUMENT;
     if (N * seq * n_kv_head > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
-    if (!workspace || workspace_bytes < rg::workspace_bytes(D)) return RG_HIP_E_WORKSPACE;
+    if (!part || !counters) return RG_HIP_E_WORKSPACE;
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) ||
         (k_cache && (!aligned16(k_cache) || !aligned16(v_cache))))
         return RG_HIP_E_ARGUMENT;
 
-    hipStream_t s = as_stream(stream);
     // many query rows per batch row: the tiled MFMA kernel (K/V staged once per query tile)
     if (seq >= kPrefillMinSeq && prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head),
                                                    static_cast<uint32_t>(D))) {
@@ -950,12 +976,11 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
     p.cap = static_cast<uint32_t>(cap);
     p.group = p.H / p.Hkv;
     p.scale_log2e = scale * 1.4426950408889634f;
-    p.part = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
-    if (sync_state) {
-        p.counters = static_cast<uint32_t *>(sync_state);
-    } else {
-        p.counters = static_cast<uint32_t *>(workspace);
-        attn_clear<<<4, 256, 0, s>>>(p.counters, kMaxWorkgroups);
+    p.part = part;
+    p.counters = counters;
+    p.n_workgroups = max_workgroups;  // upper bound; launch() lowers it to what is resident
+    if (clear_counters) {
+        attn_clear<<<1, 256, 0, s>>>(counters, max_workgroups);
         const int rc = launch_status();
         if (rc) return rc;
     }
@@ -963,4 +988,49 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
         return D == 128 ? dispatch_group<__half, 128>(p, s) : dispatch_group<__half, 64>(p, s);
     }
     return D == 128 ? dispatch_group<__hip_bfloat16, 128>(p, s) : dispatch_group<__hip_bfloat16, 64>(p, s);
+}
+
+}  // namespace
+}  // namespace rg
+
+extern "C" size_t rg_hip_attention_kvcache_workspace(size_t, size_t, size_t, size_t, size_t, size_t D) {
+    return rg::workspace_bytes(D);
+}
+
+extern "C" size_t rg_hip_attention_kvcache_state_bytes(void) { return rg::kCounterBytes; }
+
+extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *v,
+                                        void *k_cache, void *v_cache, const int64_t *past_lens,
+                                        int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
+                                        size_t seq, size_t cap, size_t D, float scale, int dtype,
+                                        void *workspace, size_t workspace_bytes, void *sync_state,
+                                        void *stream) {
+    using namespace rg;
+    // a workspace that is missing or too small is reported after the argument checks
+    const bool usable = workspace && (D == 64 || D == 128) && workspace_bytes >= rg::workspace_bytes(D);
+    float *part = usable ? reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes) : nullptr;
+    uint32_t *counters = static_cast<uint32_t *>(sync_state ? sync_state : workspace);
+    return attention_call(o, q, k, v, k_cache, v_cache, past_lens, past_per_row, N, n_head, n_kv_head, seq, cap, D,
+                          scale, dtype, part, counters, kMaxWorkgroups, sync_state == nullptr, as_stream(stream));
+}
+
+extern "C" size_t rg_hip_attention_kvcache_static_scratch_bytes(void) { return rg::kStaticBytes; }
+
+extern "C" int rg_hip_attention_kvcache_static(void *o, const void *q, const void *k, const void *v,
+                                               void *k_cache, void *v_cache, const int64_t *past_lens,
+                                               int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
+                                               size_t seq, size_t cap, size_t D, float scale, int dtype,
+                                               void *stream) {
+    using namespace rg;
+    // the scratch is sized for head dimensions up to 128 and head groups of four per launch
+    if (D > 128) return RG_HIP_E_WORKSPACE;
+    void *base = nullptr;
+    const int rc = static_scratch(&base);
+    if (rc) return rc;
+    uint32_t *counters = static_cast<uint32_t *>(base);
+    float *part = reinterpret_cast<float *>(static_cast<char *>(base) + kStaticCounterBytes);
+    // The counters are cleared by a small fill kernel on every call (no memset: the call may be
+    // under stream capture), so that whatever an earlier call left there cannot matter.
+    return attention_call(o, q, k, v, k_cache, v_cache, past_lens, past_per_row, N, n_head, n_kv_head, seq, cap, D,
+                          scale, dtype, part, counters, kStaticWorkgroups, true, as_stream(stream));
 }
