@@ -4,9 +4,9 @@
 // reference: q, o [N, H, seq, D]; k, v [N, Hkv, seq, D]; caches [N, Hkv, cap, D]; query row r
 // attends positions 0 .. past + r; new rows appended at past .. past + seq - 1).
 //
-// A workgroup of four wavefronts works on one kv head: wavefront w owns 32 query rows of one of
-// the query heads that share this kv head (GQA), so a K/V tile staged once in LDS serves up to
-// four query heads.  Keys are walked 32 at a time; a tile of K and V rows is copied from global
+// A workgroup of four wavefronts works on one kv head at a time: wavefront w owns 32 query rows of
+// one of the query heads that share this kv head (GQA), so a K/V tile staged once in LDS serves up
+// to four query heads.  Keys are walked 64 at a time; a tile of K and V rows is copied from global
 // memory straight into one of two LDS buffers (global_load_lds_dwordx4: lane L of a wavefront-wide
 // copy fills bytes 16 L .. 16 L + 15 behind a wave-uniform LDS base from an address of its own),
 // one tile ahead of its use, with the 16-byte chunks of a row XOR-swizzled so that the fragment
@@ -17,8 +17,20 @@
 // In this form a lane holds one query row of S^T / O^T in its accumulator registers, so the
 // softmax row statistics need no cross-lane reduction beyond one exchange between the two
 // half-wavefronts, and P^T is already in B-operand position.  Softmax is online in float with
-// the lazily raised reference of the split kernel.  O^T is transposed through LDS at the end so
-// that the global stores are 128-bit and row-contiguous.
+// the lazily raised reference of the split kernel.
+//
+// The workgroups are persistent.  The unit of work is an item = 32 query rows x 4 heads of one
+// (batch row, kv head) stream; moving the query rows in and the output rows out is pure memory
+// latency, which a workgroup that did one item would pay in full (a launch of one-item workgroups
+// spent two thirds of its time there).  So a workgroup walks a list of items, and the two LDS
+// buffers carry one continuous sequence of slots across them: [Q of item 0] [tile 0] [tile 1] ...
+// [Q of item 1] [tile 0] ...  While a slot is worked on, the next one is copied in; the query rows
+// of the next item therefore arrive under the last key tile of the current one, the output rows
+// leave from registers (16-byte stores, no staging) while tile 0 of the next item is on its way,
+// and nothing waits for memory except the very first slot.  Items are dealt so that every
+// workgroup gets the same number of key tiles (query tile t is paired with tile q_tiles - 1 - t)
+// and so that the workgroups of an XCD walk few streams at a time, which keeps the K/V rows that
+// the query tiles of a stream share in that XCD's L2.
 #include "attention_prefill.hpp"
 
 namespace rg {
@@ -29,8 +41,7 @@ typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int D = 128;
-constexpr int BN = 32;                 // keys per tile (32 or 64); 32 keeps the kernel within the registers and
-                                       // LDS of three workgroups per CU, which hides more of the memory latency
+constexpr int BN = 64;                 // keys per tile: two blocks of 32
 constexpr int KB = BN / 32;            // blocks of 32 keys per tile
 constexpr int CPI = BN / 16;           // K (and V) copy instructions per wavefront and tile
 constexpr int ROWB = 2 * D;            // bytes of a K or V row (unpadded in LDS)
@@ -70,6 +81,12 @@ template <> struct Ops<__half> {
         const h2 v = {static_cast<_Float16>(lo), static_cast<_Float16>(hi)};
         return __builtin_bit_cast(uint32_t, v);
     }
+    // running row sum: the two rounded probabilities of a packed word, exactly as the PV product sees them
+    static __device__ __forceinline__ float add_pair(float sum, uint32_t packed, float, float) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 ones = {static_cast<_Float16>(1.f), static_cast<_Float16>(1.f)};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), ones, sum, false);
+    }
 };
 template <> struct Ops<__hip_bfloat16> {
     static __device__ __forceinline__ f16v mfma(const Raw16 &a, const Raw16 &b, f16v c) {
@@ -80,317 +97,601 @@ template <> struct Ops<__hip_bfloat16> {
         const uint32_t h = __builtin_bit_cast(uint16_t, __float2bfloat16(hi));
         return l | (h << 16);
     }
+    static __device__ __forceinline__ float add_pair(float sum, uint32_t, float p0, float p1) { return sum + (p0 + p1); }
 };
+
+// Sum and maximum over the two half-wavefronts (lanes i and i + 32), on the vector ALU.
+struct HalfPair {
+    float a, b;
+};
+__device__ __forceinline__ HalfPair half_swap(float x, float y) {
+    // a: lanes 0-31 keep x, lanes 32-63 receive y of lanes 0-31; b: lanes 0-31 receive x of lanes 32-63, 32-63 keep y
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, y), false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return {__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1)};
+}
+__device__ __forceinline__ float half_max(float v) {
+    const HalfPair r = half_swap(v, v);
+    return fmaxf(r.a, r.b);
+}
+__device__ __forceinline__ float half_sum(float v) {
+    const HalfPair r = half_swap(v, v);
+    return r.a + r.b;
+}
+
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint32_t div_magic(uint32_t x, uint32_t magic) { return magic ? uni(__umulhi(x, magic)) : x; }
+
+// How the items are dealt to the workgroups (computed on the host).
+struct PrefillPlan {
+    uint32_t group;        // query heads per kv head
+    uint32_t head_chunks;  // group / HW
+    uint32_t q_tiles;      // query tiles (of ROWS rows) per stream
+    uint32_t pairs;        // (q_tiles + 1) / 2: workgroups that share a stream
+    uint32_t xcds;         // 8 when the streams divide evenly over the XCDs, else 1
+    uint32_t spx;          // streams per XCD
+    uint32_t groups;       // sets of `pairs` workgroups per XCD; set g walks streams g, g + groups, ...
+    // floor(2^32 / d) + 1 for d = head_chunks and d = Hkv: x / d = mulhi(x, magic) for every x with
+    // x * d < 2^32, which the host checks (0 stands for d = 1)
+    uint32_t magic_chunks, magic_hkv;
+};
+
+// One item: query tile qt of stream (kv head `kvhead` = b * Hkv + kvh of the batch, head chunk hc).
+// Kept to four scalars: the workgroup holds two of them across its whole life.
+constexpr uint32_t kNoItem = 0xffffffffu;
+struct Item {
+    uint32_t kvhead, hc;
+    uint32_t qt;    // kNoItem: there is no such item
+    uint32_t base;  // history length of the batch row, moved into [0, cap - seq]
+    __device__ bool valid() const { return qt != kNoItem; }
+};
+
+// Copy of 16 bytes per lane from global memory into LDS (lane L of the wavefront fills bytes
+// 16 L .. 16 L + 15 behind the wave-uniform LDS address; OFFSET is added to the global address and
+// to the LDS address alike).  Issued as inline assembly: the compiler
+// then does not know that a vector-memory operation writes LDS and adds no waits of its own between
+// the copies and the LDS reads; every wait for a copy in this file is an explicit s_waitcnt before a
+// barrier.  (Writing M0 needs one wait state before the copy reads it.)
+template <int OFFSET>
+__device__ __forceinline__ void copy16(const void *sbase, uint32_t voffset, uint32_t lds_addr) {
+    // the base and the LDS address are wave-uniform by construction; they are pinned to scalar registers
+    // here because the assembly needs them there, wherever the compiler has computed them
+    const uint64_t b = reinterpret_cast<uint64_t>(sbase);
+    sbase = reinterpret_cast<const void *>((static_cast<uint64_t>(uni(static_cast<uint32_t>(b >> 32))) << 32) |
+                                           uni(static_cast<uint32_t>(b)));
+    lds_addr = uni(lds_addr);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :
+                 : "v"(voffset), "s"(sbase), "s"(lds_addr), "n"(OFFSET)
+                 : "memory", "m0");
+}
+
+#define RG_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 // HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
 // query sub-tiles of the same heads.
 template <class T, int HW>
-__global__ __launch_bounds__(256, 3) void attn_prefill(const PrefillArgs a, uint32_t group,
-                                                    uint32_t q_tiles, uint32_t head_chunks) {
+__global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, const PrefillPlan plan) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
-    constexpr int ROWS = 32 * QS;   // query rows per workgroup
-    __shared__ __align__(1024) uint8_t lds0[BUF_BYTES];
-    __shared__ __align__(1024) uint8_t lds1[BUF_BYTES];
+    constexpr int ROWS = 32 * QS;   // query rows per item
+    __shared__ __align__(1024) uint8_t lds[2 * BUF_BYTES];
+    const uint32_t lds_addr0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (__attribute__((address_space(3))) uint8_t *)lds));
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t half = lane >> 5, l32 = lane & 31;
+    const uint32_t wave_u = uni(wave);
 
-    // Workgroup order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, so every
-    // XCD is given whole (batch row, kv head, head chunk) streams, one after the other and the
-    // heaviest query tile (longest key range) of each first.  The query tiles of a stream then
-    // run close together on one XCD and find the K/V rows they share in its L2.
-    const uint32_t n_rest = a.N * a.Hkv * head_chunks;
-    uint32_t rest, qt;
-    if (n_rest % 8 == 0) {
-        const uint32_t xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
-        rest = (slot / q_tiles) * 8 + xcd;
-        qt = q_tiles - 1 - slot % q_tiles;
-    } else {
-        rest = blockIdx.x / q_tiles;
-        qt = q_tiles - 1 - blockIdx.x % q_tiles;
-    }
-    const uint32_t hc = rest % head_chunks;
-    rest /= head_chunks;
-    const uint32_t kvh = rest % a.Hkv, b = rest / a.Hkv;
+    // Workgroup w: consecutive ids are dealt round-robin to the XCDs.  Within an XCD, set g of
+    // `pairs` workgroups walks the XCD's streams g, g + groups, ...; member j of a set takes query
+    // tiles q_tiles - 1 - j and j of each of them (the heavy one first).
+    const uint32_t xcd = uni(blockIdx.x % plan.xcds), lw = uni(blockIdx.x / plan.xcds);
+    const uint32_t pj = uni(lw % plan.pairs), set = uni(lw / plan.pairs);
+    uint32_t en_k = set, en_sub = 0;
+    // The history length of an item's batch row is read when the item is enumerated and clamped
+    // when the item becomes the current one (an item later), so that nobody waits for the load.
+    auto next_item = [&](uint64_t &raw_past) __attribute__((always_inline)) -> Item {
+        Item it{0, 0, kNoItem, 0};
+        raw_past = 0;
+        while (en_k < plan.spx) {
+            const uint32_t heavy = plan.q_tiles - 1 - pj;
+            const uint32_t qt = en_sub == 0 ? heavy : pj;
+            const bool ok = en_sub == 0 || pj != heavy;
+            const uint32_t stream = en_k * plan.xcds + xcd;
+            if (en_sub == 0) {
+                en_sub = 1;
+            } else {
+                en_sub = 0;
+                en_k += plan.groups;
+            }
+            if (!ok) continue;
+            // (a plain integer division would run on the vector ALU and leave its results, and every
+            // address derived from them, in vector registers)
+            it.kvhead = div_magic(stream, plan.magic_chunks);
+            it.hc = stream - it.kvhead * plan.head_chunks;
+            it.qt = qt;
+            if (a.kc && a.past) raw_past = static_cast<uint64_t>(a.past[a.past_per_row ? div_magic(it.kvhead, plan.magic_hkv) : 0]);
+            break;
+        }
+        return it;
+    };
+    auto clamp_past = [&](uint64_t raw) __attribute__((always_inline)) -> uint32_t {
+        // the two words are moved to scalar registers one by one and compared there (a 64-bit signed
+        // comparison would be done on the vector ALU and drag everything that depends on the history
+        // length into vector registers)
+        const uint32_t lo = uni(static_cast<uint32_t>(raw)), hi = uni(static_cast<uint32_t>(raw >> 32));
+        const uint32_t room = a.cap > a.seq ? a.cap - a.seq : 0;
+        const uint32_t len = hi == 0 ? lo : (hi >> 31 ? 0u : room);  // negative: 0; beyond 32 bits: the upper end
+        return len < room ? len : room;
+    };
 
-    const T *Q = static_cast<const T *>(a.q);
-    const T *Kn = static_cast<const T *>(a.k);
-    const T *Vn = static_cast<const T *>(a.v);
-    T *Kc = static_cast<T *>(a.kc);
-    T *Vc = static_cast<T *>(a.vc);
+    const uint8_t *Q = static_cast<const uint8_t *>(a.q);
+    const uint8_t *Kn = static_cast<const uint8_t *>(a.k);
+    const uint8_t *Vn = static_cast<const uint8_t *>(a.v);
+    uint8_t *Kc = static_cast<uint8_t *>(a.kc);
+    uint8_t *Vc = static_cast<uint8_t *>(a.vc);
     T *O = static_cast<T *>(a.o);
-    const uint64_t kv_head = static_cast<uint64_t>(b) * a.Hkv + kvh;
-    const T *k_new = Kn + kv_head * a.seq * D;
-    const T *v_new = Vn + kv_head * a.seq * D;
-    const T *k_hist = Kc ? Kc + kv_head * a.cap * D : nullptr;
-    const T *v_hist = Vc ? Vc + kv_head * a.cap * D : nullptr;
-
-    const uint32_t head = kvh * group + hc * HW + wave % HW;
-    const uint32_t r0 = qt * ROWS + 32 * (wave / HW);  // first query row of this wavefront
-    const bool wave_active = r0 < a.seq;
-    const uint32_t wg_rows_end = (qt + 1) * ROWS < a.seq ? (qt + 1) * ROWS : a.seq;
-
-    // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
-    Raw16 qf[8];
-    {
-        const uint32_t qrow = r0 + l32 < a.seq ? r0 + l32 : a.seq - 1;
-        const T *qp = Q + ((static_cast<uint64_t>(b) * a.H + head) * a.seq + qrow) * D + 8 * half;
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qp + 16 * kk);
-    }
-
-    // history length of this batch row, clamped so that the new rows fit the cache (read after the
-    // query loads are on their way: they do not depend on it)
-    uint32_t base = 0;
-    if (a.kc && a.past) {
-        int64_t raw = a.past[a.past_per_row ? b : 0];
-        if (raw < 0) raw = 0;
-        const int64_t room = static_cast<int64_t>(a.cap) - static_cast<int64_t>(a.seq);
-        if (raw > room) raw = room < 0 ? 0 : room;
-        base = static_cast<uint32_t>(raw);
-    }
-
-    const uint32_t wg_last_key = base + wg_rows_end - 1;  // inclusive
-    const uint32_t n_tiles = wg_last_key / BN + 1;
-    const uint32_t wave_last_row = r0 + 31 < a.seq ? r0 + 31 : a.seq - 1;
-    const uint32_t wave_tiles = wave_active ? (base + wave_last_row) / BN + 1 : 0;
-    const uint32_t qpos = base + r0 + l32;  // absolute position of this lane's query row
     const float c_log2e = a.scale * 1.4426950408889634f;
 
-    // Tile copies: wavefront w copies key rows 16 w .. 16 w + 15 of K and of V, four rows (1 KiB)
-    // per instruction; this lane brings chunk position lane % 16 of row 16 w + 4 i + lane / 16.
-    // A tile that lies inside the history or inside the new rows is addressed as a uniform base
-    // plus a per-lane byte offset prepared once (rows of the new tensors beyond the workgroup's last
-    // key are read along: they are masked); only a tile that straddles the two tensors or the end
-    // of the new rows computes its addresses row by row.
-    const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // ---- copies.  Tile: wavefront w copies key rows 16 w .. 16 w + 15 of K and of V, four rows
+    // (1 KiB) per instruction; this lane brings chunk position lane % 16 of row 16 w + 4 i + lane / 16.
+    // A tile that lies inside the history or inside the new rows is addressed as a uniform base plus
+    // a per-lane byte offset prepared once (rows of the new tensors beyond the last key are read
+    // along: they are masked); only a tile that straddles the two tensors or the end of the new rows
+    // computes its addresses row by row.  The tensors' addresses are formed from the kernel arguments
+    // by scalar arithmetic at every call: scalar registers are what this kernel is short of, scalar
+    // instructions it has to spare.
     const uint32_t cp_row = (BN / 4) * wave_u + (lane >> 4);
     const uint32_t v_lane = cp_row * ROWB + 16 * ((lane & 15) ^ v_swizzle(lane >> 4));
     // K: chunk position lane % 16 of row r holds chunk (lane % 16) ^ (r & 15); rows 4 i further on flip
     // bits 2-3 of the chunk index, i.e. bits 6-7 of the byte offset
     const uint32_t k_lane = cp_row * ROWB + 16 * ((lane & 15) ^ (cp_row & 15));
-    const uint32_t total_keys = base + a.seq;
-    typedef const __attribute__((address_space(1))) void *GlobalPtr;
-    typedef __attribute__((address_space(3))) void *LdsPtr;
-    auto copy_tile = [&](uint32_t kt, uint8_t *buf) {
-        const uint32_t first = kt * BN;
-        const bool in_hist = first + BN <= base, in_new = first >= base && first + BN <= total_keys;
+    auto copy_tile = [&](const Item &it, uint32_t kt, uint32_t buf) __attribute__((always_inline)) {
+        const uint32_t first = kt * BN, total_keys = it.base + a.seq;
+        const bool in_hist = first + BN <= it.base, in_new = first >= it.base && first + BN <= total_keys;
+        const uint32_t kdst = lds_addr0 + buf + CPI * wave_u * 1024, vdst = kdst + TILE;
         if (in_hist || in_new) {  // uniform
-            const uint64_t tile_off = static_cast<uint64_t>(in_hist ? first : first - base) * ROWB;
-            const uint8_t *kb_ = reinterpret_cast<const uint8_t *>(in_hist ? k_hist : k_new) + tile_off;
-            const uint8_t *vb_ = reinterpret_cast<const uint8_t *>(in_hist ? v_hist : v_new) + tile_off;
-#pragma unroll
-            for (int i = 0; i < CPI; ++i) {
-                __builtin_amdgcn_global_load_lds((GlobalPtr)(kb_ + ((k_lane ^ (64 * i)) + 4 * i * ROWB)), (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((GlobalPtr)(vb_ + v_lane + 4 * i * ROWB), (LdsPtr)(buf + TILE + (CPI * wave_u + i) * 1024), 16, 0, 0);
-            }
+            const uint64_t row0 = in_hist ? static_cast<uint64_t>(it.kvhead) * a.cap + first
+                                          : static_cast<uint64_t>(it.kvhead) * a.seq + (first - it.base);
+            const uint8_t *kb_ = (in_hist ? Kc : Kn) + row0 * ROWB;
+            const uint8_t *vb_ = (in_hist ? Vc : Vn) + row0 * ROWB;
+            static_assert(CPI == 4, "four copies of four rows per wavefront and tensor");
+            // (the instruction's offset moves the global and the LDS address alike: four rows are 1 KiB in both)
+            copy16<0>(kb_, k_lane, kdst);
+            copy16<0>(vb_, v_lane, vdst);
+            copy16<4 * ROWB>(kb_, k_lane ^ 64, kdst);
+            copy16<4 * ROWB>(vb_, v_lane, vdst);
+            copy16<8 * ROWB>(kb_, k_lane ^ 128, kdst);
+            copy16<8 * ROWB>(vb_, v_lane, vdst);
+            copy16<12 * ROWB>(kb_, k_lane ^ 192, kdst);
+            copy16<12 * ROWB>(vb_, v_lane, vdst);
         } else {
+            const uint8_t *kh = Kc + static_cast<uint64_t>(it.kvhead) * a.cap * ROWB;
+            const uint8_t *vh = Vc + static_cast<uint64_t>(it.kvhead) * a.cap * ROWB;
+            const uint8_t *kn = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
+            const uint8_t *vn = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
 #pragma unroll
             for (int i = 0; i < CPI; ++i) {
                 uint32_t pos = first + cp_row + 4 * i;
                 pos = pos < total_keys ? pos : total_keys - 1;
-                const bool old = pos < base;
-                const uint64_t row_off = static_cast<uint64_t>(old ? pos : pos - base) * D;
+                // a wavefront's 16 rows may lie on both sides of the seam: the side is chosen per lane
+                // by handing the copy the lane's full address (no scalar base)
+                const bool old = pos < it.base;
+                const uint32_t row_off = (old ? pos : pos - it.base) * ROWB;  // within one kv head: below 2^32
                 const uint32_t kc = (lane & 15) ^ ((cp_row + 4 * i) & 15), vc = (lane & 15) ^ v_swizzle(lane >> 4);
-                const T *ksrc = (old ? k_hist : k_new) + row_off + 8 * kc;
-                const T *vsrc = (old ? v_hist : v_new) + row_off + 8 * vc;
-                __builtin_amdgcn_global_load_lds((GlobalPtr)ksrc, (LdsPtr)(buf + (CPI * wave_u + i) * 1024), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((GlobalPtr)vsrc, (LdsPtr)(buf + TILE + (CPI * wave_u + i) * 1024), 16, 0, 0);
+                const uint8_t *ksrc = (old ? kh : kn) + (row_off + 16 * kc);
+                const uint8_t *vsrc = (old ? vh : vn) + (row_off + 16 * vc);
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(ksrc), "s"(kdst + i * 1024) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(vsrc), "s"(vdst + i * 1024) : "memory", "m0");
+            }
+        }
+    };
+    // Query rows of an item: every wavefront copies its own 32 rows (8 KiB, contiguous in memory)
+    // into its quarter of the buffer, laid out like a K tile (chunk c of row r at position c ^ (r & 15)).
+    auto copy_q = [&](const Item &it, uint32_t buf) __attribute__((always_inline)) {
+        // (b * H + head) = kvhead * group + the head's index within the group
+        const uint32_t bh = uni(it.kvhead * plan.group + it.hc * HW + wave_u % HW);
+        const uint32_t r0 = it.qt * ROWS + 32 * (wave_u / HW);
+        const uint8_t *qh = Q + static_cast<uint64_t>(bh) * a.seq * ROWB;
+        const uint32_t dst = lds_addr0 + buf + wave_u * (32 * ROWB);
+        if (r0 + 32 <= a.seq) {
+            // rows 4 i + lane / 16: the same offset pattern as a K tile's
+            const uint8_t *qb = qh + static_cast<uint64_t>(r0) * ROWB;
+            const uint32_t q_lane = (lane >> 4) * ROWB + 16 * ((lane & 15) ^ (lane >> 4));
+            copy16<0>(qb, q_lane, dst);
+            copy16<4 * ROWB>(qb, q_lane ^ 64, dst);
+            copy16<8 * ROWB>(qb, q_lane ^ 128, dst);
+            copy16<12 * ROWB>(qb, q_lane ^ 192, dst);
+            const uint8_t *qb2 = qb + 16 * ROWB;  // (the instruction's offset field ends at 4095)
+            copy16<0>(qb2, q_lane, dst + 4096);
+            copy16<4 * ROWB>(qb2, q_lane ^ 64, dst + 4096);
+            copy16<8 * ROWB>(qb2, q_lane ^ 128, dst + 4096);
+            copy16<12 * ROWB>(qb2, q_lane ^ 192, dst + 4096);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t row = 4 * i + (lane >> 4);
+                uint32_t grow = r0 + row;
+                grow = grow < a.seq ? grow : a.seq - 1;
+                copy16<0>(qh, grow * ROWB + 16 * ((lane & 15) ^ (row & 15)), dst + i * 1024);  // within one head: below 2^32
             }
         }
     };
 
-    f16v o[4];
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
-    float m = 0.f, l = 0.f;
-    bool fresh = true;
-
-    copy_tile(0, lds0);
-    // query fragments and tile 0 have landed
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-
-    // fragment addresses inside a buffer: K row l32 (+ 32 kb), chunk 2 kk + half; V see below
+    // fragment addresses inside a buffer: K (or Q) row l32 (+ 32 kb), chunk 2 kk + half; V see below
     const uint32_t k_off = l32 * ROWB + 16 * (half ^ (l32 & 15));
     // V piece of block db: row 4 half + r (+ 32 kb + 16 jj, + 8), chunk 4 db + cl; the swizzle leaves
     // 4 db to bits 6-7 of the byte offset, so a block is reached by XOR with 64 db
     const uint32_t s16 = lane & 15, v_r = s16 >> 2, v_cl = 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1);
     const uint32_t v_off = TILE + (4 * half + v_r) * ROWB + 16 * (v_cl ^ v_swizzle(v_r)) + 8 * (s16 & 1);
 
-    auto tile = [&]<int P>(uint32_t kt) __attribute__((always_inline)) {
-        uint8_t *const buf = P ? lds1 : lds0, *const other = P ? lds0 : lds1;
-        // The copy of tile kt+1 into the other buffer (free since the barrier that ended tile kt-1)
-        // is issued behind this tile's first fragment reads: the compiler waits for every copy in
-        // flight before the first read of a buffer that a copy has written, and at that point
-        // none is.
-        if (kt >= wave_tiles && kt + 1 < n_tiles) copy_tile(kt + 1, other);
-        if (kt < wave_tiles) {
-            // S^T block kb: keys BN kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32.  With two
-            // blocks per tile (BN = 64) both are issued first; the softmax of a block then runs on
-            // the VALU while the matrix core still works on the next product (S^T of block 1, or
-            // the PV update of block 0), and a block entirely above the diagonal is skipped.
-            const bool second = KB > 1 && kt * BN + 32 <= base + r0 + 31;
-            f16v s[KB];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
-                if (kb == 0 || second) {
-#pragma unroll
-                    for (int kk = 0; kk < 8; ++kk) {
-                        const Raw16 kf = *reinterpret_cast<const Raw16 *>(buf + 32 * kb * ROWB + (k_off ^ (32 * kk)));
-                        s[kb] = Ops<T>::mfma(kf, qf[kk], s[kb]);
-                    }
-                }
-            }
-            if (kt + 1 < n_tiles) copy_tile(kt + 1, other);
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                if (kb == 1 && !second) break;
-                // scale, causal mask (only blocks that reach past the wavefront's first query position)
-                const bool need_mask = kt * BN + 32 * kb + 31 > base + r0;
-                float over = -__builtin_inff();
-                if (need_mask) {  // wave-uniform: only the blocks on the diagonal pay for the comparisons
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
-                        const float t = key > qpos ? -__builtin_inff() : fmaf(s[kb][e], c_log2e, -m);
-                        s[kb][e] = t;
-                        over = fmaxf(over, t);
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const float t = fmaf(s[kb][e], c_log2e, -m);
-                        s[kb][e] = t;
-                        over = fmaxf(over, t);
-                    }
-                }
-                over = fmaxf(over, __shfl_xor(over, 32, kWave));  // both halves hold the same query row
-                if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
-                    const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
-                    const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
-                    m += up;
-                    l *= alpha;
-#pragma unroll
-                    for (int db = 0; db < 4; ++db)
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) s[kb][e] -= up;
-                    fresh = false;
-                }
-                // P^T in B-operand position: element i of MFMA (kb, jj) is accumulator register 8 jj + i
-                Raw16 pf[2];
-#pragma unroll
-                for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                    for (int i2 = 0; i2 < 4; ++i2) {
-                        const float p0 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2]);
-                        const float p1 = __builtin_amdgcn_exp2f(s[kb][8 * jj + 2 * i2 + 1]);
-                        l += p0 + p1;
-                        pf[jj].w[i2] = Ops<T>::pack2(p0, p1);
-                    }
-                // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
-                // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
-                // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
-                // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
-#pragma unroll
-                for (int db = 0; db < 4; ++db)
-#pragma unroll
-                    for (int jj = 0; jj < 2; ++jj) {
-                        const uint8_t *vp = buf + (32 * kb + 16 * jj) * ROWB + (v_off ^ (64 * db));
-                        const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * ROWB);
-                        const Raw16 vf{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
-                        o[db] = Ops<T>::mfma(vf, pf[jj], o[db]);
-                    }
-            }
-        }
-
-        // This wavefront's copies of tile kt+1 have landed and its reads of this buffer are done;
-        // after the barrier that holds for the workgroup.
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-    };
-    for (uint32_t kt = 0; kt < n_tiles; kt += 2) {
-        tile.template operator()<0>(kt);
-        if (kt + 1 < n_tiles) tile.template operator()<1>(kt + 1);
-    }
-
-    // The new rows that correspond to this workgroup's query rows are appended to the caches (once
-    // per kv head): thread owns 16-byte chunk tid % 16 of rows tid / 16 + 16 j.  The loads are
-    // issued here and the stores follow the output write-out, which hides their latency.
+    // ---- state of the item being worked on
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    const bool do_append = Kc && hc == 0;
-    const uint32_t own_lo = base + qt * ROWS, own_hi = base + wg_rows_end;
-    u32x4 ak[ROWS / 16], av[ROWS / 16];
-    if (do_append) {
-#pragma unroll
-        for (int j = 0; j < ROWS / 16; ++j) {
-            uint32_t pos = own_lo + (tid >> 4) + 16 * j;
-            pos = pos < own_hi ? pos : own_hi - 1;  // loads stay unconditional, the stores are guarded
-            const uint64_t off = static_cast<uint64_t>(pos - base) * D + (tid & 15) * 8;
-            ak[j] = *reinterpret_cast<const u32x4 *>(k_new + off);
-            av[j] = *reinterpret_cast<const u32x4 *>(v_new + off);
-        }
-    }
-
-    // ---- normalise, transpose O^T -> O through LDS, 128-bit row-contiguous stores
-    l += __shfl_xor(l, 32, kWave);
-    const float inv = 1.f / l;
-    // the K/V tiles are no longer needed (barrier above, no copy in flight): two wavefronts per buffer
-    uint8_t *ldsO = (wave & 2 ? lds1 : lds0) + (wave & 1) * (32 * ROWB);  // chunk c of row r at chunk position c ^ (r & 15)
-    if (wave_active) {
+    Raw16 qf[8];   // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
+    f16v o[4];
+    float m = 0.f, l = 0.f;
+    bool fresh = true;
+    Item cur{0, 0, kNoItem, 0};
+    uint64_t nxt_raw = 0, nn_raw = 0;
+    Item nxt = next_item(nxt_raw);
+    if (!nxt.valid()) return;
+    nxt.base = clamp_past(nxt_raw);
+    uint32_t r0 = 0, n_tiles = 0, wave_tiles = 0, qpos = 0;
+    auto begin_item = [&]() __attribute__((always_inline)) {
+        r0 = cur.qt * ROWS + 32 * (wave_u / HW);
+        const uint32_t rows_end = (cur.qt + 1) * ROWS < a.seq ? (cur.qt + 1) * ROWS : a.seq;
+        n_tiles = uni((cur.base + rows_end - 1) / BN + 1);
+        const uint32_t wave_last_row = r0 + 31 < a.seq ? r0 + 31 : a.seq - 1;
+        wave_tiles = uni(r0 < a.seq ? (cur.base + wave_last_row) / BN + 1 : 0);
+        qpos = cur.base + r0 + l32;  // absolute position of this lane's query row
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const uint32_t d = 32 * db + 8 * (e / 4) + 4 * half + (e % 4);
-                *reinterpret_cast<uint32_t *>(ldsO + l32 * ROWB + ((2 * d) ^ (16 * (l32 & 15)))) =
-                    Ops<T>::pack2(o[db][e] * inv, o[db][e + 1] * inv);
-            }
-    }
-    // (each wavefront reads back only what it wrote itself: no barrier)
-    if (wave_active) {
-        // computed afresh from an opaque copy of the wavefront index: otherwise the address is built in the
-        // prologue, next to the query pointer it resembles, and kept in scratch memory across the tile loop
-        uint32_t wave_e = wave;
-        asm volatile("" : "+v"(wave_e));
-        const uint32_t head_e = kvh * group + hc * HW + wave_e % HW, r0_e = qt * ROWS + 32 * (wave_e / HW);
-        T *op = O + ((static_cast<uint64_t>(b) * a.H + head_e) * a.seq + r0_e) * D;
+            for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+        m = 0.f;
+        l = 0.f;
+        fresh = true;
+    };
+
+    // ---- the new k/v rows that correspond to an item's query rows go to the caches (once per kv head):
+    // thread owns 16-byte chunk tid % 16 of rows tid / 16 + 16 j.  They are picked up behind the
+    // item's last key tile, whose buffer still holds them unless the item's rows straddle two tiles
+    // (then they are loaded from the inputs again), and stored when the item goes out.
+    auto load_own_rows = [&](const Item &it, uint32_t buf, u32x4 (&ak)[ROWS / 16], u32x4 (&av)[ROWS / 16]) __attribute__((always_inline)) {
+        if (!(Kc && it.hc == 0)) return;
+        const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
+        const uint32_t lo = it.qt * ROWS;
+        const uint32_t tile_first = (n_tiles - 1) * BN;  // first key of the last tile
+        uint32_t tid = threadIdx.x;  // (opaque copy, see finish_item)
+        asm volatile("" : "+v"(tid));
+        if (it.base + lo >= tile_first) {
+            const uint8_t *tb = lds + buf;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t idx = lane + 64 * i, row = idx / 16, c = idx % 16;
-            if (r0 + row < a.seq)
-                *reinterpret_cast<Raw16 *>(op + static_cast<uint64_t>(row) * D + c * 8) =
-                    *reinterpret_cast<const Raw16 *>(ldsO + row * ROWB + 16 * (c ^ (row & 15)));
+            for (int jr = 0; jr < ROWS / 16; ++jr) {
+                uint32_t row = lo + (tid >> 4) + 16 * jr;
+                row = row < rows_end ? row : rows_end - 1;  // reads stay unconditional, the stores are guarded
+                const uint32_t r = it.base + row - tile_first, c = tid & 15;
+                ak[jr] = *reinterpret_cast<const u32x4 *>(tb + r * ROWB + 16 * (c ^ (r & 15)));
+                av[jr] = *reinterpret_cast<const u32x4 *>(tb + TILE + r * ROWB + 16 * (c ^ v_swizzle(r & 3)));
+            }
+        } else {
+            const uint8_t *k_new = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
+            const uint8_t *v_new = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
+#pragma unroll
+            for (int jr = 0; jr < ROWS / 16; ++jr) {
+                uint32_t row = lo + (tid >> 4) + 16 * jr;
+                row = row < rows_end ? row : rows_end - 1;
+                const uint32_t off = row * ROWB + (tid & 15) * 16;
+                ak[jr] = *reinterpret_cast<const u32x4 *>(k_new + off);
+                av[jr] = *reinterpret_cast<const u32x4 *>(v_new + off);
+            }
         }
-    }
-    if (do_append) {
+    };
+
+    // ---- output of a finished item: normalise and transpose through LDS, so that a store instruction
+    // covers four whole rows (1 KiB contiguous) instead of 64 scattered pieces.  The wavefront uses
+    // its own quarter of the query buffer (`stage`), which nobody else touches and whose query rows
+    // it has already taken: chunk c of row r at chunk position c ^ (r & 15).  Then the item's own new rows.
+    auto finish_item = [&](const Item &it, const u32x4 (&ak)[ROWS / 16], const u32x4 (&av)[ROWS / 16], uint8_t *stage) __attribute__((always_inline)) {
+        const uint32_t bh = uni(it.kvhead * plan.group + it.hc * HW + wave_u % HW);
+        const uint32_t fr0 = it.qt * ROWS + 32 * (wave_u / HW);
+        const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
+        const bool do_append = Kc && it.hc == 0;
+        const uint32_t own_lo = it.base + it.qt * ROWS, own_hi = it.base + rows_end;
+        // (lane indices from an opaque copy: the addresses below are then formed here, once per item, and
+        // not ahead of the loops, where they would occupy registers all the time)
+        uint32_t tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const uint32_t lane = tid & 63, l32 = tid & 31, half = (tid >> 5) & 1;
+        if (fr0 < a.seq) {
+            const float inv = 1.f / half_sum(l);
 #pragma unroll
-        for (int j = 0; j < ROWS / 16; ++j) {
-            const uint32_t pos = own_lo + (tid >> 4) + 16 * j;
-            if (pos < own_hi) {
-                const uint64_t dst = (kv_head * a.cap + pos) * D + (tid & 15) * 8;
-                *reinterpret_cast<u32x4 *>(Kc + dst) = ak[j];
-                *reinterpret_cast<u32x4 *>(Vc + dst) = av[j];
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // registers 4 g .. 4 g + 3 of a block: d = 32 db + 8 g + 4 half + 0..3 of row l32
+                    const uint2 w = make_uint2(Ops<T>::pack2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv),
+                                               Ops<T>::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv));
+                    *reinterpret_cast<uint2 *>(stage + l32 * ROWB + 16 * ((4 * db + g) ^ (l32 & 15)) + 8 * half) = w;
+                }
+            // (each wavefront reads back only what it wrote itself: no barrier)
+            uint8_t *op = reinterpret_cast<uint8_t *>(O) + (static_cast<uint64_t>(bh) * a.seq + fr0) * ROWB;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t row = 4 * i + (lane >> 4), c = lane & 15;
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + 16 * (c ^ (row & 15)));
+                if (fr0 + row < a.seq) *reinterpret_cast<u32x4 *>(op + row * ROWB + 16 * c) = v;
             }
+        }
+        if (do_append) {
+#pragma unroll
+            for (int jr = 0; jr < ROWS / 16; ++jr) {
+                const uint32_t pos = own_lo + (tid >> 4) + 16 * jr;
+                if (pos < own_hi) {
+                    const uint64_t dst = (static_cast<uint64_t>(it.kvhead) * a.cap + pos) * ROWB + (tid & 15) * 16;
+                    *reinterpret_cast<u32x4 *>(Kc + dst) = ak[jr];
+                    *reinterpret_cast<u32x4 *>(Vc + dst) = av[jr];
+                }
+            }
+        }
+    };
+
+    // ---- one key tile in buffer `buf` (byte offset of the buffer within `lds`).  The scheduling
+    // fences keep the order written here: fragment reads four ahead of the products that use them.
+    auto tile = [&](uint32_t buf, uint32_t kt) __attribute__((always_inline)) {
+        const uint32_t other = buf ^ BUF_BYTES;
+        // The copy of the next slot (the next key tile, or the next item's query rows) is issued in
+        // eight parts, one behind each of the first eight products: a copy instruction that finds the
+        // memory pipeline busy holds the wavefront, and there it waits under a product instead of
+        // ahead of them.  Both kinds of copy have the same shape: parts 0, 2, 4, 6 take four rows each
+        // from `base_a`, parts 1, 3, 5, 7 from `base_b`.  A key tile that straddles the seam between
+        // history and new rows, or ragged query rows, are copied at once (mode 2).
+        uint32_t mode = 0, dst_a = 0, dst_b = 0;
+        bool is_q = false;
+        const uint8_t *base_a = nullptr, *base_b = nullptr;
+        const uint32_t q_lane = (lane >> 4) * ROWB + 16 * ((lane & 15) ^ (lane >> 4));
+        const uint32_t vq_lane = (lane >> 4) * ROWB + 16 * ((lane & 15) ^ v_swizzle(lane >> 4));
+        if (kt + 1 < n_tiles) {
+            const uint32_t first = (kt + 1) * BN, total_keys = cur.base + a.seq;
+            const bool in_hist = first + BN <= cur.base, in_new = first >= cur.base && first + BN <= total_keys;
+            if (in_hist || in_new) {
+                const uint64_t row0 = (in_hist ? static_cast<uint64_t>(cur.kvhead) * a.cap + first
+                                               : static_cast<uint64_t>(cur.kvhead) * a.seq + (first - cur.base)) +
+                                      (BN / 4) * wave_u;
+                base_a = (in_hist ? Kc : Kn) + row0 * ROWB;
+                base_b = (in_hist ? Vc : Vn) + row0 * ROWB;
+                dst_a = lds_addr0 + other + CPI * wave_u * 1024;
+                dst_b = dst_a + TILE;
+                mode = 1;
+            } else {
+                mode = 2;
+            }
+        } else if (nxt.valid()) {
+            const uint32_t nr0 = nxt.qt * ROWS + 32 * (wave_u / HW);
+            if (nr0 + 32 <= a.seq) {
+                const uint32_t bh = uni(nxt.kvhead * plan.group + nxt.hc * HW + wave_u % HW);
+                base_a = Q + (static_cast<uint64_t>(bh) * a.seq + nr0) * ROWB;
+                base_b = base_a + 16 * ROWB;
+                dst_a = lds_addr0 + other + wave_u * (32 * ROWB);
+                dst_b = dst_a + 16 * ROWB;
+                is_q = true;
+                mode = 1;
+            } else {
+                mode = 2;
+            }
+        }
+        auto copy_part = [&]<int I>() __attribute__((always_inline)) {
+            if (mode != 1) return;
+            constexpr int J = I / 2;
+            if (I % 2 == 0) copy16<J * 4 * ROWB>(base_a, q_lane ^ (64 * J), dst_a);
+            else copy16<J * 4 * ROWB>(base_b, is_q ? q_lane ^ (64 * J) : vq_lane, dst_b);
+        };
+        auto copy_rest = [&]() __attribute__((always_inline)) {  // what the parts do not cover
+            if (mode != 2) return;
+            if (kt + 1 < n_tiles) copy_tile(cur, kt + 1, other);
+            else copy_q(nxt, other);
+        };
+        if (kt >= wave_tiles) {
+            copy_part.template operator()<0>();
+            copy_part.template operator()<1>();
+            copy_part.template operator()<2>();
+            copy_part.template operator()<3>();
+            copy_part.template operator()<4>();
+            copy_part.template operator()<5>();
+            copy_part.template operator()<6>();
+            copy_part.template operator()<7>();
+            copy_rest();
+            return;
+        }
+        const uint8_t *const tb = lds + buf;
+        // a block entirely above the diagonal is skipped
+        const bool second = KB > 1 && kt * BN + 32 <= cur.base + r0 + 31;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb == 1 && !second) break;
+            // S^T block kb: keys BN kt + 32 kb + (8 (e/4) + 4 half + e%4), query row l32
+            Raw16 kf[4];
+            const uint8_t *kb_base = tb + 32 * kb * ROWB;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) kf[kk] = *reinterpret_cast<const Raw16 *>(kb_base + (k_off ^ (32 * kk)));
+            if (kb == 0) copy_rest();
+            RG_SCHED_FENCE();
+            f16v sc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sc[e] = 0.f;
+            auto product = [&]<int KK>() __attribute__((always_inline)) {
+                sc = Ops<T>::mfma(kf[KK % 4], qf[KK], sc);
+                if (KK + 4 < 8) kf[KK % 4] = *reinterpret_cast<const Raw16 *>(kb_base + (k_off ^ (32 * (KK + 4))));
+                if (kb == 0) copy_part.template operator()<KK>();
+                RG_SCHED_FENCE();
+            };
+            product.template operator()<0>();
+            product.template operator()<1>();
+            product.template operator()<2>();
+            product.template operator()<3>();
+            product.template operator()<4>();
+            product.template operator()<5>();
+            product.template operator()<6>();
+            product.template operator()<7>();
+            // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
+            // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
+            // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
+            // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
+            // (product index i = 4 jj + db; the first four fragments are requested before the softmax)
+            auto read_v = [&](int i) __attribute__((always_inline)) {
+                const int jj = i / 4, db = i % 4;
+                const uint8_t *vp = tb + (32 * kb + 16 * jj) * ROWB + (v_off ^ (64 * db));
+                const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * ROWB);
+                return Raw16{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
+            };
+            Raw16 vf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vf[i] = read_v(i);
+            RG_SCHED_FENCE();
+            // scale, causal mask (only blocks that reach past the wavefront's first query position)
+            const bool need_mask = kt * BN + 32 * kb + 31 > cur.base + r0;
+            float over = -__builtin_inff();
+            if (need_mask) {  // wave-uniform: only the blocks on the diagonal pay for the comparisons
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
+                    const float t = key > qpos ? -__builtin_inff() : fmaf(sc[e], c_log2e, -m);
+                    sc[e] = t;
+                    over = fmaxf(over, t);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float t = fmaf(sc[e], c_log2e, -m);
+                    sc[e] = t;
+                    over = fmaxf(over, t);
+                }
+            }
+            over = half_max(over);  // both halves hold the same query row
+            if (fresh || __builtin_amdgcn_ballot_w64(over > kSlack) != 0) {
+                const float up = fresh ? fmaxf(over, kMinusBig) : fmaxf(over, 0.f);
+                const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-up);
+                m += up;
+                l *= alpha;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) sc[e] -= up;
+                fresh = false;
+            }
+            // P^T in B-operand position: element i of MFMA (kb, jj) is accumulator register 8 jj + i
+            Raw16 pf[2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int i2 = 0; i2 < 4; ++i2) {
+                    const float p0 = __builtin_amdgcn_exp2f(sc[8 * jj + 2 * i2]);
+                    const float p1 = __builtin_amdgcn_exp2f(sc[8 * jj + 2 * i2 + 1]);
+                    pf[jj].w[i2] = Ops<T>::pack2(p0, p1);
+                    l = Ops<T>::add_pair(l, pf[jj].w[i2], p0, p1);
+                }
+            RG_SCHED_FENCE();
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                o[i % 4] = Ops<T>::mfma(vf[i % 4], pf[i / 4], o[i % 4]);
+                if (i + 4 < 8) vf[i % 4] = read_v(i + 4);
+                RG_SCHED_FENCE();
+            }
+        }
+    };
+
+    // ---- the slot of the next item's query rows (in buffer `buf`; the other buffer still holds the
+    // last key tile of the item just finished): every wavefront takes its query fragments and the
+    // finished item's own new rows out of LDS; after a barrier tile 0 of the next item is requested
+    // into the buffer thus freed, and the finished item goes out while it travels
+    bool have_cur = false;
+    auto q_slot = [&](uint32_t buf) __attribute__((always_inline)) -> bool {
+        Item nn{0, 0, kNoItem, 0};
+        u32x4 ak[ROWS / 16], av[ROWS / 16];
+        if (have_cur) load_own_rows(cur, buf ^ BUF_BYTES, ak, av);
+        if (nxt.valid()) {
+            const uint8_t *qb = lds + buf + wave_u * (32 * ROWB);
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qb + (k_off ^ (32 * kk)));
+            if (have_cur) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+            }
+            copy_tile(nxt, 0, buf ^ BUF_BYTES);
+            nn = next_item(nn_raw);  // its history length is on its way while the output goes out
+        }
+        if (have_cur) finish_item(cur, ak, av, lds + buf + wave_u * (32 * ROWB));
+        if (!nxt.valid()) return false;
+        cur = nxt;
+        nxt = nn;
+        nxt.base = clamp_past(nn_raw);
+        have_cur = true;
+        begin_item();
+        return true;
+    };
+    auto end_slot = [&]() __attribute__((always_inline)) {
+        // this wavefront's copies for the next slot have landed and its reads of this slot's buffer
+        // are done; after the barrier that holds for the workgroup
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    };
+
+    // slot sequence: the query slot of an item, then its key tiles; the buffer alternates with every slot
+    copy_q(nxt, 0);
+    end_slot();
+    uint32_t buf = 0;
+    for (;;) {
+        if (!q_slot(buf)) break;
+        end_slot();
+        buf ^= BUF_BYTES;
+        for (uint32_t kt = 0; kt < n_tiles; ++kt) {
+            tile(buf, kt);
+            end_slot();
+            buf ^= BUF_BYTES;
         }
     }
 }
 
 template <class T, int HW>
+uint32_t resident_prefill_workgroups() {
+    static uint32_t cached = [] {
+        int per_cu = 0, dev = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_prefill<T, HW>, 256, 0) != hipSuccess || per_cu <= 0)
+            per_cu = 2;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+        return static_cast<uint32_t>(per_cu) * static_cast<uint32_t>(cus);
+    }();
+    return cached;
+}
+
+template <class T, int HW>
 int launch_hw(const PrefillArgs &a, hipStream_t s) {
-    const uint32_t group = a.H / a.Hkv;
-    const uint32_t head_chunks = group / HW;
     constexpr uint32_t ROWS = 32 * (4 / HW);
-    const uint32_t q_tiles = (a.seq + ROWS - 1) / ROWS;
-    const uint64_t grid = static_cast<uint64_t>(a.N) * a.Hkv * head_chunks * q_tiles;
-    if (grid > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
-    attn_prefill<T, HW><<<static_cast<unsigned>(grid), 256, 0, s>>>(a, group, q_tiles, head_chunks);
+    PrefillPlan plan{};
+    plan.group = a.H / a.Hkv;
+    plan.head_chunks = plan.group / HW;
+    plan.q_tiles = (a.seq + ROWS - 1) / ROWS;
+    plan.pairs = (plan.q_tiles + 1) / 2;
+    const uint64_t streams = static_cast<uint64_t>(a.N) * a.Hkv * plan.head_chunks;
+    if (streams * plan.pairs > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+    plan.xcds = streams % 8 == 0 ? 8 : 1;
+    plan.spx = static_cast<uint32_t>(streams / plan.xcds);
+    // as many sets of `pairs` workgroups per XCD as stay resident together (at least one)
+    const uint32_t per_xcd = resident_prefill_workgroups<T, HW>() / plan.xcds;
+    uint32_t groups = per_xcd / plan.pairs;
+    if (groups < 1) groups = 1;
+    if (groups > plan.spx) groups = plan.spx;
+    plan.groups = groups;
+    const uint64_t widest = plan.head_chunks > a.Hkv ? plan.head_chunks : a.Hkv;
+    if (streams * widest >= (1ull << 32)) return RG_HIP_E_UNSUPPORTED;
+    plan.magic_chunks = plan.head_chunks > 1 ? static_cast<uint32_t>((1ull << 32) / plan.head_chunks + 1) : 0;
+    plan.magic_hkv = a.Hkv > 1 ? static_cast<uint32_t>((1ull << 32) / a.Hkv + 1) : 0;
+    const uint32_t grid = plan.xcds * plan.groups * plan.pairs;
+    attn_prefill<T, HW><<<grid, 256, 0, s>>>(a, plan);
     return launch_status();
 }
 
