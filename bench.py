@@ -493,8 +493,9 @@ def main():
         ops_out["transpose"] = e
         del xs, ys
 
-    if (want("matmul_integer") or want("matmul_integer_dequantize") or want("matmul_integer_few_rows")
-            or want("matmul_integer_one_row")):
+    if any(want(nm) for nm in ("matmul_integer", "matmul_integer_dequantize", "matmul_integer_few_rows", "matmul_integer_one_row",
+                               "matmul_integer_zero_operands", "matmul_integer_small_operands", "matmul_integer_8192",
+                               "matmul_integer_mfma_ceiling")):
         a = torch.randint(0, 256, (4096, 4096), device=dev, dtype=torch.uint8)
         b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
         az = torch.tensor([128], device=dev, dtype=torch.uint8)
@@ -531,6 +532,67 @@ def main():
             ops_out["matmul_integer"]["cpu_baseline_all_cores"] = {
                 "value": round(2 * ma * 4096 * 4096 / dt / 1e12, 5), "unit": "TOP/s", "cores": CPU_THREADS, "kind": "port",
                 "sample": f"first {ma} rows of A against all of B, rows split over the threads ({dt:.1f} s)"}
+        def mmi_entry(name, workload, aa, bb, yy, ops_count):
+            """Further MatMulInteger rows through the same kernel: what the matrix pipe sustains depends on the
+            operand values (power) and on how many tiles a CU gets (one tile per CU leaves its write-out bare)."""
+            wall, d_ms, md = time_steps(torch, lambda i: ops.matmul_integer(aa, bb, az, bz, out=yy), steps, warmup, 1)
+            t_ops = ops_count / (d_ms * 1e-3) / 1e12
+            ent = {"bound": "mfma", "achieved": round(t_ops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                   "frac": round(t_ops / INT8_PEAK_TOPS, 4), "traffic": None, "workload": workload,
+                   "device_ms_per_launch": round(d_ms, 5), "timing": md, "observed_sclk_mhz": LAST["clock"],
+                   "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
+            if LAST["clock"]:
+                at = INT8_PEAK_TOPS * LAST["clock"]["median"] / 2400.0
+                ent["peak_at_observed_clock"] = round(at, 1)
+                ent["frac_at_observed_clock"] = round(t_ops / at, 4)
+            ops_out[name] = ent
+
+        if want("matmul_integer_zero_operands"):
+            a0 = torch.full((4096, 4096), 128, device=dev, dtype=torch.uint8)   # a - a_zp = 0
+            b0 = torch.zeros((4096, 4096), device=dev, dtype=torch.int8)
+            mmi_entry("matmul_integer_zero_operands", "MatMulInteger 4096^3, every operand byte 0 after the zero point "
+                      "(same kernel, same launches: what the operand values cost)", a0, b0, y, 2 * 4096 ** 3)
+            del a0, b0
+        if want("matmul_integer_small_operands"):
+            a0 = torch.randint(121, 136, (4096, 4096), device=dev, dtype=torch.uint8)   # |a - a_zp| < 8
+            b0 = torch.randint(-7, 8, (4096, 4096), device=dev, dtype=torch.int8)
+            mmi_entry("matmul_integer_small_operands", "MatMulInteger 4096^3, operands uniform in -7..7 after the zero point",
+                      a0, b0, y, 2 * 4096 ** 3)
+            del a0, b0
+        if want("matmul_integer_8192"):
+            a0 = torch.randint(0, 256, (8192, 4096), device=dev, dtype=torch.uint8)
+            b0 = torch.randint(-128, 128, (4096, 8192), device=dev, dtype=torch.int8)
+            y0 = torch.empty((8192, 8192), device=dev, dtype=torch.int32)
+            mmi_entry("matmul_integer_8192", "MatMulInteger u8 [8192,4096] x i8 [4096,8192] -> i32 (uniform random bytes; four "
+                      "256 x 256 tiles per CU instead of one)", a0, b0, y0, 2 * 8192 * 8192 * 4096)
+            del a0, b0, y0
+        if want("matmul_integer_mfma_ceiling"):
+            # what the matrix pipe itself sustains: the same 4 x 4 blocks of products from registers (no LDS,
+            # no copies, no write-out), as many per wavefront as the 4096^3 kernel issues, one workgroup per CU
+            from refactorgraph_amd import abi as _abi
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            outp = torch.empty(cus * 256, device=dev, dtype=torch.int32)
+            for nm, opnd, what in (
+                    ("matmul_integer_mfma_ceiling", torch.randint(-128, 128, (8192,), device=dev, dtype=torch.int8),
+                     "uniform random operand bytes"),
+                    ("matmul_integer_mfma_ceiling_zero", torch.zeros(8192, device=dev, dtype=torch.int8), "all-zero operands")):
+                def probe(i, opnd=opnd):
+                    rc = _abi.lib().rg_hip_probe_mfma_i8(outp.data_ptr(), opnd.data_ptr(), cus, 128,
+                                                         torch.cuda.current_stream().cuda_stream)
+                    assert rc == 0, rc
+                wall, d_ms, md = time_steps(torch, probe, steps, warmup, 1)
+                t_ops = cus * 4 * 128 * 16 * 2 * 32 ** 3 / (d_ms * 1e-3) / 1e12
+                ent = {"bound": "mfma", "achieved": round(t_ops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                       "frac": round(t_ops / INT8_PEAK_TOPS, 4), "traffic": None,
+                       "workload": f"register-only loop of 2048 v_mfma_i32_32x32x32_i8 per wavefront, {cus} workgroups of 4 "
+                                   f"wavefronts, {what}: the ceiling of any int8 GEMM on this part for such data",
+                       "device_ms_per_launch": round(d_ms, 5), "timing": md, "observed_sclk_mhz": LAST["clock"],
+                       "warmup_ms": LAST["warmup_ms"]}
+                if LAST["clock"]:
+                    at = INT8_PEAK_TOPS * LAST["clock"]["median"] / 2400.0
+                    ent["peak_at_observed_clock"] = round(at, 1)
+                    ent["frac_at_observed_clock"] = round(t_ops / at, 4)
+                ops_out[nm] = ent
         if want("matmul_integer_dequantize"):
             # the same product with DequantizeLinear (per-column scale) folded into the epilogue, against
             # the two operators one after the other
