@@ -493,6 +493,69 @@ def main():
         ops_out["transpose"] = e
         del xs, ys
 
+    if want("split") or want("concat"):
+        # a fused QKV projection's output taken apart (and put together again): [4096, 12288] fp16 <-> 3 x [4096, 4096];
+        # every byte is read once and written once
+        nb = 3  # 3 x 201 MB
+        xs = [torch.randn((4096, 12288), device=dev).half() for _ in range(nb)]
+        parts = [[torch.empty((4096, 4096), device=dev, dtype=torch.float16) for _ in range(3)] for _ in range(nb)]
+        mv_bytes = 2 * 4096 * 12288 * 2
+        if not args.no_cpu:
+            import oracle
+            xn = xs[0][:512].cpu().numpy()
+            pn = oracle.split(xn, [4096] * 3, 1)
+        if want("split"):
+            wall, dms, mode = time_steps(torch, lambda i: ops.split(xs[i], [4096] * 3, 1, outs=parts[i]), steps, warmup, nb)
+            e = hbm_entry(mv_bytes, dms, "split")
+            e.update(workload="Split fp16 [4096,12288] -> 3 x [4096,4096] along the last axis",
+                     device_ms_per_launch=round(dms, 5), timing=mode)
+            if not args.no_cpu:
+                e["cpu_baseline"] = cpu_leg(lambda: oracle.split(xn, [4096] * 3, 1), mv_bytes // 8, "512 of the 4096 rows")
+            ops_out["split"] = e
+        if want("concat"):
+            wall, dms, mode = time_steps(torch, lambda i: ops.concat(parts[i], 1, out=xs[i]), steps, warmup, nb)
+            e = hbm_entry(mv_bytes, dms, "concat")
+            e.update(workload="Concat fp16 3 x [4096,4096] -> [4096,12288] along the last axis",
+                     device_ms_per_launch=round(dms, 5), timing=mode)
+            if not args.no_cpu:
+                e["cpu_baseline"] = cpu_leg(lambda: oracle.concat(pn, 1), mv_bytes // 8, "512 of the 4096 rows")
+            ops_out["concat"] = e
+        del xs, parts
+
+    if want("where"):
+        # a mask applied to attention scores: c bool [512, 512] broadcast over [32, 32, 512, 512] f32 x, scalar y
+        nb = 3
+        c = torch.ones((512, 512), device=dev).tril().bool()
+        xs = [torch.randn((32, 32, 512, 512), device=dev) for _ in range(nb)]
+        ys = [torch.empty_like(xs[0]) for _ in range(nb)]
+        fill = torch.full((1,), -1e9, device=dev)
+        wall, dms, mode = time_steps(torch, lambda i: ops.where(c, xs[i], fill, out=ys[i]), steps, warmup, nb)
+        wh_bytes = 32 * 32 * 512 * 512 * 8 + 512 * 512 + 4
+        e = hbm_entry(wh_bytes, dms, "where")
+        e.update(workload="Where bool [512,512], f32 [32,32,512,512], f32 [1] -> f32 [32,32,512,512]",
+                 device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            cn, xn, fn = c.cpu().numpy(), xs[0][:1, :4].cpu().numpy(), fill.cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.where(cn, xn, fn), wh_bytes // 256, "4 of the 1024 [512,512] slabs")
+        ops_out["where"] = e
+        del xs, ys
+
+    if want("expand"):
+        # a bias row laid out over a batch of activations: fp16 [1, 4096] -> [32768, 4096]; only the output is traffic
+        y = torch.empty((32768, 4096), device=dev, dtype=torch.float16)
+        x = torch.randn((1, 4096), device=dev).half()
+        wall, dms, mode = time_steps(torch, lambda i: ops.expand(x, (32768, 4096), out=y), steps, warmup, 1)
+        ex_bytes = 32768 * 4096 * 2 + 4096 * 2
+        e = hbm_entry(ex_bytes, dms, "expand")
+        e.update(workload="Expand fp16 [1,4096] -> [32768,4096]", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn = x.cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.expand(xn, (4096, 4096)), ex_bytes // 8, "4096 of the 32768 rows")
+        ops_out["expand"] = e
+        del x, y
+
     if any(want(nm) for nm in ("matmul_integer", "matmul_integer_dequantize", "matmul_integer_few_rows", "matmul_integer_one_row",
                                "matmul_integer_zero_operands", "matmul_integer_small_operands", "matmul_integer_8192",
                                "matmul_integer_mfma_ceiling")):

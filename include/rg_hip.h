@@ -177,6 +177,39 @@ int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtyp
 int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o,
                      size_t dims, size_t block_size, size_t block_count, void *stream);
 
+/* ---- Split / Concat ----------------------------------------------------------------------
+ * replace src/04kernel/cuda/src/split.cu:7-50 and concat.cu:7-50 (+ the launchers in
+ * src/04kernel/src/kernels/{split,concat}/cuda_kernel.cc); contract
+ * src/04kernel/src/kernels/{split,concat}/cpu_kernel.cc with SplitInfo
+ * (src/04kernel/src/attributes/split_info.cc:5-30): the joined tensor is block_count blocks of `sum`
+ * bytes, block i being the segments of the `count` parts one after the other; part j holds
+ * block_count segments of segments[j] bytes.  outputs / inputs and segments: HOST arrays [count]
+ * (device pointers, bytes); the segments add up to `sum`. */
+int rg_hip_split(void *const *outputs, const void *x, const uint32_t *segments, size_t count,
+                 size_t block_count, size_t sum, void *stream);
+int rg_hip_concat(void *y, const void *const *inputs, const uint32_t *segments, size_t count,
+                  size_t block_count, size_t sum, void *stream);
+
+/* ---- Expand ------------------------------------------------------------------------------
+ * replaces src/04kernel/cuda/src/expand.cu:1-56 + src/04kernel/src/kernels/expand/cuda_kernel.cu:9-26;
+ * contract src/04kernel/src/kernels/expand/cpu_kernel.cc:27-46 with ExpandInfo
+ * (src/04kernel/src/attributes/expand_info.cc:14-60): output block i (block_size bytes) is input
+ * block j, where for d = 0 .. dims-1: j += (rem / stride_o[d]) * stride_i[d]; rem %= stride_o[d]
+ * (stride_i[d] == 0 where the input is broadcast).  stride_i / stride_o: HOST arrays [dims],
+ * dims <= 8; dims == 0 copies.  y != x. */
+int rg_hip_expand(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o,
+                  size_t dims, size_t block_size, size_t block_count, void *stream);
+
+/* ---- Where -------------------------------------------------------------------------------
+ * replaces src/04kernel/cuda/src/where.cu:1-62 + src/04kernel/src/kernels/where/where_cuda.cu;
+ * contract src/04kernel/src/kernels/where/cpu_kernel.cc:32-47: output element i (element_size
+ * bytes: 1, 2, 4 or 8) is x[at1] where condition[at0] != 0 (one byte per element), else y[at2],
+ * with (at0, at1, at2) = Broadcaster::locate(i) (src/04kernel/src/attributes/broadcaster.cc:87-100).
+ * strides: HOST array [dims][4] = per merged dimension the strides of condition, x, y and of the
+ * output (Broadcaster::strides as it stands); dims == 0: nothing is broadcast, at = (i, i, i). */
+int rg_hip_where(void *out, const void *condition, const void *x, const void *y, const uint32_t *strides,
+                 size_t dims, size_t outputs_count, size_t element_size, void *stream);
+
 /* ---- MatMulInteger -----------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/mat_mul_integer/cublas_kernel.cu:87-184 (Thrust
  * zero-point pre-pass + cublasGemmEx); arithmetic contract

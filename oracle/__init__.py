@@ -61,6 +61,18 @@ def lib() -> C.CDLL:
         L.oracle_transpose_info.restype = i32
         L.oracle_transpose.argtypes = [vp, vp, vp, vp, i32, C.c_uint32]
         L.oracle_transpose.restype = None
+        u32 = C.c_uint32
+        L.oracle_split_info.argtypes = [vp, vp, vp, vp, i32, i32, i32, u32]
+        L.oracle_split.argtypes = [vp, vp, vp, sz, sz, sz]
+        L.oracle_concat.argtypes = [vp, vp, vp, sz, sz, sz]
+        L.oracle_expand_info.argtypes = [vp, vp, vp, vp, vp, i32, vp, i32, u32]
+        L.oracle_expand_info.restype = i32
+        L.oracle_expand.argtypes = [vp, vp, vp, vp, i32, u32, u32]
+        L.oracle_broadcaster.argtypes = [vp, vp, vp, vp, i32]
+        L.oracle_broadcaster.restype = i32
+        L.oracle_where.argtypes = [vp, vp, vp, vp, vp, i32, u32, u32]
+        for name in ("oracle_split_info", "oracle_split", "oracle_concat", "oracle_expand", "oracle_where"):
+            getattr(L, name).restype = None
         for name in ("oracle_rms_norm_f32", "oracle_rms_norm_f64", "oracle_softmax_f32",
                      "oracle_softmax_f64", "oracle_softmax_literal_f32", "oracle_softmax_causal_f32",
                      "oracle_matmul_integer", "oracle_matmul_f32", "oracle_mul_f32",
@@ -424,3 +436,85 @@ def transpose(x, perm):
     y = np.empty(tuple(x.shape[p] for p in perm), dtype=x.dtype)
     lib().oracle_transpose(_p(y), _p(x), _p(sh), _p(pm), x.ndim, x.dtype.itemsize)
     return y
+
+
+def split_info(part_shapes, axis, elem_size):
+    """The reference's SplitInfo of parts with the given shapes: (block count, bytes per joined block, segment bytes)."""
+    shapes = np.asarray(part_shapes, np.uint32)
+    count, rank = shapes.shape
+    blocks, total = np.zeros(1, np.uint32), np.zeros(1, np.uint32)
+    segments = np.zeros(count, np.uint32)
+    lib().oracle_split_info(_p(blocks), _p(total), _p(segments), _p(shapes), count, rank, axis, elem_size)
+    return int(blocks[0]), int(total[0]), [int(v) for v in segments]
+
+
+def split(x, sizes, axis):
+    """numpy.split(x, cumsum(sizes)[:-1], axis) made contiguous, computed the reference's way."""
+    x = np.ascontiguousarray(x)
+    shapes = [x.shape[:axis] + (n,) + x.shape[axis + 1:] for n in sizes]
+    blocks, total, segments = split_info(shapes, axis, x.dtype.itemsize)
+    outs = [np.empty(sh, x.dtype) for sh in shapes]
+    ptrs = (C.c_void_p * len(outs))(*[o.ctypes.data for o in outs])
+    seg = np.asarray(segments, np.uint32)
+    lib().oracle_split(ptrs, _p(x), _p(seg), len(outs), blocks, total)
+    return outs
+
+
+def concat(parts, axis):
+    """numpy.concatenate(parts, axis), computed the reference's way."""
+    parts = [np.ascontiguousarray(p) for p in parts]
+    blocks, total, segments = split_info([p.shape for p in parts], axis, parts[0].dtype.itemsize)
+    shape = list(parts[0].shape)
+    shape[axis] = sum(p.shape[axis] for p in parts)
+    y = np.empty(shape, parts[0].dtype)
+    ptrs = (C.c_void_p * len(parts))(*[p.ctypes.data for p in parts])
+    seg = np.asarray(segments, np.uint32)
+    lib().oracle_concat(_p(y), ptrs, _p(seg), len(parts), blocks, total)
+    return y
+
+
+def expand_info(in_shape, out_shape, elem_size):
+    """The reference's ExpandInfo: ([(i, o), ...], block bytes, block count)."""
+    a, b = np.asarray(in_shape, np.uint32).reshape(-1), np.asarray(out_shape, np.uint32).reshape(-1)
+    si, so = np.zeros(18, np.uint32), np.zeros(18, np.uint32)
+    block, count = np.zeros(1, np.uint32), np.zeros(1, np.uint32)
+    dims = lib().oracle_expand_info(_p(si), _p(so), _p(block), _p(count), _p(a), len(a), _p(b), len(b), elem_size)
+    return [(int(si[d]), int(so[d])) for d in range(dims)], int(block[0]), int(count[0])
+
+
+def expand(x, out_shape):
+    """numpy.broadcast_to(x, out_shape) made contiguous, computed the reference's way."""
+    x = np.require(x, requirements="C")
+    pairs, block, count = expand_info(x.shape, out_shape, x.dtype.itemsize)
+    y = np.empty(out_shape, x.dtype)
+    si = np.asarray([p[0] for p in pairs] + [0], np.uint32)
+    so = np.asarray([p[1] for p in pairs] + [1], np.uint32)
+    lib().oracle_expand(_p(y), _p(x), _p(si), _p(so), len(pairs), block, count)
+    return y
+
+
+def broadcaster(shapes):
+    """The reference's Broadcaster of the given input shapes: (rows of strides: one per input, then the output's;
+    output element count).  No rows: nothing is broadcast."""
+    n = len(shapes)
+    table = np.ones((n, 8), np.uint32)
+    ranks = np.zeros(n, np.int32)
+    for i, sh in enumerate(shapes):
+        ranks[i] = len(sh)
+        table[i, :len(sh)] = sh
+    strides, count = np.zeros(16 * (n + 1), np.uint32), np.zeros(1, np.uint32)
+    dims = lib().oracle_broadcaster(_p(strides), _p(count), _p(table), _p(ranks), n)
+    return strides[:dims * (n + 1)].reshape(dims, n + 1).astype(np.int64).tolist(), int(count[0])
+
+
+def where(c, x, y):
+    """numpy.where(c, x, y) with multidirectional broadcasting, computed the reference's way."""
+    c = np.require(np.asarray(c).astype(np.bool_), requirements="C")   # (keeps 0-d arrays 0-d)
+    x, y = np.require(x, requirements="C"), np.require(y, requirements="C")
+    assert x.dtype == y.dtype
+    rows, count = broadcaster([c.shape, x.shape, y.shape])
+    out = np.empty(np.broadcast_shapes(c.shape, x.shape, y.shape), x.dtype)
+    assert out.size == count
+    st = np.asarray(rows, np.uint32).reshape(-1) if rows else np.zeros(4, np.uint32)
+    lib().oracle_where(_p(out), _p(c.view(np.uint8)), _p(x), _p(y), _p(st), len(rows), count, x.dtype.itemsize)
+    return out

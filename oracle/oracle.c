@@ -522,3 +522,176 @@ void oracle_transpose(void *y, const void *x, const uint32_t *shape, const uint3
     }
 }
 
+
+/* ------------------------------------------------------- split / concat */
+
+/* split_info.cc:5-24: blockCount = product of the dimensions before the axis, segment j = shape_j[axis] times
+ * the bytes behind the axis, sum = their total.  shapes: count rows of `rank` entries. */
+void oracle_split_info(uint32_t *block_count, uint32_t *sum, uint32_t *segments, const uint32_t *shapes, int count,
+                       int rank, int axis, uint32_t elem_size) {
+    uint32_t blocks = 1, postfix = elem_size, total = 0;
+    for (int d = 0; d < axis; ++d) blocks *= shapes[d];
+    for (int d = axis + 1; d < rank; ++d) postfix *= shapes[d];
+    for (int j = 0; j < count; ++j) {
+        segments[j] = shapes[j * rank + axis] * postfix;
+        total += segments[j];
+    }
+    *block_count = blocks;
+    *sum = total;
+}
+
+/* split/cpu_kernel.cc:27-42 */
+void oracle_split(void *const *outputs, const void *x, const uint32_t *segments, size_t count, size_t block_count,
+                  size_t sum) {
+    for (size_t i = 0; i < block_count; ++i) {
+        size_t offset = i * sum;
+        for (size_t j = 0; j < count; ++j) {
+            const size_t len = segments[j];
+            memcpy((uint8_t *) outputs[j] + i * len, (const uint8_t *) x + offset, len);
+            offset += len;
+        }
+    }
+}
+
+/* concat/cpu_kernel.cc:27-42 */
+void oracle_concat(void *y, const void *const *inputs, const uint32_t *segments, size_t count, size_t block_count,
+                   size_t sum) {
+    for (size_t i = 0; i < block_count; ++i) {
+        size_t offset = i * sum;
+        for (size_t j = 0; j < count; ++j) {
+            const size_t len = segments[j];
+            memcpy((uint8_t *) y + offset, (const uint8_t *) inputs[j] + i * len, len);
+            offset += len;
+        }
+    }
+}
+
+/* ------------------------------------------------------- expand */
+
+/* expand_info.cc:14-60.  Returns the number of (i, o) stride pairs (0: nothing is broadcast). */
+int oracle_expand_info(uint32_t *stride_i, uint32_t *stride_o, uint32_t *block_size, uint32_t *block_count,
+                       const uint32_t *input, int in_rank, const uint32_t *output, int out_rank, uint32_t elem_size) {
+    uint32_t si[18], so[18];
+    int n = 1;
+    si[0] = so[0] = 1;
+    uint32_t count = 1, stride = 1;
+    int i = in_rank;
+    for (int o = out_rank; o != 0;) {
+        const uint32_t i_ = i == 0 ? 1 : input[--i], o_ = output[--o];
+        if (o_ == 1) continue;
+        if (i_ == 1) {
+            if (si[n - 1]) { si[n] = 0; so[n] = count; ++n; }
+        } else {
+            if (!si[n - 1]) { si[n] = stride; so[n] = count; ++n; }
+            stride *= i_;
+        }
+        count *= o_;
+    }
+    *block_size = elem_size;
+    if (n == 1) {  /* nothing is broadcast */
+        *block_size *= count;
+        *block_count = 1;
+        return 0;
+    }
+    /* reversed, the initial {1, 1} dropped; the last pair left is a broadcast one and becomes the block */
+    int dims = n - 1;
+    for (int d = 0; d < dims; ++d) { stride_i[d] = si[n - 1 - d]; stride_o[d] = so[n - 1 - d]; }
+    const uint32_t tail_o = stride_o[dims - 1];
+    *block_size *= tail_o;
+    *block_count = count / tail_o;
+    for (int d = 0; d < dims; ++d) { stride_i[d] /= tail_o; stride_o[d] /= tail_o; }
+    return dims;
+}
+
+/* expand/cpu_kernel.cc:27-46 */
+void oracle_expand(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o, int dims,
+                   uint32_t block_size, uint32_t block_count) {
+    for (uint32_t k = 0; k < block_count; ++k) {
+        long rem = k, j = 0;
+        for (int d = 0; d < dims; ++d) {
+            if (stride_i[d]) {
+                j += rem / stride_o[d] * stride_i[d];
+                rem %= stride_o[d];
+            } else {
+                rem %= stride_o[d];
+            }
+        }
+        memcpy((uint8_t *) y + (size_t) k * block_size, (const uint8_t *) x + (size_t) j * block_size, block_size);
+    }
+}
+
+/* ------------------------------------------------------- broadcaster / where */
+
+/* broadcaster.cc:17-79: shapes of `inputs` tensors (ranks[i] entries each, rows of 8).  strides receives
+ * dims x (inputs + 1) values; returns dims (0: nothing is broadcast) and the output element count. */
+int oracle_broadcaster(uint32_t *strides, uint32_t *outputs_count, const uint32_t *shapes, const int *ranks, int inputs) {
+    uint32_t rev[16 * 9];
+    int used = 0, end[8], state[8], next[8];
+    uint32_t muls[8], count = 1;
+    for (int i = 0; i < inputs; ++i) { end[i] = ranks[i]; state[i] = 0; muls[i] = 1; }
+    for (;;) {
+        uint32_t shape = 1;
+        int all_end = 1;
+        for (int i = 0; i < inputs; ++i) next[i] = 0;
+        for (int i = 0; i < inputs; ++i) {
+            if (end[i] == 0) continue;
+            const uint32_t dim = shapes[i * 8 + --end[i]];
+            next[i] = dim != 1;
+            if (next[i]) shape = dim;  /* (a mismatch between inputs is the caller's error) */
+            all_end = 0;
+        }
+        if (all_end) break;
+        if (shape == 1) continue;
+        int same = 1;
+        for (int i = 0; i < inputs; ++i) same &= next[i] == state[i];
+        if (!same) {
+            /* a new group of (inputs + 1) strides, written back to front: output stride first */
+            for (int i = 0; i < inputs; ++i) state[i] = next[i];
+            uint32_t *group = rev + used;
+            used += inputs + 1;
+            for (int i = 0; i < inputs; ++i) {
+                group[i] = 0;
+                if (state[inputs - 1 - i]) { group[i] = muls[inputs - 1 - i]; muls[inputs - 1 - i] *= shape; }
+            }
+            group[inputs] = count;
+        } else {
+            for (int i = 0; i < inputs; ++i)
+                if (state[i]) muls[i] *= shape;
+        }
+        count *= shape;
+    }
+    *outputs_count = count;
+    /* `rev` holds what the reference's vector holds read from its end; reversing the whole vector gives, per
+     * group from the slowest dimension on, the input strides in input order followed by the output stride */
+    int all_one = used == inputs + 1;
+    for (int t = 0; t < used && all_one; ++t) all_one = rev[t] == 1;
+    if (all_one || used == 0) return 0;
+    const int dims = used / (inputs + 1);
+    for (int g = 0; g < dims; ++g) {
+        const uint32_t *group = rev + (dims - 1 - g) * (inputs + 1);
+        for (int i = 0; i < inputs; ++i) strides[g * (inputs + 1) + i] = group[inputs - 1 - i];
+        strides[g * (inputs + 1) + inputs] = group[inputs];
+    }
+    return dims;
+}
+
+/* where/cpu_kernel.cc:32-47 with broadcaster.cc:87-100 */
+void oracle_where(void *out, const uint8_t *c, const void *x, const void *y, const uint32_t *strides, int dims,
+                  uint32_t count, uint32_t elem_size) {
+    for (uint32_t i = 0; i < count; ++i) {
+        uint32_t at[3] = {i, i, i};
+        if (dims) {
+            long rem = i;
+            at[0] = at[1] = at[2] = 0;
+            for (int d = 0; d < dims; ++d) {
+                const uint32_t *dim = strides + 4 * d;
+                const long q = rem / dim[3];
+                for (int j = 0; j < 3; ++j) at[j] += dim[j] * (uint32_t) q;
+                rem %= dim[3];
+            }
+        }
+        memcpy((uint8_t *) out + (size_t) i * elem_size,
+               c[at[0]] ? (const uint8_t *) x + (size_t) at[1] * elem_size : (const uint8_t *) y + (size_t) at[2] * elem_size,
+               elem_size);
+    }
+}

@@ -33,6 +33,9 @@
  *                              src/08-01llm/README.md:29-63.  PARITY UNPINNED by the reference.
  *   oracle_rope_f32            no reference item exists; closed-form rotate-half rotary
  *                              embedding.  PARITY UNPINNED by the reference.
+ *   oracle_split / _concat     src/04kernel/src/kernels/{split,concat}/cpu_kernel.cc + attributes/split_info.cc
+ *   oracle_expand(_info)       src/04kernel/src/kernels/expand/cpu_kernel.cc + attributes/expand_info.cc
+ *   oracle_where, _broadcaster src/04kernel/src/kernels/where/cpu_kernel.cc + attributes/broadcaster.cc
  *   oracle_transpose(_info)    src/04kernel/src/attributes/transpose_info.cc:7-126
  *                              + src/04kernel/src/kernels/transpose/cpu_kernel.cc:27-37
  *
@@ -147,6 +150,35 @@ int oracle_transpose_info(uint32_t *stride_i, uint32_t *stride_o, uint32_t *bloc
                           const uint32_t *shape, const uint32_t *perm, int rank, uint32_t elem_size);
 void oracle_transpose(void *y, const void *x, const uint32_t *shape, const uint32_t *perm, int rank,
                       uint32_t elem_size);
+
+/* Split / Concat as the reference computes them: src/04kernel/src/attributes/split_info.cc:5-24
+ * (digest) and src/04kernel/src/kernels/{split,concat}/cpu_kernel.cc:27-42 (copies).  shapes: `count`
+ * rows of `rank` entries (the parts).  Pinned by the reference's vectors
+ * (src/04kernel/test/attributes/test_split_info.cpp:7-30, test/kernels/{split,concat}/test_cpu.cpp)
+ * and by numpy.split / numpy.concatenate. */
+void oracle_split_info(uint32_t *block_count, uint32_t *sum, uint32_t *segments, const uint32_t *shapes, int count,
+                       int rank, int axis, uint32_t elem_size);
+void oracle_split(void *const *outputs, const void *x, const uint32_t *segments, size_t count, size_t block_count,
+                  size_t sum);
+void oracle_concat(void *y, const void *const *inputs, const uint32_t *segments, size_t count, size_t block_count,
+                   size_t sum);
+
+/* Expand: src/04kernel/src/attributes/expand_info.cc:14-60 (digest; returns the number of stride pairs)
+ * and src/04kernel/src/kernels/expand/cpu_kernel.cc:27-46.  Pinned by
+ * src/04kernel/test/attributes/test_expand_info.cpp:7-18, test/kernels/expand/test_cpu.cpp and
+ * numpy.broadcast_to. */
+int oracle_expand_info(uint32_t *stride_i, uint32_t *stride_o, uint32_t *block_size, uint32_t *block_count,
+                       const uint32_t *input, int in_rank, const uint32_t *output, int out_rank, uint32_t elem_size);
+void oracle_expand(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o, int dims,
+                   uint32_t block_size, uint32_t block_count);
+
+/* Broadcaster (src/04kernel/src/attributes/broadcaster.cc:17-100; shapes: rows of 8 entries, at most 8
+ * inputs; returns the number of merged dimensions) and Where
+ * (src/04kernel/src/kernels/where/cpu_kernel.cc:32-47; strides rows of 4).  Pinned by
+ * src/04kernel/test/attributes/test_broadcaster.cpp:7-36, test/kernels/where/test_cpu.cpp and numpy.where. */
+int oracle_broadcaster(uint32_t *strides, uint32_t *outputs_count, const uint32_t *shapes, const int *ranks, int inputs);
+void oracle_where(void *out, const uint8_t *c, const void *x, const void *y, const uint32_t *strides, int dims,
+                  uint32_t count, uint32_t elem_size);
 
 #ifdef __cplusplus
 }

@@ -48,6 +48,10 @@ SIGNATURES = {
     "rg_hip_cast": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rg_hip_transpose": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "rg_hip_split": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "rg_hip_concat": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "rg_hip_expand": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "rg_hip_where": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul_integer_workspace": (_sz, [_sz, _sz, _sz, _sz, _u]),
     "rg_hip_matmul_integer": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
     "rg_hip_matmul_integer_dequantize": (_i, [_vp, _vp, _vp, _vp, _vp, _u, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _i,

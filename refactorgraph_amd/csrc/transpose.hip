@@ -252,6 +252,48 @@ int launch(void *y, const void *x, const Plan &p, const uint32_t *stride_i, cons
 }  // namespace
 }  // namespace rg
 
+// Expand (one-directional broadcast), contract src/04kernel/src/kernels/expand/cpu_kernel.cc:27-46 with the
+// digest of src/04kernel/src/attributes/expand_info.cc:14-60: output block i is input block
+// j = sum over the dimensions of (rem / o) * i, rem %= o — the arithmetic of the transposition's locate()
+// with input strides that are 0 where the input is broadcast, so the word kernel above serves as it is.
+extern "C" int rg_hip_expand(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o, size_t dims,
+                             size_t block_size, size_t block_count, void *stream) {
+    using namespace rg;
+    if (!y || !x || (dims && (!stride_i || !stride_o))) return RG_HIP_E_ARGUMENT;
+    if (dims > static_cast<size_t>(kMaxDims)) return RG_HIP_E_UNSUPPORTED;
+    if (block_size == 0 || block_count == 0) return 0;
+    if (y == x) return RG_HIP_E_ARGUMENT;
+    const uint64_t bytes = static_cast<uint64_t>(block_size) * block_count;
+    if (block_count > 0xffffffffull) return RG_HIP_E_UNSUPPORTED;
+    hipStream_t s = as_stream(stream);
+    if (dims == 0) return static_cast<int>(hipMemcpyAsync(y, x, bytes, hipMemcpyDeviceToDevice, s));  // nothing is broadcast
+    const uintptr_t misalign = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(x) | block_size;
+    uint32_t w = 16;
+    while (misalign & (w - 1)) w >>= 1;
+    const uint64_t words = bytes / w;
+    if (words > 0xffffffffull) return RG_HIP_E_UNSUPPORTED;
+    Plan p{};
+    p.dims = static_cast<uint32_t>(dims);
+    p.words = words;
+    p.words_per_block = make_divisor(static_cast<uint32_t>(block_size / w));
+    for (size_t d = 0; d < dims; ++d) {
+        if (stride_o[d] == 0) return RG_HIP_E_ARGUMENT;
+        p.stride_o[d] = make_divisor(stride_o[d]);
+        p.stride_i[d] = stride_i[d];
+    }
+    const uint64_t grid = (p.words + 256ull * UNROLL - 1) / (256ull * UNROLL);
+    if (grid > 0x7fffffffull) return RG_HIP_E_UNSUPPORTED;
+    const unsigned g = static_cast<unsigned>(grid);
+    switch (w) {
+        case 16: transpose_words<u32x4><<<g, 256, 0, s>>>(static_cast<u32x4 *>(y), static_cast<const u32x4 *>(x), p); break;
+        case 8: transpose_words<uint64_t><<<g, 256, 0, s>>>(static_cast<uint64_t *>(y), static_cast<const uint64_t *>(x), p); break;
+        case 4: transpose_words<uint32_t><<<g, 256, 0, s>>>(static_cast<uint32_t *>(y), static_cast<const uint32_t *>(x), p); break;
+        case 2: transpose_words<uint16_t><<<g, 256, 0, s>>>(static_cast<uint16_t *>(y), static_cast<const uint16_t *>(x), p); break;
+        default: transpose_words<uint8_t><<<g, 256, 0, s>>>(static_cast<uint8_t *>(y), static_cast<const uint8_t *>(x), p); break;
+    }
+    return launch_status();
+}
+
 extern "C" int rg_hip_transpose(void *y, const void *x, const uint32_t *stride_i, const uint32_t *stride_o,
                                 size_t dims, size_t block_size, size_t block_count, void *stream) {
     using namespace rg;

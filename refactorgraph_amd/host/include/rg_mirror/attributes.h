@@ -1,6 +1,7 @@
 // Shape pre-digestion used by the hot-path collectors.  Semantics follow
 // src/04kernel/src/attributes/{softmax_info.cc:6-13, broadcaster.cc:17-105,
-// mat_mul_integer_info.cc:5-40, mat_mul_info.cc:5-43, transpose_info.cc:7-126}.
+// mat_mul_integer_info.cc:5-40, mat_mul_info.cc:5-43, transpose_info.cc:7-126, split_info.cc:5-24,
+// expand_info.cc:14-60}.
 #pragma once
 
 #include <optional>
@@ -63,6 +64,28 @@ namespace refactor::kernel {
 
         TransposeInfo(DataType, std::vector<dim_t> const &shape, Permutation const &);
         dim_t locate(dim_t) const noexcept;
+    };
+
+    // Digest of Split and Concat (src/04kernel/include/kernel/attributes/split_info.h:9-21): the joined
+    // tensor is blockCount blocks of `sum` bytes, block i being one segment of every part in turn.
+    struct SplitInfo {
+        dim_t blockCount, sum;
+        std::vector<dim_t> segments;
+        SplitInfo(dim_t axis, TensorRefs const &parts);
+    };
+
+    // Digest of a one-directional broadcast (src/04kernel/include/kernel/attributes/expand_info.h:9-25):
+    // the output is blockCount blocks of blockSize bytes; output block k is input block
+    // sum over the strides of (rem / o) * i with rem %= o.  No strides: nothing is broadcast.
+    struct ExpandInfo {
+        struct Dim {
+            dim_t i, o;
+            bool operator==(Dim const &rhs) const noexcept { return i == rhs.i && o == rhs.o; }
+        };
+        std::vector<Dim> strides;
+        dim_t blockCount, blockSize;
+        ExpandInfo(DataType, std::vector<dim_t> const &input, std::vector<dim_t> const &output);
+        ExpandInfo(Tensor const &input, Tensor const &output);
     };
 
     struct MatMulIntegerInfo {

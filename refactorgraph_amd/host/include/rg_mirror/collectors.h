@@ -72,6 +72,34 @@ namespace refactor::kernel {
         std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
     };
 
+    // inputs: data; outputs: its parts along `axis` (src/04kernel/include/kernel/collectors/split.h:8-16)
+    struct SplitCollector final : public InfoCollector {
+        dim_t axis;
+        constexpr SplitCollector(hardware::Device::Type target, dim_t axis_) noexcept
+            : InfoCollector(target), axis(axis_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: the parts; outputs: them joined along `axis` (src/04kernel/include/kernel/collectors/concat.h:8-16)
+    struct ConcatCollector final : public InfoCollector {
+        dim_t axis;
+        constexpr ConcatCollector(hardware::Device::Type target, dim_t axis_) noexcept
+            : InfoCollector(target), axis(axis_) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: data; outputs: data broadcast to the output's shape (src/04kernel/include/kernel/collectors/expand.h)
+    struct ExpandCollector final : public InfoCollector {
+        constexpr explicit ExpandCollector(hardware::Device::Type target) noexcept : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
+    // inputs: condition (Bool), x, y; outputs: the selection, broadcast (src/04kernel/include/kernel/collectors/where.h)
+    struct WhereCollector final : public InfoCollector {
+        constexpr explicit WhereCollector(hardware::Device::Type target) noexcept : InfoCollector(target) {}
+        std::vector<KernelBox> filter(TensorRefs inputs, TensorRefs outputs) const final;
+    };
+
     // inputs: query, key, value [, past_seq_len [, k_cache, v_cache]]; outputs: output
     // [, k_cache, v_cache] (src/08-01llm/README.md:29-63).
     struct AttentionCollector final : public InfoCollector {

@@ -107,6 +107,30 @@ namespace refactor::computation {
         std::string serialize() const final;
     };
 
+    // src/05computation/include/computation/operators/{split,concat,expand,where}.h
+    struct Split final : public Operator {
+        dim_t axis;
+        constexpr explicit Split(dim_t axis_) noexcept : axis(axis_) {}
+        RG_OPERATOR_COMMON
+        kernel::CollectorBox candidateKernels(Target) const final;
+        std::string serialize() const final;
+    };
+    struct Concat final : public Operator {
+        dim_t axis;
+        constexpr explicit Concat(dim_t axis_) noexcept : axis(axis_) {}
+        RG_OPERATOR_COMMON
+        kernel::CollectorBox candidateKernels(Target) const final;
+        std::string serialize() const final;
+    };
+    struct Expand final : public Operator {
+        RG_OPERATOR_COMMON
+        kernel::CollectorBox candidateKernels(Target) const final;
+    };
+    struct Where final : public Operator {
+        RG_OPERATOR_COMMON
+        kernel::CollectorBox candidateKernels(Target) const final;
+    };
+
     struct RotaryEmbedding final : public Operator {
         float theta;
         constexpr explicit RotaryEmbedding(float theta_) noexcept : theta(theta_) {}

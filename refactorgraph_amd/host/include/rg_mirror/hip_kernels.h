@@ -128,6 +128,51 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // mirror SplitCuda and ConcatCuda (src/04kernel/src/kernels/{split,concat}/cuda_kernel.hh): outputs of
+    // Split / inputs of Concat are the parts of the digest, in order
+    struct SplitHip final : public Kernel {
+        SplitInfo info;
+        explicit SplitHip(SplitInfo) noexcept;
+        static KernelBox build(SplitInfo) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+    struct ConcatHip final : public Kernel {
+        SplitInfo info;
+        explicit ConcatHip(SplitInfo) noexcept;
+        static KernelBox build(SplitInfo) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    // mirrors ExpandCuda (src/04kernel/src/kernels/expand/cuda_kernel.hh); the stride table travels in
+    // the kernel arguments, nothing is uploaded at lower() time
+    struct ExpandHip final : public Kernel {
+        ExpandInfo info;
+        explicit ExpandHip(ExpandInfo) noexcept;
+        static KernelBox build(ExpandInfo) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
+    // mirrors WhereCuda (src/04kernel/src/kernels/where/where_cuda.hh): inputs condition (Bool), x, y
+    struct WhereHip final : public Kernel {
+        DataType dataType;
+        Broadcaster broadcaster;
+        WhereHip(DataType, Broadcaster) noexcept;
+        static KernelBox build(TensorRefs const &inputs) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct AttentionHip final : public Kernel {
         // the reference's parameter block (src/04kernel/src/kernels/attention/cuda_kernel.hh:10-14)
         // plus what it leaves to the run time: where past_seq_len comes from

@@ -221,4 +221,62 @@ namespace refactor::kernel {
         return ans;
     }
 
+    // ------------------------------------------------------------------ SplitInfo
+
+    SplitInfo::SplitInfo(dim_t axis, TensorRefs const &parts) : blockCount(1), sum(0), segments() {
+        ASSERT(!parts.empty(), "SplitInfo: no parts");
+        auto const &shape = parts[0].get().shape;
+        ASSERT(axis < shape.size(), "SplitInfo: axis out of range");
+        for (size_t d = 0; d < axis; ++d) { blockCount *= shape[d]; }
+        dim_t postfix = static_cast<dim_t>(parts[0].get().dataType.size());
+        for (size_t d = axis + 1; d < shape.size(); ++d) { postfix *= shape[d]; }
+        segments.reserve(parts.size());
+        for (auto const &part : parts) {
+            segments.push_back(part.get().shape[axis] * postfix);
+            sum += segments.back();
+        }
+    }
+
+    // ------------------------------------------------------------------ ExpandInfo
+
+    ExpandInfo::ExpandInfo(DataType dataType, std::vector<dim_t> const &input, std::vector<dim_t> const &output)
+        : strides(), blockCount(1), blockSize(static_cast<dim_t>(dataType.size())) {
+        ASSERT(input.size() <= output.size(), "ExpandInfo: the input has more dimensions than the output");
+        // from the innermost dimension outwards: a run of dimensions that are all kept or all broadcast is one
+        // stride pair; `kept` tells what the innermost run so far is (it starts as a kept run of extent 1)
+        std::vector<Dim> reversed;
+        bool kept = true, any = false;
+        dim_t stride = 1;
+        auto i = input.size();
+        for (auto o = output.size(); o != 0;) {
+            auto const i_ = i == 0 ? dim_t(1) : input[--i], o_ = output[--o];
+            if (o_ == 1) { continue; }
+            if (i_ == 1) {
+                if (kept) { reversed.push_back({0, blockCount}); kept = false; any = true; }
+            } else {
+                ASSERT(i_ == o_, "ExpandInfo: shapes do not broadcast");
+                if (!kept) { reversed.push_back({stride, blockCount}); kept = true; }
+                stride *= i_;
+            }
+            blockCount *= o_;
+        }
+        if (!any) {// nothing is broadcast: one block
+            blockSize *= blockCount;
+            blockCount = 1;
+            return;
+        }
+        strides.assign(reversed.rbegin(), reversed.rend());
+        // the innermost pair is a broadcast one (a kept innermost run is implicit): it becomes the block
+        auto const tail = strides.back();
+        blockSize *= tail.o;
+        blockCount /= tail.o;
+        for (auto &s : strides) {
+            s.i /= tail.o;
+            s.o /= tail.o;
+        }
+    }
+
+    ExpandInfo::ExpandInfo(Tensor const &input, Tensor const &output)
+        : ExpandInfo(input.dataType, input.shape, output.shape) {}
+
 }// namespace refactor::kernel

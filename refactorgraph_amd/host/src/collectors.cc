@@ -159,6 +159,68 @@ namespace refactor::kernel {
     }
 
     std::vector<KernelBox>
+    SplitCollector::filter(TensorRefs, TensorRefs outputs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                if (!outputs.empty() && axis < outputs[0].get().shape.size()) { ADD(SplitHip::build(SplitInfo(axis, outputs))) }
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    ConcatCollector::filter(TensorRefs inputs, TensorRefs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                if (!inputs.empty() && axis < inputs[0].get().shape.size()) { ADD(ConcatHip::build(SplitInfo(axis, inputs))) }
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    ExpandCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                if (inputs[0].get().shape.size() <= outputs[0].get().shape.size()) {
+                    ADD(ExpandHip::build(ExpandInfo(inputs[0], outputs[0])))
+                }
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
+    WhereCollector::filter(TensorRefs inputs, TensorRefs) const {
+        std::vector<KernelBox> ans;
+        switch (_target) {
+            case Target::Cpu:
+                break;
+            case Target::Amd:
+                ADD(WhereHip::build(inputs))
+                break;
+            default:
+                UNREACHABLEX(void, "Unknown target");
+        }
+        return ans;
+    }
+
+    std::vector<KernelBox>
     AttentionCollector::filter(TensorRefs inputs, TensorRefs outputs) const {
         auto const &query = inputs[0].get();
         auto const &key = inputs[1].get();

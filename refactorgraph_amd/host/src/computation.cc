@@ -27,6 +27,10 @@ namespace refactor::computation {
     RG_OPERATOR_IDS(Attention, "Attention")
     RG_OPERATOR_IDS(RotaryEmbedding, "RotaryEmbedding")
     RG_OPERATOR_IDS(Transpose, "Transpose")
+    RG_OPERATOR_IDS(Split, "Split")
+    RG_OPERATOR_IDS(Concat, "Concat")
+    RG_OPERATOR_IDS(Expand, "Expand")
+    RG_OPERATOR_IDS(Where, "Where")
     RG_OPERATOR_IDS(Identity, "Identity")
     RG_OPERATOR_IDS(Reshape, "Reshape")
 #undef RG_OPERATOR_IDS
@@ -76,6 +80,21 @@ namespace refactor::computation {
         s += "([";
         for (auto p : perm) s += ' ' + std::to_string(p);
         return s + " ])";
+    }
+
+    kernel::CollectorBox Split::candidateKernels(Target target) const {
+        return std::make_unique<kernel::SplitCollector>(target, axis);
+    }
+    std::string Split::serialize() const { return detail::cat(name(), '(', axis, ')'); }
+    kernel::CollectorBox Concat::candidateKernels(Target target) const {
+        return std::make_unique<kernel::ConcatCollector>(target, axis);
+    }
+    std::string Concat::serialize() const { return detail::cat(name(), '(', axis, ')'); }
+    kernel::CollectorBox Expand::candidateKernels(Target target) const {
+        return std::make_unique<kernel::ExpandCollector>(target);
+    }
+    kernel::CollectorBox Where::candidateKernels(Target target) const {
+        return std::make_unique<kernel::WhereCollector>(target);
     }
 
     kernel::CollectorBox RotaryEmbedding::candidateKernels(Target target) const {

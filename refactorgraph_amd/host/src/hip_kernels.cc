@@ -131,6 +131,72 @@ namespace refactor::kernel {
         };
     }
 
+    // ------------------------------------------------------------------ Split / Concat / Expand / Where
+
+    SplitHip::SplitHip(SplitInfo info_) noexcept : Kernel(), info(std::move(info_)) {}
+    KernelBox SplitHip::build(SplitInfo info) noexcept { return std::make_unique<SplitHip>(std::move(info)); }
+    size_t SplitHip::typeId() noexcept { return idOf<SplitHip>(); }
+    size_t SplitHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view SplitHip::description() const noexcept { return "Performing split operation on AMD gfx950"; }
+    RoutineWorkspace SplitHip::lower(Resources &) const {
+        return [info = this->info](Resources &res, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_split(outputs, inputs[0], info.segments.data(), info.segments.size(), info.blockCount, info.sum,
+                                  streamOf(res)));
+        };
+    }
+
+    ConcatHip::ConcatHip(SplitInfo info_) noexcept : Kernel(), info(std::move(info_)) {}
+    KernelBox ConcatHip::build(SplitInfo info) noexcept { return std::make_unique<ConcatHip>(std::move(info)); }
+    size_t ConcatHip::typeId() noexcept { return idOf<ConcatHip>(); }
+    size_t ConcatHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view ConcatHip::description() const noexcept { return "Performing concat operation on AMD gfx950"; }
+    RoutineWorkspace ConcatHip::lower(Resources &) const {
+        return [info = this->info](Resources &res, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_concat(outputs[0], inputs, info.segments.data(), info.segments.size(), info.blockCount, info.sum,
+                                   streamOf(res)));
+        };
+    }
+
+    ExpandHip::ExpandHip(ExpandInfo info_) noexcept : Kernel(), info(std::move(info_)) {}
+    KernelBox ExpandHip::build(ExpandInfo info) noexcept {
+        return info.strides.size() <= 8 ? std::make_unique<ExpandHip>(std::move(info)) : nullptr;
+    }
+    size_t ExpandHip::typeId() noexcept { return idOf<ExpandHip>(); }
+    size_t ExpandHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view ExpandHip::description() const noexcept { return "Performing expand operation on AMD gfx950"; }
+    RoutineWorkspace ExpandHip::lower(Resources &) const {
+        std::vector<uint32_t> strideI, strideO;
+        for (auto [i, o] : info.strides) {
+            strideI.push_back(i);
+            strideO.push_back(o);
+        }
+        return [strideI = std::move(strideI), strideO = std::move(strideO), blockSize = info.blockSize,
+                blockCount = info.blockCount](Resources &res, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_expand(outputs[0], inputs[0], strideI.data(), strideO.data(), strideI.size(), blockSize, blockCount,
+                                   streamOf(res)));
+        };
+    }
+
+    WhereHip::WhereHip(DataType dataType_, Broadcaster b) noexcept : Kernel(), dataType(dataType_), broadcaster(std::move(b)) {}
+    KernelBox WhereHip::build(TensorRefs const &inputs) noexcept {
+        if (inputs.size() != 3 || inputs[1].get().dataType != inputs[2].get().dataType) { return nullptr; }
+        auto const size = inputs[1].get().dataType.size();
+        if (size != 1 && size != 2 && size != 4 && size != 8) { return nullptr; }
+        Broadcaster b(inputs);
+        if (b.strides.size() / 4 > 8) { return nullptr; }
+        return std::make_unique<WhereHip>(inputs[1].get().dataType, std::move(b));
+    }
+    size_t WhereHip::typeId() noexcept { return idOf<WhereHip>(); }
+    size_t WhereHip::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view WhereHip::description() const noexcept { return "Performing where operation on AMD gfx950"; }
+    RoutineWorkspace WhereHip::lower(Resources &) const {
+        return [strides = broadcaster.strides, count = broadcaster.outputsCount,
+                eleSize = dataType.size()](Resources &res, void *, void const *const *inputs, void *const *outputs) {
+            HIP_CALL(rg_hip_where(outputs[0], inputs[0], inputs[1], inputs[2], strides.data(), strides.size() / 4, count, eleSize,
+                                  streamOf(res)));
+        };
+    }
+
     // ------------------------------------------------------------------ MatMulInteger + DequantizeLinear
 
     using MMD = MatMulIntegerDequantizeHip;

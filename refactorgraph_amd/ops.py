@@ -203,6 +203,124 @@ def transpose(x, perm, out=None):
     return y
 
 
+def split_info(part_shapes, axis, itemsize):
+    """(block count, bytes of a joined block, segment bytes): SplitInfo of the host layer, restated for this driver."""
+    first = part_shapes[0]
+    blocks = math.prod(first[:axis])
+    postfix = itemsize * math.prod(first[axis + 1:])
+    segments = [sh[axis] * postfix for sh in part_shapes]
+    return blocks, sum(segments), segments
+
+
+def _pointer_array(tensors):
+    return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def split(x, sizes, axis, outs=None):
+    """The parts of x along `axis` with the given sizes, each contiguous (any dtype: bytes are moved)."""
+    _need_gpu(x)
+    axis %= x.dim()
+    assert sum(sizes) == x.shape[axis]
+    shapes = [tuple(x.shape[:axis]) + (n,) + tuple(x.shape[axis + 1:]) for n in sizes]
+    if outs is None:
+        outs = [torch.empty(sh, dtype=x.dtype, device=x.device) for sh in shapes]
+    blocks, total, segments = split_info(shapes, axis, x.element_size())
+    seg = np.asarray(segments, np.uint32)
+    check(lib().rg_hip_split(_pointer_array(outs), _ptr(x), seg.ctypes.data_as(C.c_void_p), len(outs), blocks, total,
+                             _stream()), "rg_hip_split")
+    return outs
+
+
+def concat(parts, axis, out=None):
+    _need_gpu(*parts)
+    axis %= parts[0].dim()
+    shape = list(parts[0].shape)
+    shape[axis] = sum(p.shape[axis] for p in parts)
+    y = torch.empty(shape, dtype=parts[0].dtype, device=parts[0].device) if out is None else out
+    blocks, total, segments = split_info([tuple(p.shape) for p in parts], axis, parts[0].element_size())
+    seg = np.asarray(segments, np.uint32)
+    check(lib().rg_hip_concat(_ptr(y), _pointer_array(parts), seg.ctypes.data_as(C.c_void_p), len(parts), blocks, total,
+                              _stream()), "rg_hip_concat")
+    return y
+
+
+def expand_info(in_shape, out_shape, itemsize):
+    """(stride_i, stride_o, block bytes, block count): ExpandInfo of the host layer, restated for this driver.
+    Walks the dimensions from the last one; runs of dimensions that are all broadcast or all kept become one
+    stride pair; the innermost run becomes the block."""
+    pairs, count, stride, broadcast_run = [], 1, 1, None
+    ins = [1] * (len(out_shape) - len(in_shape)) + list(in_shape)
+    for i_, o_ in zip(reversed(ins), reversed(list(out_shape))):
+        if o_ == 1:
+            continue
+        is_broadcast = i_ == 1
+        if broadcast_run is None:
+            if is_broadcast:            # the innermost run is a broadcast one: it starts a pair of its own
+                pairs.append((0, count))
+        elif is_broadcast != broadcast_run:
+            pairs.append((0 if is_broadcast else stride, count))
+        broadcast_run = is_broadcast
+        if not is_broadcast:
+            stride *= i_
+        count *= o_
+    if not any(p[0] == 0 for p in pairs):
+        return [], [], itemsize * count, 1
+    # slowest dimension first; the innermost explicit pair is a broadcast one (a kept innermost run is the
+    # implicit pair (1, 1)) and becomes the block
+    pairs.reverse()
+    tail_o = pairs[-1][1]
+    return [p[0] // tail_o for p in pairs], [p[1] // tail_o for p in pairs], itemsize * tail_o, count // tail_o
+
+
+def expand(x, out_shape, out=None):
+    _need_gpu(x)
+    y = torch.empty(tuple(out_shape), dtype=x.dtype, device=x.device) if out is None else out
+    si, so, block, count = expand_info(list(x.shape), list(out_shape), x.element_size())
+    si_, so_ = np.asarray(si + [0], np.uint32), np.asarray(so + [1], np.uint32)
+    check(lib().rg_hip_expand(_ptr(y), _ptr(x), si_.ctypes.data_as(C.c_void_p), so_.ctypes.data_as(C.c_void_p), len(si),
+                              block, count, _stream()), "rg_hip_expand")
+    return y
+
+
+def broadcaster(shapes):
+    """(rows of strides: one per input, then the output's; output element count): the host layer's Broadcaster,
+    restated for this driver.  Dimensions where every input is 1 vanish; neighbouring dimensions in which the same
+    inputs are broadcast merge.  No rows: nothing is broadcast."""
+    n, rank = len(shapes), max((len(sh) for sh in shapes), default=0)
+    padded = [[1] * (rank - len(sh)) + list(sh) for sh in shapes]
+    rows, muls, count, state = [], [1] * n, 1, [False] * n
+    for d in reversed(range(rank)):
+        dims = [padded[i][d] for i in range(n)]
+        extent = max(dims)
+        if extent == 1:
+            continue
+        nxt = [v != 1 for v in dims]
+        if nxt != state:
+            state = nxt
+            rows.append([muls[i] if state[i] else 0 for i in range(n)] + [count])
+        for i in range(n):
+            if state[i]:
+                muls[i] *= extent
+        count *= extent
+    rows.reverse()
+    if len(rows) == 1 and all(v == 1 for v in rows[0]):
+        rows = []
+    return rows, count
+
+
+def where(c, x, y, out=None):
+    """torch.where(c, x, y) with multidirectional broadcasting; c: bool."""
+    _need_gpu(c, x, y)
+    assert c.dtype == torch.bool and x.dtype == y.dtype
+    rows, count = broadcaster([list(c.shape), list(x.shape), list(y.shape)])
+    shape = torch.broadcast_shapes(c.shape, x.shape, y.shape)
+    o = torch.empty(shape, dtype=x.dtype, device=x.device) if out is None else out
+    st = np.asarray(rows if rows else [[0, 0, 0, 1]], np.uint32).reshape(-1)
+    check(lib().rg_hip_where(_ptr(o), _ptr(c), _ptr(x), _ptr(y), st.ctypes.data_as(C.c_void_p), len(rows), count,
+                             x.element_size(), _stream()), "rg_hip_where")
+    return o
+
+
 def matmul_integer(a, b, a_zp=None, b_zp=None, out=None, dequant_scale=None):
     """a [..., m, k], b [..., k, n] (uint8/int8).  Zero points: None, one element, or one per
     (batch, row) of the operand as the reference's CPU kernel reads them.  dequant_scale (float32,

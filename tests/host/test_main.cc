@@ -10,6 +10,13 @@
 #include "kernel/attributes/softmax_info.h"
 #include "kernel/attributes/transpose_info.h"
 #include "kernel/collectors/transpose.h"
+#include "kernel/attributes/expand_info.h"
+#include "kernel/attributes/split_info.h"
+#include "kernel/collectors/concat.h"
+#include "kernel/collectors/expand.h"
+#include "kernel/collectors/split.h"
+#include "kernel/collectors/where.h"
+#include "computation/operators/split.h"
 #include "computation/operators/transpose.h"
 #include "kernel/collectors/attention.h"
 #include "kernel/collectors/dequantize_linear.h"
@@ -725,6 +732,46 @@ static void computationGraphLowers() {
     };
     EXPECT(quantised(1, 4, false) == 1 && quantised(1, 1, false) == 1 && quantised(-1, 4, false) == 1);
     EXPECT(quantised(0, 4, false) == 2 && quantised(1, 4, true) == 2);
+}
+
+// Split / Concat / Expand digests against the reference's vectors
+// (src/04kernel/test/attributes/test_split_info.cpp:7-30, test_expand_info.cpp:7-18) and the collectors
+static void dataMoverDigests() {
+    using T = Device::Type;
+    std::vector<Arc<Tensor>> parts{
+        Tensor::share(DataType::I64, Shape{2, 3, 1, 1, 7, 7}), Tensor::share(DataType::I64, Shape{2, 3, 1, 9, 7, 7}),
+        Tensor::share(DataType::I64, Shape{2, 3, 1, 3, 7, 7}), Tensor::share(DataType::I64, Shape{2, 3, 1, 7, 7, 7})};
+    TensorRefs refs;
+    for (auto const &t : parts) refs.emplace_back(*t);
+    SplitInfo info(3, refs);
+    dim_t const postfix = 49 * 8;
+    EXPECT(info.blockCount == 6 && info.sum == 20 * postfix);
+    EXPECT((info.segments == std::vector<dim_t>{1 * postfix, 9 * postfix, 3 * postfix, 7 * postfix}));
+
+    auto in = Tensor::share(DataType::F32, Shape{3, 4, 1, 6}), out = Tensor::share(DataType::F32, Shape{2, 3, 4, 5, 6});
+    ExpandInfo e(*in, *out);
+    EXPECT(e.blockSize == 24 && e.blockCount == 120);
+    EXPECT((e.strides == std::vector<ExpandInfo::Dim>{{0, 60}, {1, 5}, {0, 1}}));
+    ExpandInfo same(*out, *out);
+    EXPECT(same.strides.empty() && same.blockCount == 1 && same.blockSize == 720 * 4);
+    ExpandInfo bias(DataType::F32, {4096}, {512, 4096});
+    EXPECT(bias.blockSize == 16384 && bias.blockCount == 512 && (bias.strides == std::vector<ExpandInfo::Dim>{{0, 1}}));
+
+    auto joined = Tensor::share(DataType::I64, Shape{2, 3, 1, 20, 7, 7});
+    auto sp = SplitCollector(T::Amd, 3).filter({*joined}, refs);
+    EXPECT(sp.size() == 1 && sp[0]->is<SplitHip>() && static_cast<SplitHip const &>(*sp[0]).info.sum == 20 * postfix);
+    auto cc = ConcatCollector(T::Amd, 3).filter(refs, {*joined});
+    EXPECT(cc.size() == 1 && cc[0]->is<ConcatHip>());
+    EXPECT(SplitCollector(T::Cpu, 3).filter({*joined}, refs).empty() && ConcatCollector(T::Cpu, 3).filter(refs, {*joined}).empty());
+    EXPECT(SplitCollector(T::Amd, 9).filter({*joined}, refs).empty());// no such axis
+    EXPECT(ExpandCollector(T::Amd).filter({*in}, {*out}).size() == 1 && ExpandCollector(T::Amd).filter({*out}, {*in}).empty());
+    auto c = Tensor::share(DataType::Bool, Shape{2, 5});
+    auto x = Tensor::share(DataType::F32, Shape{2, 3, 2, 5}), y = Tensor::share(DataType::F32, Shape{3, 2, 5});
+    auto wh = WhereCollector(T::Amd).filter({*c, *x, *y}, {*x});
+    EXPECT(wh.size() == 1 && wh[0]->is<WhereHip>() && static_cast<WhereHip const &>(*wh[0]).broadcaster.outputsCount == 60);
+    auto yi = Tensor::share(DataType::I32, Shape{3, 2, 5});
+    EXPECT(WhereCollector(T::Amd).filter({*c, *x, *yi}, {*x}).empty());// x and y of different types
+    EXPECT(throws<UnreachableError>([&] { SplitCollector(T::Nvidia, 3).filter({*joined}, refs); }));
 }
 
 static Device &amd() { return *device::init(Device::Type::Amd, 0, "pool=4294967296"); }
@@ -1624,6 +1671,208 @@ static void prefillAttentionStream() {
     EXPECT(ok);
 }
 
+// The reference's test shapes (src/04kernel/test/kernels/{split,concat,expand,where}/test_cpu.cpp) through
+// build -> lower -> routine on the AMD device, against the oracle's restatement of the CPU kernels
+static void dataMoversHip() {
+    auto &dev = amd();
+    runtime::Resources res;
+    std::vector<dim_t> const sizes{1, 9, 3, 7};
+    auto joined = Tensor::share(DataType::F32, Shape{2, 3, 1, 20, 7, 7});
+    std::vector<Arc<Tensor>> parts;
+    TensorRefs refs;
+    for (auto n : sizes) parts.push_back(Tensor::share(DataType::F32, Shape{2, 3, 1, n, 7, 7}));
+    for (auto const &t : parts) refs.emplace_back(*t);
+    SplitInfo info(3, refs);
+    std::vector<float> data(joined->elementsSize());
+    std::iota(data.begin(), data.end(), 0.f);
+    auto dJoined = dev.malloc(joined->bytesSize());
+    dJoined->copyFromHost(data.data());
+    std::vector<Arc<Device::Blob>> dParts;
+    std::vector<std::vector<float>> want, got;
+    std::vector<void *> wantPtr, outPtr;
+    for (auto const &t : parts) {
+        dParts.push_back(dev.malloc(t->bytesSize()));
+        want.emplace_back(t->elementsSize());
+        got.emplace_back(t->elementsSize(), -1.f);
+    }
+    for (size_t j = 0; j < parts.size(); ++j) {
+        wantPtr.push_back(want[j].data());
+        outPtr.push_back(dParts[j]->get());
+    }
+    {// Split
+        auto kernel = SplitHip::build(info);
+        EXPECT(kernel != nullptr);
+        auto routine = kernel->lower(res).routine;
+        void const *inputs[]{dJoined->get()};
+        routine(res, nullptr, inputs, outPtr.data());
+        oracle_split(wantPtr.data(), data.data(), info.segments.data(), info.segments.size(), info.blockCount, info.sum);
+        bool ok = true;
+        for (size_t j = 0; j < parts.size(); ++j) {
+            dParts[j]->copyToHost(got[j].data());
+            ok &= got[j] == want[j];
+        }
+        EXPECT(ok);
+        EXPECT(want[1][0] == 49.f && want[3][7 * 49] == 20 * 49 + 13 * 49);// the reference's own expectation (offsets 0, 1, 10, 13)
+    }
+    {// Concat of the parts gives the joined tensor back
+        auto kernel = ConcatHip::build(info);
+        auto routine = kernel->lower(res).routine;
+        auto dOut = dev.malloc(joined->bytesSize());
+        std::vector<void const *> inputs(outPtr.begin(), outPtr.end());
+        void *outputs[]{dOut->get()};
+        routine(res, nullptr, inputs.data(), outputs);
+        std::vector<float> back(data.size(), -1.f), ref(data.size());
+        dOut->copyToHost(back.data());
+        std::vector<void const *> hostParts(wantPtr.begin(), wantPtr.end());
+        oracle_concat(ref.data(), hostParts.data(), info.segments.data(), info.segments.size(), info.blockCount, info.sum);
+        EXPECT(back == ref && back == data);
+    }
+    {// Expand {3, 4, 1, 6} -> {2, 3, 4, 5, 6}
+        auto in = Tensor::share(DataType::F32, Shape{3, 4, 1, 6}), out = Tensor::share(DataType::F32, Shape{2, 3, 4, 5, 6});
+        ExpandInfo e(*in, *out);
+        auto kernel = ExpandHip::build(e);
+        EXPECT(kernel != nullptr);
+        auto routine = kernel->lower(res).routine;
+        std::vector<float> x(in->elementsSize()), y(out->elementsSize(), -1.f), ref(out->elementsSize());
+        std::iota(x.begin(), x.end(), 0.f);
+        auto dx = dev.malloc(in->bytesSize()), dy = dev.malloc(out->bytesSize());
+        dx->copyFromHost(x.data());
+        void const *inputs[]{dx->get()};
+        void *outputs[]{dy->get()};
+        routine(res, nullptr, inputs, outputs);
+        dy->copyToHost(y.data());
+        std::vector<uint32_t> si, so;
+        for (auto [i, o] : e.strides) { si.push_back(i); so.push_back(o); }
+        oracle_expand(ref.data(), x.data(), si.data(), so.data(), static_cast<int>(si.size()), e.blockSize, e.blockCount);
+        bool pattern = true;// test_cpu.cpp:27-38: result[i][j][k][m] = 6 j + m
+        for (size_t idx = 0; idx < y.size(); ++idx) pattern &= y[idx] == static_cast<float>((idx / 30) % 12 * 6 + idx % 6);
+        EXPECT(y == ref && pattern);
+    }
+    {// Where: c {2, 5}, x {2, 3, 2, 5}, y {3, 2, 5}
+        auto c = Tensor::share(DataType::Bool, Shape{2, 5});
+        auto x = Tensor::share(DataType::F32, Shape{2, 3, 2, 5}), y = Tensor::share(DataType::F32, Shape{3, 2, 5});
+        auto kernel = WhereHip::build({*c, *x, *y});
+        EXPECT(kernel != nullptr);
+        auto const &b = static_cast<WhereHip const &>(*kernel).broadcaster;
+        auto routine = kernel->lower(res).routine;
+        std::mt19937 rng(5);
+        std::vector<uint8_t> c_(10);
+        std::vector<float> x_(60), y_(30), out(60, -1.f), ref(60);
+        for (auto &v : c_) v = rng() & 1;
+        for (auto &v : x_) v = static_cast<float>(rng() % 100);
+        for (auto &v : y_) v = static_cast<float>(100 + rng() % 100);
+        auto dc = dev.malloc(10), dx = dev.malloc(240), dy = dev.malloc(120), dout = dev.malloc(240);
+        dc->copyFromHost(c_.data());
+        dx->copyFromHost(x_.data());
+        dy->copyFromHost(y_.data());
+        void const *inputs[]{dc->get(), dx->get(), dy->get()};
+        void *outputs[]{dout->get()};
+        routine(res, nullptr, inputs, outputs);
+        dout->copyToHost(out.data());
+        oracle_where(ref.data(), c_.data(), x_.data(), y_.data(), b.strides.data(), static_cast<int>(b.strides.size() / 4),
+                     b.outputsCount, 4);
+        bool direct = true;// numpy semantics written out: c broadcasts over the first two dimensions, y over the first
+        for (size_t i = 0; i < 60; ++i) direct &= ref[i] == (c_[i % 10] ? x_[i] : y_[i % 30]);
+        EXPECT(out == ref && direct);
+    }
+}
+
+// A decode step whose projection leaves q, k and v in one tensor: Split -> RotaryEmbedding (q, k) -> Attention,
+// lowered for the AMD device and stepped, against the oracle chain
+static void fusedQkvDecodeStream() {
+    using namespace computation;
+    constexpr dim_t N = 2, H = 8, Hkv = 2, D = 128, S = 48;
+    constexpr float theta = 10000.f;
+    auto qkv = Tensor::share(DataType::FP16, Shape{N, 1, (H + 2 * Hkv) * D});
+    auto qFlat = Tensor::share(DataType::FP16, Shape{N, 1, H * D}), kFlat = Tensor::share(DataType::FP16, Shape{N, 1, Hkv * D});
+    auto q = Tensor::share(DataType::FP16, Shape{N, 1, H, D}), qa = Tensor::share(DataType::FP16, Shape{N, H, 1, D});
+    auto k = Tensor::share(DataType::FP16, Shape{N, 1, Hkv, D}), ka = Tensor::share(DataType::FP16, Shape{N, Hkv, 1, D});
+    auto pos = Tensor::share(DataType::I64, Shape{N, 1}), past = Tensor::share(DataType::I64, Shape{N});
+    auto cache = Tensor::share(DataType::FP16, Shape{N, Hkv, S, D});
+    // edges: 0 qkv 1 pos 2 past | 3 q 4 k 5 v (split) | 6 q4 | 7 k4 | 8 qr | 9 kr | 10 q' | 11 k' | 12 v' | 13 o 14 kc 15 vc
+    graph_topo::GraphTopo topo(3, 3);
+    topo.pushNode({0}, 0, 3);      // Split
+    topo.pushNode({3}, 0, 1);      // Reshape q -> [N, 1, H, D]
+    topo.pushNode({4}, 0, 1);      // Reshape k
+    topo.pushNode({6, 1}, 0, 1);   // rope q
+    topo.pushNode({7, 1}, 0, 1);   // rope k
+    topo.pushNode({8}, 0, 1);      // heads first (seq is 1: a reshape)
+    topo.pushNode({9}, 0, 1);
+    topo.pushNode({5}, 0, 1);
+    topo.pushNode({10, 11, 12, 2}, 0, 3);
+    for (count_t i = 0; i < 3; ++i) topo.setGlobalOutput(i, 13 + i);
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<Split>(2), "split_qkv"});
+    ops.push_back({std::make_unique<Reshape>(), "q_heads"});
+    ops.push_back({std::make_unique<Reshape>(), "k_heads"});
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_q"});
+    ops.push_back({std::make_unique<RotaryEmbedding>(theta), "rope_k"});
+    ops.push_back({std::make_unique<Reshape>(), "q_heads_first"});
+    ops.push_back({std::make_unique<Reshape>(), "k_heads_first"});
+    ops.push_back({std::make_unique<Reshape>(), "v_heads_first"});
+    ops.push_back({std::make_unique<Attention>(S), "attention"});
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    auto stream = computation::Graph(std::move(topo), std::move(ops),
+                                     {{qkv, "qkv"}, {pos, "pos"}, {past, "past"}, {qFlat, "q"}, {kFlat, "k"}, {kFlat, "v"},
+                                      {q, "q4"}, {k, "k4"}, {q, "qr"}, {k, "kr"}, {qa, "q'"}, {ka, "k'"}, {ka, "v'"},
+                                      {qa, "o"}, {cache, "k_cache"}, {cache, "v_cache"}})
+                      .lower(Target::Amd)
+                      .lower(dev, reusableAllocate);
+    std::mt19937 rng(44);
+    std::normal_distribution<float> n01;
+    auto randomHalf = [&](size_t n) { std::vector<uint16_t> v(n); for (auto &e : v) e = f2h(n01(rng)); return v; };
+    auto kc = randomHalf(cache->elementsSize()), vc = randomHalf(cache->elementsSize());
+    stream.getData(14)->copyFromHost(kc.data());
+    stream.getData(15)->copyFromHost(vc.data());
+    int64_t pastLen[N] = {9, 30};
+    float const scale = 1.0f / std::sqrt(static_cast<float>(D));
+    for (int step = 0; step < 3; ++step) {
+        auto x = randomHalf(qkv->elementsSize());
+        stream.setData(0, x.data(), x.size() * 2);
+        stream.setData(1, pastLen, sizeof pastLen);
+        stream.setData(2, pastLen, sizeof pastLen);
+        stream.run();
+        device::sync(Device::Type::Amd);
+        std::vector<uint16_t> o(N * H * D), kcOut(kc.size()), vcOut(vc.size());
+        EXPECT(stream.copyData(13, o.data(), o.size() * 2) && stream.copyData(14, kcOut.data(), kc.size() * 2) &&
+               stream.copyData(15, vcOut.data(), vc.size() * 2));
+        // the oracle chain: split by hand (rows of q | k | v), rope on up-cast values with one rounding back, attention
+        constexpr dim_t row = (H + 2 * Hkv) * D;
+        std::vector<float> qf(N * H * D), kf(N * Hkv * D), qr(qf.size()), kr(kf.size());
+        for (dim_t b = 0; b < N; ++b) {
+            for (dim_t i = 0; i < H * D; ++i) qf[b * H * D + i] = h2f(x[b * row + i]);
+            for (dim_t i = 0; i < Hkv * D; ++i) kf[b * Hkv * D + i] = h2f(x[b * row + H * D + i]);
+        }
+        oracle_rope_f32(qr.data(), qf.data(), pastLen, 1, N, 1, H, D, theta, 1);
+        oracle_rope_f32(kr.data(), kf.data(), pastLen, 1, N, 1, Hkv, D, theta, 1);
+        bool rowsOk = true;
+        for (dim_t b = 0; b < N; ++b)
+            for (dim_t h = 0; h < Hkv; ++h) {
+                auto const at = ((b * Hkv + h) * S + pastLen[b]) * D;
+                for (dim_t i = 0; i < D; ++i) rowsOk &= std::fabs(h2f(kcOut[at + i]) - h2f(f2h(kr[(b * Hkv + h) * D + i]))) <= 2e-3f;
+                std::memcpy(&kc[at], &kcOut[at], D * 2);
+                std::memcpy(&vc[at], &x[b * row + (H + Hkv) * D + h * D], D * 2);// v rows appended bit for bit
+            }
+        EXPECT(rowsOk && kcOut == kc && vcOut == vc);
+        bool ok = true;
+        std::vector<float> scratch(2 * S), ref(D), q1(D);
+        for (dim_t b = 0; b < N; ++b)
+            for (dim_t h = 0; h < H; ++h) {
+                dim_t const len = pastLen[b] + 1, kh = h / (H / Hkv);
+                std::vector<float> kk(len * D), vv(len * D);
+                for (size_t i = 0; i < len * D; ++i) {
+                    kk[i] = h2f(kc[(b * Hkv + kh) * S * D + i]);
+                    vv[i] = h2f(vc[(b * Hkv + kh) * S * D + i]);
+                }
+                for (dim_t i = 0; i < D; ++i) q1[i] = h2f(f2h(qr[(b * H + h) * D + i]));
+                oracle_attention_head_f32(ref.data(), q1.data(), kk.data(), vv.data(), 1, pastLen[b], D, scale, 1, scratch.data());
+                for (dim_t i = 0; i < D; ++i) ok &= std::fabs(h2f(o[(b * H + h) * D + i]) - ref[i]) <= 4e-3f;
+            }
+        EXPECT(ok);
+        for (auto &p : pastLen) ++p;
+    }
+}
+
 static void amdDeviceAndPool() {
     auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
     EXPECT(dev && dev->type() == Device::Type::Amd && device::fetch(Device::Type::Amd) == dev);
@@ -1657,6 +1906,7 @@ int main(int argc, char **argv) {
     RUN(executorOnCpu);
     RUN(transposeInfoDigest);
     RUN(computationGraphLowers);
+    RUN(dataMoverDigests);
     if (mode == "gpu") {
         RUN(amdDeviceAndPool);
         RUN(rmsNormalizationHip);
@@ -1669,6 +1919,8 @@ int main(int argc, char **argv) {
         RUN(attentionHip);
         RUN(rotaryEmbeddingHip);
         RUN(transposeHip);
+        RUN(dataMoversHip);
+        RUN(fusedQkvDecodeStream);
         RUN(quantisedLinearStream);
         RUN(executorOnGpu);
         RUN(decodeAttentionStream);

@@ -575,6 +575,94 @@ def test_transpose_full_config():
     assert np.array_equal(host(y[sl]), oracle.transpose(host(x[sl]), (0, 2, 1, 3)))
 
 
+# ------------------------------------------------------------------ Split / Concat / Expand / Where
+_MOVER_DTYPES = [np.uint8, np.int16, np.float32, np.float64]
+
+
+@pytest.mark.parametrize("shape,axis,sizes", [
+    ((2, 3, 1, 20, 7, 7), 3, [1, 9, 3, 7]),          # the reference's test shape
+    ((4096, 12288), 1, [4096, 4096, 4096]),           # fused q, k, v of 4096 tokens: segments of 8 KiB
+    ((64, 6144), 1, [4096, 1024, 1024]),              # grouped-query projection (32 + 8 + 8 heads of 128)
+    ((5, 7, 33), 2, [1, 0, 30, 2]),                   # odd sizes, an empty part
+    ((3, 40, 5), 1, list(range(1, 9)) + [4]),         # nine parts
+    ((2, 50, 3), 1, [2] * 25),                        # more parts than one launch takes
+    ((10,), 0, [3, 7]),                               # one block
+    ((7, 2, 4), 0, [5, 2]),                           # split of the slowest axis: two contiguous halves
+])
+def test_split_and_concat_bit_exact(shape, axis, sizes):
+    rng = np.random.default_rng(len(shape) * 100 + axis)
+    for dt in _MOVER_DTYPES:
+        x = rng.integers(0, 1 << 15, shape).astype(dt)
+        want = oracle.split(x, sizes, axis)
+        got = ops.split(dev(x), sizes, axis)
+        for g, w in zip(got, want):
+            assert np.array_equal(host(g), w)
+        assert np.array_equal(host(ops.concat([dev(w) for w in want], axis)), oracle.concat(want, axis))
+        assert np.array_equal(host(ops.concat(got, axis)), x)          # inverse of each other
+
+
+def test_split_concat_misaligned_views():
+    # parts and joined tensor two bytes off a four-byte boundary: the unit falls back to 2 bytes
+    x = torch.arange(3 * 10 * 6, device=DEV, dtype=torch.int16).reshape(3, 10, 6)
+    buf = torch.empty(3 * 4 * 6 + 1, device=DEV, dtype=torch.int16)
+    a = buf[1:].view(3, 4, 6)
+    b = torch.empty((3, 6, 6), device=DEV, dtype=torch.int16)
+    ops.split(x, [4, 6], 1, outs=[a, b])
+    assert torch.equal(a, x[:, :4]) and torch.equal(b, x[:, 4:])
+    jb = torch.empty(3 * 10 * 6 + 1, device=DEV, dtype=torch.int16)
+    y = ops.concat([a, b], 1, out=jb[1:].view(3, 10, 6))
+    assert torch.equal(y, x)
+
+
+@pytest.mark.parametrize("inp,out", [
+    ((3, 4, 1, 6), (2, 3, 4, 5, 6)),                  # the reference's test shape
+    ((4096,), (512, 4096)),                           # a bias over rows
+    ((32, 1, 128), (32, 512, 128)),
+    ((1, 8, 1, 128), (4, 8, 16, 128)),                # a kv head repeated
+    ((5, 1), (3, 5, 7)),                              # innermost dimension broadcast: blocks of 7 elements
+    ((1,), (9, 11)),
+    ((2, 3, 4), (2, 3, 4)),                           # nothing to do: a copy
+    ((), (4, 5)),
+])
+def test_expand_bit_exact(inp, out):
+    rng = np.random.default_rng(sum(out))
+    for dt in _MOVER_DTYPES:
+        x = rng.integers(0, 1 << 15, inp).astype(dt)
+        assert np.array_equal(host(ops.expand(dev(x), out)), oracle.expand(x, out))
+
+
+@pytest.mark.parametrize("c_shape,x_shape,y_shape", [
+    ((2, 5), (2, 3, 2, 5), (3, 2, 5)),                # the reference's test shape
+    ((512, 512), (8, 512, 512), (1,)),                # a causal mask over scores, scalar fill
+    ((64, 1024), (64, 1024), (64, 1024)),             # nothing broadcast: the vector kernel
+    ((1000,), (1000,), (1000,)),
+    ((3, 1, 5), (1, 4, 5), (3, 4, 1)),
+    ((), (7, 9), (9,)),
+    ((4, 1, 64), (1, 6, 64), (4, 6, 1)),              # 16-byte groups: c and x run along the last axis, y does not
+    ((5, 1), (5, 48), (3, 1, 48)),                    # c constant within a group
+    ((8,), (3, 5, 8), (5, 8)),                        # groups for elements of 2 bytes and wider only
+    ((2, 1, 3, 32), (1, 7, 1, 32), (32,)),
+])
+def test_where_bit_exact(c_shape, x_shape, y_shape):
+    rng = np.random.default_rng(len(x_shape))
+    for dt in _MOVER_DTYPES:
+        c = rng.integers(0, 2, c_shape).astype(bool)
+        x = rng.integers(0, 100, x_shape).astype(dt)
+        y = rng.integers(100, 200, y_shape).astype(dt)
+        assert np.array_equal(host(ops.where(dev(c), dev(x), dev(y))), oracle.where(c, x, y))
+
+
+def test_data_movers_full_size():
+    # the fused q, k, v projection of 32 x 128 tokens split into its three tensors and joined again
+    # (numpy.split is the checker at this size, the oracle on a slab)
+    x = torch.randn((4096, 3 * 4096), device=DEV).half()
+    q, k, v = ops.split(x, [4096, 4096, 4096], 1)
+    assert torch.equal(q, x[:, :4096]) and torch.equal(k, x[:, 4096:8192]) and torch.equal(v, x[:, 8192:])
+    assert torch.equal(ops.concat([q, k, v], 1), x)
+    slab = host(x[:64])
+    assert all(np.array_equal(host(t[:64]), w) for t, w in zip((q, k, v), oracle.split(slab, [4096] * 3, 1)))
+
+
 # ------------------------------------------------------------------ AttentionKVCache
 
 def _attention_case(N, H, Hkv, seq, cap, D, past, dt=torch.float16, seed=9, per_row=True, pairs=None,

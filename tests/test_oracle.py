@@ -576,3 +576,80 @@ def test_transpose_against_numpy_and_its_invariants():
     assert np.array_equal(oracle.transpose(x, (2, 3, 0, 1)), np.transpose(x, (2, 3, 0, 1)))
     assert np.array_equal(oracle.transpose(x, (0, 1, 2, 3)), x)
 
+
+
+# ------------------------------------------------------------------ Split / Concat / Expand / Where
+def test_split_concat_reference_vectors_and_numpy():
+    c = GOLDEN["split_info"]
+    assert oracle.split_info(c["parts"], c["axis"], 8) == (c["block_count"], c["sum"], c["segments"])
+    k = GOLDEN["split_concat"]
+    x = np.arange(np.prod(k["joined_shape"]), dtype=np.float32).reshape(k["joined_shape"])
+    parts = oracle.split(x, k["sizes"], k["axis"])
+    offsets = np.concatenate([[0], np.cumsum(k["sizes"])])
+    for j, part in enumerate(parts):              # the reference's own check, split/test_cpu.cpp:60-68
+        flat = part.reshape(6, -1)
+        for i in range(6):
+            assert np.array_equal(flat[i], i * 20 * 49 + offsets[j] * 49 + np.arange(k["sizes"][j] * 49))
+    iotas = [np.arange(p.size, dtype=np.float32).reshape(p.shape) for p in parts]
+    joined = oracle.concat(iotas, k["axis"]).reshape(6, -1)
+    for i in range(6):                            # concat/test_cpu.cpp:61-69
+        for j, n in enumerate(k["sizes"]):
+            assert np.array_equal(joined[i, offsets[j] * 49:offsets[j + 1] * 49], i * n * 49 + np.arange(n * 49))
+    # numpy.split / numpy.concatenate are the library routines; the two are inverse to each other
+    rng = np.random.default_rng(5)
+    for t in range(200):
+        rank = int(rng.integers(1, 6))
+        shape = [int(v) for v in rng.integers(1, 6, rank)]
+        axis = int(rng.integers(0, rank))
+        sizes = [int(v) for v in rng.integers(0, 5, int(rng.integers(1, 6)))]
+        shape[axis] = sum(sizes)
+        x = rng.integers(0, 1 << 15, shape).astype([np.uint8, np.int16, np.float32, np.float64][t % 4])
+        parts = oracle.split(x, sizes, axis)
+        ref = np.split(x, np.cumsum(sizes)[:-1], axis=axis)
+        assert all(np.array_equal(a, b) for a, b in zip(parts, ref))
+        assert np.array_equal(oracle.concat(ref, axis), x)
+
+
+def test_expand_reference_vectors_and_numpy():
+    c = GOLDEN["expand_info"]
+    pairs, block, count = oracle.expand_info(c["input"], c["output"], 4)
+    assert (pairs, block, count) == ([tuple(v) for v in c["strides"]], c["block_size"], c["block_count"])
+    d = np.arange(72, dtype=np.float32).reshape(c["input"])
+    y = oracle.expand(d, c["output"]).reshape(2, 12, 5, 6)
+    for j in range(12):                            # expand/test_cpu.cpp:27-38
+        assert np.array_equal(y[:, j], np.broadcast_to(6 * j + np.arange(6, dtype=np.float32), (2, 5, 6)))
+    rng = np.random.default_rng(6)
+    for t in range(300):
+        rank = int(rng.integers(1, 7))
+        out = [int(rng.choice([1, 1, 2, 3, 4, 5])) for _ in range(rank)]
+        keep = int(rng.integers(0, rank + 1))
+        inp = [o if rng.random() < 0.5 else 1 for o in out[rank - keep:]]
+        x = rng.integers(0, 1 << 15, inp).astype([np.uint8, np.int16, np.float32, np.float64][t % 4])
+        assert np.array_equal(oracle.expand(x, out), np.broadcast_to(x, out))
+
+
+def test_broadcaster_and_where_reference_vectors_and_numpy():
+    c = GOLDEN["broadcaster"]
+    rows, count = oracle.broadcaster(c["shapes"])
+    assert rows == c["strides"] and count == c["outputs_count"]
+    for k, want in c["locate"].items():             # broadcaster.cc:87-100
+        rem, at = int(k), [0] * 4
+        for row in rows:
+            q, rem = divmod(rem, row[4])
+            at = [a + s * q for a, s in zip(at, row[:4])]
+        assert at == want
+    w = GOLDEN["where"]
+    out = oracle.where(np.ones(w["c_shape"], bool), np.full(w["x_shape"], w["x"], np.float32), np.full(w["y_shape"], w["y"], np.float32))
+    assert out.shape == tuple(w["x_shape"]) and np.all(out == w["expected"])
+    rng = np.random.default_rng(7)
+    for t in range(300):
+        rank = int(rng.integers(0, 5))
+        out_shape = [int(rng.choice([1, 2, 3, 4])) for _ in range(rank)]
+        shapes = []
+        for _ in range(3):
+            keep = int(rng.integers(0, rank + 1))
+            shapes.append([o if rng.random() < 0.6 else 1 for o in out_shape[rank - keep:]])
+        dt = [np.uint8, np.int16, np.float32, np.float64][t % 4]
+        cnd = rng.integers(0, 2, shapes[0]).astype(bool)
+        x, y = rng.integers(0, 100, shapes[1]).astype(dt), rng.integers(100, 200, shapes[2]).astype(dt)
+        assert np.array_equal(oracle.where(cnd, x, y), np.where(cnd, x, y))
