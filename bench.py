@@ -396,6 +396,23 @@ def main():
         ops_out["softmax_causal_data_masked"] = e
         del x, y
 
+    if want("softmax_long_rows"):
+        # the scores of one decode step over a long context: [32 x 32 heads, 1, 32768] fp16, 64 KiB a row
+        nb = 6  # 6 x 134 MB
+        xs = [(3 * torch.randn((1024, 32768), device=dev)).half() for _ in range(nb)]
+        ys = [torch.empty_like(xs[0]) for _ in range(nb)]
+        wall, dms, mode = time_steps(torch, lambda i: ops.softmax(xs[i], out=ys[i]), steps, warmup, nb)
+        sl_bytes = 2 * 1024 * 32768 * 2
+        e = hbm_entry(sl_bytes, dms)
+        e.update(workload="Softmax fp16 [1024,32768] (one workgroup per row, row kept in LDS between the two sweeps)",
+                 device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn = xs[0][:64].float().cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.softmax(xn), sl_bytes // 16, "64 of the 1024 rows, fp32 on up-cast input")
+        ops_out["softmax_long_rows"] = e
+        del xs, ys
+
     if want("rope"):
         nb = 2
         xs = [torch.randn((16, 2048, 32, 128), device=dev).half() for _ in range(nb)]

@@ -116,6 +116,90 @@ __global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *
     }
 }
 
+// Rows too long for the register kernel (more than 1024 16-byte vectors; post == 1): one workgroup of 1024
+// threads per row.  One sweep over the row keeps a running (max, sum of exp) per thread, rescaling the sum
+// when the maximum rises, and leaves the first 64 KiB of the row in LDS as read; the threads' pairs are merged
+// once; the second sweep takes the row from LDS (what did not fit, from memory again) and writes the result.
+// A thread visits the same vectors in both sweeps, so the LDS copy needs no barrier of its own.  CACHED is
+// 4096 vectors (two workgroups per CU) for rows that fit in them, else 8192.
+template <class T, uint32_t CACHED>
+__global__ __launch_bounds__(1024) void softmax_long(T *__restrict__ y, const T *__restrict__ x, uint32_t mid,
+                                                     uint32_t causal_rows) {
+    using CT = typename Compute<T>::type;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr uint32_t THREADS = 1024, AHEAD = 4;
+    __shared__ Vec16<T> cache[CACHED];
+    __shared__ CT smem[THREADS / kWave];
+
+    const uint32_t t = threadIdx.x;
+    const uint64_t row = blockIdx.x;
+    const uint32_t nvec = mid / VEC;
+    uint32_t keep = mid;
+    if (causal_rows) keep = static_cast<uint32_t>(row % causal_rows) + (mid - causal_rows) + 1;
+    const uint32_t kvec = (keep + VEC - 1) / VEC;  // vectors that hold at least one kept column
+    const T *xr = x + row * mid;
+    T *yr = y + row * mid;
+
+    CT mx = neg_inf<CT>(), sum = 0;
+    for (uint32_t i0 = t; i0 < kvec; i0 += THREADS * AHEAD) {
+        Vec16<T> xv[AHEAD];
+#pragma unroll
+        for (uint32_t a = 0; a < AHEAD; ++a) {
+            const uint32_t idx = i0 + a * THREADS;
+            if (idx < kvec) xv[a] = load16_stream(xr + static_cast<size_t>(idx) * VEC);
+        }
+#pragma unroll
+        for (uint32_t a = 0; a < AHEAD; ++a) {
+            const uint32_t idx = i0 + a * THREADS;
+            if (idx >= kvec) break;
+            if (idx < CACHED) cache[idx] = xv[a];
+            CT f[VEC], vm = neg_inf<CT>();
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                f[e] = idx * VEC + e < keep ? to_compute(xv[a].v[e]) : neg_inf<CT>();
+                vm = vm < f[e] ? f[e] : vm;
+            }
+            if (mx < vm) {  // exp(-inf - vm) = 0 clears the (still zero) sum of a thread that had no maximum yet
+                sum *= Exp<T>::eval(mx - vm);
+                mx = vm;
+            }
+            if (mx > neg_inf<CT>()) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) sum += Exp<T>::eval(f[e] - mx);
+            }
+        }
+    }
+    auto wmax = [](CT v) { return wave_max(v); };
+    auto wsum = [](CT v) { return wave_sum(v); };
+    const CT row_max = block_allreduce<THREADS / kWave>(mx, smem, wmax, [](CT a, CT b) { return a < b ? b : a; });
+    // a thread without a maximum contributes 0 * exp(-inf) = 0; a row of -inf only gives NaN throughout, as
+    // in the kernel above and in the reference
+    const CT share = sum * Exp<T>::eval(mx - row_max);
+    const CT total = block_allreduce<THREADS / kWave>(share, smem, wsum, [](CT a, CT b) { return a + b; });
+    const Normalise<T> norm(total);
+
+    for (uint32_t i0 = t; i0 < nvec; i0 += THREADS * AHEAD) {
+        Vec16<T> xv[AHEAD];
+#pragma unroll
+        for (uint32_t a = 0; a < AHEAD; ++a) {
+            const uint32_t idx = i0 + a * THREADS;
+            if (idx < kvec) xv[a] = idx < CACHED ? cache[idx] : load16_stream(xr + static_cast<size_t>(idx) * VEC);
+        }
+#pragma unroll
+        for (uint32_t a = 0; a < AHEAD; ++a) {
+            const uint32_t idx = i0 + a * THREADS;
+            if (idx >= nvec) break;
+            Vec16<T> out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const bool kept = idx < kvec && idx * VEC + e < keep;
+                out.v[e] = from_compute<T>(kept ? norm(Exp<T>::eval(to_compute(xv[a].v[e]) - row_max)) : CT(0));
+            }
+            store16_stream(yr + static_cast<size_t>(idx) * VEC, out);
+        }
+    }
+}
+
 // Any mid / post / alignment: one thread per (pre, post) slice, three passes, neighbouring
 // threads touch neighbouring `post` positions.
 template <class T>
@@ -165,6 +249,13 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
         if (nvec <= 256) launch_rows<T, 256, 1>(y, x, pre, mid, causal_rows, s);
         else if (nvec <= 512) launch_rows<T, 256, 2>(y, x, pre, mid, causal_rows, s);
         else launch_rows<T, 256, 4>(y, x, pre, mid, causal_rows, s);
+    } else if (rows_ok && pre <= 0x7fffffffu) {
+        if (nvec <= 4096)
+            softmax_long<T, 4096><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, static_cast<uint32_t>(mid),
+                                                                             static_cast<uint32_t>(causal_rows));
+        else
+            softmax_long<T, 8192><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, static_cast<uint32_t>(mid),
+                                                                             static_cast<uint32_t>(causal_rows));
     } else {
         const uint64_t slices = static_cast<uint64_t>(pre) * post;
         const uint64_t grid = (slices + 255) / 256;

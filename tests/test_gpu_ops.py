@@ -129,6 +129,38 @@ def test_softmax_16bit_plain_and_causal(dt, tol):
         assert torch.all(yc[..., mask] == 0)
 
 
+def test_softmax_long_rows():
+    # rows beyond what the register kernel holds (1024 16-byte vectors): the looped kernel, with the row cached in
+    # 64 KiB or 128 KiB of LDS or, beyond that, read twice
+    rng = np.random.default_rng(31)
+    for shape, dt in [((5, 16384), torch.float16), ((3, 32768), torch.float16), ((2, 40000), torch.bfloat16),
+                      ((2, 2, 70000), torch.float16), ((3, 8192), torch.float32), ((2, 50000), torch.float32),
+                      ((2, 4104), torch.float64)]:
+        x = dev(3 * rng.standard_normal(shape)).to(dt)
+        x[0, ..., 5:9000:7] = float("-inf")        # masked entries inside the row
+        x[-1, ..., 100] = 40.0                     # a late maximum far above what came before it
+        ref = oracle.softmax(host(x.double() if dt == torch.float64 else x.float()), threads=8)
+        y = ops.softmax(x)
+        if dt == torch.float32:
+            # the oracle adds the 50000 terms of a row one after the other in float, as the reference does, which
+            # alone costs up to n * 2^-24 of the sum: the float64 softmax is the tighter check at this length
+            assert_rel(host(y), ref, 1e-4)
+            assert_rel(host(y), oracle.softmax(host(x.double()), threads=8), REL_F32)
+        elif dt == torch.float64:
+            assert_rel(host(y), ref, 1e-13)
+        else:
+            assert np.max(np.abs(host(y.float()) - ref)) <= (ABS_F16 if dt == torch.float16 else 8e-3)
+        assert float((y.double().sum(-1) - 1).abs().max()) < 2e-2
+        assert torch.all(y[0, ..., 5:9000:7] == 0)
+    # causal over a long row: 24 query rows against 16408 keys, flag == data-masked input bit for bit
+    x16 = dev(3 * rng.standard_normal((2, 24, 16408)).astype(np.float32)).half()
+    yc = ops.softmax(x16, causal=True)
+    mask = torch.arange(16408, device=DEV)[None, :] > torch.arange(24, device=DEV)[:, None] + (16408 - 24)
+    assert torch.equal(yc, ops.softmax(x16.masked_fill(mask, float("-inf"))))
+    assert np.max(np.abs(host(yc.float()) - oracle.softmax_causal(host(x16.float()), threads=8))) <= ABS_F16
+    assert torch.all(yc[..., mask] == 0)
+
+
 def test_softmax_full_config_properties():
     # [8,32,2048,2048] fp16: a slab against the oracle, the whole tensor through row sums
     g = torch.Generator(device=DEV).manual_seed(3)
