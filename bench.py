@@ -42,7 +42,7 @@ MEASURED_TRAFFIC = {
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
     "matmul_integer": (2 * 49313 + 65638) * 1024,
-    "attention_prefill": (2 * 100058 + 200612) * 1024,
+    "attention_prefill": (2 * 110058 + 196608) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
     "matmul_few_rows": (2 * 17456 + 256) * 1024,
@@ -53,6 +53,12 @@ MEASURED_TRAFFIC = {
     "matmul_integer_one_row": (2 * 8242 + 512 + 2 * 10 + 16) * 1024,
     "matmul_one_row_kn": (2 * 16460 + 8) * 1024,
     "matmul_four_rows_kn": (2 * 16565 + 32) * 1024,
+    "dynamic_quantize_linear": (2 * 32798 + 32 + 2 * 32889 + 16384) * 1024,
+    "softmax_long_rows": (2 * 32828 + 65602) * 1024,
+    "split": (2 * 49176 + 98312) * 1024,
+    "concat": (2 * 49181 + 98318) * 1024,
+    "where": (2 * 524433 + 1048576) * 1024,
+    "expand": (2 * 118 + 262162) * 1024,
 }
 
 
@@ -403,7 +409,7 @@ def main():
         ys = [torch.empty_like(xs[0]) for _ in range(nb)]
         wall, dms, mode = time_steps(torch, lambda i: ops.softmax(xs[i], out=ys[i]), steps, warmup, nb)
         sl_bytes = 2 * 1024 * 32768 * 2
-        e = hbm_entry(sl_bytes, dms)
+        e = hbm_entry(sl_bytes, dms, "softmax_long_rows")
         e.update(workload="Softmax fp16 [1024,32768] (one workgroup per row, row kept in LDS between the two sweeps)",
                  device_ms_per_launch=round(dms, 5), timing=mode)
         if not args.no_cpu:

@@ -1081,7 +1081,8 @@ def test_matmul_full_config_fp16():
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160), (200, 256, 96)])
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160), (200, 256, 96),
+                                   (5, 128, 16), (16, 11008, 48), (17, 384, 80), (31, 4224, 1040), (9, 2176, 32)])
 def test_matmul_few_rows_weight_streaming(m, k, n, dt):
     # weights as [n, k] (trans_b), fewer than 256 rows of A: the kernel that reads W once per 32 rows
     rng = np.random.default_rng(17)
