@@ -508,6 +508,9 @@ def test_empty_inputs_are_no_ops_and_bad_arguments_are_refused():
     out = torch.full((4096,), -3.0, device=DEV)
     i64 = torch.zeros(64, device=DEV, dtype=torch.int64)
     d, o = p(buf), p(out)
+    parts = (C.c_void_p * 2)(out.data_ptr(), out.data_ptr() + 8192)     # two parts inside `out`
+    null_part = (C.c_void_p * 2)(out.data_ptr(), None)
+    seg = np.array([8, 8], np.uint32).ctypes.data_as(C.c_void_p)
     calls = {
         "rms_norm rows=0": L.rg_hip_rms_norm(o, d, d, 0, 64, 1e-5, abi.F32, None),
         "softmax mid=0": L.rg_hip_softmax(o, d, 4, 0, 1, abi.F32, 0, None),
@@ -517,6 +520,10 @@ def test_empty_inputs_are_no_ops_and_bad_arguments_are_refused():
         "matmul batch=0": L.rg_hip_matmul(o, d, d, None, abi.FP16, 0, 0, 1.0, 0.0, 0, 4, 4, 4, None, None, 0, 0, 0, None),
         "matmul_integer m=0": L.rg_hip_matmul_integer(o, d, d, None, None, 0, 1, 0, 8, 8, None, None, None, None),
         "transpose no blocks": L.rg_hip_transpose(o, d, p(i64), p(i64), 1, 16, 0, None),
+        "split no blocks": L.rg_hip_split(parts, d, seg, 2, 0, 16, None),
+        "concat no parts": L.rg_hip_concat(o, parts, seg, 0, 4, 16, None),
+        "expand no blocks": L.rg_hip_expand(o, d, p(i64), p(i64), 1, 16, 0, None),
+        "where no outputs": L.rg_hip_where(o, d, d, d, None, 0, 0, 4, None),
         "attention N=0": L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 0, 8, 2, 1, 0, 128, 0.1, abi.FP16,
                                                      None, 0, None, None),
     }
@@ -545,6 +552,13 @@ def test_empty_inputs_are_no_ops_and_bad_arguments_are_refused():
                                                                               None, 0, None, None), E_ARGUMENT),
         "transpose in place": (L.rg_hip_transpose(d, d, one, one, 1, 16, 4, None), E_ARGUMENT),
         "transpose of nine dimensions": (L.rg_hip_transpose(o, d, p(i64), p(i64), 9, 16, 4, None), E_UNSUPPORTED),
+        "split segments that do not add up": (L.rg_hip_split(parts, d, seg, 2, 4, 24, None), E_ARGUMENT),
+        "split into a null part": (L.rg_hip_split(null_part, d, seg, 2, 4, 16, None), E_ARGUMENT),
+        "concat into null": (L.rg_hip_concat(None, parts, seg, 2, 4, 16, None), E_ARGUMENT),
+        "expand in place": (L.rg_hip_expand(d, d, one, one, 1, 16, 4, None), E_ARGUMENT),
+        "expand of nine dimensions": (L.rg_hip_expand(o, d, p(i64), p(i64), 9, 16, 4, None), E_UNSUPPORTED),
+        "where of three-byte elements": (L.rg_hip_where(o, d, d, d, None, 0, 16, 3, None), E_UNSUPPORTED),
+        "where without a condition": (L.rg_hip_where(o, None, d, d, None, 0, 16, 4, None), E_ARGUMENT),
         "attention head dim 96": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 2, 1, 0, 96, 0.1, abi.FP16,
                                                               d, 1 << 14, None, None), E_UNSUPPORTED),
         "attention heads not a multiple": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 3, 1, 0, 128, 0.1,
