@@ -122,6 +122,15 @@ constexpr int D_STAGE = 2 * D_TILE;      // one LDS buffer
 
 __device__ __forceinline__ uint32_t b_swizzle(uint32_t x) { return ((x & 3) << 1) | ((x >> 2) * 9); }  // x < 8
 
+// A wave-uniform pointer, moved to scalar registers (so that what is added to it later is scalar arithmetic).
+// (The builtin returns int: without the casts the low word would be sign-extended over the high one.)
+__device__ __forceinline__ const uint8_t *scalar_pointer(const uint8_t *p) {
+    const uint64_t bits = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits)));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32)));
+    return reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 template <int A_MODE, bool B_ZP>
 __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, uint8_t *lds1,
                                               const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t lda, uint32_t n,
@@ -133,24 +142,39 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
     const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
     // copy q < 8: A rows 8 (8 wave + q) .. + 7, this lane row + lane / 8, chunk position lane % 8;
     // copy 8 + p: B k-rows 4 (8 wave + p) .. + 3, this lane k-row + lane / 16, chunk position lane % 16
-    const uint8_t *a_wave = A + static_cast<uint64_t>(wave * 64) * lda;
+    const uint8_t *a_wave = scalar_pointer(A + static_cast<uint64_t>(wave * 64) * lda);
     const uint32_t a_lane = (lane >> 3) * lda + 16 * ((lane & 7) ^ (lane >> 3));
-    const uint8_t *b_wave = B + static_cast<uint64_t>(wave * 32) * n;
+    const uint8_t *b_wave = scalar_pointer(B + static_cast<uint64_t>(wave * 32) * n);
     uint32_t b_lane[2];
 #pragma unroll
     for (int p = 0; p < 2; ++p) b_lane[p] = (lane >> 4) * n + 16 * ((lane & 15) ^ b_swizzle(4 * p + (lane >> 4)));
+    // The copies are issued as assembly, a scalar base plus a 32-bit lane offset (the host keeps 8 rows of A and
+    // 4 k-rows of B below 2^31 bytes): no vector arithmetic per copy, and the compiler, which then does not know
+    // that a vector-memory instruction writes LDS, adds no waits of its own; the waits for copies in this file are
+    // the explicit ones in front of the barriers.  (Writing M0 needs one wait state before the copy reads it.)
+    const uint32_t a_lane2[2] = {a_lane, a_lane ^ 16u};
+    const uint32_t lds_addr[2] = {
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t *)lds0)),
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t *)lds1))};
     auto copy = [&](uint8_t *base, uint32_t k0, int q) {
+        const uint32_t to = base == lds0 ? lds_addr[0] : lds_addr[1];
         const uint8_t *src;
-        uint8_t *dst;
+        uint32_t lane_off, dst;
         if (q < 8) {
-            src = a_wave + (k0 + 8 * q * lda) + (a_lane ^ (16 * (q & 1)));
-            dst = base + (wave * 8 + q) * 1024;
+            src = a_wave + (k0 + static_cast<uint64_t>(8 * q) * lda);
+            lane_off = a_lane2[q & 1];
+            dst = to + (wave * 8 + q) * 1024;
         } else {
-            src = b_wave + static_cast<uint64_t>(k0 + 4 * (q - 8)) * n + b_lane[q & 1];
-            dst = base + D_TILE + (wave * 8 + (q - 8)) * 1024;
+            src = b_wave + static_cast<uint64_t>(k0 + 4 * (q - 8)) * n;
+            lane_off = b_lane[q & 1];
+            dst = to + D_TILE + (wave * 8 + (q - 8)) * 1024;
         }
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                         (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+        src = scalar_pointer(src);
+        dst = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(dst));
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(lane_off), "s"(src), "s"(dst)
+                     : "memory", "m0");
     };
     // A fragment i of k-step ks: row wm 128 + 32 i + lane % 32, chunk 2 ks + h
     const uint32_t a_off = (wm * 128 + (lane & 31)) * 128 + 16 * (h ^ (lane & 7) ^ ((lane >> 3) & 1));
@@ -209,8 +233,8 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
 
     // Tile kt is in buffer RB, tile kt+1 arrives in WB.
     auto step = [&](uint32_t kt_, uint8_t *RB, const uint8_t *WB) __attribute__((always_inline)) {
-        const uint32_t k_cp = (kt_ + 2) * BK;
-        const bool more = kt_ + 2 < k_tiles;  // uniform
+        // the tile after next; behind the end, tile 0 once more (never multiplied): no branch around the copies
+        const uint32_t k_cp = kt_ + 2 < k_tiles ? (kt_ + 2) * BK : 0;
         auto slot = [&]<int s>() __attribute__((always_inline)) {
             // rows walk the columns back and forth, so that only one operand changes between MFMAs
             constexpr int ks = s / 16, o = s % 16, row = o / 4, col = (row & 1) ? 3 - o % 4 : o % 4;
@@ -226,7 +250,7 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
             constexpr int nks = (ks + 1) % 4;
             if constexpr (o < 4) fa[nxt][o] = read_a(src, nks, o);
             else if constexpr (o < 12) read_b(src, nks, (o - 4) / 2, (o - 4) % 2, fb[nxt][(o - 4) / 2]);
-            if constexpr (s >= 48) if (more) copy(RB, k_cp, s - 48);
+            if constexpr (s >= 48) copy(RB, k_cp, s - 48);
             __builtin_amdgcn_sched_barrier(0);
         };
         [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) {
@@ -669,7 +693,8 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     const ZeroPoint za{static_cast<const uint8_t *>(a_zp), (flags & RG_MMI_A_ZP_SCALAR) ? 0u : 1u};
     const ZeroPoint zb{static_cast<const uint8_t *>(b_zp), (flags & RG_MMI_B_ZP_SCALAR) ? 0u : 1u};
     // B rows start on 16-byte boundaries when n is a multiple of 16
-    const bool fast = m >= BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b);
+    const bool fast = m >= BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b) &&
+                      k < (1u << 27) && n < (1u << 28);  // lane offsets of the tile copies stay below 2^31
 
     // fewer rows than a tile: stream B once per slab of 32 rows
     const bool skinny = !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
