@@ -41,7 +41,7 @@ MEASURED_TRAFFIC = {
     "softmax_causal": (2 * 540713 + 2097158) * 1024,
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
-    "matmul_integer": (2 * 49313 + 65638) * 1024,
+    "matmul_integer": (2 * 50834 + 65647) * 1024,
     "attention_prefill": (2 * 110058 + 196608) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
