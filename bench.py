@@ -454,6 +454,23 @@ def main():
         ops_out["dequantize_linear"] = e
         del xs, ys
 
+    if want("dequantize_linear_i32"):
+        # the same operator on the int32 sums of a MatMulInteger (the quantised layer without the fused epilogue)
+        nb = 4  # 4 x 134 MB
+        xs = [torch.randint(-(1 << 20), 1 << 20, (4096, 4096), device=dev, dtype=torch.int32) for _ in range(nb)]
+        ys = [torch.empty((4096, 4096), device=dev, dtype=torch.float32) for _ in range(nb)]
+        sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
+        wall, dms, mode = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
+        dq_bytes = 4096 * 4096 * 8 + 4096 * 4
+        e = hbm_entry(dq_bytes, dms)
+        e.update(workload="DequantizeLinear i32->f32 [4096,4096] per-axis scale", device_ms_per_launch=round(dms, 5), timing=mode)
+        if not args.no_cpu:
+            import oracle
+            xn, sn = xs[0].cpu().numpy(), sc.cpu().numpy()
+            e["cpu_baseline"] = cpu_leg(lambda: oracle.dequantize_linear(xn, sn, axis=1), dq_bytes, "the whole tensor once")
+        ops_out["dequantize_linear_i32"] = e
+        del xs, ys
+
     if want("dynamic_quantize_linear"):
         # producer of MatMulInteger's A operand; rotate inputs so that the first pass (min/max)
         # streams from HBM; the second pass re-reads the 67 MB it has just seen

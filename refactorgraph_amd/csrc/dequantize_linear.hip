@@ -72,6 +72,47 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
     }
 }
 
+// 32-bit input (the sums of a MatMulInteger), groups of 4 consecutive elements: 16 bytes in, 16 bytes out per lane,
+// UNROLL groups per thread 256 lanes apart.  Same arithmetic, same sharing of the scale as above.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+template <bool PER_AXIS, int UNROLL>
+__global__ __launch_bounds__(256) void dequant32_vec(float *__restrict__ y, const int32_t *__restrict__ x,
+                                                     const float *__restrict__ scale, const int32_t *__restrict__ zp,
+                                                     uint64_t groups, uint32_t axis_len) {
+    const uint64_t g0 = static_cast<uint64_t>(blockIdx.x) * (256 * UNROLL) + threadIdx.x;
+    i32x4 in[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g = g0 + u * 256;
+        if (g < groups) in[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4 *>(x + g * 4));
+    }
+    float s_scalar = 0.f;
+    int z_scalar = 0;
+    if constexpr (!PER_AXIS) {
+        s_scalar = scale[0];
+        z_scalar = zp ? zp[0] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g = g0 + u * 256;
+        if (g < groups) {
+            Float4 out;
+            if constexpr (PER_AXIS) {
+                const uint32_t a0 = static_cast<uint32_t>((g * 4) % axis_len);
+                const Float4 s = *reinterpret_cast<const Float4 *>(scale + a0);
+                i32x4 z = {0, 0, 0, 0};
+                if (zp) z = *reinterpret_cast<const i32x4 *>(zp + a0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(in[u][e] - z[e]) * s.v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(in[u][e] - z_scalar) * s_scalar;
+            }
+            __builtin_nontemporal_store(__builtin_bit_cast(f32x4, out), reinterpret_cast<f32x4 *>(y + g * 4));
+        }
+    }
+}
+
 // Every other case: one element per thread-iteration.
 template <class TI>
 __global__ __launch_bounds__(256) void dequant_generic(float *__restrict__ y, const TI *__restrict__ x,
@@ -119,6 +160,24 @@ template <class TI>
 int dispatch_wide(float *y, const void *x, const float *scale, const void *zp, size_t outer,
                   size_t axis_len, size_t inner, int per_axis, hipStream_t s) {
     const uint64_t n = static_cast<uint64_t>(outer) * axis_len * inner;
+    if constexpr (sizeof(TI) == 4) {
+        constexpr int UNROLL = 4;
+        const uint64_t groups = n / 4;
+        const uint64_t grid = (groups + 256 * UNROLL - 1) / (256 * UNROLL);
+        if (n % 4 == 0 && aligned16(y) && aligned16(x) && grid <= 0x7fffffffu) {
+            auto *xi = static_cast<const int32_t *>(x);
+            auto *zi = static_cast<const int32_t *>(zp);
+            if (!per_axis) {
+                dequant32_vec<false, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups, 1);
+                return launch_status();
+            }
+            if (inner == 1 && axis_len % 4 == 0 && aligned16(scale) && (!zp || aligned16(zp)) && axis_len <= 0xffffffffu) {
+                dequant32_vec<true, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups,
+                                                                                         static_cast<uint32_t>(axis_len));
+                return launch_status();
+            }
+        }
+    }
     uint64_t g = (n + 255) / 256;
     if (g > 65536) g = 65536;
     dequant_generic<TI><<<static_cast<unsigned>(g), 256, 0, s>>>(
