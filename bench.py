@@ -137,7 +137,10 @@ def time_steps(torch, fn, steps, warmup, n_sets):
     graph: the GPU leaves its idle clocks only after a few hundred milliseconds of load, so a
     short warm-up would time the clock ramp, not the kernel.  Two measurements of exactly `steps`
     steps each follow: the wall clock between two device synchronisations, and HIP events on the
-    replay stream around replays that follow an untimed one without a gap.
+    replay stream around replays that follow an untimed one without a gap.  A replay costs a few
+    microseconds between its last kernel and the next replay's first one; with fewer than 100 steps
+    the events therefore surround a graph that holds the step sequence several times over (at least
+    100 launches), so that this gap weighs on a launch as little as it does in a long run.
     Returns (wall ms per step, device ms per step, "graph" | "eager")."""
     steps = max(int(steps), 1)
     chunk = max(d for d in range(1, min(steps, 100) + 1) if steps % d == 0)
@@ -179,16 +182,29 @@ def time_steps(torch, fn, steps, warmup, n_sets):
     # (b) device time of exactly `steps` steps from HIP events on the launch stream.  The timed replays are
     #     queued directly behind one untimed replay, so the events see the kernels back to back, as a
     #     profiler's per-kernel durations do, and not the start-up of a queue that had run dry.
+    run_b, reps_b, per_b = run, steps // chunk, chunk
+    if mode == "graph" and steps < 100:
+        times = -(-100 // steps)                      # whole repetitions of the step sequence
+        try:
+            graph_b = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph_b):
+                for _ in range(times):
+                    for i in range(steps):
+                        fn(i % n_sets)
+            run_b, reps_b, per_b = graph_b.replay, 1, times * steps
+            run_b()
+        except Exception as exc:
+            sys.stderr.write(f"bench.py: second capture failed ({exc}); device time from the short graph\n")
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with ClockSampler() as clock:
-        run()
+        run_b()
         start.record()
-        for _ in range(steps // chunk):
-            run()
+        for _ in range(reps_b):
+            run_b()
         stop.record()
         torch.cuda.synchronize()
     LAST["clock"] = clock.result()
-    dev_ms = start.elapsed_time(stop) / steps
+    dev_ms = start.elapsed_time(stop) / (reps_b * per_b)
     return wall_ms, dev_ms, mode
 
 
