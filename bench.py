@@ -808,6 +808,18 @@ def main():
         ops_out["matmul_few_rows"] = e
         del a, ws, y
 
+    if want("matmul_eight_rows"):
+        # eight sequences in the decode step: operands straight from memory into block products, no pass through LDS
+        nb = 10
+        a = torch.randn((8, 4096), device=dev).half()
+        ws = [(torch.randn((4096, 4096), device=dev) * 0.05).half() for _ in range(nb)]
+        y = torch.empty((8, 4096), device=dev, dtype=torch.float16)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, ws[i], trans_b=True, out=y), steps, warmup, nb)
+        e = hbm_entry((4096 * 4096 + 2 * 8 * 4096) * 2, dms, "matmul_eight_rows")
+        e.update(workload="MatMul fp16 [8,4096] x [4096,4096]^T (trans_b)", device_ms_per_launch=round(dms, 5), timing=mode)
+        ops_out["matmul_eight_rows"] = e
+        del a, ws, y
+
     if want("matmul_one_row"):
         # the projection of a single sequence's decode step: one row of activations (matrix-vector product)
         nb = 10

@@ -19,6 +19,9 @@
 //           (8 consecutive k of one column per lane) is formed by two ds_read_b64_tr_b16, which
 //           transpose 16-bit elements inside 16 lanes (lane i receives element i % 4 of the 8-byte
 //           pieces addressed by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12).
+// Few rows of A with the weights as [n, k] (a decode step) are bound by reading the weights once: one row goes
+// through a matrix-vector kernel on the vector ALUs, 2 to 16 rows through 4x4x4 block products whose operands
+// come straight from global memory, up to 255 rows through 32x32x16 products with the tiles passed through LDS.
 // Everything else (F32, F64, transposed A, other shapes) goes through a plain tiled kernel.
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
@@ -453,6 +456,140 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
     }
 }
 
+// ---------------------------------------------------------------- two to sixteen rows of A: blocks of k
+//
+// Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 16, FP16 / BF16, with operands that need no pass through
+// LDS.  v_mfma_f32_4x4x4 multiplies sixteen independent 4x4 blocks; here the sixteen blocks stand for sixteen
+// pieces of k.  Lane l holds row l % 4 of a group of four rows and the eight elements of k-piece l / 4, so one
+// 128-bit load per lane (four rows of 256 contiguous bytes per instruction) is already the operand of two
+// instructions, for W (rows of W as the first operand) and for A (rows of A as the second) alike.  A workgroup
+// owns 16 rows of W, its wavefronts each a share of k; a wavefront keeps 4 x G accumulators of four registers
+// (rows of W 4 r + register index, row of A 4 g + l % 4, block l / 4) and streams steps of 128 k, DEPTH ahead.
+// At the end the sixteen blocks are added by two halving lane swaps and two rotations inside the 16-lane rows,
+// and the wavefronts' sums meet in LDS.  Every workgroup reads all of A from L2, and that traffic adds to the
+// time: beyond 16 rows of A the kernel above, with half as many workgroups, is faster.
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+template <class T> struct Mfma4;
+template <> struct Mfma4<__half> {
+    static __device__ __forceinline__ f4v run(u32x2 a, u32x2 b, f4v c) {
+        return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma4<__hip_bfloat16> {
+    static __device__ __forceinline__ f4v run(u32x2 a, u32x2 b, f4v c) {
+        return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s4, a), __builtin_bit_cast(s4, b), c, 0, 0, 0);
+    }
+};
+// lanes 0-31 receive lo_keeps summed over both halves of the wavefront, lanes 32-63 hi_keeps
+__device__ __forceinline__ float swap32_sum(float lo_keeps, float hi_keeps) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, lo_keeps),
+                                                    __builtin_bit_cast(uint32_t, hi_keeps), false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+// the same between neighbouring rows of 16 lanes: even rows receive even_keeps, odd rows odd_keeps
+__device__ __forceinline__ float swap16_sum(float even_keeps, float odd_keeps) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, even_keeps),
+                                                    __builtin_bit_cast(uint32_t, odd_keeps), false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+template <class T, int G, int WAVES, int DEPTH>  // G groups of four rows of A
+__global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
+                                                      Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                                                      uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    constexpr int ROWS = 4 * G, PITCH = 20;  // floats per row of a partial block [row of A][16 columns]
+    __shared__ __align__(16) float part[WAVES * ROWS * PITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t n0 = blockIdx.x * 16;
+    const uint32_t pitch = 2 * k;
+    const uint8_t *W = reinterpret_cast<const uint8_t *>(w + (bm * n + n0) * static_cast<uint64_t>(k));
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + am * m * static_cast<uint64_t>(k));
+    const uint32_t steps = k / 128;
+    const uint32_t s0 = steps * wave / WAVES, s1 = steps * (wave + 1) / WAVES, cnt = s1 - s0;
+    const uint32_t i4 = lane & 3, blk = lane >> 2;
+    uint32_t w_off[4], a_off[G];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w_off[r] = (4 * r + i4) * pitch + 16 * blk + 256 * s0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) a_off[g] = (4 * g + i4 < m ? 4 * g + i4 : m - 1) * pitch + 16 * blk + 256 * s0;
+    struct Step {
+        u32x4 w[4], a[G];
+    };
+    auto load = [&](Step &t, uint32_t j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            t.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(W + (w_off[r] + 256 * j)));
+#pragma unroll
+        for (int g = 0; g < G; ++g) t.a[g] = *reinterpret_cast<const u32x4 *>(A + (a_off[g] + 256 * j));
+    };
+    f4v acc[4][G];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int g = 0; g < G; ++g) acc[r][g] = f4v{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const Step &t) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int g = 0; g < G; ++g) acc[r][g] = Mfma4<T>::run(u32x2{t.w[r][0], t.w[r][1]}, u32x2{t.a[g][0], t.a[g][1]}, acc[r][g]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int g = 0; g < G; ++g) acc[r][g] = Mfma4<T>::run(u32x2{t.w[r][2], t.w[r][3]}, u32x2{t.a[g][2], t.a[g][3]}, acc[r][g]);
+    };
+    Step st[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < cnt) load(st[d], d);
+    for (uint32_t j = 0; j < cnt; j += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (j + d < cnt) {
+                multiply(st[d]);
+                if (j + d + DEPTH < cnt) load(st[d], j + d + DEPTH);
+            }
+        }
+    }
+    // The sixteen blocks of a register hold sixteen parts of k.  Two halving exchanges leave a lane with the sums
+    // over the four rows of 16 lanes, for the rows of W 4 rr .. 4 rr + 3; two rotations inside the row of lanes
+    // add the four blocks that are left.
+    const uint32_t rr = 2 * (lane >> 5) + ((lane >> 4) & 1);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        f4v t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float u0 = swap32_sum(acc[0][g][e], acc[2][g][e]);
+            const float u1 = swap32_sum(acc[1][g][e], acc[3][g][e]);
+            float v = swap16_sum(u0, u1);
+            v += dpp_f32<0x124>(v);  // row_ror:4
+            v += dpp_f32<0x128>(v);  // row_ror:8
+            t[e] = v;
+        }
+        if ((blk & 3) == 0) *reinterpret_cast<f4v *>(part + (wave * ROWS + 4 * g + i4) * PITCH + 4 * rr) = t;
+    }
+    __syncthreads();
+    const T *C = static_cast<const T *>(bias.ptr);
+    for (uint32_t idx = tid; idx < ROWS * 16; idx += 64 * WAVES) {
+        const uint32_t row = idx >> 4, col = idx & 15;
+        if (row < m) {
+            float v = 0.f;
+#pragma unroll
+            for (int p = 0; p < WAVES; ++p) v += part[(p * ROWS + row) * PITCH + col];
+            v *= alpha;
+            if (C) v += beta * up(C[ym * bias.sb + row * bias.sm + (n0 + col) * bias.sn]);
+            y[(ym * m + row) * n + n0 + col] = down<T>(v);
+        }
+    }
+}
+
+
 // ---------------------------------------------------------------- one to four rows of A: matrix-vector products
 //
 // Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 4, FP16 / BF16.  A matrix core would spend
@@ -757,6 +894,14 @@ int launch_gemv_kn(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t
     return launch_gemv_kn_l<T, M, 2>(y, a, b, bias, m, k, n, alpha, beta, am0, bm0, ym0, count, row0, rows, s);
 }
 
+template <class T, int G, int WAVES, int DEPTH>
+int launch_rows(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float al, float be, uint32_t am0,
+                uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+    const dim3 grid(n / 16, 1, count);
+    mm_rows<T, G, WAVES, DEPTH><<<grid, 64 * WAVES, 0, s>>>(y, a, b, bias, m, k, n, al, be, am0, bm0, ym0);
+    return launch_status();
+}
+
 constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
 
 template <class T, int M>
@@ -795,8 +940,8 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool skinny = narrow && !fast && !trans_a && trans_b && m < BM && n % 32 == 0 && k % SK_TK == 0 &&
                         aligned16(a) && aligned16(b);
 
-    // one to four rows: matrix-vector products on the vector ALUs, A (padded to 1, 2 or 4 rows) in LDS; from five
-    // rows on the matrix-core kernel below is as fast
+    // one row (and up to four where the block-product kernel below does not apply): matrix-vector products on the
+    // vector ALUs, A (padded to 1, 2 or 4 rows) in LDS
     const uint32_t gv_m = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const bool gemv = narrow && !trans_a && trans_b && m <= 4 && k > 0 && k % 8 == 0 && aligned16(a) && aligned16(b);
 
@@ -806,8 +951,20 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool gemv_kn = narrow && !trans_a && !trans_b && m <= 32 && k > 0 && k % 8 == 0 && n % 8 == 0 && aligned16(a) &&
                          aligned16(b);
 
+    // two to sixteen rows, weights as [n, k]: operands straight from global memory into 4x4x4 block products
+    const bool rows = narrow && !trans_a && trans_b && m >= 2 && m <= 16 && n % 16 == 0 && k % 128 == 0 && k > 0 &&
+                      k < (1u << 26) && aligned16(a) && aligned16(b);
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            if (rows) {
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                if (m <= 4) return launch_rows<T, 1, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                if (m <= 8) return launch_rows<T, 2, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                // many workgroups per CU: small ones, several of which run side by side
+                if (n / 16 > 384) return launch_rows<T, 4, 4, 3>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                return launch_rows<T, 4, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+            }
             if (gemv_kn) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
                 for (uint32_t r0 = 0; r0 < m32; r0 += 4) {
