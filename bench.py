@@ -46,6 +46,8 @@ MEASURED_TRAFFIC = {
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
     "matmul_few_rows": (2 * 17456 + 256) * 1024,
+    "matmul_eight_rows": (2 * 16661 + 64) * 1024,
+    "dequantize_linear_i32": (2 * 32869 + 65611) * 1024,
     "transpose": (2 * 65552 + 131217) * 1024,
     "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
@@ -478,7 +480,7 @@ def main():
         sc = torch.rand(4096, device=dev) * 9e-3 + 1e-3
         wall, dms, mode = time_steps(torch, lambda i: ops.dequantize_linear(xs[i], sc, axis=1, out=ys[i]), steps, warmup, nb)
         dq_bytes = 4096 * 4096 * 8 + 4096 * 4
-        e = hbm_entry(dq_bytes, dms)
+        e = hbm_entry(dq_bytes, dms, "dequantize_linear_i32")
         e.update(workload="DequantizeLinear i32->f32 [4096,4096] per-axis scale", device_ms_per_launch=round(dms, 5), timing=mode)
         if not args.no_cpu:
             import oracle
