@@ -952,13 +952,16 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
                          aligned16(b);
 
     // two to sixteen rows, weights as [n, k]: operands straight from global memory into 4x4x4 block products
-    const bool rows = narrow && !trans_a && trans_b && m >= 2 && m <= 16 && n % 16 == 0 && k % 128 == 0 && k > 0 &&
-                      k < (1u << 26) && aligned16(a) && aligned16(b);
+    // (a single row too when k is long: the matrix-vector kernel keeps a whole row of W per wavefront in flight,
+    // which stops paying beyond 16 KiB)
+    const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
+                      k > 0 && k < (1u << 26) && aligned16(a) && aligned16(b);
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
             if (rows) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                if (m <= 4 && k > 8192) return launch_rows<T, 1, 16, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
                 if (m <= 4) return launch_rows<T, 1, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
                 if (m <= 8) return launch_rows<T, 2, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
                 // many workgroups per CU: small ones, several of which run side by side

@@ -1098,7 +1098,7 @@ def test_matmul_full_config_fp16():
 @pytest.mark.parametrize("m,k,n", [(1, 256, 32), (7, 1024, 96), (32, 4096, 4096), (33, 512, 64), (100, 768, 160), (200, 256, 96),
                                    (5, 128, 16), (16, 11008, 48), (17, 384, 80), (31, 4224, 1040), (9, 2176, 32),
                                    (2, 4096, 1024), (4, 384, 48), (3, 128, 16), (8, 256, 4096), (13, 256, 6400),
-                                   (16, 2176, 16), (12, 1152, 6160)])
+                                   (16, 2176, 16), (12, 1152, 6160), (1, 11008, 64), (3, 16384, 32)])
 def test_matmul_few_rows_weight_streaming(m, k, n, dt):
     # weights as [n, k] (trans_b), fewer than 256 rows of A: the kernels that read W once (block products with
     # operands straight from memory up to 16 rows, in every workgroup size they are launched with; tiles through
