@@ -22,6 +22,8 @@
 // Few rows of A with the weights as [n, k] (a decode step) are bound by reading the weights once: one row goes
 // through a matrix-vector kernel on the vector ALUs, 2 to 16 rows through 4x4x4 block products whose operands
 // come straight from global memory, up to 255 rows through 32x32x16 products with the tiles passed through LDS.
+// With the weights as [k, n] the block products sit behind a transposition in registers (32 rows a pass).  Where
+// those passes would take longer than one launch of the 256 x 256 tiles, fewer than 256 rows run on one row of tiles.
 // Everything else (F32, F64, transposed A, other shapes) goes through a plain tiled kernel.
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
@@ -119,10 +121,12 @@ constexpr int M_STAGE = 2 * M_TILE;
 
 __device__ __forceinline__ uint32_t n_swizzle(uint32_t r) { return 4 * (r & 1) + 10 * ((r >> 1) & 1); }  // r < 4
 
-// A, B: byte pointers to this workgroup's first row / first column; pitches in bytes.
-template <class T, bool TRANS_B>
+// A, B: byte pointers to this workgroup's first row / first column; pitches in bytes.  SHORT_M: A has only
+// a_rows < 256 rows; the tile's rows beyond them are copied from the last one (their results are not stored).
+template <class T, bool TRANS_B, bool SHORT_M>
 __device__ __forceinline__ void mm_tile_loop(f16v (&acc)[4][4], uint8_t *lds0, uint8_t *lds1, const uint8_t *A,
-                                             const uint8_t *B, uint32_t k, uint32_t pitch_a, uint32_t pitch_b) {
+                                             const uint8_t *B, uint32_t k, uint32_t pitch_a, uint32_t pitch_b,
+                                             uint32_t a_rows) {
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
@@ -143,7 +147,12 @@ __device__ __forceinline__ void mm_tile_loop(f16v (&acc)[4][4], uint8_t *lds0, u
         const uint8_t *src;
         uint8_t *dst;
         if (q < 8) {
-            src = a_wave + (kt * 128 + 8 * q * pitch_a) + (a_lane ^ (16 * (q & 1)));
+            if constexpr (SHORT_M) {
+                const uint32_t row = wave * 64 + 8 * q + (lane >> 3);
+                src = A + ((row < a_rows ? row : a_rows - 1) * pitch_a + kt * 128 + (16 * ((lane & 7) ^ (lane >> 3) ^ (q & 1))));
+            } else {
+                src = a_wave + (kt * 128 + 8 * q * pitch_a) + (a_lane ^ (16 * (q & 1)));
+            }
             dst = base + (wave * 8 + q) * 1024;
         } else if constexpr (TRANS_B) {
             src = b_wave + (kt * 128 + 8 * (q - 8) * pitch_b) + (b_lane[0] ^ (16 * (q & 1)));
@@ -231,7 +240,7 @@ __device__ __forceinline__ void mm_tile_loop(f16v (&acc)[4][4], uint8_t *lds0, u
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
 }
 
-template <class T, bool TRANS_B>
+template <class T, bool TRANS_B, bool SHORT_M = false>  // SHORT_M: fewer than 256 rows of A, one row of tiles
 __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, const T *__restrict__ a,
                                                           const T *__restrict__ b, Bias bias, uint32_t m, uint32_t k,
                                                           uint32_t n, float alpha, float beta, uint32_t a_matrix0,
@@ -257,7 +266,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     // m and n need not be multiples of the tile: the last tile of a row or column of tiles is moved back
     // so that it ends with the matrix (m, n >= 256); the outputs it shares with its neighbour are
     // computed twice, to the same values
-    const uint32_t tile_row0 = tile_m * BM + BM <= m ? tile_m * BM : m - BM;
+    const uint32_t tile_row0 = SHORT_M ? 0 : tile_m * BM + BM <= m ? tile_m * BM : m - BM;
     const uint32_t tile_col0 = tile_n * BN + BN <= n ? tile_n * BN : n - BN;
     const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m + tile_row0) * k);
     const T *b_matrix = b + bm * static_cast<uint64_t>(k) * n;
@@ -272,7 +281,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    mm_tile_loop<T, TRANS_B>(acc, lds0, lds1, A, B, k, 2 * k, TRANS_B ? 2 * k : 2 * n);
+    mm_tile_loop<T, TRANS_B, SHORT_M>(acc, lds0, lds1, A, B, k, 2 * k, TRANS_B ? 2 * k : 2 * n, m);
 
     // 32x32 accumulator layout: lane holds column (lane % 32); register e holds row
     // 8*(e/4) + 4*(lane/32) + e%4.  The 128x128 block of a wavefront is transposed through LDS (its
@@ -297,7 +306,8 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
                 for (int e = 0; e < 4; ++e) {
                     const uint32_t row = i * 32 + 8 * eg + 4 * (lane >> 5) + e, col = j * 32 + (lane & 31);
                     v[e] = alpha * acc[i][j][4 * eg + e];
-                    if (C) v[e] += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
+                    if (C && (!SHORT_M || row0 + row < m))
+                        v[e] += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
                 }
                 // even lanes keep rows 0 and 1, odd lanes rows 2 and 3 of the group of four
                 const float give0 = odd ? v[0] : v[2], give1 = odd ? v[1] : v[3];
@@ -320,7 +330,8 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     for (int it = 0; it < 32; ++it) {
         const uint32_t idx = lane + 64 * it, row = idx / 16, chunk = idx % 16;
         const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * 256 + 16 * (chunk ^ (row & 15)));
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(Y + static_cast<uint64_t>(row) * n + chunk * 8));
+        if (!SHORT_M || row0 + row < m)
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(Y + static_cast<uint64_t>(row) * n + chunk * 8));
     }
 }
 
@@ -589,6 +600,129 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T
     }
 }
 
+
+// ---------------------------------------------------------------- up to 32 rows of A, weights as [k, n]: blocks of k
+//
+// The same block products with the weights as ONNX MatMul stores them, B [k, n]: Y[rows <= 32, n] = alpha * A @ B
+// (+ bias).  The contraction index runs down the columns of B, so a lane cannot load an operand (four
+// consecutive k of one column) in one piece; it loads CW columns of eight consecutive k-rows (eight loads of 8 or
+// 16 bytes; four lanes cover a strip of 4 CW columns, the sixteen blocks sixteen groups of eight k-rows) and
+// transposes them in registers, two byte permutes per operand.  A (rows of A as the first operand) is loaded as
+// in mm_rows.  A workgroup owns a strip and all of k, its wavefronts a share of k each, so no sums cross
+// workgroups: strips of 16 columns (32-byte pieces of a row of B) where that is needed to cover the chip, of 32
+// columns for wide B.  Strips are numbered so that neighbours, which share 128-byte lines, run on the same XCD.
+// More than 32 rows take several passes over B.
+template <int CW> struct ColumnWord;
+template <> struct ColumnWord<4> { typedef u32x2 type; };
+template <> struct ColumnWord<8> { typedef u32x4 type; };
+
+template <class T, int G, int WAVES, int CW>  // G groups of four rows of A; CW columns per lane (4 or 8)
+__global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b,
+                                                         Bias bias, uint32_t m, uint32_t m_total, uint32_t row_first, uint32_t k,
+                                                         uint32_t n, float alpha, float beta, uint32_t a_matrix0,
+                                                         uint32_t b_matrix0, uint32_t y_matrix0) {
+    constexpr int ROWS = 4 * G, SW = 4 * CW, PITCH = SW + 1;  // strip width; floats per row of a partial block
+    constexpr int DEPTH = 2;  // steps of 128 k in flight
+    typedef typename ColumnWord<CW>::type Word;
+    __shared__ float part[WAVES * ROWS * PITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    uint32_t strip = blockIdx.x;
+    if (gridDim.x % 8 == 0) strip = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const uint32_t n0 = strip * SW;
+    const uint32_t pitch_a = 2 * k, pitch_b = 2 * n;
+    const uint8_t *B = reinterpret_cast<const uint8_t *>(b + bm * k * static_cast<uint64_t>(n) + n0);
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m_total + row_first) * static_cast<uint64_t>(k));
+    const uint32_t steps = k / 128;
+    const uint32_t s0 = steps * wave / WAVES, s1 = steps * (wave + 1) / WAVES, cnt = s1 - s0;
+    const uint32_t j4 = lane & 3, blk = lane >> 2;
+    // this lane: k-rows 128 s + 8 blk .. + 7, columns n0 + CW j4 .. + CW - 1 of B; rows 4 g + j4 of A at the same k
+    const uint32_t b_off = (128 * s0 + 8 * blk) * pitch_b + 2 * CW * j4;
+    uint32_t a_off[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) a_off[g] = (4 * g + j4 < m ? 4 * g + j4 : m - 1) * pitch_a + 16 * blk + 256 * s0;
+    struct Step {
+        Word w[8];
+        u32x4 a[G];
+    };
+    auto load = [&](Step &t, uint32_t j) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            t.w[r] = __builtin_nontemporal_load(reinterpret_cast<const Word *>(B + (b_off + (128 * j + r) * pitch_b)));
+#pragma unroll
+        for (int g = 0; g < G; ++g) t.a[g] = *reinterpret_cast<const u32x4 *>(A + (a_off[g] + 256 * j));
+    };
+    f4v acc[CW][G];
+#pragma unroll
+    for (int c = 0; c < CW; ++c)
+#pragma unroll
+        for (int g = 0; g < G; ++g) acc[c][g] = f4v{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const Step &t) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            // four k-rows of CW columns become CW columns of four k
+            u32x2 col[CW];
+#pragma unroll
+            for (int p = 0; p < CW / 2; ++p) {
+                const uint32_t d0 = t.w[4 * q][p], d1 = t.w[4 * q + 1][p], d2 = t.w[4 * q + 2][p], d3 = t.w[4 * q + 3][p];
+                col[2 * p] = u32x2{__builtin_amdgcn_perm(d1, d0, 0x05040100u), __builtin_amdgcn_perm(d3, d2, 0x05040100u)};
+                col[2 * p + 1] = u32x2{__builtin_amdgcn_perm(d1, d0, 0x07060302u), __builtin_amdgcn_perm(d3, d2, 0x07060302u)};
+            }
+#pragma unroll
+            for (int c = 0; c < CW; ++c)
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    acc[c][g] = Mfma4<T>::run(u32x2{t.a[g][2 * q], t.a[g][2 * q + 1]}, col[c], acc[c][g]);
+        }
+    };
+    Step st[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < cnt) load(st[d], d);
+    for (uint32_t j = 0; j < cnt; j += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (j + d < cnt) {
+                multiply(st[d]);
+                if (j + d + DEPTH < cnt) load(st[d], j + d + DEPTH);
+            }
+        }
+    }
+    // sixteen blocks = sixteen parts of k: two halving swaps leave a lane with the columns
+    // (CW / 4) (2 (lane / 32) + (lane / 16) % 2) + x of its CW, two rotations inside the 16-lane row add the four
+    // blocks that remain
+    constexpr int Q = CW / 4;
+    const uint32_t cc = Q * (2 * (lane >> 5) + ((lane >> 4) & 1));
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int x = 0; x < Q; ++x) {
+                const float u0 = swap32_sum(acc[x][g][e], acc[2 * Q + x][g][e]);
+                const float u1 = swap32_sum(acc[Q + x][g][e], acc[3 * Q + x][g][e]);
+                float v = swap16_sum(u0, u1);
+                v += dpp_f32<0x124>(v);  // row_ror:4
+                v += dpp_f32<0x128>(v);  // row_ror:8
+                if ((blk & 3) == 0) part[(wave * ROWS + 4 * g + e) * PITCH + CW * j4 + cc + x] = v;
+            }
+    __syncthreads();
+    const T *C = static_cast<const T *>(bias.ptr);
+    for (uint32_t idx = tid; idx < ROWS * SW; idx += 64 * WAVES) {
+        const uint32_t row = idx / SW, col = idx % SW;
+        if (row < m) {
+            float v = 0.f;
+#pragma unroll
+            for (int p = 0; p < WAVES; ++p) v += part[(p * ROWS + row) * PITCH + col];
+            v *= alpha;
+            const uint64_t yrow = row_first + row;
+            if (C) v += beta * up(C[ym * bias.sb + yrow * bias.sm + (n0 + col) * bias.sn]);
+            y[(ym * m_total + yrow) * n + n0 + col] = down<T>(v);
+        }
+    }
+}
 
 // ---------------------------------------------------------------- one to four rows of A: matrix-vector products
 //
@@ -902,6 +1036,14 @@ int launch_rows(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k,
     return launch_status();
 }
 
+template <class T, int G, int WAVES, int CW>
+int launch_rows_kn(T *y, const T *a, const T *b, Bias bias, uint32_t rows, uint32_t m, uint32_t row_first, uint32_t k, uint32_t n,
+                   float al, float be, uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+    const dim3 grid(n / (4 * CW), 1, count);
+    mm_rows_kn<T, G, WAVES, CW><<<grid, 64 * WAVES, 0, s>>>(y, a, b, bias, rows, m, row_first, k, n, al, be, am0, bm0, ym0);
+    return launch_status();
+}
+
 constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
 
 template <class T, int M>
@@ -957,8 +1099,51 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
                       k > 0 && k < (1u << 26) && aligned16(a) && aligned16(b);
 
+    // fewer than 256 rows, weights as [k, n]: the same block products behind a transposition in registers, 32 rows a
+    // pass (one to four rows against a wide B stay with the matrix-vector kernel, which is a little faster there)
+    const bool rows_kn = narrow && !trans_a && !trans_b && m < BM && !(m <= 4 && n >= 8192) && n % 16 == 0 && k % 128 == 0 &&
+                         k > 0 && static_cast<uint64_t>(k) * n < (1ull << 31) && k < (1u << 26) && aligned16(a) && aligned16(b);
+
+    // fewer than 256 rows on the 256 x 256 tiles (one row of tiles, A's missing rows repeated, their results not
+    // stored): a launch costs what a full tile costs, about 93 us at k = 4096, whatever m is, so it is taken where
+    // the passes of the few-rows kernels would take longer (measured per pass at k = 4096: 5.5 ns per column for 32
+    // rows with B as [k, n], 3.4 to 4.7 ns for 64 rows with B as [n, k]) and where the plain kernel is the alternative
+    const bool short_ok = narrow && !trans_a && m < BM && n >= BN && n % 8 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
+                          aligned16(b) && aligned16(y_) && !(n % BN != 0 && bias.ptr == y_);
+    bool short_tile = false;
+    if (short_ok) {
+        if (trans_b) short_tile = rows ? false : skinny ? ((m + 63) / 64) * n > 23000 : !gemv;
+        else short_tile = rows_kn ? ((m + 31) / 32) * n > 17000 : gemv_kn ? m > 16 : true;
+    }
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            if (short_tile) {
+                const dim3 grid(static_cast<unsigned>((n + BN - 1) / BN), 1, count);
+                if (trans_b)
+                    mm_mfma_256x256<T, true, true><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                                        static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                else
+                    mm_mfma_256x256<T, false, true><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                                         static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                return launch_status();
+            }
+            if (rows_kn) {
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                const bool wide = n % 32 == 0 && n >= 8192;
+                for (uint32_t r0 = 0; r0 < m32; r0 += 32) {
+                    const uint32_t rows = m32 - r0 < 32 ? m32 - r0 : 32;
+                    int e;
+#define RG_ROWS_KN(G, CW) launch_rows_kn<T, G, 8, CW>(y, a, b, bias, rows, m32, r0, k32, n32, al, be, am0, bm0, ym0, count, s)
+                    if (rows <= 4) e = wide ? RG_ROWS_KN(1, 8) : RG_ROWS_KN(1, 4);
+                    else if (rows <= 8) e = wide ? RG_ROWS_KN(2, 8) : RG_ROWS_KN(2, 4);
+                    else if (rows <= 16) e = wide ? RG_ROWS_KN(4, 8) : RG_ROWS_KN(4, 4);
+                    else e = RG_ROWS_KN(8, 4);
+#undef RG_ROWS_KN
+                    if (e) return e;
+                }
+                return 0;
+            }
             if (rows) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
                 if (m <= 4 && k > 8192) return launch_rows<T, 1, 16, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);

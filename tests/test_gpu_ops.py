@@ -1039,9 +1039,12 @@ def test_matmul_generic_transposes_bias_broadcast(dt):
 
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
-# the last three: m and n that are no multiples of the 256 x 256 tile (last tiles moved back, overlapping)
+# (300, 64, 256) to (513, 192, 520): m and n that are no multiples of the 256 x 256 tile (last tiles moved back,
+# overlapping); after them fewer than 256 rows on one row of tiles (where the passes of the few-rows kernels would
+# take longer, or k and n fit none of them)
 @pytest.mark.parametrize("m,k,n", [(256, 64, 256), (256, 192, 512), (512, 128, 256), (300, 64, 256), (256, 128, 264),
-                                   (513, 192, 520)])
+                                   (513, 192, 520), (200, 128, 2560), (100, 64, 264), (40, 192, 512), (10, 64, 256),
+                                   (255, 128, 11008), (129, 320, 1032)])
 def test_matmul_mfma_path_fp16_bf16(m, k, n, dt, tb):
     rng = np.random.default_rng(14)
     a = rng.standard_normal((2, m, k)).astype(np.float32)
@@ -1126,9 +1129,15 @@ def test_matmul_few_rows_weight_streaming(m, k, n, dt):
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 8, 8), (1, 4096, 4096), (2, 520, 40), (3, 1000, 248), (4, 4096, 1024), (4, 11008, 72),
                                    (1, 8200, 16), (2, 12288, 104), (2, 264, 10248), (3, 512, 5120), (4, 136, 2568),
-                                   (5, 520, 40), (13, 4096, 264), (32, 1000, 248), (30, 264, 10248)])
-def test_matmul_one_to_four_rows_weights_as_k_by_n(m, k, n, dt):
-    # B as [k, n] (not transposed), at most four rows of A at a time (up to 32 rows as passes of four, the last
+                                   (5, 520, 40), (13, 4096, 264), (32, 1000, 248), (30, 264, 10248),
+                                   (1, 128, 16), (3, 256, 48), (5, 128, 16), (8, 1152, 272), (13, 256, 6400), (16, 2176, 16),
+                                   (17, 384, 80), (31, 4224, 1040), (32, 1024, 2048), (9, 11008, 64), (12, 256, 8192),
+                                   (3, 384, 8224), (6, 128, 8224), (33, 256, 64), (64, 384, 48), (40, 128, 8192),
+                                   (255, 128, 32)])
+def test_matmul_few_rows_weights_as_k_by_n(m, k, n, dt):
+    # B as [k, n] (not transposed), fewer than 256 rows of A.  With k a multiple of 128 and n of 16: block products
+    # behind a transposition in registers, 32 rows a pass, strips of 16 or (n from 8192) 32 columns.  Otherwise at
+    # most four rows of A at a time (up to 32 rows as passes of four, the last
     # one of fewer): a workgroup walks all of k for a strip of columns
     # (fixed order of summation, no atomics); k beyond one LDS segment of A (4096), k and n that end inside a
     # workgroup's step and strip; strips of 16, 32 and 64 columns (the widest that still gives 160 workgroups
