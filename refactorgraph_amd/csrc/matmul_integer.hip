@@ -11,6 +11,7 @@
 // LDS buffers.  B [k,n] stays as in memory and is byte-transposed by the LDS read, so that both
 // MFMA operands are k-contiguous.  Zero points are applied to the operand fragments, so there is
 // no pre-pass over A or B and no workspace.  Everything else goes through a plain tiled kernel.
+#include <type_traits>
 #include <utility>
 
 #include "common.hpp"
@@ -131,11 +132,13 @@ __device__ __forceinline__ const uint8_t *scalar_pointer(const uint8_t *p) {
     return reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(hi) << 32) | lo);
 }
 
-template <int A_MODE, bool B_ZP>
+// SHORT_M: A has only a_rows < 256 rows; the tile's rows beyond them are copied from the last one (their results
+// are not stored).
+template <int A_MODE, bool B_ZP, bool SHORT_M>
 __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, uint8_t *lds1,
                                               const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t lda, uint32_t n,
                                               uint32_t a_xor, const uint32_t (&za_f)[4], ZeroPoint zb,
-                                              uint64_t zb_row0) {
+                                              uint64_t zb_row0, uint32_t a_rows) {
     // k: length of the range of k walked here (A, B and zb_row0 point at its start); lda: bytes per row of A
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -161,8 +164,14 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
         const uint8_t *src;
         uint32_t lane_off, dst;
         if (q < 8) {
-            src = a_wave + (k0 + static_cast<uint64_t>(8 * q) * lda);
-            lane_off = a_lane2[q & 1];
+            if constexpr (SHORT_M) {
+                const uint32_t row = wave * 64 + 8 * q + (lane >> 3);
+                src = A + k0;
+                lane_off = (row < a_rows ? row : a_rows - 1) * lda + 16 * ((lane & 7) ^ (lane >> 3) ^ (q & 1));
+            } else {
+                src = a_wave + (k0 + static_cast<uint64_t>(8 * q) * lda);
+                lane_off = a_lane2[q & 1];
+            }
             dst = to + (wave * 8 + q) * 1024;
         } else {
             src = b_wave + static_cast<uint64_t>(k0 + 4 * (q - 8)) * n;
@@ -268,7 +277,8 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
 
 // SPLIT: blockIdx.y picks a range of `split_tiles` k-tiles and the sums are added to a zeroed Y with integer atomics
 // (exact in any order): for products with too few output tiles to occupy the chip.
-template <bool DEQ, bool SPLIT>
+// SHORT_M: fewer than 256 rows of A, one row of tiles.
+template <bool DEQ, bool SPLIT, bool SHORT_M = false>
 __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__ y, const uint8_t *__restrict__ a,
                                                            const uint8_t *__restrict__ b, ZeroPoint za, ZeroPoint zb,
                                                            Dequant dq, uint32_t m, uint32_t k, uint32_t n, uint32_t split_tiles,
@@ -295,7 +305,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     // m and n need not be multiples of the tile: the last tile of a row or column of tiles is moved back
     // so that it ends with the matrix (m, n >= 256); the outputs it shares with its neighbour are
     // computed twice, to the same values
-    const uint32_t row0 = tile_m * BM + BM <= m ? tile_m * BM : m - BM;
+    const uint32_t row0 = SHORT_M ? 0 : tile_m * BM + BM <= m ? tile_m * BM : m - BM;
     const uint32_t col0 = tile_n * BN + BN <= n ? tile_n * BN : n - BN;
     uint32_t k_begin = 0, k_len = k;
     if constexpr (SPLIT) {
@@ -322,8 +332,11 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
         if (za.per_row) {
             a_simple = false;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                za_f[i] = splat(za.ptr[am * m + row0 + wm * 128 + 32 * i + (lane & 31)]);
+            for (int i = 0; i < 4; ++i) {
+                uint32_t row = row0 + wm * 128 + 32 * i + (lane & 31);
+                if (SHORT_M && row >= m) row = m - 1;
+                za_f[i] = splat(za.ptr[am * m + row]);
+            }
         } else {
             const uint32_t z = za.ptr[0];
             if (z == 0 || z == 128) {
@@ -340,11 +353,11 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     const uint64_t zb_row0 = bm * k + k_begin;
 
     if (a_simple) {
-        if (!b_zp) mmi_tile_loop<0, false>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
-        else mmi_tile_loop<0, true>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<0, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
+        else mmi_tile_loop<0, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
     } else {
-        if (!b_zp) mmi_tile_loop<1, false>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
-        else mmi_tile_loop<1, true>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0);
+        if (!b_zp) mmi_tile_loop<1, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
+        else mmi_tile_loop<1, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
     }
 
     int32_t *Y = y + (ym * m + row0 + wm * 128) * n + col0 + wn * 128;
@@ -362,6 +375,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
             for (int e = 0; e < 16; ++e) {
                 const uint32_t row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
                 const uint32_t col = j * 32 + (lane & 31);
+                if (SHORT_M && wm * 128 + row >= m) continue;
                 if constexpr (SPLIT)
                     __hip_atomic_fetch_add(Y + static_cast<uint64_t>(row) * n + col, acc[i][j][e], __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
@@ -700,11 +714,58 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     const bool skinny = !fast && m < BM && n % 256 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
                         aligned16(b);
 
+    // fewer than 256 rows on one row of 256 x 256 tiles (A's missing rows repeated, their results not stored): for
+    // more than 64 rows (at 4096 x 4096: 128 rows 31 us through the weight-streaming kernel, 255 rows, two passes,
+    // 60 us, against 22 to 25 us here) and for shapes that kernel does not fit
+    const bool short_ok = m < BM && n >= BN && n % 16 == 0 && k % BK == 0 && k > 0 && aligned16(a) && aligned16(b) &&
+                          k < (1u << 23) && n < (1u << 28);
+
     // one to four rows: matrix-vector products on the vector ALUs
     const bool gemv = m <= 4 && n % 16 == 0 && k % 16 == 0 && k > 0 && aligned16(b) && (reinterpret_cast<uintptr_t>(a) & 3u) == 0 &&
                       (!zb.ptr || !zb.per_row || (reinterpret_cast<uintptr_t>(zb.ptr) & 3u) == 0);
 
+    const bool short_tile = short_ok && !gemv && (skinny ? m > 64 : true);
+
+    // the 256 x 256 tiles, with k split between workgroups when the tiles are few
+    auto launch_tiles = [&](auto short_m, uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        constexpr bool SHORT = decltype(short_m)::value;
+        const uint64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+        const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
+        // too few tiles for the chip: split k as well, up to kSplitMax ways with at least two k-tiles each
+        uint32_t splits = static_cast<uint32_t>(kSplitFill / (tiles * count));
+        splits = splits > kSplitMax ? kSplitMax : splits;
+        splits = splits > k_tiles / 2 ? k_tiles / 2 : splits;
+        // tiles moved back overlap: their outputs would be added twice
+        if ((!SHORT && m % BM != 0) || n % BN != 0) splits = 1;
+        if (splits > 1) {
+            const uint32_t split_tiles = (k_tiles + splits - 1) / splits;
+            splits = (k_tiles + split_tiles - 1) / split_tiles;
+            const uint64_t outputs = static_cast<uint64_t>(count) * m * n, zero_grid = (outputs + 1023) / 1024;
+            int32_t *y0 = y + static_cast<uint64_t>(ym0) * m * n;
+            mmi_zero<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(y0, outputs);
+            int rc = launch_status();
+            if (rc) return rc;
+            mmi_mfma_256x256<false, true, SHORT><<<dim3(static_cast<unsigned>(tiles), splits, count), 256, 0, s>>>(
+                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
+                static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), split_tiles, am0, bm0, ym0);
+            rc = launch_status();
+            if (rc) return rc;
+            if constexpr (DEQ) {
+                mmi_dequantize_in_place<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(
+                    y0, dq, static_cast<uint64_t>(count) * m, static_cast<uint32_t>(n));
+                return launch_status();
+            }
+            return 0;
+        }
+        const dim3 grid(static_cast<unsigned>(tiles), 1, count);
+        mmi_mfma_256x256<DEQ, false, SHORT><<<grid, 256, 0, s>>>(
+            y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
+            static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), 0, am0, bm0, ym0);
+        return launch_status();
+    };
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if (short_tile) return launch_tiles(std::true_type{}, am0, bm0, ym0, count);
         if (gemv) {
             const auto *a8 = static_cast<const uint8_t *>(a);
             const auto *b8 = static_cast<const uint8_t *>(b);
@@ -758,37 +819,7 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
             return 0;
         }
         if (fast) {
-            const uint64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
-            const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
-            // too few tiles for the chip: split k as well, up to kSplitMax ways with at least two k-tiles each
-            uint32_t splits = static_cast<uint32_t>(kSplitFill / (tiles * count));
-            splits = splits > kSplitMax ? kSplitMax : splits;
-            splits = splits > k_tiles / 2 ? k_tiles / 2 : splits;
-            if (m % BM != 0 || n % BN != 0) splits = 1;  // tiles moved back overlap: their outputs would be added twice
-            if (splits > 1) {
-                const uint32_t split_tiles = (k_tiles + splits - 1) / splits;
-                splits = (k_tiles + split_tiles - 1) / split_tiles;
-                const uint64_t outputs = static_cast<uint64_t>(count) * m * n, zero_grid = (outputs + 1023) / 1024;
-                int32_t *y0 = y + static_cast<uint64_t>(ym0) * m * n;
-                mmi_zero<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(y0, outputs);
-                int rc = launch_status();
-                if (rc) return rc;
-                mmi_mfma_256x256<false, true><<<dim3(static_cast<unsigned>(tiles), splits, count), 256, 0, s>>>(
-                    y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
-                    static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), split_tiles, am0, bm0, ym0);
-                rc = launch_status();
-                if (rc) return rc;
-                if constexpr (DEQ) {
-                    mmi_dequantize_in_place<<<static_cast<unsigned>(zero_grid > 4096 ? 4096 : zero_grid), 256, 0, s>>>(
-                        y0, dq, static_cast<uint64_t>(count) * m, static_cast<uint32_t>(n));
-                    return launch_status();
-                }
-                return 0;
-            }
-            const dim3 grid(static_cast<unsigned>(tiles), 1, count);
-            mmi_mfma_256x256<DEQ, false><<<grid, 256, 0, s>>>(
-                y, static_cast<const uint8_t *>(a), static_cast<const uint8_t *>(b), za, zb, dq,
-                static_cast<uint32_t>(m), static_cast<uint32_t>(k), static_cast<uint32_t>(n), 0, am0, bm0, ym0);
+            return launch_tiles(std::false_type{}, am0, bm0, ym0, count);
         } else {
             const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
             mmi_generic<DEQ><<<grid, 256, 0, s>>>(

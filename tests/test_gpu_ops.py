@@ -428,10 +428,13 @@ def test_matmul_integer_ragged_rows_and_columns(m, k, n):
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 128, 256), (7, 1024, 512), (32, 4096, 4096), (33, 256, 256), (64, 256, 256), (100, 384, 512),
-                                   (200, 384, 768), (255, 128, 256)])
+                                   (200, 384, 768), (255, 128, 256), (129, 256, 512), (250, 1024, 256), (100, 128, 272),
+                                   (40, 256, 1040), (5, 384, 528)])
 def test_matmul_integer_few_rows_weight_streaming(m, k, n):
     # fewer than 256 rows of A: B is streamed once per 32 rows, the k-tiles of a column block are added up with
-    # integer atomics (exact in any order); every zero-point form, equal and broadcast batches
+    # integer atomics (exact in any order); every zero-point form, equal and broadcast batches.  More than 128
+    # rows, and column counts that are no multiple of 256, run on one row of 256 x 256 tiles instead (with k split
+    # between workgroups where n is a multiple of the tile)
     rng = np.random.default_rng(m + k)
     a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
     b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
