@@ -850,7 +850,22 @@ uint32_t resident_workgroups() {
 }
 
 constexpr uint32_t kMaxWorkgroups = 4096;  // bound used by the workspace query
-constexpr size_t kPrefillMinSeq = 16;      // query rows per batch row from which the tiled kernel is used
+// Several query rows per batch row: the tiled kernel stages K/V once per 32 query rows x 4 heads, but an item walks
+// all of its keys by itself, while the split kernel reads K/V once per query row and spreads the keys over every
+// CU.  With the history length h: tiled about rounds * h * 0.020 us (rounds = items over the 512 workgroups that
+// are resident), split about N * Hkv * seq * h * 512 B at 7 TB/s; h cancels.  Measured at N = 32, 8 kv heads,
+// h = 4000: 4 rows 109 us tiled against 318 us split, 2 rows 108 against 159; at N = 1: 4 rows 84 against 20.
+constexpr size_t kPrefillAlways = 32;  // query rows from which the tiled kernel is used whatever the batch
+
+bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq) {
+    if (seq >= kPrefillAlways) return true;
+    if (seq < 2) return false;
+    const size_t group = n_head / n_kv_head, heads_per_item = group == 1 ? 1 : group == 2 ? 2 : 4;
+    const size_t rows_per_item = 32 * (4 / heads_per_item);
+    const size_t items = N * n_kv_head * ((group + heads_per_item - 1) / heads_per_item) * ((seq + rows_per_item - 1) / rows_per_item);
+    const size_t rounds = (items + 511) / 512;
+    return N * n_kv_head * seq >= 280 * rounds;
+}
 
 template <class T, int D, int G>
 int launch(AttnParams p, hipStream_t s) {
@@ -949,8 +964,8 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
         return RG_HIP_E_ARGUMENT;
 
     // many query rows per batch row: the tiled MFMA kernel (K/V staged once per query tile)
-    if (seq >= kPrefillMinSeq && prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head),
-                                                   static_cast<uint32_t>(D))) {
+    if (prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head), static_cast<uint32_t>(D)) &&
+        prefill_pays(N, n_head, n_kv_head, seq)) {
         PrefillArgs a{};
         a.q = q; a.k = k; a.v = v; a.o = o; a.kc = k_cache; a.vc = v_cache;
         a.past = past_lens;

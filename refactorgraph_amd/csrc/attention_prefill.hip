@@ -286,11 +286,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             }
         }
     };
+    // This wavefront's head within the group of the item's kv head.  A group that is no multiple of HW leaves the
+    // last chunk short: the wavefronts beyond it repeat the group's last head and store nothing.
+    auto head_in_group = [&](const Item &it) __attribute__((always_inline)) -> uint32_t {
+        const uint32_t h = it.hc * HW + wave_u % HW;
+        return h < plan.group ? h : plan.group - 1;
+    };
     // Query rows of an item: every wavefront copies its own 32 rows (8 KiB, contiguous in memory)
     // into its quarter of the buffer, laid out like a K tile (chunk c of row r at position c ^ (r & 15)).
     auto copy_q = [&](const Item &it, uint32_t buf) __attribute__((always_inline)) {
         // (b * H + head) = kvhead * group + the head's index within the group
-        const uint32_t bh = uni(it.kvhead * plan.group + it.hc * HW + wave_u % HW);
+        const uint32_t bh = uni(it.kvhead * plan.group + head_in_group(it));
         const uint32_t r0 = it.qt * ROWS + 32 * (wave_u / HW);
         const uint8_t *qh = Q + static_cast<uint64_t>(bh) * a.seq * ROWB;
         const uint32_t dst = lds_addr0 + buf + wave_u * (32 * ROWB);
@@ -393,7 +399,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     // its own quarter of the query buffer (`stage`), which nobody else touches and whose query rows
     // it has already taken: chunk c of row r at chunk position c ^ (r & 15).  Then the item's own new rows.
     auto finish_item = [&](const Item &it, const u32x4 (&ak)[ROWS / 16], const u32x4 (&av)[ROWS / 16], uint8_t *stage) __attribute__((always_inline)) {
-        const uint32_t bh = uni(it.kvhead * plan.group + it.hc * HW + wave_u % HW);
+        const uint32_t bh = uni(it.kvhead * plan.group + head_in_group(it));
+        const bool head_ok = it.hc * HW + wave_u % HW < plan.group;  // else a repeated head: nothing to store
         const uint32_t fr0 = it.qt * ROWS + 32 * (wave_u / HW);
         const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
         const bool do_append = Kc && it.hc == 0;
@@ -403,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         uint32_t tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
         const uint32_t lane = tid & 63, l32 = tid & 31, half = (tid >> 5) & 1;
-        if (fr0 < a.seq) {
+        if (fr0 < a.seq && head_ok) {
             const float inv = 1.f / half_sum(l);
 #pragma unroll
             for (int db = 0; db < 4; ++db)
@@ -469,7 +476,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         } else if (nxt.valid()) {
             const uint32_t nr0 = nxt.qt * ROWS + 32 * (wave_u / HW);
             if (nr0 + 32 <= a.seq) {
-                const uint32_t bh = uni(nxt.kvhead * plan.group + nxt.hc * HW + wave_u % HW);
+                const uint32_t bh = uni(nxt.kvhead * plan.group + head_in_group(nxt));
                 base_a = Q + (static_cast<uint64_t>(bh) * a.seq + nr0) * ROWB;
                 base_b = base_a + 16 * ROWB;
                 dst_a = lds_addr0 + other + wave_u * (32 * ROWB);
@@ -673,7 +680,7 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
     constexpr uint32_t ROWS = 32 * (4 / HW);
     PrefillPlan plan{};
     plan.group = a.H / a.Hkv;
-    plan.head_chunks = plan.group / HW;
+    plan.head_chunks = (plan.group + HW - 1) / HW;
     plan.q_tiles = (a.seq + ROWS - 1) / ROWS;
     plan.pairs = (plan.q_tiles + 1) / 2;
     const uint64_t streams = static_cast<uint64_t>(a.N) * a.Hkv * plan.head_chunks;
@@ -698,16 +705,15 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
 template <class T>
 int launch_t(const PrefillArgs &a, hipStream_t s) {
     const uint32_t group = a.H / a.Hkv;
-    if (group % 4 == 0) return launch_hw<T, 4>(a, s);
+    if (group == 1) return launch_hw<T, 1>(a, s);
     if (group == 2) return launch_hw<T, 2>(a, s);
-    return launch_hw<T, 1>(a, s);
+    return launch_hw<T, 4>(a, s);  // chunks of four heads; the last one is short when group % 4 != 0
 }
 
 }  // namespace
 
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D_) {
-    const uint32_t group = H / Hkv;
-    return D_ == D && (group % 4 == 0 || group == 2 || group == 1);
+    return D_ == D && Hkv != 0 && H % Hkv == 0;
 }
 
 int launch_prefill(const PrefillArgs &a, hipStream_t s) {

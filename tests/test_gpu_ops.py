@@ -833,11 +833,28 @@ def test_attention_decode_invariants_full_size():
     (1, 4, 2, 64, 200, 128, [100], torch.float16),        # group of 2
     (2, 16, 2, 96, 96, 128, [0, 0], torch.float16),       # group of 8: two head chunks per kv head
     (2, 8, 2, 70, 256, 128, [3, 150], torch.bfloat16),
-    (1, 6, 2, 48, 64, 128, [7], torch.float16),           # group of 3: split-KV fallback
+    (1, 6, 2, 48, 64, 128, [7], torch.float16),           # group of 3: a short chunk of heads
     (1, 8, 2, 129, 512, 128, [300], torch.float16),
 ])
 def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
     o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt)
+    assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,dt", [
+    (40, 32, 8, 2, 200, 128, torch.float16),    # two new rows per sequence, many sequences: the tiled kernel pays
+    (36, 8, 8, 3, 96, 128, torch.float16),      # MHA, three rows
+    (24, 12, 4, 5, 70, 128, torch.bfloat16),    # group of 3: the last wavefront of a chunk repeats a head, stores nothing
+    (12, 40, 8, 4, 130, 128, torch.float16),    # group of 5: two chunks, the second with one head
+    (10, 28, 4, 7, 64, 128, torch.float16),     # group of 7
+    (3, 8, 2, 9, 300, 128, torch.float16),      # few sequences: the split kernel (one segment per query row)
+])
+def test_attention_few_new_rows_either_kernel(N, H, Hkv, seq, cap, D, dt):
+    # 2 to 31 new rows per sequence run through the tiled kernel when there are enough sequences and kv heads to
+    # occupy the chip with one item each, else through the split kernel; any head group size
+    past = np.random.default_rng(33).integers(0, cap - seq + 1, N)
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt, seed=34)
     assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
 
