@@ -28,6 +28,7 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA, published
 FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 MFMA, published
+FP32_PEAK_TFLOPS = 157.3       # MI355X fp32 MFMA, published
 
 # HBM-side bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, one run each,
 # KiB per dispatch) on the workloads below and scaled by what the same counters read for a plain
@@ -789,6 +790,32 @@ def main():
                 "value": round(2 * rows * CPU_THREADS * 4096 * 4096 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": CPU_THREADS,
                 "kind": "port", "sample": f"first {rows * CPU_THREADS} rows of A, {rows} per thread ({dt:.1f} s)"}
         del a, b, y
+
+    if want("matmul_f32"):
+        # the same products in float, as an f32 graph asks for them: 4096^3 with the weights as ONNX MatMul stores
+        # them ([k, n]) on 32x32x2 matrix instructions, and one row of activations (bound by reading the weights once)
+        a = torch.randn((4096, 4096), device=dev)
+        b = torch.randn((4096, 4096), device=dev) * 0.05
+        y = torch.empty((4096, 4096), device=dev)
+        f32_steps = max(steps // 10, 1)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a, b, out=y), f32_steps, max(warmup // 10, 1), 1)
+        tflops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
+        ops_out["matmul_f32"] = {
+            "bound": "mfma", "achieved": round(tflops, 1), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+            "workload": "MatMul f32 [4096,4096] x [4096,4096] (weights as [k,n]), alpha 1, no bias",
+            "device_ms_per_launch": round(dms, 5), "timing": mode, "steps": f32_steps, "observed_sclk_mhz": LAST["clock"],
+            "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
+        del a, y
+        nb = 5  # 5 x 67 MB of weights: beyond the memory-side cache
+        a1 = torch.randn((1, 4096), device=dev)
+        ws = [b] + [torch.randn((4096, 4096), device=dev) * 0.05 for _ in range(nb - 1)]
+        y1 = torch.empty((1, 4096), device=dev)
+        wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a1, ws[i], out=y1), steps, warmup, nb)
+        e = hbm_entry((4096 * 4096 + 2 * 4096) * 4, dms)
+        e.update(workload="MatMul f32 [1,4096] x [4096,4096] (weights as [k,n])", device_ms_per_launch=round(dms, 5), timing=mode)
+        ops_out["matmul_f32_one_row"] = e
+        del a1, ws, y1, b
 
     if want("matmul_few_rows"):
         # the same projection in a decode step: 32 rows of activations; bound by reading the weights once

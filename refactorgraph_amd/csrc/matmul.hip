@@ -24,10 +24,12 @@
 // come straight from global memory, up to 255 rows through 32x32x16 products with the tiles passed through LDS.
 // With the weights as [k, n] the block products sit behind a transposition in registers (32 rows a pass).  Where
 // those passes would take longer than one launch of the 256 x 256 tiles, fewer than 256 rows run on one row of tiles.
-// Everything else (F32, F64, transposed A, other shapes) goes through a plain tiled kernel.
+// F32 (A not transposed) has 128 x 128 tiles of 32x32x2 products and the block-product kernels for few rows.
+// Everything else (F64, transposed A, other shapes) goes through a plain tiled kernel.
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
 #include <utility>
 
 #include "common.hpp"
@@ -102,6 +104,118 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef short s4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---------------------------------------------------------------- F32 on the matrix cores
+//
+// Y = alpha * A @ op(B) (+ bias) for float operands, A not transposed, k a multiple of 16: 128 x 128 outputs per
+// workgroup of four wavefronts (64 x 64 each, 2 x 2 blocks of v_mfma_f32_32x32x2_f32, whose operands are one float
+// per lane: row or column lane % 32, k lane / 32).  k is walked in tiles of 16 through two LDS buffers, filled from
+// registers (128-bit loads a tile ahead); tiles that come as [row][k] are kept with a pitch of 20 floats, B as
+// [k, n] with a pitch of 132.  Rows and columns beyond the matrix are loaded from its last ones and not stored.
+constexpr int FT = 128, FK = 16, FP_RK = 20, FP_KN = 132;
+
+template <bool TRANS_B>
+__global__ __launch_bounds__(256) void mm_f32_tiles(float *__restrict__ y, const float *__restrict__ a,
+                                                    const float *__restrict__ b, Bias bias, uint32_t m, uint32_t k, uint32_t n,
+                                                    float alpha, float beta, uint32_t a_matrix0, uint32_t b_matrix0,
+                                                    uint32_t y_matrix0) {
+    constexpr int B_TILE = TRANS_B ? FT * FP_RK : FK * FP_KN;
+    __shared__ __align__(16) float As[2][FT * FP_RK];
+    __shared__ __align__(16) float Bs[2][B_TILE];
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t row0 = blockIdx.y * FT, col0 = blockIdx.x * FT;
+    const float *A = a + am * m * static_cast<uint64_t>(k);
+    const float *B = b + bm * static_cast<uint64_t>(k) * n;
+
+    // a thread's pieces of a tile: [row][k] tiles: rows tid / 4 and + 64, k 4 (tid % 4) .. + 3;
+    // B as [k, n]: k-rows tid / 32 and + 8, columns 4 (tid % 32) .. + 3
+    const uint32_t pr = tid >> 2, pk = 4 * (tid & 3);
+    const float *a_src[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t r = row0 + pr + 64 * i;
+        a_src[i] = A + static_cast<uint64_t>(r < m ? r : m - 1) * k + pk;
+    }
+    const float *b_src[2];
+    if constexpr (TRANS_B) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t c = col0 + pr + 64 * i;
+            b_src[i] = B + static_cast<uint64_t>(c < n ? c : n - 1) * k + pk;
+        }
+    } else {
+        const uint32_t c = col0 + 4 * (tid & 31);
+        const uint32_t cc = c + 4 <= n ? c : n - 4;  // n is a multiple of 4
+#pragma unroll
+        for (int i = 0; i < 2; ++i) b_src[i] = B + static_cast<uint64_t>((tid >> 5) + 8 * i) * n + cc;
+    }
+    f32x4 ra[2], rb[2];
+    auto fetch = [&](uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            ra[i] = *reinterpret_cast<const f32x4 *>(a_src[i] + k0);
+            rb[i] = *reinterpret_cast<const f32x4 *>(TRANS_B ? b_src[i] + k0 : b_src[i] + static_cast<uint64_t>(k0) * n);
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<f32x4 *>(&As[buf][(pr + 64 * i) * FP_RK + pk]) = ra[i];
+            if constexpr (TRANS_B) *reinterpret_cast<f32x4 *>(&Bs[buf][(pr + 64 * i) * FP_RK + pk]) = rb[i];
+            else *reinterpret_cast<f32x4 *>(&Bs[buf][((tid >> 5) + 8 * i) * FP_KN + 4 * (tid & 31)]) = rb[i];
+        }
+    };
+
+    f16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const uint32_t l32 = lane & 31, kh = lane >> 5;
+    const uint32_t tiles = k / FK;
+    fetch(0);
+    for (uint32_t t = 0; t < tiles; ++t) {
+        const int buf = t & 1;
+        stash(buf);
+        __syncthreads();  // the tile is complete; the other buffer's readers of two tiles ago have passed this point
+        if (t + 1 < tiles) fetch((t + 1) * FK);
+#pragma unroll
+        for (int kk = 0; kk < FK; kk += 2) {
+            float fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = As[buf][(wm * 64 + 32 * i + l32) * FP_RK + kk + kh];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                fb[j] = TRANS_B ? Bs[buf][(wn * 64 + 32 * j + l32) * FP_RK + kk + kh] : Bs[buf][(kk + kh) * FP_KN + wn * 64 + 32 * j + l32];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
+    const float *C = static_cast<const float *>(bias.ptr);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t row = row0 + wm * 64 + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
+                const uint32_t col = col0 + wn * 64 + 32 * j + l32;
+                if (row < m && col < n) {
+                    float v = alpha * acc[i][j][e];
+                    if (C) v += beta * C[ym * bias.sb + row * bias.sm + col * bias.sn];
+                    y[(ym * m + row) * n + col] = v;
+                }
+            }
+}
 
 template <class T> struct Mfma;
 template <> struct Mfma<__half> {
@@ -481,15 +595,35 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
 // time: beyond 16 rows of A the kernel above, with half as many workgroups, is faster.
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+// Block products on a 128-bit piece of each operand (the sixteen blocks are sixteen pieces of k): PARTS
+// instructions, part q on the q-th share of the piece.
 template <class T> struct Mfma4;
 template <> struct Mfma4<__half> {
+    static constexpr int PARTS = 2;
+    template <int Q> static __device__ __forceinline__ f4v part(const u32x4 &a, const u32x4 &b, f4v c) {
+        return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, u32x2{a[2 * Q], a[2 * Q + 1]}),
+                                                  __builtin_bit_cast(h4, u32x2{b[2 * Q], b[2 * Q + 1]}), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ f4v run(u32x2 a, u32x2 b, f4v c) {
         return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(h4, a), __builtin_bit_cast(h4, b), c, 0, 0, 0);
     }
 };
 template <> struct Mfma4<__hip_bfloat16> {
+    static constexpr int PARTS = 2;
+    template <int Q> static __device__ __forceinline__ f4v part(const u32x4 &a, const u32x4 &b, f4v c) {
+        return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s4, u32x2{a[2 * Q], a[2 * Q + 1]}),
+                                                      __builtin_bit_cast(s4, u32x2{b[2 * Q], b[2 * Q + 1]}), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ f4v run(u32x2 a, u32x2 b, f4v c) {
         return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s4, a), __builtin_bit_cast(s4, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma4<float> {  // v_mfma_f32_4x4x1_16B_f32: one k per block and instruction
+    static constexpr int PARTS = 4;
+    template <int Q> static __device__ __forceinline__ f4v part(const u32x4 &a, const u32x4 &b, f4v c) {
+        // (elements copied into scalars first: reinterpreting a vector element in place reads element 0)
+        const uint32_t ua = a[Q], ub = b[Q];
+        return __builtin_amdgcn_mfma_f32_4x4x1f32(__builtin_bit_cast(float, ua), __builtin_bit_cast(float, ub), c, 0, 0, 0);
     }
 };
 // lanes 0-31 receive lo_keeps summed over both halves of the wavefront, lanes 32-63 hi_keeps
@@ -509,8 +643,10 @@ __device__ __forceinline__ float swap16_sum(float even_keeps, float odd_keeps) {
 
 template <class T, int G, int WAVES, int DEPTH>  // G groups of four rows of A
 __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ w,
-                                                      Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
-                                                      uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+                                                      Bias bias, uint32_t m, uint32_t m_total, uint32_t row_first, uint32_t k,
+                                                      uint32_t n, float alpha, float beta, uint32_t a_matrix0,
+                                                      uint32_t b_matrix0, uint32_t y_matrix0) {
+    // rows row_first .. row_first + m - 1 of each m_total-row matrix
     constexpr int ROWS = 4 * G, PITCH = 20;  // floats per row of a partial block [row of A][16 columns]
     __shared__ __align__(16) float part[WAVES * ROWS * PITCH];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -518,10 +654,10 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
     const uint32_t n0 = blockIdx.x * 16;
-    const uint32_t pitch = 2 * k;
+    const uint32_t pitch = sizeof(T) * k;
     const uint8_t *W = reinterpret_cast<const uint8_t *>(w + (bm * n + n0) * static_cast<uint64_t>(k));
-    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + am * m * static_cast<uint64_t>(k));
-    const uint32_t steps = k / 128;
+    const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m_total + row_first) * static_cast<uint64_t>(k));
+    const uint32_t steps = pitch / 256;  // a step is 256 bytes of every row: 128 or (float) 64 k
     const uint32_t s0 = steps * wave / WAVES, s1 = steps * (wave + 1) / WAVES, cnt = s1 - s0;
     const uint32_t i4 = lane & 3, blk = lane >> 2;
     uint32_t w_off[4], a_off[G];
@@ -545,14 +681,18 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T
 #pragma unroll
         for (int g = 0; g < G; ++g) acc[r][g] = f4v{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const Step &t) {
+        auto sweep = [&]<int Q>() __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+            for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int g = 0; g < G; ++g) acc[r][g] = Mfma4<T>::run(u32x2{t.w[r][0], t.w[r][1]}, u32x2{t.a[g][0], t.a[g][1]}, acc[r][g]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int g = 0; g < G; ++g) acc[r][g] = Mfma4<T>::run(u32x2{t.w[r][2], t.w[r][3]}, u32x2{t.a[g][2], t.a[g][3]}, acc[r][g]);
+                for (int g = 0; g < G; ++g) acc[r][g] = Mfma4<T>::template part<Q>(t.w[r], t.a[g], acc[r][g]);
+        };
+        sweep.template operator()<0>();
+        sweep.template operator()<1>();
+        if constexpr (Mfma4<T>::PARTS == 4) {
+            sweep.template operator()<2>();
+            sweep.template operator()<3>();
+        }
     };
     Step st[DEPTH];
 #pragma unroll
@@ -594,12 +734,12 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T
 #pragma unroll
             for (int p = 0; p < WAVES; ++p) v += part[(p * ROWS + row) * PITCH + col];
             v *= alpha;
-            if (C) v += beta * up(C[ym * bias.sb + row * bias.sm + (n0 + col) * bias.sn]);
-            y[(ym * m + row) * n + n0 + col] = down<T>(v);
+            const uint64_t yrow = row_first + row;
+            if (C) v += beta * up(C[ym * bias.sb + yrow * bias.sm + (n0 + col) * bias.sn]);
+            y[(ym * m_total + yrow) * n + n0 + col] = down<T>(v);
         }
     }
 }
-
 
 // ---------------------------------------------------------------- up to 32 rows of A, weights as [k, n]: blocks of k
 //
@@ -612,9 +752,9 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows(T *__restrict__ y, const T
 // workgroups: strips of 16 columns (32-byte pieces of a row of B) where that is needed to cover the chip, of 32
 // columns for wide B.  Strips are numbered so that neighbours, which share 128-byte lines, run on the same XCD.
 // More than 32 rows take several passes over B.
-template <int CW> struct ColumnWord;
-template <> struct ColumnWord<4> { typedef u32x2 type; };
-template <> struct ColumnWord<8> { typedef u32x4 type; };
+template <int BYTES> struct ColumnWord;  // CW columns of one k-row
+template <> struct ColumnWord<8> { typedef u32x2 type; };
+template <> struct ColumnWord<16> { typedef u32x4 type; };
 
 template <class T, int G, int WAVES, int CW>  // G groups of four rows of A; CW columns per lane (4 or 8)
 __global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b,
@@ -623,7 +763,10 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, cons
                                                          uint32_t b_matrix0, uint32_t y_matrix0) {
     constexpr int ROWS = 4 * G, SW = 4 * CW, PITCH = SW + 1;  // strip width; floats per row of a partial block
     constexpr int DEPTH = 2;  // steps of 128 k in flight
-    typedef typename ColumnWord<CW>::type Word;
+    constexpr bool F32 = sizeof(T) == 4;  // floats: four columns per lane, one k per block and instruction, no transposition
+    static_assert(!F32 || CW == 4, "floats come four columns to a lane");
+    constexpr int AW = F32 ? 2 : 1;       // 128-bit pieces of a row of A per step: eight k
+    typedef typename ColumnWord<sizeof(T) * CW>::type Word;
     __shared__ float part[WAVES * ROWS * PITCH];
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -632,27 +775,30 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, cons
     uint32_t strip = blockIdx.x;
     if (gridDim.x % 8 == 0) strip = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     const uint32_t n0 = strip * SW;
-    const uint32_t pitch_a = 2 * k, pitch_b = 2 * n;
+    const uint32_t pitch_a = sizeof(T) * k, pitch_b = sizeof(T) * n;
     const uint8_t *B = reinterpret_cast<const uint8_t *>(b + bm * k * static_cast<uint64_t>(n) + n0);
     const uint8_t *A = reinterpret_cast<const uint8_t *>(a + (am * m_total + row_first) * static_cast<uint64_t>(k));
     const uint32_t steps = k / 128;
     const uint32_t s0 = steps * wave / WAVES, s1 = steps * (wave + 1) / WAVES, cnt = s1 - s0;
     const uint32_t j4 = lane & 3, blk = lane >> 2;
     // this lane: k-rows 128 s + 8 blk .. + 7, columns n0 + CW j4 .. + CW - 1 of B; rows 4 g + j4 of A at the same k
-    const uint32_t b_off = (128 * s0 + 8 * blk) * pitch_b + 2 * CW * j4;
+    const uint32_t b_off = (128 * s0 + 8 * blk) * pitch_b + sizeof(T) * CW * j4;
     uint32_t a_off[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) a_off[g] = (4 * g + j4 < m ? 4 * g + j4 : m - 1) * pitch_a + 16 * blk + 256 * s0;
+    for (int g = 0; g < G; ++g)
+        a_off[g] = (4 * g + j4 < m ? 4 * g + j4 : m - 1) * pitch_a + 16 * AW * blk + 256 * AW * s0;
     struct Step {
         Word w[8];
-        u32x4 a[G];
+        u32x4 a[G][AW];
     };
     auto load = [&](Step &t, uint32_t j) {
 #pragma unroll
         for (int r = 0; r < 8; ++r)
             t.w[r] = __builtin_nontemporal_load(reinterpret_cast<const Word *>(B + (b_off + (128 * j + r) * pitch_b)));
 #pragma unroll
-        for (int g = 0; g < G; ++g) t.a[g] = *reinterpret_cast<const u32x4 *>(A + (a_off[g] + 256 * j));
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int x = 0; x < AW; ++x) t.a[g][x] = *reinterpret_cast<const u32x4 *>(A + (a_off[g] + 256 * AW * j + 16 * x));
     };
     f4v acc[CW][G];
 #pragma unroll
@@ -660,6 +806,20 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, cons
 #pragma unroll
         for (int g = 0; g < G; ++g) acc[c][g] = f4v{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const Step &t) {
+        if constexpr (F32) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r)
+#pragma unroll
+                for (int c = 0; c < CW; ++c) {
+                    const uint32_t wv = t.w[r][c];
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const uint32_t av = t.a[g][r / 4][r % 4];
+                        acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(__builtin_bit_cast(float, av), __builtin_bit_cast(float, wv),
+                                                                       acc[c][g], 0, 0, 0);
+                    }
+                }
+        } else {
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             // four k-rows of CW columns become CW columns of four k
@@ -674,7 +834,8 @@ __global__ __launch_bounds__(64 * WAVES) void mm_rows_kn(T *__restrict__ y, cons
             for (int c = 0; c < CW; ++c)
 #pragma unroll
                 for (int g = 0; g < G; ++g)
-                    acc[c][g] = Mfma4<T>::run(u32x2{t.a[g][2 * q], t.a[g][2 * q + 1]}, col[c], acc[c][g]);
+                    acc[c][g] = Mfma4<T>::run(u32x2{t.a[g][0][2 * q], t.a[g][0][2 * q + 1]}, col[c], acc[c][g]);
+        }
         }
     };
     Step st[DEPTH];
@@ -1029,10 +1190,10 @@ int launch_gemv_kn(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t
 }
 
 template <class T, int G, int WAVES, int DEPTH>
-int launch_rows(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float al, float be, uint32_t am0,
-                uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
+int launch_rows(T *y, const T *a, const T *b, Bias bias, uint32_t rows, uint32_t m, uint32_t row_first, uint32_t k, uint32_t n,
+                float al, float be, uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, hipStream_t s) {
     const dim3 grid(n / 16, 1, count);
-    mm_rows<T, G, WAVES, DEPTH><<<grid, 64 * WAVES, 0, s>>>(y, a, b, bias, m, k, n, al, be, am0, bm0, ym0);
+    mm_rows<T, G, WAVES, DEPTH><<<grid, 64 * WAVES, 0, s>>>(y, a, b, bias, rows, m, row_first, k, n, al, be, am0, bm0, ym0);
     return launch_status();
 }
 
@@ -1116,6 +1277,26 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
         else short_tile = rows_kn ? ((m + 31) / 32) * n > 17000 : gemv_kn ? m > 16 : true;
     }
 
+    // F32 on the matrix cores.  A launch of the 128 x 128 tiles walks all of k in every workgroup and takes about
+    // 300 us at k = 4096 however few tiles there are; up to that cost few rows go through the block products of
+    // mm_rows / mm_rows_kn (one k per block and instruction; no transposition needed for B as [k, n], an operand
+    // being one float), 32 rows a pass: 27 us (B as [n, k]) and 33 us (as [k, n]) per pass and 4096 columns.
+    constexpr bool is_f32 = std::is_same<T, float>::value;
+    const bool f32_tiles_ok = is_f32 && !trans_a && k % FK == 0 && k > 0 && aligned16(a) && aligned16(b) &&
+                              (trans_b || (n % 4 == 0 && n >= 4));
+    const bool rows_f32_ok = is_f32 && !trans_a && trans_b && n % 16 == 0 && k % 64 == 0 && k > 0 && k < (1u << 25) &&
+                             aligned16(a) && aligned16(b);
+    const bool rows_kn_f32_ok = is_f32 && !trans_a && !trans_b && n % 16 == 0 && k % 128 == 0 && k > 0 &&
+                                static_cast<uint64_t>(k) * n < (1ull << 30) && k < (1u << 25) && aligned16(a) && aligned16(b);
+    // (microseconds, from those figures, with 3 us for a launch; 768 tiles run side by side)
+    const double kn4096 = static_cast<double>(n) / 4096 * static_cast<double>(k) / 4096;
+    const double f32_tile_rounds = static_cast<double>((((m + FT - 1) / FT) * ((n + FT - 1) / FT) + 767) / 768);
+    const double f32_cost_tiles = f32_tiles_ok ? 3.0 + 300.0 * static_cast<double>(k) / 4096 * f32_tile_rounds : 1e30;
+    const double f32_passes = static_cast<double>((m + 31) / 32);
+    const bool rows_f32 = rows_f32_ok && f32_passes * (3.0 + 27.0 * kn4096) <= f32_cost_tiles;
+    const bool rows_kn_f32 = rows_kn_f32_ok && f32_passes * (3.0 + 33.0 * kn4096) <= f32_cost_tiles;
+    const bool f32_tiles = f32_tiles_ok && m > 8;
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
             if (short_tile) {
@@ -1146,12 +1327,12 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
             }
             if (rows) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
-                if (m <= 4 && k > 8192) return launch_rows<T, 1, 16, 2>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
-                if (m <= 4) return launch_rows<T, 1, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
-                if (m <= 8) return launch_rows<T, 2, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                if (m <= 4 && k > 8192) return launch_rows<T, 1, 16, 2>(y, a, b, bias, m32, m32, 0, k32, n32, al, be, am0, bm0, ym0, count, s);
+                if (m <= 4) return launch_rows<T, 1, 16, 1>(y, a, b, bias, m32, m32, 0, k32, n32, al, be, am0, bm0, ym0, count, s);
+                if (m <= 8) return launch_rows<T, 2, 16, 1>(y, a, b, bias, m32, m32, 0, k32, n32, al, be, am0, bm0, ym0, count, s);
                 // many workgroups per CU: small ones, several of which run side by side
-                if (n / 16 > 384) return launch_rows<T, 4, 4, 3>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
-                return launch_rows<T, 4, 16, 1>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0, count, s);
+                if (n / 16 > 384) return launch_rows<T, 4, 4, 3>(y, a, b, bias, m32, m32, 0, k32, n32, al, be, am0, bm0, ym0, count, s);
+                return launch_rows<T, 4, 16, 1>(y, a, b, bias, m32, m32, 0, k32, n32, al, be, am0, bm0, ym0, count, s);
             }
             if (gemv_kn) {
                 const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
@@ -1199,6 +1380,47 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
                 else
                     mm_mfma_256x256<T, false><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
                                                                    static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                return launch_status();
+            }
+        }
+        if constexpr (std::is_same<T, float>::value) {
+            if (rows_f32) {
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                for (uint32_t r0 = 0; r0 < m32; r0 += 32) {
+                    const uint32_t rows = m32 - r0 < 32 ? m32 - r0 : 32;
+                    int e;
+#define RG_ROWS_F32(G, W, DP) launch_rows<T, G, W, DP>(y, a, b, bias, rows, m32, r0, k32, n32, al, be, am0, bm0, ym0, count, s)
+                    if (rows <= 4) e = RG_ROWS_F32(1, 16, 1);
+                    else if (rows <= 8) e = RG_ROWS_F32(2, 16, 1);
+                    else if (rows <= 16) e = n / 16 > 384 ? RG_ROWS_F32(4, 4, 3) : RG_ROWS_F32(4, 16, 1);
+                    else e = RG_ROWS_F32(8, 4, 3);
+#undef RG_ROWS_F32
+                    if (e) return e;
+                }
+                return 0;
+            }
+            if (rows_kn_f32) {
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                for (uint32_t r0 = 0; r0 < m32; r0 += 32) {
+                    const uint32_t rows = m32 - r0 < 32 ? m32 - r0 : 32;
+                    int e;
+#define RG_ROWS_KN_F32(G, W) launch_rows_kn<T, G, W, 4>(y, a, b, bias, rows, m32, r0, k32, n32, al, be, am0, bm0, ym0, count, s)
+                    if (rows <= 4) e = RG_ROWS_KN_F32(1, 8);
+                    else if (rows <= 8) e = RG_ROWS_KN_F32(2, 8);
+                    else if (rows <= 16) e = RG_ROWS_KN_F32(4, 8);
+                    else e = RG_ROWS_KN_F32(8, 4);  // 128 accumulators and two steps of operands: one wavefront per SIMD
+#undef RG_ROWS_KN_F32
+                    if (e) return e;
+                }
+                return 0;
+            }
+            if (f32_tiles) {
+                const dim3 grid(static_cast<unsigned>((n + FT - 1) / FT), static_cast<unsigned>((m + FT - 1) / FT), count);
+                if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
+                if (trans_b) mm_f32_tiles<true><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                                    static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                else mm_f32_tiles<false><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
+                                                              static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
                 return launch_status();
             }
         }

@@ -1058,6 +1058,29 @@ def test_matmul_generic_transposes_bias_broadcast(dt):
 
 
 @pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("m,k,n", [(130, 64, 260), (65, 16, 4), (256, 128, 128), (100, 48, 36), (70, 32, 8), (300, 4096, 132),
+                                   (1, 64, 16), (3, 4096, 64), (7, 192, 48), (13, 128, 6400), (16, 1024, 32), (31, 320, 80),
+                                   (32, 4096, 256), (50, 128, 32), (64, 64, 16), (5, 128, 16), (40, 256, 48), (2, 4096, 64)])
+def test_matmul_f32_on_the_matrix_cores(m, k, n, tb):
+    # float operands.  More than 64 rows, k a multiple of 16 (and n of 4 for B as [k, n]): 128 x 128 tiles of 32x32x2
+    # products, rows and columns beyond the matrix loaded from its last ones.  Up to 64 rows against B as [n, k]
+    # (k a multiple of 64, n of 16): 4x4x1 block products, 32 rows a pass.  Batches, bias forms, alpha and beta as
+    # everywhere
+    rng = np.random.default_rng(m + n)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    b = rng.standard_normal((2, n, k) if tb else (2, k, n)).astype(np.float32)
+    for bias in (None, rng.standard_normal((n,)).astype(np.float32), rng.standard_normal((2, m, n)).astype(np.float32)):
+        ref = oracle.matmul(a, b, bias, False, tb, 0.5, 2.0, "f32")
+        got = host(ops.matmul(dev(a), dev(b), None if bias is None else dev(bias), False, tb, 0.5, 2.0))
+        _matmul_check(got, ref, _absprod(a, b, False, tb), 1e-5)
+    # integer-valued operands: every product and sum is exact
+    ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    bi = rng.integers(-8, 9, (n, k) if tb else (k, n)).astype(np.float32)
+    want = ai.astype(np.int64) @ (bi.T if tb else bi).astype(np.int64)
+    assert np.array_equal(host(ops.matmul(dev(ai), dev(bi), trans_b=tb)), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 # (300, 64, 256) to (513, 192, 520): m and n that are no multiples of the 256 x 256 tile (last tiles moved back,
 # overlapping); after them fewer than 256 rows on one row of tiles (where the passes of the few-rows kernels would
