@@ -53,6 +53,9 @@ MEASURED_TRAFFIC = {
     "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
     "matmul_one_row": (2 * 16444 + 8) * 1024,
+    "matmul_one_row_kn": (2 * 16499 + 20) * 1024,
+    "matmul_f32_one_row": (2 * 35255 + 16) * 1024,
+    "matmul_few_rows_kn": (2 * 17591 + 256) * 1024,
     "matmul_integer_one_row": (2 * 8242 + 512 + 2 * 10 + 16) * 1024,
     "dynamic_quantize_linear": (2 * 32798 + 32 + 2 * 32889 + 16384) * 1024,
     "softmax_long_rows": (2 * 32828 + 65602) * 1024,
@@ -802,7 +805,7 @@ def main():
         tflops = 2 * 4096 ** 3 / (dms * 1e-3) / 1e12
         ops_out["matmul_f32"] = {
             "bound": "mfma", "achieved": round(tflops, 1), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+            "frac": round(tflops / FP32_PEAK_TFLOPS, 4), "traffic": (2 * 378527 + 65536) * 1024,
             "workload": "MatMul f32 [4096,4096] x [4096,4096] (weights as [k,n]), alpha 1, no bias",
             "device_ms_per_launch": round(dms, 5), "timing": mode, "steps": f32_steps, "observed_sclk_mhz": LAST["clock"],
             "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
@@ -812,7 +815,7 @@ def main():
         ws = [b] + [torch.randn((4096, 4096), device=dev) * 0.05 for _ in range(nb - 1)]
         y1 = torch.empty((1, 4096), device=dev)
         wall, dms, mode = time_steps(torch, lambda i: ops.matmul(a1, ws[i], out=y1), steps, warmup, nb)
-        e = hbm_entry((4096 * 4096 + 2 * 4096) * 4, dms)
+        e = hbm_entry((4096 * 4096 + 2 * 4096) * 4, dms, "matmul_f32_one_row")
         e.update(workload="MatMul f32 [1,4096] x [4096,4096] (weights as [k,n])", device_ms_per_launch=round(dms, 5), timing=mode)
         ops_out["matmul_f32_one_row"] = e
         del a1, ws, y1, b
