@@ -975,6 +975,7 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
         a.Hkv = static_cast<uint32_t>(n_kv_head);
         a.seq = static_cast<uint32_t>(seq);
         a.cap = static_cast<uint32_t>(cap);
+        a.D = static_cast<uint32_t>(D);
         a.scale = scale;
         a.dtype = dtype;
         return launch_prefill(a, s);

@@ -1,4 +1,4 @@
-// Tiled causal attention for many query rows per batch row (prefill), head dim 128, gfx950.
+// Tiled causal attention for many query rows per batch row (prefill), head dim 128 or 64, gfx950.
 //
 // Same contract as the split-KV kernel (layouts of src/08-01llm/README.md:29-63 of the
 // reference: q, o [N, H, seq, D]; k, v [N, Hkv, seq, D]; caches [N, Hkv, cap, D]; query row r
@@ -40,11 +40,12 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int D = 128;
 constexpr int BN = 64;                 // keys per tile: two blocks of 32
 constexpr int KB = BN / 32;            // blocks of 32 keys per tile
 constexpr int CPI = BN / 16;           // K (and V) copy instructions per wavefront and tile
-constexpr int ROWB = 2 * D;            // bytes of a K or V row (unpadded in LDS)
+constexpr int ROWB = 256;              // bytes of a K, V or Q row in LDS: head dim 128, unpadded.  Head dim 64 keeps
+                                       // this pitch and the layout below and uses chunks 0-7 of a row only (the
+                                       // copies fill the other positions with chunks they fetch a second time)
 constexpr int TILE = BN * ROWB;        // 16384: one K or V tile
 constexpr int BUF_BYTES = 2 * TILE;    // K tile + V tile; two such buffers, reused for the output transposition
 constexpr float kSlack = 6.0f;
@@ -170,10 +171,17 @@ __device__ __forceinline__ void copy16(const void *sbase, uint32_t voffset, uint
 
 // HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
 // query sub-tiles of the same heads.
-template <class T, int HW>
+template <class T, int HW, int DH>
 __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, const PrefillPlan plan) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
     constexpr int ROWS = 32 * QS;   // query rows per item
+    constexpr int GROWB = 2 * DH;   // bytes of a row in memory
+    constexpr int KSTEPS = DH / 16; // products of a S^T block
+    constexpr int DBLK = DH / 32;   // blocks of 32 rows of O^T
+    constexpr uint32_t CM = DH / 8 - 1;  // mask of a row's chunk indices in memory
+    constexpr uint32_t OWN_CHUNKS = DH / 8, OWN_ROWS = 256 / OWN_CHUNKS;  // the new rows on their way to the caches
+    constexpr int OWN_PASSES = (ROWS + OWN_ROWS - 1) / OWN_ROWS;
+    static_assert(DH == 128 || DH == 64, "head dim 128 or 64");
     __shared__ __align__(1024) uint8_t lds[2 * BUF_BYTES];
     const uint32_t lds_addr0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) uint8_t *)lds));
@@ -253,23 +261,32 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         if (in_hist || in_new) {  // uniform
             const uint64_t row0 = in_hist ? static_cast<uint64_t>(it.kvhead) * a.cap + first
                                           : static_cast<uint64_t>(it.kvhead) * a.seq + (first - it.base);
-            const uint8_t *kb_ = (in_hist ? Kc : Kn) + row0 * ROWB;
-            const uint8_t *vb_ = (in_hist ? Vc : Vn) + row0 * ROWB;
+            const uint8_t *kb_ = (in_hist ? Kc : Kn) + row0 * GROWB;
+            const uint8_t *vb_ = (in_hist ? Vc : Vn) + row0 * GROWB;
             static_assert(CPI == 4, "four copies of four rows per wavefront and tensor");
-            // (the instruction's offset moves the global and the LDS address alike: four rows are 1 KiB in both)
-            copy16<0>(kb_, k_lane, kdst);
-            copy16<0>(vb_, v_lane, vdst);
-            copy16<4 * ROWB>(kb_, k_lane ^ 64, kdst);
-            copy16<4 * ROWB>(vb_, v_lane, vdst);
-            copy16<8 * ROWB>(kb_, k_lane ^ 128, kdst);
-            copy16<8 * ROWB>(vb_, v_lane, vdst);
-            copy16<12 * ROWB>(kb_, k_lane ^ 192, kdst);
-            copy16<12 * ROWB>(vb_, v_lane, vdst);
+            if constexpr (DH == 128) {
+                // (the instruction's offset moves the global and the LDS address alike: four rows are 1 KiB in both)
+                copy16<0>(kb_, k_lane, kdst);
+                copy16<0>(vb_, v_lane, vdst);
+                copy16<4 * ROWB>(kb_, k_lane ^ 64, kdst);
+                copy16<4 * ROWB>(vb_, v_lane, vdst);
+                copy16<8 * ROWB>(kb_, k_lane ^ 128, kdst);
+                copy16<8 * ROWB>(vb_, v_lane, vdst);
+                copy16<12 * ROWB>(kb_, k_lane ^ 192, kdst);
+                copy16<12 * ROWB>(vb_, v_lane, vdst);
+            } else {
+#pragma unroll
+                for (int i = 0; i < CPI; ++i) {
+                    const uint32_t r = cp_row + 4 * i;
+                    copy16<0>(kb_, r * GROWB + 16 * (((lane & 15) ^ (r & 15)) & CM), kdst + i * 1024);
+                    copy16<0>(vb_, r * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) & CM), vdst + i * 1024);
+                }
+            }
         } else {
-            const uint8_t *kh = Kc + static_cast<uint64_t>(it.kvhead) * a.cap * ROWB;
-            const uint8_t *vh = Vc + static_cast<uint64_t>(it.kvhead) * a.cap * ROWB;
-            const uint8_t *kn = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
-            const uint8_t *vn = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
+            const uint8_t *kh = Kc + static_cast<uint64_t>(it.kvhead) * a.cap * GROWB;
+            const uint8_t *vh = Vc + static_cast<uint64_t>(it.kvhead) * a.cap * GROWB;
+            const uint8_t *kn = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * GROWB;
+            const uint8_t *vn = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * GROWB;
 #pragma unroll
             for (int i = 0; i < CPI; ++i) {
                 uint32_t pos = first + cp_row + 4 * i;
@@ -277,8 +294,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 // a wavefront's 16 rows may lie on both sides of the seam: the side is chosen per lane
                 // by handing the copy the lane's full address (no scalar base)
                 const bool old = pos < it.base;
-                const uint32_t row_off = (old ? pos : pos - it.base) * ROWB;  // within one kv head: below 2^32
-                const uint32_t kc = (lane & 15) ^ ((cp_row + 4 * i) & 15), vc = (lane & 15) ^ v_swizzle(lane >> 4);
+                const uint32_t row_off = (old ? pos : pos - it.base) * GROWB;  // within one kv head: below 2^32
+                const uint32_t kc = ((lane & 15) ^ ((cp_row + 4 * i) & 15)) & CM, vc = ((lane & 15) ^ v_swizzle(lane >> 4)) & CM;
                 const uint8_t *ksrc = (old ? kh : kn) + (row_off + 16 * kc);
                 const uint8_t *vsrc = (old ? vh : vn) + (row_off + 16 * vc);
                 asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(ksrc), "s"(kdst + i * 1024) : "memory", "m0");
@@ -298,28 +315,36 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         // (b * H + head) = kvhead * group + the head's index within the group
         const uint32_t bh = uni(it.kvhead * plan.group + head_in_group(it));
         const uint32_t r0 = it.qt * ROWS + 32 * (wave_u / HW);
-        const uint8_t *qh = Q + static_cast<uint64_t>(bh) * a.seq * ROWB;
+        const uint8_t *qh = Q + static_cast<uint64_t>(bh) * a.seq * GROWB;
         const uint32_t dst = lds_addr0 + buf + wave_u * (32 * ROWB);
         if (r0 + 32 <= a.seq) {
             // rows 4 i + lane / 16: the same offset pattern as a K tile's
-            const uint8_t *qb = qh + static_cast<uint64_t>(r0) * ROWB;
-            const uint32_t q_lane = (lane >> 4) * ROWB + 16 * ((lane & 15) ^ (lane >> 4));
-            copy16<0>(qb, q_lane, dst);
-            copy16<4 * ROWB>(qb, q_lane ^ 64, dst);
-            copy16<8 * ROWB>(qb, q_lane ^ 128, dst);
-            copy16<12 * ROWB>(qb, q_lane ^ 192, dst);
-            const uint8_t *qb2 = qb + 16 * ROWB;  // (the instruction's offset field ends at 4095)
-            copy16<0>(qb2, q_lane, dst + 4096);
-            copy16<4 * ROWB>(qb2, q_lane ^ 64, dst + 4096);
-            copy16<8 * ROWB>(qb2, q_lane ^ 128, dst + 4096);
-            copy16<12 * ROWB>(qb2, q_lane ^ 192, dst + 4096);
+            const uint8_t *qb = qh + static_cast<uint64_t>(r0) * GROWB;
+            if constexpr (DH == 128) {
+                const uint32_t q_lane = (lane >> 4) * ROWB + 16 * ((lane & 15) ^ (lane >> 4));
+                copy16<0>(qb, q_lane, dst);
+                copy16<4 * ROWB>(qb, q_lane ^ 64, dst);
+                copy16<8 * ROWB>(qb, q_lane ^ 128, dst);
+                copy16<12 * ROWB>(qb, q_lane ^ 192, dst);
+                const uint8_t *qb2 = qb + 16 * ROWB;  // (the instruction's offset field ends at 4095)
+                copy16<0>(qb2, q_lane, dst + 4096);
+                copy16<4 * ROWB>(qb2, q_lane ^ 64, dst + 4096);
+                copy16<8 * ROWB>(qb2, q_lane ^ 128, dst + 4096);
+                copy16<12 * ROWB>(qb2, q_lane ^ 192, dst + 4096);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t row = 4 * i + (lane >> 4);
+                    copy16<0>(qb, row * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM), dst + i * 1024);
+                }
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const uint32_t row = 4 * i + (lane >> 4);
                 uint32_t grow = r0 + row;
                 grow = grow < a.seq ? grow : a.seq - 1;
-                copy16<0>(qh, grow * ROWB + 16 * ((lane & 15) ^ (row & 15)), dst + i * 1024);  // within one head: below 2^32
+                copy16<0>(qh, grow * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM), dst + i * 1024);  // within one head: below 2^32
             }
         }
     };
@@ -333,8 +358,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
 
     // ---- state of the item being worked on
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    Raw16 qf[8];   // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
-    f16v o[4];
+    Raw16 qf[KSTEPS];   // Q fragments (B operand): lane holds query row r0 + l32, d = 16 kk + 8 half .. +7
+    f16v o[DBLK];
     float m = 0.f, l = 0.f;
     bool fresh = true;
     Item cur{0, 0, kNoItem, 0};
@@ -351,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         wave_tiles = uni(r0 < a.seq ? (cur.base + wave_last_row) / BN + 1 : 0);
         qpos = cur.base + r0 + l32;  // absolute position of this lane's query row
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < DBLK; ++db)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
         m = 0.f;
@@ -370,24 +395,25 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         const uint32_t tile_first = (n_tiles - 1) * BN;  // first key of the last tile
         uint32_t tid = threadIdx.x;  // (opaque copy, see finish_item)
         asm volatile("" : "+v"(tid));
+        // a pass of the workgroup covers OWN_ROWS rows: 16 chunks a row at head dim 128, 8 at head dim 64
         if (it.base + lo >= tile_first) {
             const uint8_t *tb = lds + buf;
 #pragma unroll
-            for (int jr = 0; jr < ROWS / 16; ++jr) {
-                uint32_t row = lo + (tid >> 4) + 16 * jr;
+            for (int jr = 0; jr < OWN_PASSES; ++jr) {
+                uint32_t row = lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
                 row = row < rows_end ? row : rows_end - 1;  // reads stay unconditional, the stores are guarded
-                const uint32_t r = it.base + row - tile_first, c = tid & 15;
+                const uint32_t r = it.base + row - tile_first, c = tid % OWN_CHUNKS;
                 ak[jr] = *reinterpret_cast<const u32x4 *>(tb + r * ROWB + 16 * (c ^ (r & 15)));
                 av[jr] = *reinterpret_cast<const u32x4 *>(tb + TILE + r * ROWB + 16 * (c ^ v_swizzle(r & 3)));
             }
         } else {
-            const uint8_t *k_new = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
-            const uint8_t *v_new = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * ROWB;
+            const uint8_t *k_new = Kn + static_cast<uint64_t>(it.kvhead) * a.seq * GROWB;
+            const uint8_t *v_new = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * GROWB;
 #pragma unroll
-            for (int jr = 0; jr < ROWS / 16; ++jr) {
-                uint32_t row = lo + (tid >> 4) + 16 * jr;
+            for (int jr = 0; jr < OWN_PASSES; ++jr) {
+                uint32_t row = lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
                 row = row < rows_end ? row : rows_end - 1;
-                const uint32_t off = row * ROWB + (tid & 15) * 16;
+                const uint32_t off = row * GROWB + (tid % OWN_CHUNKS) * 16;
                 ak[jr] = *reinterpret_cast<const u32x4 *>(k_new + off);
                 av[jr] = *reinterpret_cast<const u32x4 *>(v_new + off);
             }
@@ -413,7 +439,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         if (fr0 < a.seq && head_ok) {
             const float inv = 1.f / half_sum(l);
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < DBLK; ++db)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     // registers 4 g .. 4 g + 3 of a block: d = 32 db + 8 g + 4 half + 0..3 of row l32
@@ -422,20 +448,21 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                     *reinterpret_cast<uint2 *>(stage + l32 * ROWB + 16 * ((4 * db + g) ^ (l32 & 15)) + 8 * half) = w;
                 }
             // (each wavefront reads back only what it wrote itself: no barrier)
-            uint8_t *op = reinterpret_cast<uint8_t *>(O) + (static_cast<uint64_t>(bh) * a.seq + fr0) * ROWB;
+            uint8_t *op = reinterpret_cast<uint8_t *>(O) + (static_cast<uint64_t>(bh) * a.seq + fr0) * GROWB;
+            constexpr uint32_t OC = DH / 8;  // chunks of an output row; a store instruction covers 64 / OC rows
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const uint32_t row = 4 * i + (lane >> 4), c = lane & 15;
+            for (int i = 0; i < 32 * OC / 64; ++i) {
+                const uint32_t row = (64 / OC) * i + lane / OC, c = lane % OC;
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + 16 * (c ^ (row & 15)));
-                if (fr0 + row < a.seq) *reinterpret_cast<u32x4 *>(op + row * ROWB + 16 * c) = v;
+                if (fr0 + row < a.seq) *reinterpret_cast<u32x4 *>(op + row * GROWB + 16 * c) = v;
             }
         }
         if (do_append) {
 #pragma unroll
-            for (int jr = 0; jr < ROWS / 16; ++jr) {
-                const uint32_t pos = own_lo + (tid >> 4) + 16 * jr;
+            for (int jr = 0; jr < OWN_PASSES; ++jr) {
+                const uint32_t pos = own_lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
                 if (pos < own_hi) {
-                    const uint64_t dst = (static_cast<uint64_t>(it.kvhead) * a.cap + pos) * ROWB + (tid & 15) * 16;
+                    const uint64_t dst = (static_cast<uint64_t>(it.kvhead) * a.cap + pos) * GROWB + (tid % OWN_CHUNKS) * 16;
                     *reinterpret_cast<u32x4 *>(Kc + dst) = ak[jr];
                     *reinterpret_cast<u32x4 *>(Vc + dst) = av[jr];
                 }
@@ -465,8 +492,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 const uint64_t row0 = (in_hist ? static_cast<uint64_t>(cur.kvhead) * a.cap + first
                                                : static_cast<uint64_t>(cur.kvhead) * a.seq + (first - cur.base)) +
                                       (BN / 4) * wave_u;
-                base_a = (in_hist ? Kc : Kn) + row0 * ROWB;
-                base_b = (in_hist ? Vc : Vn) + row0 * ROWB;
+                base_a = (in_hist ? Kc : Kn) + row0 * GROWB;
+                base_b = (in_hist ? Vc : Vn) + row0 * GROWB;
                 dst_a = lds_addr0 + other + CPI * wave_u * 1024;
                 dst_b = dst_a + TILE;
                 mode = 1;
@@ -477,8 +504,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             const uint32_t nr0 = nxt.qt * ROWS + 32 * (wave_u / HW);
             if (nr0 + 32 <= a.seq) {
                 const uint32_t bh = uni(nxt.kvhead * plan.group + head_in_group(nxt));
-                base_a = Q + (static_cast<uint64_t>(bh) * a.seq + nr0) * ROWB;
-                base_b = base_a + 16 * ROWB;
+                base_a = Q + (static_cast<uint64_t>(bh) * a.seq + nr0) * GROWB;
+                base_b = base_a + 16 * GROWB;
                 dst_a = lds_addr0 + other + wave_u * (32 * ROWB);
                 dst_b = dst_a + 16 * ROWB;
                 is_q = true;
@@ -490,8 +517,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         auto copy_part = [&]<int I>() __attribute__((always_inline)) {
             if (mode != 1) return;
             constexpr int J = I / 2;
-            if (I % 2 == 0) copy16<J * 4 * ROWB>(base_a, q_lane ^ (64 * J), dst_a);
-            else copy16<J * 4 * ROWB>(base_b, is_q ? q_lane ^ (64 * J) : vq_lane, dst_b);
+            if constexpr (DH == 128) {
+                if (I % 2 == 0) copy16<J * 4 * ROWB>(base_a, q_lane ^ (64 * J), dst_a);
+                else copy16<J * 4 * ROWB>(base_b, is_q ? q_lane ^ (64 * J) : vq_lane, dst_b);
+            } else {
+                // rows 4 J + lane / 16 of the wavefront's sixteen: K and Q rows swizzled by the row, V rows by lane / 16
+                const uint32_t row = 4 * J + (lane >> 4);
+                const uint32_t k_like = row * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM);
+                const uint32_t v_like = row * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) & CM);
+                if (I % 2 == 0) copy16<0>(base_a, k_like, dst_a + 1024 * J);
+                else copy16<0>(base_b, is_q ? k_like : v_like, dst_b + 1024 * J);
+            }
         };
         auto copy_rest = [&]() __attribute__((always_inline)) {  // what the parts do not cover
             if (mode != 2) return;
@@ -528,25 +564,34 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             for (int e = 0; e < 16; ++e) sc[e] = 0.f;
             auto product = [&]<int KK>() __attribute__((always_inline)) {
                 sc = Ops<T>::mfma(kf[KK % 4], qf[KK], sc);
-                if (KK + 4 < 8) kf[KK % 4] = *reinterpret_cast<const Raw16 *>(kb_base + (k_off ^ (32 * (KK + 4))));
-                if (kb == 0) copy_part.template operator()<KK>();
+                if constexpr (KK + 4 < KSTEPS) kf[KK % 4] = *reinterpret_cast<const Raw16 *>(kb_base + (k_off ^ (32 * (KK + 4))));
+                if (kb == 0) {  // the eight parts of the copy spread over the products
+                    if constexpr (KSTEPS == 8) {
+                        copy_part.template operator()<KK>();
+                    } else {
+                        copy_part.template operator()<2 * KK>();
+                        copy_part.template operator()<2 * KK + 1>();
+                    }
+                }
                 RG_SCHED_FENCE();
             };
             product.template operator()<0>();
             product.template operator()<1>();
             product.template operator()<2>();
             product.template operator()<3>();
-            product.template operator()<4>();
-            product.template operator()<5>();
-            product.template operator()<6>();
-            product.template operator()<7>();
+            if constexpr (KSTEPS == 8) {
+                product.template operator()<4>();
+                product.template operator()<5>();
+                product.template operator()<6>();
+                product.template operator()<7>();
+            }
             // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
             // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
             // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
             // keys each: lane s of the group addresses key s / 4, columns 4 (s % 4) .. +3.
-            // (product index i = 4 jj + db; the first four fragments are requested before the softmax)
+            // (product index i = DBLK jj + db; the first four fragments are requested before the softmax)
             auto read_v = [&](int i) __attribute__((always_inline)) {
-                const int jj = i / 4, db = i % 4;
+                const int jj = i / DBLK, db = i % DBLK;
                 const uint8_t *vp = tb + (32 * kb + 16 * jj) * ROWB + (v_off ^ (64 * db));
                 const U2 lo = read_tr16(vp), hi = read_tr16(vp + 8 * ROWB);
                 return Raw16{{lo.w[0], lo.w[1], hi.w[0], hi.w[1]}};
@@ -581,7 +626,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 m += up;
                 l *= alpha;
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                for (int db = 0; db < DBLK; ++db)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
 #pragma unroll
@@ -601,9 +646,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 }
             RG_SCHED_FENCE();
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                o[i % 4] = Ops<T>::mfma(vf[i % 4], pf[i / 4], o[i % 4]);
-                if (i + 4 < 8) vf[i % 4] = read_v(i + 4);
+            for (int i = 0; i < 2 * DBLK; ++i) {
+                o[i % DBLK] = Ops<T>::mfma(vf[i % 4], pf[i / DBLK], o[i % DBLK]);
+                if (i + 4 < 2 * DBLK) vf[i % 4] = read_v(i + 4);
                 RG_SCHED_FENCE();
             }
         }
@@ -621,7 +666,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         if (nxt.valid()) {
             const uint8_t *qb = lds + buf + wave_u * (32 * ROWB);
 #pragma unroll
-            for (int kk = 0; kk < 8; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qb + (k_off ^ (32 * kk)));
+            for (int kk = 0; kk < KSTEPS; ++kk) qf[kk] = *reinterpret_cast<const Raw16 *>(qb + (k_off ^ (32 * kk)));
             if (have_cur) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_s_barrier();
@@ -661,11 +706,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     }
 }
 
-template <class T, int HW>
+template <class T, int HW, int DH>
 uint32_t resident_prefill_workgroups() {
     static uint32_t cached = [] {
         int per_cu = 0, dev = 0, cus = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_prefill<T, HW>, 256, 0) != hipSuccess || per_cu <= 0)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_prefill<T, HW, DH>, 256, 0) != hipSuccess || per_cu <= 0)
             per_cu = 2;
         hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
@@ -675,7 +720,7 @@ uint32_t resident_prefill_workgroups() {
     return cached;
 }
 
-template <class T, int HW>
+template <class T, int HW, int DH>
 int launch_hw(const PrefillArgs &a, hipStream_t s) {
     constexpr uint32_t ROWS = 32 * (4 / HW);
     PrefillPlan plan{};
@@ -688,7 +733,7 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
     plan.xcds = streams % 8 == 0 ? 8 : 1;
     plan.spx = static_cast<uint32_t>(streams / plan.xcds);
     // as many sets of `pairs` workgroups per XCD as stay resident together (at least one)
-    const uint32_t per_xcd = resident_prefill_workgroups<T, HW>() / plan.xcds;
+    const uint32_t per_xcd = resident_prefill_workgroups<T, HW, DH>() / plan.xcds;
     uint32_t groups = per_xcd / plan.pairs;
     if (groups < 1) groups = 1;
     if (groups > plan.spx) groups = plan.spx;
@@ -698,22 +743,27 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
     plan.magic_chunks = plan.head_chunks > 1 ? static_cast<uint32_t>((1ull << 32) / plan.head_chunks + 1) : 0;
     plan.magic_hkv = a.Hkv > 1 ? static_cast<uint32_t>((1ull << 32) / a.Hkv + 1) : 0;
     const uint32_t grid = plan.xcds * plan.groups * plan.pairs;
-    attn_prefill<T, HW><<<grid, 256, 0, s>>>(a, plan);
+    attn_prefill<T, HW, DH><<<grid, 256, 0, s>>>(a, plan);
     return launch_status();
+}
+
+template <class T, int DH>
+int launch_d(const PrefillArgs &a, hipStream_t s) {
+    const uint32_t group = a.H / a.Hkv;
+    if (group == 1) return launch_hw<T, 1, DH>(a, s);
+    if (group == 2) return launch_hw<T, 2, DH>(a, s);
+    return launch_hw<T, 4, DH>(a, s);  // chunks of four heads; the last one is short when group % 4 != 0
 }
 
 template <class T>
 int launch_t(const PrefillArgs &a, hipStream_t s) {
-    const uint32_t group = a.H / a.Hkv;
-    if (group == 1) return launch_hw<T, 1>(a, s);
-    if (group == 2) return launch_hw<T, 2>(a, s);
-    return launch_hw<T, 4>(a, s);  // chunks of four heads; the last one is short when group % 4 != 0
+    return a.D == 64 ? launch_d<T, 64>(a, s) : launch_d<T, 128>(a, s);
 }
 
 }  // namespace
 
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D_) {
-    return D_ == D && Hkv != 0 && H % Hkv == 0;
+    return (D_ == 128 || D_ == 64) && Hkv != 0 && H % Hkv == 0;
 }
 
 int launch_prefill(const PrefillArgs &a, hipStream_t s) {

@@ -10,12 +10,12 @@ struct PrefillArgs {
     void *o, *kc, *vc;
     const int64_t *past;
     int past_per_row;
-    uint32_t N, H, Hkv, seq, cap;
+    uint32_t N, H, Hkv, seq, cap, D;
     float scale;
     int dtype;  // RG_FP16 or RG_BF16
 };
 
-// True when launch_prefill handles the shape (head dim 128, group size 1, 2 or a multiple of 4).
+// True when launch_prefill handles the shape (head dim 128 or 64, any group size).
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D);
 
 // Enqueues the kernel; returns a hipError_t as int.

@@ -752,7 +752,7 @@ def test_attention_decode_and_small_prefill(N, H, Hkv, seq, cap, D, past):
     (16, 8, 8, 8, 32, 64, torch.float16),     # many short segments: several pieces per range, several passes
     (70, 4, 2, 1, 96, 128, torch.float16),    # more than 64 batch rows: the partition is built by the whole workgroup
     (24, 12, 4, 3, 40, 128, torch.bfloat16),  # group of 3 heads (two launches), short segments, bf16
-    (4, 8, 8, 200, 256, 64, torch.float16),   # head dim 64 prefill through the split kernel: ~25 segments per range
+    (4, 8, 8, 200, 256, 64, torch.float16),   # head dim 64, 200 new rows (the tiled kernel)
     (200, 2, 1, 1, 48, 64, torch.float16),    # 200 batch rows
 ])
 def test_attention_split_many_segments(N, H, Hkv, seq, cap, D, dt):
@@ -835,6 +835,13 @@ def test_attention_decode_invariants_full_size():
     (2, 8, 2, 70, 256, 128, [3, 150], torch.bfloat16),
     (1, 6, 2, 48, 64, 128, [7], torch.float16),           # group of 3: a short chunk of heads
     (1, 8, 2, 129, 512, 128, [300], torch.float16),
+    (2, 8, 2, 40, 128, 64, [0, 20], torch.float16),       # head dim 64: the same kernel on half rows
+    (2, 4, 4, 33, 64, 64, [5, 31], torch.float16),        # MHA
+    (1, 4, 2, 64, 200, 64, [100], torch.float16),         # group of 2
+    (2, 16, 2, 96, 96, 64, [0, 0], torch.float16),        # group of 8
+    (2, 10, 2, 70, 256, 64, [3, 150], torch.bfloat16),    # group of 5
+    (1, 8, 2, 129, 512, 64, [300], torch.float16),
+    (3, 4, 1, 200, 333, 64, [0, 70, 133], torch.float16), # odd capacity and history lengths: the seam inside tiles
 ])
 def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
     o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt)
@@ -849,6 +856,8 @@ def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
     (12, 40, 8, 4, 130, 128, torch.float16),    # group of 5: two chunks, the second with one head
     (10, 28, 4, 7, 64, 128, torch.float16),     # group of 7
     (3, 8, 2, 9, 300, 128, torch.float16),      # few sequences: the split kernel (one segment per query row)
+    (40, 16, 8, 3, 150, 64, torch.float16),     # head dim 64
+    (12, 20, 4, 6, 90, 64, torch.bfloat16),     # head dim 64, group of 5
 ])
 def test_attention_few_new_rows_either_kernel(N, H, Hkv, seq, cap, D, dt):
     # 2 to 31 new rows per sequence run through the tiled kernel when there are enough sequences and kv heads to
