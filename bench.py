@@ -923,6 +923,29 @@ def main():
                 402653184 * len(pa) // (Np * H), f"{len(pa)} of the 1024 (batch row, head) pairs, one per thread")
         ops_out["attention_prefill"] = e
 
+    if want("attention_prefill_d64"):
+        # the same prefill for a model with 64-wide heads (the tiled kernel on half rows)
+        Np, seq, D64 = 32, 512, 64
+        q = torch.randn((Np, H, seq, D64), device=dev).half()
+        k = torch.randn((Np, Hkv, seq, D64), device=dev).half()
+        v = torch.randn((Np, Hkv, seq, D64), device=dev).half()
+        kc = torch.zeros((Np, Hkv, cap, D64), device=dev, dtype=torch.float16)
+        vc = torch.zeros_like(kc)
+        o = torch.empty_like(q)
+        zero = torch.zeros(Np, device=dev, dtype=torch.int64)
+        wsp = ops.attention_workspace(Np, H, Hkv, seq, cap, D64, dev)
+        wall, dms, mode = time_steps(
+            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, zero, 1.0 / math.sqrt(D64), out=o, workspace=wsp,
+                                                   sync_state=state),
+            max(steps // 10, 20), max(warmup // 80, 2), 1)
+        e = hbm_entry(402653184 // 2, dms)
+        flops = 68853694464 // 2
+        e.update(workload="AttentionKVCache prefill fp16 seq=512 past=0 causal N=32 H=32 Hkv=8 D=64",
+                 device_ms_per_launch=round(dms, 5), timing=mode,
+                 mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
+                 mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
+        ops_out["attention_prefill_d64"] = e
+
     if ops_out:
         result["ops"] = ops_out
     print(json.dumps(result))

@@ -859,12 +859,16 @@ constexpr size_t kPrefillAlways = 32;  // query rows from which the tiled kernel
 
 bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq) {
     if (seq >= kPrefillAlways) return true;
-    if (seq < 2) return false;
     const size_t group = n_head / n_kv_head, heads_per_item = group == 1 ? 1 : group == 2 ? 2 : 4;
+    // the split kernel takes at most four heads of a group per launch and reads K/V again in every launch
+    // (a group of 8: twice), while the chunks of a group on the tiled kernel find them in L2
+    size_t split_launches = 0;
+    for (size_t left = group; left > 0; left -= left >= 4 ? 4 : left >= 2 ? 2 : 1) ++split_launches;
+    if (seq < 2 && split_launches < 2) return false;
     const size_t rows_per_item = 32 * (4 / heads_per_item);
     const size_t items = N * n_kv_head * ((group + heads_per_item - 1) / heads_per_item) * ((seq + rows_per_item - 1) / rows_per_item);
     const size_t rounds = (items + 511) / 512;
-    return N * n_kv_head * seq >= 280 * rounds;
+    return N * n_kv_head * seq * split_launches >= 280 * rounds;
 }
 
 template <class T, int D, int G>

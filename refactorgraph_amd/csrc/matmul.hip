@@ -1270,7 +1270,8 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     // the passes of the few-rows kernels would take longer (measured per pass at k = 4096: 5.5 ns per column for 32
     // rows with B as [k, n], 3.4 to 4.7 ns for 64 rows with B as [n, k]) and where the plain kernel is the alternative
     const bool short_ok = narrow && !trans_a && m < BM && n >= BN && n % 8 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
-                          aligned16(b) && aligned16(y_) && !(n % BN != 0 && bias.ptr == y_);
+                          aligned16(b) && aligned16(y_) && !(n % BN != 0 && bias.ptr == y_) &&
+                          k < (1u << 22);  // a lane's offset into A (up to 255 rows) stays below 2^31
     bool short_tile = false;
     if (short_ok) {
         if (trans_b) short_tile = rows ? false : skinny ? ((m + 63) / 64) * n > 23000 : !gemv;

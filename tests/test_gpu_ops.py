@@ -856,12 +856,15 @@ def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
     (12, 40, 8, 4, 130, 128, torch.float16),    # group of 5: two chunks, the second with one head
     (10, 28, 4, 7, 64, 128, torch.float16),     # group of 7
     (3, 8, 2, 9, 300, 128, torch.float16),      # few sequences: the split kernel (one segment per query row)
+    (40, 24, 8, 1, 96, 128, torch.float16),     # one new row, group of 3: the split kernel would take two launches
+    (36, 64, 8, 1, 200, 128, torch.float16),    # one new row, group of 8
     (40, 16, 8, 3, 150, 64, torch.float16),     # head dim 64
     (12, 20, 4, 6, 90, 64, torch.bfloat16),     # head dim 64, group of 5
 ])
 def test_attention_few_new_rows_either_kernel(N, H, Hkv, seq, cap, D, dt):
-    # 2 to 31 new rows per sequence run through the tiled kernel when there are enough sequences and kv heads to
-    # occupy the chip with one item each, else through the split kernel; any head group size
+    # up to 31 new rows per sequence run through the tiled kernel when there are enough sequences and kv heads to
+    # occupy the chip with one item each (a single new row only where the split kernel would need several launches
+    # for the head group), else through the split kernel; any head group size
     past = np.random.default_rng(33).integers(0, cap - seq + 1, N)
     o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt, seed=34)
     assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
