@@ -200,6 +200,97 @@ __global__ __launch_bounds__(1024) void softmax_long(T *__restrict__ y, const T 
     }
 }
 
+// Contiguous rows (post == 1) whose length or addresses do not fit 128-bit vectors throughout (a row of scores
+// over a history of 1025 positions, a vocabulary of 50257): THREADS threads per row, the row swept twice (a running
+// maximum and sum per thread, merged once; then the results - the second read comes from L2).  The middle of a row,
+// from the first 16-byte boundary of its addresses on, still moves in aligned 128-bit vectors; only the elements
+// before and after go one by one (all of them when x and y are aligned differently).
+template <class T, int THREADS>
+__global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_ragged(T *__restrict__ y, const T *__restrict__ x,
+                                                                               uint64_t rows, uint32_t mid, uint32_t causal_rows) {
+    using CT = typename Compute<T>::type;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int BLOCK = THREADS < 256 ? 256 : THREADS, RPB = BLOCK / THREADS;
+    static_assert(THREADS == kWave || THREADS == BLOCK, "a row belongs to one wavefront or to the whole workgroup");
+    __shared__ CT smem[BLOCK / kWave];
+    const uint32_t t = threadIdx.x % THREADS;
+    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * RPB + threadIdx.x / THREADS;
+    const bool live = row < rows;
+    uint32_t keep = mid;
+    if (causal_rows) keep = static_cast<uint32_t>(row % causal_rows) + (mid - causal_rows) + 1;
+    if (!live) keep = 0;  // (a workgroup's surplus rows take part in the barriers only)
+    const T *xr = x + (live ? row : 0) * mid;
+    T *yr = y + (live ? row : 0) * mid;
+    const uint32_t to_boundary = static_cast<uint32_t>((16 - (reinterpret_cast<uintptr_t>(xr) & 15)) & 15) / sizeof(T);
+    const bool same = ((reinterpret_cast<uintptr_t>(xr) ^ reinterpret_cast<uintptr_t>(yr)) & 15) == 0;
+    const uint32_t head = same && to_boundary < mid ? to_boundary : mid;  // elements before the first vector
+    const uint32_t vecs = (mid - head) / VEC, tail = head + vecs * VEC;  // elements from `tail` on follow the last vector
+
+    CT mx = neg_inf<CT>(), sum = 0;
+    auto take = [&](CT f) {
+        if (mx < f) {  // exp(-inf - f) = 0 clears the (still zero) sum of a thread that had no maximum yet
+            sum *= Exp<T>::eval(mx - f);
+            mx = f;
+        }
+        if (mx > neg_inf<CT>()) sum += Exp<T>::eval(f - mx);
+    };
+    for (uint32_t i = t; i < head; i += THREADS)
+        if (i < keep) take(to_compute(xr[i]));
+    for (uint32_t i = tail + t; i < mid; i += THREADS)
+        if (i < keep) take(to_compute(xr[i]));
+#pragma unroll 4
+    for (uint32_t v = t; v < vecs; v += THREADS) {
+        const uint32_t c0 = head + v * VEC;
+        if (c0 >= keep) break;  // this thread's further vectors lie beyond the kept columns as well
+        const Vec16<T> xv = load16_stream(xr + c0);
+        CT f[VEC], vm = neg_inf<CT>();
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            f[e] = c0 + e < keep ? to_compute(xv.v[e]) : neg_inf<CT>();
+            vm = vm < f[e] ? f[e] : vm;
+        }
+        if (mx < vm) {
+            sum *= Exp<T>::eval(mx - vm);
+            mx = vm;
+        }
+        if (mx > neg_inf<CT>()) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sum += Exp<T>::eval(f[e] - mx);
+        }
+    }
+    auto wmax = [](CT v) { return wave_max(v); };
+    auto wsum = [](CT v) { return wave_sum(v); };
+    CT row_max, total;
+    if constexpr (THREADS == kWave) {
+        row_max = wave_max(mx);
+        total = wave_sum(sum * Exp<T>::eval(mx - row_max));
+    } else {
+        row_max = block_allreduce<THREADS / kWave>(mx, smem, wmax, [](CT a, CT b) { return a < b ? b : a; });
+        total = block_allreduce<THREADS / kWave>(sum * Exp<T>::eval(mx - row_max), smem, wsum, [](CT a, CT b) { return a + b; });
+    }
+    if (!live) return;
+    const Normalise<T> norm(total);
+    auto result = [&](T v, uint32_t i) {
+        return from_compute<T>(i < keep ? norm(Exp<T>::eval(to_compute(v) - row_max)) : CT(0));
+    };
+    for (uint32_t i = t; i < head; i += THREADS) yr[i] = result(xr[i], i);
+    for (uint32_t i = tail + t; i < mid; i += THREADS) yr[i] = result(xr[i], i);
+#pragma unroll 4
+    for (uint32_t v = t; v < vecs; v += THREADS) {
+        const uint32_t c0 = head + v * VEC;
+        Vec16<T> out;
+        if (c0 < keep) {
+            const Vec16<T> xv = load16_stream(xr + c0);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out.v[e] = result(xv.v[e], c0 + e);
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out.v[e] = from_compute<T>(CT(0));
+        }
+        store16_stream(yr + c0, out);
+    }
+}
+
 // Any mid / post / alignment: one thread per (pre, post) slice, three passes, neighbouring
 // threads touch neighbouring `post` positions.
 template <class T>
@@ -256,6 +347,11 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
         else
             softmax_long<T, 8192><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, static_cast<uint32_t>(mid),
                                                                              static_cast<uint32_t>(causal_rows));
+    } else if (post == 1 && pre <= 0x7fffffffu) {
+        const uint32_t m32 = static_cast<uint32_t>(mid), c32 = static_cast<uint32_t>(causal_rows);
+        if (mid <= 2048) softmax_ragged<T, 64><<<static_cast<unsigned>((pre + 3) / 4), 256, 0, s>>>(y, x, pre, m32, c32);
+        else if (mid <= 32768) softmax_ragged<T, 256><<<static_cast<unsigned>(pre), 256, 0, s>>>(y, x, pre, m32, c32);
+        else softmax_ragged<T, 1024><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, pre, m32, c32);
     } else {
         const uint64_t slices = static_cast<uint64_t>(pre) * post;
         const uint64_t grid = (slices + 255) / 256;

@@ -161,6 +161,41 @@ def test_softmax_long_rows():
     assert torch.all(yc[..., mask] == 0)
 
 
+def test_softmax_rows_that_fit_no_vectors():
+    # row lengths that are no multiple of a 128-bit vector (scores over 1025 positions, a vocabulary of 50257) and rows
+    # that start off a 16-byte boundary: aligned vectors in the middle of a row, single elements at its ends
+    rng = np.random.default_rng(41)
+    for shape, dt in [((5, 1025), torch.float16), ((3, 7, 33), torch.float32), ((4, 2047), torch.bfloat16),
+                      ((3, 50257), torch.float16), ((2, 3, 4097), torch.float32), ((6, 5), torch.float64),
+                      ((2, 40001), torch.float32), ((9, 1), torch.float16), ((3, 2049), torch.float64)]:
+        x = dev(3 * rng.standard_normal(shape)).to(dt)
+        if shape[-1] > 40:
+            x[0, ..., 5:40:7] = float("-inf")
+        ref = oracle.softmax(host(x.double() if dt == torch.float64 else x.float()), threads=8)
+        y = ops.softmax(x)
+        if dt == torch.float32:
+            assert_rel(host(y), oracle.softmax(host(x.double()), threads=8), REL_F32)
+        elif dt == torch.float64:
+            assert_rel(host(y), ref, 1e-13)
+        else:
+            assert np.max(np.abs(host(y.float()) - ref)) <= (ABS_F16 if dt == torch.float16 else 8e-3)
+    # rows of a multiple of the vector length that start two bytes off a boundary; output aligned alike, then differently
+    base = dev(3 * rng.standard_normal(4 * 1024 + 1).astype(np.float32)).half()
+    x = base[1:].view(4, 1024)
+    ref = oracle.softmax(host(x.float()), threads=8)
+    out_alike = torch.empty(4 * 1024 + 1, dtype=torch.float16, device=DEV)[1:].view(4, 1024)
+    out_other = torch.empty((4, 1024), dtype=torch.float16, device=DEV)
+    for out in (out_alike, out_other):
+        assert np.max(np.abs(host(ops.softmax(x, out=out).float()) - ref)) <= ABS_F16
+    # causal flag on ragged rows: equal to the data-masked input bit for bit
+    x16 = dev(3 * rng.standard_normal((2, 130, 135)).astype(np.float32)).half()
+    yc = ops.softmax(x16, causal=True)
+    mask = torch.arange(135, device=DEV)[None, :] > torch.arange(130, device=DEV)[:, None] + 5
+    assert torch.equal(yc, ops.softmax(x16.masked_fill(mask, float("-inf"))))
+    assert np.max(np.abs(host(yc.float()) - oracle.softmax_causal(host(x16.float()), threads=8))) <= ABS_F16
+    assert torch.all(yc[..., mask] == 0)
+
+
 def test_softmax_full_config_properties():
     # [8,32,2048,2048] fp16: a slab against the oracle, the whole tensor through row sums
     g = torch.Generator(device=DEV).manual_seed(3)
