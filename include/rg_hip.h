@@ -262,7 +262,7 @@ int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, con
  *   cap - seq (the new rows then replace the last seq rows of the cache and the queries see the
  *   history shortened accordingly); nothing is ever read or written outside the caches.
  * k_cache == v_cache == NULL: no cache (past = 0, attends k/v directly).  past_lens == NULL: 0.
- * n_head % n_kv_head == 0; D in {64, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
+ * n_head % n_kv_head == 0; D in {64, 80, 96, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
  * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials), contents irrelevant.
  * sync_state: NULL, or rg_hip_attention_kvcache_state_bytes() bytes of device memory that the
  *   caller zeroed once and keeps for this purpose (a runtime::Resource of the stream, like the

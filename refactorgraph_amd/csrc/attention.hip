@@ -957,7 +957,9 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
     if ((k_cache == nullptr) != (v_cache == nullptr)) return RG_HIP_E_ARGUMENT;
     if (N == 0 || n_head == 0 || seq == 0) return 0;
     if (n_kv_head == 0 || n_head % n_kv_head != 0) return RG_HIP_E_ARGUMENT;
-    if (D != 64 && D != 128) return RG_HIP_E_UNSUPPORTED;
+    // head dims 64 and 128 have both kernels; 80 and 96 the tiled one only (the split kernel gives 8 or 16 lanes to a row)
+    const bool split_ok = D == 64 || D == 128;
+    if (!split_ok && D != 80 && D != 96) return RG_HIP_E_UNSUPPORTED;
     if (dtype != RG_FP16 && dtype != RG_BF16) return RG_HIP_E_UNSUPPORTED;
     if (N > kMaxBatch || seq > 0xffffu || cap > 0x3fffffffu || n_head > 0xffffu) return RG_HIP_E_UNSUPPORTED;
     if (k_cache && cap < seq) return RG_HIP_E_ARGUMENT;
@@ -969,7 +971,7 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
 
     // many query rows per batch row: the tiled MFMA kernel (K/V staged once per query tile)
     if (prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head), static_cast<uint32_t>(D)) &&
-        prefill_pays(N, n_head, n_kv_head, seq)) {
+        (!split_ok || prefill_pays(N, n_head, n_kv_head, seq))) {
         PrefillArgs a{};
         a.q = q; a.k = k; a.v = v; a.o = o; a.kc = k_cache; a.vc = v_cache;
         a.past = past_lens;
@@ -1027,7 +1029,7 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
                                         void *stream) {
     using namespace rg;
     // a workspace that is missing or too small is reported after the argument checks
-    const bool usable = workspace && (D == 64 || D == 128) && workspace_bytes >= rg::workspace_bytes(D);
+    const bool usable = workspace && D <= 128 && workspace_bytes >= rg::workspace_bytes(D);
     float *part = usable ? reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes) : nullptr;
     uint32_t *counters = static_cast<uint32_t *>(sync_state ? sync_state : workspace);
     return attention_call(o, q, k, v, k_cache, v_cache, past_lens, past_per_row, N, n_head, n_kv_head, seq, cap, D,

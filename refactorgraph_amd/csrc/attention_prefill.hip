@@ -177,11 +177,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     constexpr int ROWS = 32 * QS;   // query rows per item
     constexpr int GROWB = 2 * DH;   // bytes of a row in memory
     constexpr int KSTEPS = DH / 16; // products of a S^T block
-    constexpr int DBLK = DH / 32;   // blocks of 32 rows of O^T
-    constexpr uint32_t CM = DH / 8 - 1;  // mask of a row's chunk indices in memory
-    constexpr uint32_t OWN_CHUNKS = DH / 8, OWN_ROWS = 256 / OWN_CHUNKS;  // the new rows on their way to the caches
-    constexpr int OWN_PASSES = (ROWS + OWN_ROWS - 1) / OWN_ROWS;
-    static_assert(DH == 128 || DH == 64, "head dim 128 or 64");
+    constexpr int DBLK = (DH + 31) / 32;  // blocks of 32 rows of O^T (the last one half used at head dim 80)
+    constexpr uint32_t NCH = DH / 8;      // 16-byte chunks of a row in memory; a copy's lanes beyond them fetch
+                                          // chunk (position's chunk) % NCH of the same row a second time
+    constexpr int OWN_PASSES = (ROWS * NCH + 255) / 256;  // the new rows on their way to the caches: chunks per thread
+    static_assert(DH % 16 == 0 && DH >= 64 && DH <= 128, "head dim 64 to 128 in steps of 16");
     __shared__ __align__(1024) uint8_t lds[2 * BUF_BYTES];
     const uint32_t lds_addr0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (__attribute__((address_space(3))) uint8_t *)lds));
@@ -278,8 +278,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
 #pragma unroll
                 for (int i = 0; i < CPI; ++i) {
                     const uint32_t r = cp_row + 4 * i;
-                    copy16<0>(kb_, r * GROWB + 16 * (((lane & 15) ^ (r & 15)) & CM), kdst + i * 1024);
-                    copy16<0>(vb_, r * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) & CM), vdst + i * 1024);
+                    copy16<0>(kb_, r * GROWB + 16 * (((lane & 15) ^ (r & 15)) % NCH), kdst + i * 1024);
+                    copy16<0>(vb_, r * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) % NCH), vdst + i * 1024);
                 }
             }
         } else {
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 // by handing the copy the lane's full address (no scalar base)
                 const bool old = pos < it.base;
                 const uint32_t row_off = (old ? pos : pos - it.base) * GROWB;  // within one kv head: below 2^32
-                const uint32_t kc = ((lane & 15) ^ ((cp_row + 4 * i) & 15)) & CM, vc = ((lane & 15) ^ v_swizzle(lane >> 4)) & CM;
+                const uint32_t kc = ((lane & 15) ^ ((cp_row + 4 * i) & 15)) % NCH, vc = ((lane & 15) ^ v_swizzle(lane >> 4)) % NCH;
                 const uint8_t *ksrc = (old ? kh : kn) + (row_off + 16 * kc);
                 const uint8_t *vsrc = (old ? vh : vn) + (row_off + 16 * vc);
                 asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(ksrc), "s"(kdst + i * 1024) : "memory", "m0");
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const uint32_t row = 4 * i + (lane >> 4);
-                    copy16<0>(qb, row * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM), dst + i * 1024);
+                    copy16<0>(qb, row * GROWB + 16 * (((lane & 15) ^ (row & 15)) % NCH), dst + i * 1024);
                 }
             }
         } else {
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 const uint32_t row = 4 * i + (lane >> 4);
                 uint32_t grow = r0 + row;
                 grow = grow < a.seq ? grow : a.seq - 1;
-                copy16<0>(qh, grow * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM), dst + i * 1024);  // within one head: below 2^32
+                copy16<0>(qh, grow * GROWB + 16 * (((lane & 15) ^ (row & 15)) % NCH), dst + i * 1024);  // within one head: below 2^32
             }
         }
     };
@@ -395,14 +395,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         const uint32_t tile_first = (n_tiles - 1) * BN;  // first key of the last tile
         uint32_t tid = threadIdx.x;  // (opaque copy, see finish_item)
         asm volatile("" : "+v"(tid));
-        // a pass of the workgroup covers OWN_ROWS rows: 16 chunks a row at head dim 128, 8 at head dim 64
+        // thread tid takes chunks tid, tid + 256, ... of the ROWS x NCH chunks of the item's rows
         if (it.base + lo >= tile_first) {
             const uint8_t *tb = lds + buf;
 #pragma unroll
             for (int jr = 0; jr < OWN_PASSES; ++jr) {
-                uint32_t row = lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
+                const uint32_t idx = tid + 256 * jr;
+                uint32_t row = lo + idx / NCH;
                 row = row < rows_end ? row : rows_end - 1;  // reads stay unconditional, the stores are guarded
-                const uint32_t r = it.base + row - tile_first, c = tid % OWN_CHUNKS;
+                const uint32_t r = it.base + row - tile_first, c = idx % NCH;
                 ak[jr] = *reinterpret_cast<const u32x4 *>(tb + r * ROWB + 16 * (c ^ (r & 15)));
                 av[jr] = *reinterpret_cast<const u32x4 *>(tb + TILE + r * ROWB + 16 * (c ^ v_swizzle(r & 3)));
             }
@@ -411,9 +412,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             const uint8_t *v_new = Vn + static_cast<uint64_t>(it.kvhead) * a.seq * GROWB;
 #pragma unroll
             for (int jr = 0; jr < OWN_PASSES; ++jr) {
-                uint32_t row = lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
+                const uint32_t idx = tid + 256 * jr;
+                uint32_t row = lo + idx / NCH;
                 row = row < rows_end ? row : rows_end - 1;
-                const uint32_t off = row * GROWB + (tid % OWN_CHUNKS) * 16;
+                const uint32_t off = row * GROWB + (idx % NCH) * 16;
                 ak[jr] = *reinterpret_cast<const u32x4 *>(k_new + off);
                 av[jr] = *reinterpret_cast<const u32x4 *>(v_new + off);
             }
@@ -442,6 +444,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             for (int db = 0; db < DBLK; ++db)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
+                    if (4 * db + g >= static_cast<int>(NCH)) continue;  // (head dim 80: the second half of the last block)
                     // registers 4 g .. 4 g + 3 of a block: d = 32 db + 8 g + 4 half + 0..3 of row l32
                     const uint2 w = make_uint2(Ops<T>::pack2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv),
                                                Ops<T>::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv));
@@ -449,20 +452,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 }
             // (each wavefront reads back only what it wrote itself: no barrier)
             uint8_t *op = reinterpret_cast<uint8_t *>(O) + (static_cast<uint64_t>(bh) * a.seq + fr0) * GROWB;
-            constexpr uint32_t OC = DH / 8;  // chunks of an output row; a store instruction covers 64 / OC rows
+            // lane takes chunks lane, lane + 64, ... of the 32 x NCH chunks of the wavefront's rows
 #pragma unroll
-            for (int i = 0; i < 32 * OC / 64; ++i) {
-                const uint32_t row = (64 / OC) * i + lane / OC, c = lane % OC;
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + 16 * (c ^ (row & 15)));
-                if (fr0 + row < a.seq) *reinterpret_cast<u32x4 *>(op + row * GROWB + 16 * c) = v;
+            for (int i = 0; i < (32 * static_cast<int>(NCH) + 63) / 64; ++i) {
+                const uint32_t idx = lane + 64 * i, row = idx / NCH, c = idx % NCH;
+                if (idx < 32 * NCH) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * ROWB + 16 * (c ^ (row & 15)));
+                    if (fr0 + row < a.seq) *reinterpret_cast<u32x4 *>(op + row * GROWB + 16 * c) = v;
+                }
             }
         }
         if (do_append) {
 #pragma unroll
             for (int jr = 0; jr < OWN_PASSES; ++jr) {
-                const uint32_t pos = own_lo + tid / OWN_CHUNKS + OWN_ROWS * jr;
-                if (pos < own_hi) {
-                    const uint64_t dst = (static_cast<uint64_t>(it.kvhead) * a.cap + pos) * GROWB + (tid % OWN_CHUNKS) * 16;
+                const uint32_t idx = tid + 256 * jr, pos = own_lo + idx / NCH;
+                if (pos < own_hi) {  // (chunks beyond the item's ROWS rows fall beyond own_hi as well)
+                    const uint64_t dst = (static_cast<uint64_t>(it.kvhead) * a.cap + pos) * GROWB + (idx % NCH) * 16;
                     *reinterpret_cast<u32x4 *>(Kc + dst) = ak[jr];
                     *reinterpret_cast<u32x4 *>(Vc + dst) = av[jr];
                 }
@@ -523,8 +528,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             } else {
                 // rows 4 J + lane / 16 of the wavefront's sixteen: K and Q rows swizzled by the row, V rows by lane / 16
                 const uint32_t row = 4 * J + (lane >> 4);
-                const uint32_t k_like = row * GROWB + 16 * (((lane & 15) ^ (row & 15)) & CM);
-                const uint32_t v_like = row * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) & CM);
+                const uint32_t k_like = row * GROWB + 16 * (((lane & 15) ^ (row & 15)) % NCH);
+                const uint32_t v_like = row * GROWB + 16 * (((lane & 15) ^ v_swizzle(lane >> 4)) % NCH);
                 if (I % 2 == 0) copy16<0>(base_a, k_like, dst_a + 1024 * J);
                 else copy16<0>(base_b, is_q ? k_like : v_like, dst_b + 1024 * J);
             }
@@ -566,12 +571,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 sc = Ops<T>::mfma(kf[KK % 4], qf[KK], sc);
                 if constexpr (KK + 4 < KSTEPS) kf[KK % 4] = *reinterpret_cast<const Raw16 *>(kb_base + (k_off ^ (32 * (KK + 4))));
                 if (kb == 0) {  // the eight parts of the copy spread over the products
-                    if constexpr (KSTEPS == 8) {
-                        copy_part.template operator()<KK>();
-                    } else {
-                        copy_part.template operator()<2 * KK>();
-                        copy_part.template operator()<2 * KK + 1>();
-                    }
+                    constexpr int P0 = KK * 8 / KSTEPS, P1 = (KK + 1) * 8 / KSTEPS;
+                    copy_part.template operator()<P0>();
+                    if constexpr (P1 - P0 > 1) copy_part.template operator()<P0 + 1>();
+                    static_assert(P1 - P0 <= 2, "at most two parts behind a product");
                 }
                 RG_SCHED_FENCE();
             };
@@ -579,12 +582,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             product.template operator()<1>();
             product.template operator()<2>();
             product.template operator()<3>();
-            if constexpr (KSTEPS == 8) {
-                product.template operator()<4>();
-                product.template operator()<5>();
-                product.template operator()<6>();
-                product.template operator()<7>();
-            }
+            if constexpr (KSTEPS > 4) product.template operator()<4>();
+            if constexpr (KSTEPS > 5) product.template operator()<5>();
+            if constexpr (KSTEPS > 6) product.template operator()<6>();
+            if constexpr (KSTEPS > 7) product.template operator()<7>();
             // O^T block db: rows d = 32 db + l32; A element i of MFMA (kb, jj) is V[key(i), d] with
             // key(i) = 32 kb + 16 jj + (i < 4 ? 4 half + i : 8 + 4 half + i - 4), the key order of pf.
             // A transposing read hands the 16 lanes of a group (16 consecutive d) four consecutive
@@ -757,13 +758,19 @@ int launch_d(const PrefillArgs &a, hipStream_t s) {
 
 template <class T>
 int launch_t(const PrefillArgs &a, hipStream_t s) {
-    return a.D == 64 ? launch_d<T, 64>(a, s) : launch_d<T, 128>(a, s);
+    switch (a.D) {
+        case 64: return launch_d<T, 64>(a, s);
+        case 80: return launch_d<T, 80>(a, s);
+        case 96: return launch_d<T, 96>(a, s);
+        case 128: return launch_d<T, 128>(a, s);
+        default: return RG_HIP_E_UNSUPPORTED;
+    }
 }
 
 }  // namespace
 
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D_) {
-    return (D_ == 128 || D_ == 64) && Hkv != 0 && H % Hkv == 0;
+    return (D_ == 128 || D_ == 96 || D_ == 80 || D_ == 64) && Hkv != 0 && H % Hkv == 0;
 }
 
 int launch_prefill(const PrefillArgs &a, hipStream_t s) {

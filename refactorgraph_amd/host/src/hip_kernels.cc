@@ -381,7 +381,7 @@ namespace refactor::kernel {
     AT::AttentionHip(Info info_) noexcept : Kernel(), info(info_) {}
     KernelBox AT::build(Info info) noexcept {
         if (info.dataType != DataType::FP16 && info.dataType != DataType::BF16) { return nullptr; }
-        if (info.headDim != 64 && info.headDim != 128) { return nullptr; }
+        if (info.headDim != 64 && info.headDim != 80 && info.headDim != 96 && info.headDim != 128) { return nullptr; }
         if (info.nKVHead == 0 || info.nHead % info.nKVHead != 0) { return nullptr; }
         if (info.cacheLen && info.cacheLen < info.seqLen) { return nullptr; }
         if (info.pastFromInput && info.pastCount != 1 && info.pastCount != info.batch) { return nullptr; }

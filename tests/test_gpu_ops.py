@@ -597,7 +597,7 @@ def test_empty_inputs_are_no_ops_and_bad_arguments_are_refused():
         "expand of nine dimensions": (L.rg_hip_expand(o, d, p(i64), p(i64), 9, 16, 4, None), E_UNSUPPORTED),
         "where of three-byte elements": (L.rg_hip_where(o, d, d, d, None, 0, 16, 3, None), E_UNSUPPORTED),
         "where without a condition": (L.rg_hip_where(o, None, d, d, None, 0, 16, 4, None), E_ARGUMENT),
-        "attention head dim 96": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 2, 1, 0, 96, 0.1, abi.FP16,
+        "attention head dim 48": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 2, 1, 0, 48, 0.1, abi.FP16,
                                                               d, 1 << 14, None, None), E_UNSUPPORTED),
         "attention heads not a multiple": (L.rg_hip_attention_kvcache(o, d, d, d, None, None, None, 0, 1, 8, 3, 1, 0, 128, 0.1,
                                                                        abi.FP16, d, 1 << 14, None, None), E_ARGUMENT),
@@ -877,6 +877,13 @@ def test_attention_decode_invariants_full_size():
     (2, 10, 2, 70, 256, 64, [3, 150], torch.bfloat16),    # group of 5
     (1, 8, 2, 129, 512, 64, [300], torch.float16),
     (3, 4, 1, 200, 333, 64, [0, 70, 133], torch.float16), # odd capacity and history lengths: the seam inside tiles
+    (2, 8, 2, 40, 128, 96, [0, 20], torch.float16),       # head dim 96: twelve chunks a row, three blocks of O^T
+    (2, 4, 4, 33, 64, 80, [5, 31], torch.float16),        # head dim 80: the third block of O^T half used
+    (1, 10, 2, 129, 512, 80, [300], torch.bfloat16),      # group of 5
+    (3, 4, 1, 200, 333, 96, [0, 70, 133], torch.float16),
+    (2, 8, 8, 1, 300, 80, [17, 299], torch.float16),      # a decode step: these head dims have the tiled kernel only
+    (3, 6, 2, 1, 64, 96, [0, 5, 63], torch.bfloat16),
+    (1, 32, 32, 7, 40, 96, [33], torch.float16),
 ])
 def test_attention_prefill_tiled_kernel(N, H, Hkv, seq, cap, D, past, dt):
     o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt)

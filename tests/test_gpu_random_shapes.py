@@ -185,7 +185,7 @@ def test_attention_on_random_shapes(seed):
         N = int(rng.integers(1, 7))
         Hkv = int(rng.choice([1, 2, 3, 4, 8]))
         H = Hkv * int(rng.choice([1, 2, 3, 4, 5, 8, 12]))
-        D = int(rng.choice([64, 128]))
+        D = int(rng.choice([64, 80, 96, 128]))
         kind = rng.integers(0, 4)
         seq = 1 if kind == 0 else int(rng.integers(1, 20)) if kind == 1 else int(rng.integers(16, 150))
         if kind == 3 and rng.integers(0, 3) == 0:

@@ -71,6 +71,6 @@ def test_static_scratch_entry_refuses_what_the_workspace_entry_refuses():
     d = torch.zeros(4096, device=DEV, dtype=torch.float16)
     p = d.data_ptr()
     L = abi.lib()
-    assert L.rg_hip_attention_kvcache_static(p, p, p, p, None, None, None, 0, 1, 8, 2, 1, 0, 96, 0.1, abi.FP16, None) == -1
+    assert L.rg_hip_attention_kvcache_static(p, p, p, p, None, None, None, 0, 1, 8, 2, 1, 0, 48, 0.1, abi.FP16, None) == -1
     assert L.rg_hip_attention_kvcache_static(p, p, p, p, None, None, None, 0, 1, 8, 2, 1, 0, 256, 0.1, abi.FP16, None) == -3
     assert L.rg_hip_attention_kvcache_static(p, p, p, p, None, None, None, 0, 1, 8, 3, 1, 0, 128, 0.1, abi.FP16, None) == -2
