@@ -449,6 +449,153 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     }
 }
 
+// ---------------------------------------------------------------- FP16 / BF16: any shape on the matrix cores
+//
+// What the kernels above do not take (fewer than 256 columns, column counts that are no multiple of 8, k that is
+// no multiple of 64, ...) as long as A is not transposed and k is a multiple of 8: 128 x 128 outputs per workgroup
+// of four wavefronts (64 x 64 each, 2 x 2 blocks of v_mfma_f32_32x32x16), k in tiles of 64 through two LDS
+// buffers filled from registers that are loaded two tiles ahead.  Both tiles are kept as [row or column][k] with a
+// pitch of 72 elements, so every fragment is one 128-bit read; B as [k, n] is turned on its way into LDS (two k-rows
+// of eight columns become eight 32-bit writes).  Loads are unconditional, from addresses clamped into the matrix,
+// so that the wait for a tile does not wait for the later ones as well; what lies beyond k is replaced by zeros,
+// rows and columns beyond the matrix are not stored.  Where rows of B as [k, n] are not 16-byte aligned its
+// elements are loaded one by one.
+constexpr int HT = 128, HK = 64, HP = 72, HF = 2;
+
+template <class T, bool TRANS_B, bool B_VEC>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
+__global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
+                                                  uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(16) uint16_t As[2][HT * HP];
+    __shared__ __align__(16) uint16_t Bs[2][HT * HP];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t row0 = blockIdx.y * HT, col0 = blockIdx.x * HT;
+    const uint16_t *A = reinterpret_cast<const uint16_t *>(a) + am * m * static_cast<uint64_t>(k);
+    const uint16_t *B = reinterpret_cast<const uint16_t *>(b) + bm * static_cast<uint64_t>(k) * n;
+
+    // [row][k] tiles: rows tid / 8 + 32 i, k 8 (tid % 8) .. + 7 (a row of a tile is one 128-byte line).
+    // B as [k, n]: k-rows 2 (tid / 16) + 32 (i / 2) + i % 2, columns 8 (tid % 16) .. + 7
+    const uint32_t pr = tid >> 3, pk = 8 * (tid & 7);
+    const uint16_t *a_src[4], *b_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t r = row0 + pr + 32 * i;
+        a_src[i] = A + static_cast<uint64_t>(r < m ? r : m - 1) * k;
+        const uint32_t c = col0 + pr + 32 * i;
+        b_src[i] = B + static_cast<uint64_t>(c < n ? c : n - 1) * k;  // (B as [n, k] only)
+    }
+    const uint32_t bk = tid >> 4, bc = col0 + 8 * (tid & 15);
+    const uint32_t bc_load = bc + 8 <= n ? bc : (n >= 8 ? n - 8 : 0);  // (vector loads only)
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    u32x4 ra[HF][4], rb[HF][4];  // HF tiles in flight
+    auto fetch = [&](auto set, uint32_t k0) {
+        constexpr int P = decltype(set)::value;
+        const uint32_t kq = k0 + pk < k ? k0 + pk : k - 8;  // k is a multiple of 8
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            ra[P][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kq);
+            if constexpr (TRANS_B) {
+                rb[P][i] = *reinterpret_cast<const u32x4 *>(b_src[i] + kq);
+            } else {
+                const uint32_t kr = k0 + 2 * bk + 32 * (i / 2) + i % 2;
+                const uint16_t *src = B + static_cast<uint64_t>(kr < k ? kr : k - 1) * n;
+                if constexpr (B_VEC) {
+                    rb[P][i] = *reinterpret_cast<const u32x4 *>(src + bc_load);
+                } else {
+                    uint16_t e[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) e[j] = src[bc + j < n ? bc + j : n - 1];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) rb[P][i][j] = e[2 * j] | (static_cast<uint32_t>(e[2 * j + 1]) << 16);
+                }
+            }
+        }
+    };
+    auto stash = [&](auto set, int buf, uint32_t k0) {
+        constexpr int P = decltype(set)::value;
+        const bool k_in = k0 + pk < k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<u32x4 *>(&As[buf][(pr + 32 * i) * HP + pk]) = k_in ? ra[P][i] : zero4;
+            if constexpr (TRANS_B) *reinterpret_cast<u32x4 *>(&Bs[buf][(pr + 32 * i) * HP + pk]) = k_in ? rb[P][i] : zero4;
+        }
+        if constexpr (!TRANS_B) {
+            // the two k-rows of a lane's eight columns as one 32-bit word per column.  The eight 16-byte pieces of a
+            // column's k are kept in an order that depends on the column (piece ^ (column / 16) % 8): the writes of
+            // a wavefront then fall into 64 different LDS banks
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii) {
+                const uint32_t kr = k0 + 2 * bk + 32 * ii;  // (k is even: both rows of the pair are in or out)
+                const uint32_t word = (bk + 16 * ii) ^ (((tid >> 1) & 7) << 2);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t col = 8 * (tid & 15) + 2 * j;
+                    const uint32_t even = __builtin_amdgcn_perm(rb[P][2 * ii + 1][j], rb[P][2 * ii][j], 0x05040100u);
+                    const uint32_t odd = __builtin_amdgcn_perm(rb[P][2 * ii + 1][j], rb[P][2 * ii][j], 0x07060302u);
+                    *reinterpret_cast<uint32_t *>(&Bs[buf][col * HP + 2 * word]) = kr < k ? even : 0u;
+                    *reinterpret_cast<uint32_t *>(&Bs[buf][(col + 1) * HP + 2 * word]) = kr < k ? odd : 0u;
+                }
+            }
+        }
+    };
+
+    f16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    const uint32_t l32 = lane & 31, kh = lane >> 5;
+    const uint32_t tiles = (k + HK - 1) / HK;
+    auto step = [&](auto set, uint32_t t) {
+        const int buf = t & 1;
+        stash(set, buf, t * HK);
+        __syncthreads();  // the tile is complete; the other buffer's readers of two tiles ago have passed this point
+        fetch(set, (t + HF) * HK);
+#pragma unroll
+        for (int ks = 0; ks < HK / 16; ++ks) {
+            u32x4 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const u32x4 *>(&As[buf][(wm * 64 + 32 * i + l32) * HP + 16 * ks + 8 * kh]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t piece = TRANS_B ? 2 * ks + kh : (2 * ks + kh) ^ ((4 * wn + 2 * j + (l32 >> 4)) & 7);
+                fb[j] = *reinterpret_cast<const u32x4 *>(&Bs[buf][(wn * 64 + 32 * j + l32) * HP + 8 * piece]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+        }
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    fetch(std::integral_constant<int, 1>{}, HK);
+    for (uint32_t t = 0; t < tiles; t += HF) {  // no branch inside: an odd count's last step multiplies zeros
+        step(std::integral_constant<int, 0>{}, t);
+        step(std::integral_constant<int, 1>{}, t + 1);
+    }
+    // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
+    const T *C = static_cast<const T *>(bias.ptr);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t row = row0 + wm * 64 + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
+                const uint32_t col = col0 + wn * 64 + 32 * j + l32;
+                if (row < m && col < n) {
+                    float v = alpha * acc[i][j][e];
+                    if (C) v += beta * up(C[ym * bias.sb + row * bias.sm + col * bias.sn]);
+                    y[(ym * m + row) * n + col] = down<T>(v);
+                }
+            }
+}
+
 // ---------------------------------------------------------------- few rows of A (decode): weight streaming
 //
 // Y[m, n] = alpha * A[m, k] @ W[n, k]^T (+ bias) for m <= 32 SLABS, FP16 / BF16: bound by reading W once
@@ -1298,6 +1445,9 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool rows_kn_f32 = rows_kn_f32_ok && f32_passes * (3.0 + 33.0 * kn4096) <= f32_cost_tiles;
     const bool f32_tiles = f32_tiles_ok && m > 8;
 
+    // FP16 / BF16 shapes that none of the kernels above takes, more than 8 rows: 128 x 128 tiles, any m and n
+    const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && m > 8 && aligned16(a) && (!trans_b || aligned16(b));
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
             if (short_tile) {
@@ -1381,6 +1531,17 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
                 else
                     mm_mfma_256x256<T, false><<<grid, 256, 0, s>>>(y, a, b, bias, static_cast<uint32_t>(m), static_cast<uint32_t>(k),
                                                                    static_cast<uint32_t>(n), al, be, am0, bm0, ym0);
+                return launch_status();
+            }
+        }
+        if constexpr (narrow) {
+            if (tiles16) {
+                const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + HT - 1) / HT), count);
+                if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
+                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+                if (trans_b) mm_tiles16<T, true, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+                else if (n % 8 == 0 && n >= 8 && aligned16(b)) mm_tiles16<T, false, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+                else mm_tiles16<T, false, false><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
                 return launch_status();
             }
         }

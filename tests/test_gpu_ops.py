@@ -1162,6 +1162,39 @@ def test_matmul_mfma_path_fp16_bf16(m, k, n, dt, tb):
     _matmul_check(got, ref, _absprod(f(ad), f(bd[:1]), False, tb), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("m,k,n", [(300, 72, 128), (130, 1000, 77), (64, 8, 5), (513, 136, 250), (9, 200, 1031), (257, 64, 8)])
+def test_matmul_any_shape_on_the_matrix_cores(m, k, n, dt, tb):
+    # fewer than 256 columns, column counts that are no multiple of 8 (rows of B as [k, n] then start on odd
+    # addresses), k that is no multiple of 64, one to three k tiles: the 128 x 128 tile kernel, against the oracle
+    rng = np.random.default_rng(41)
+    a = rng.standard_normal((2, m, k)).astype(np.float32)
+    b = rng.standard_normal((2, n, k) if tb else (2, k, n)).astype(np.float32)
+    bias = rng.standard_normal((2, m, n)).astype(np.float32)
+    ad, bd, cd = (dev(t).to(dt) for t in (a, b, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(bd), to_oracle(cd), False, tb, 0.5, 2.0, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    got = f(ops.matmul(ad, bd, cd, False, tb, 0.5, 2.0))
+    mag = 0.5 * _absprod(f(ad), f(bd), False, tb) + 2.0 * np.abs(f(cd))
+    _matmul_check(got, ref, mag, 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+
+
+def test_matmul_any_shape_exact_on_small_integers():
+    # integer-valued operands: every result is exact in fp16, so rows, columns and k beyond the matrix must
+    # contribute nothing, bit for bit (vocabulary-sized column count, both layouts of B)
+    rng = np.random.default_rng(42)
+    a = rng.integers(-2, 3, (200, 328)).astype(np.float32)
+    b = rng.integers(-2, 3, (328, 5003)).astype(np.float32)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.max(np.abs(want)) < 2048
+    assert np.array_equal(host(ops.matmul(dev(a).half(), dev(b).half()).float()), want)
+    assert np.array_equal(host(ops.matmul(dev(a).half(), dev(np.ascontiguousarray(b.T)).half(), trans_b=True).float()), want)
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
