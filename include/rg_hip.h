@@ -224,7 +224,8 @@ int rg_hip_where(void *out, const void *condition, const void *x, const void *y,
  * rg_hip_matmul_integer_workspace() returns 0 (the reference needs m*k [+ k*n] bytes).
  * Integer sums are exact in any order, so every path (matrix cores on 256 x 256 tiles, with k split
  * between workgroups when the tiles are few, also for 65 to 255 rows; weight streaming for up to 64
- * rows; vector-ALU dot products for one to four rows) returns the same bits. */
+ * rows; vector-ALU dot products for one to four rows; 128 x 128 tiles for other shapes with k a
+ * multiple of 16) returns the same bits. */
 enum {
     RG_MMI_A_ZP_SCALAR = 1u,
     RG_MMI_B_ZP_SCALAR = 2u,

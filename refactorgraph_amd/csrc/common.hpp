@@ -106,6 +106,25 @@ __device__ __forceinline__ void store16(T *p, const Vec16<T> &v) {
 // Streaming variants: data touched once, marked non-temporal so it does not displace reusable
 // lines in L2 / the memory-side cache.
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Sixteen bytes from an address of any alignment: five aligned 32-bit loads and four byte alignments.  `last_word` is
+// the last aligned word of the buffer; words behind it are not read (the bytes they would have given are arbitrary),
+// and the word in front of an unaligned `p` shares its first byte's word, so nothing outside the buffer's own words
+// is touched.
+__device__ __forceinline__ u32x4 load16_any(const void *p, const void *last_word) {
+    const uint64_t bits = reinterpret_cast<uint64_t>(p), last = reinterpret_cast<uint64_t>(last_word);
+    const uint32_t shift = static_cast<uint32_t>(bits) & 3u;
+    const uint64_t first = bits & ~3ull;
+    uint32_t w[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        const uint64_t at = first + 4 * i < last ? first + 4 * i : last;
+        w[i] = *reinterpret_cast<const uint32_t *>(at);
+    }
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __builtin_amdgcn_alignbyte(w[i + 1], w[i], shift);
+    return v;
+}
 template <class T>
 __device__ __forceinline__ Vec16<T> load16_stream(const T *p) {
     const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));

@@ -458,8 +458,8 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 // pitch of 72 elements, so every fragment is one 128-bit read; B as [k, n] is turned on its way into LDS (two k-rows
 // of eight columns become eight 32-bit writes).  Loads are unconditional, from addresses clamped into the matrix,
 // so that the wait for a tile does not wait for the later ones as well; what lies beyond k is replaced by zeros,
-// rows and columns beyond the matrix are not stored.  Where rows of B as [k, n] are not 16-byte aligned its
-// elements are loaded one by one.
+// rows and columns beyond the matrix are not stored.  Where rows of B as [k, n] are not 16-byte aligned, eight
+// elements come from five aligned words.
 constexpr int HT = 128, HK = 64, HP = 72, HF = 2;
 
 template <class T, bool TRANS_B, bool B_VEC>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
@@ -488,6 +488,7 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
     }
     const uint32_t bk = tid >> 4, bc = col0 + 8 * (tid & 15);
     const uint32_t bc_load = bc + 8 <= n ? bc : (n >= 8 ? n - 8 : 0);  // (vector loads only)
+    const uint16_t *b_last = reinterpret_cast<const uint16_t *>((reinterpret_cast<uint64_t>(B + static_cast<uint64_t>(k) * n) - 1) & ~3ull);
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     u32x4 ra[HF][4], rb[HF][4];  // HF tiles in flight
     auto fetch = [&](auto set, uint32_t k0) {
@@ -504,11 +505,7 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
                 if constexpr (B_VEC) {
                     rb[P][i] = *reinterpret_cast<const u32x4 *>(src + bc_load);
                 } else {
-                    uint16_t e[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) e[j] = src[bc + j < n ? bc + j : n - 1];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) rb[P][i][j] = e[2 * j] | (static_cast<uint32_t>(e[2 * j + 1]) << 16);
+                    rb[P][i] = load16_any(src + bc, b_last);  // (columns beyond n: arbitrary values, not stored)
                 }
             }
         }

@@ -413,6 +413,150 @@ constexpr uint64_t kSplitFill = 128;
 constexpr uint32_t kSplitMax = 4;
 constexpr uint64_t kSkinnyWorkgroups = 256;  // per launch: one per CU (512 and 128 were measured: slower)
 
+// ---------------------------------------------------------------- any shape on the matrix cores
+//
+// What the kernels around it do not take (fewer than 256 columns, column counts that are no multiple of 16, k that
+// is no multiple of 128) as long as k is a multiple of 16: 128 x 128 outputs per workgroup of four wavefronts
+// (64 x 64 each, 2 x 2 blocks of v_mfma_i32_32x32x32_i8), k in tiles of 128 through two LDS buffers filled from
+// registers that are loaded two tiles ahead.  Both tiles are kept as [row or column][k] with a pitch of 144 bytes,
+// so every fragment is one 128-bit read; B ([k, n] in memory) is turned on its way into LDS: four k-rows of sixteen
+// columns become sixteen 32-bit writes.  The zero points are subtracted (bytes, modulo 256) as the tiles pass
+// through registers.  Loads are unconditional, from addresses clamped into the matrices, so that the wait for a
+// tile does not wait for the later ones as well; what lies beyond k is replaced by zeros (after the subtraction),
+// rows and columns beyond the matrices are not stored.  Where rows of B are not 16-byte aligned, sixteen bytes
+// come from five aligned words.
+constexpr int GT = 128, GK = 128, GP = 144;
+
+template <bool DEQ, bool B_VEC>  // B_VEC: rows of B start on 16-byte boundaries, n >= 16
+__global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+                                                 ZeroPoint za, ZeroPoint zb, Dequant dq, uint32_t m, uint32_t k, uint32_t n,
+                                                 uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
+    __shared__ __align__(16) uint8_t As[2][GT * GP];
+    __shared__ __align__(16) uint8_t Bs[2][GT * GP];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t bz = blockIdx.z;
+    const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
+    const uint32_t row0 = blockIdx.y * GT, col0 = blockIdx.x * GT;
+    const uint8_t *A = a + am * m * static_cast<uint64_t>(k);
+    const uint8_t *B = b + bm * static_cast<uint64_t>(k) * n;
+
+    // A tile: rows tid / 8 + 32 i, k 16 (tid % 8) .. + 15 (a row of a tile is one 128-byte line).
+    // B tile: k-rows 4 (tid / 8) + i, columns 16 (tid % 8) .. + 15
+    const uint32_t pr = tid >> 3, pk = 16 * (tid & 7);
+    const uint8_t *a_src[4];
+    uint32_t a_zero[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t r = row0 + pr + 32 * i, row = r < m ? r : m - 1;
+        a_src[i] = A + static_cast<uint64_t>(row) * k;
+        a_zero[i] = splat(zp_byte(za, am * m + row));
+    }
+    const uint32_t bq = tid >> 3, bc = col0 + 16 * (tid & 7);
+    const uint32_t bc_load = bc + 16 <= n ? bc : (n >= 16 ? n - 16 : 0);  // (vector loads only)
+    const uint8_t *b_last = reinterpret_cast<const uint8_t *>((reinterpret_cast<uint64_t>(B) + static_cast<uint64_t>(k) * n - 1) & ~3ull);
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    u32x4 ra[2][4], rb[2][4];  // two tiles in flight
+    uint32_t b_zero[2][4];
+    auto fetch = [&](auto set, uint32_t k0) {
+        constexpr int P = decltype(set)::value;
+        const uint32_t kq = k0 + pk < k ? k0 + pk : k - 16;  // k is a multiple of 16
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            ra[P][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kq);
+            const uint32_t kr0 = k0 + 4 * bq + i, kr = kr0 < k ? kr0 : k - 1;
+            const uint8_t *src = B + static_cast<uint64_t>(kr) * n;
+            b_zero[P][i] = splat(zp_byte(zb, bm * k + kr));
+            if constexpr (B_VEC) {
+                rb[P][i] = *reinterpret_cast<const u32x4 *>(src + bc_load);
+            } else {
+                rb[P][i] = load16_any(src + bc, b_last);  // (columns beyond n: arbitrary bytes, not stored)
+            }
+        }
+    };
+    auto stash = [&](auto set, int buf, uint32_t k0) {
+        constexpr int P = decltype(set)::value;
+        const bool k_in = k0 + pk < k;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = sub_bytes(ra[P][i][j], a_zero[i]);
+            *reinterpret_cast<u32x4 *>(&As[buf][(pr + 32 * i) * GP + pk]) = k_in ? v : zero4;
+        }
+        // four k-rows of sixteen columns -> per column one word of four consecutive k.  The eight 16-byte pieces
+        // of a column's k are kept in an order that depends on the column (piece ^ (column / 16) % 8), which
+        // spreads the eight column groups of a wavefront over the LDS banks
+        const bool rows_in = k0 + 4 * bq < k;  // (k is a multiple of 4: all four rows are in or out)
+        const uint32_t word = bq ^ ((tid & 7) << 2);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t r[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r[i] = sub_bytes(rb[P][i][j], b_zero[P][i]);
+            const uint32_t lo01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+            const uint32_t c[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                                   __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t col = 16 * (tid & 7) + 4 * j + q;
+                *reinterpret_cast<uint32_t *>(&Bs[buf][col * GP + 4 * word]) = rows_in ? c[q] : 0u;
+            }
+        }
+    };
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    const uint32_t l32 = lane & 31, kh = lane >> 5;
+    const uint32_t tiles = (k + GK - 1) / GK;
+    auto step = [&](auto set, uint32_t t) {
+        const int buf = t & 1;
+        stash(set, buf, t * GK);
+        __syncthreads();  // the tile is complete; the other buffer's readers of two tiles ago have passed this point
+        fetch(set, (t + 2) * GK);
+#pragma unroll
+        for (int ks = 0; ks < GK / 32; ++ks) {
+            v4i fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const v4i *>(&As[buf][(wm * 64 + 32 * i + l32) * GP + 32 * ks + 16 * kh]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t piece = (2 * ks + kh) ^ ((4 * wn + 2 * j + (l32 >> 4)) & 7);
+                fb[j] = *reinterpret_cast<const v4i *>(&Bs[buf][(wn * 64 + 32 * j + l32) * GP + 16 * piece]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    };
+    fetch(std::integral_constant<int, 0>{}, 0);
+    fetch(std::integral_constant<int, 1>{}, GK);
+    for (uint32_t t = 0; t < tiles; t += 2) {  // no branch inside: an odd count's last step multiplies zeros
+        step(std::integral_constant<int, 0>{}, t);
+        step(std::integral_constant<int, 1>{}, t + 1);
+    }
+    // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t col = col0 + wn * 64 + 32 * j + l32;
+        const float scale = DEQ && col < n ? dq.scale[dq.per_column ? col : 0] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t row = row0 + wm * 64 + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
+                if (row < m && col < n) y[(ym * m + row) * n + col] = finish<DEQ>(acc[i][j][e], scale);
+            }
+    }
+}
+
 __global__ __launch_bounds__(256) void mmi_zero(int32_t *__restrict__ y, uint64_t count) {
     for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<uint64_t>(gridDim.x) * 256)
         y[i] = 0;
@@ -820,6 +964,13 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         }
         if (fast) {
             return launch_tiles(std::false_type{}, am0, bm0, ym0, count);
+        } else if (k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && (m + GT - 1) / GT <= 65535) {
+            const dim3 grid(static_cast<unsigned>((n + GT - 1) / GT), static_cast<unsigned>((m + GT - 1) / GT), count);
+            const auto *a8 = static_cast<const uint8_t *>(a);
+            const auto *b8 = static_cast<const uint8_t *>(b);
+            const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+            if (n % 16 == 0 && aligned16(b)) mmi_tiles<DEQ, true><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
+            else mmi_tiles<DEQ, false><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
         } else {
             const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
             mmi_generic<DEQ><<<grid, 256, 0, s>>>(

@@ -449,7 +449,7 @@ def test_matmul_integer_few_tiles_split_k(m, k, n):
 @pytest.mark.parametrize("m,k,n", [(300, 128, 256), (256, 128, 272), (700, 256, 1008), (513, 384, 528), (257, 128, 257)])
 def test_matmul_integer_ragged_rows_and_columns(m, k, n):
     # m and n beyond 256 that are no multiples of the MFMA tile: the last tiles are moved back and overlap
-    # their neighbours ((257, 128, 257): n is no multiple of 16, the plain kernel takes it)
+    # their neighbours ((257, 128, 257): n is no multiple of 16, the 128 x 128 tile kernel takes it)
     rng = np.random.default_rng(m * n)
     a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
     b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
@@ -460,6 +460,29 @@ def test_matmul_integer_ragged_rows_and_columns(m, k, n):
     scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
     y = host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale)))
     assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
+
+
+@pytest.mark.parametrize("m,k,n", [(300, 144, 128), (130, 1008, 77), (64, 16, 5), (513, 272, 250), (9, 208, 1031), (257, 128, 16),
+                                   (200, 336, 5003)])
+def test_matmul_integer_any_shape_on_the_matrix_cores(m, k, n):
+    # fewer than 256 columns, column counts that are no multiple of 16 (rows of B then start on odd addresses), k that
+    # is no multiple of 128, one to three k tiles: the 128 x 128 tile kernel, every zero-point form, both epilogues
+    rng = np.random.default_rng(m * n + k)
+    a = rng.integers(0, 256, (2, m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (2, k, n), dtype=np.int8)
+    az = rng.integers(0, 256, (2 * m,), dtype=np.uint8)        # one per (batch, row)
+    bz = rng.integers(-128, 128, (2 * k,), dtype=np.int8)
+    ref = oracle.matmul_integer(a, b, az, bz, threads=8)
+    assert np.array_equal(host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz))), ref)
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), dev(bz), dequant_scale=dev(scale)))
+    assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
+    assert np.array_equal(host(ops.matmul_integer(dev(a), dev(b))), oracle.matmul_integer(a, b, None, None, threads=8))
+    # B from an address that is no multiple of 4: the aligned words around it belong to the same buffer
+    flat = dev(np.concatenate([np.zeros(1, np.int8), b[0].reshape(-1)]))
+    b_odd = flat[1:].view(k, n)
+    got = host(ops.matmul_integer(dev(a[0]), b_odd, dev(az[:m]), dev(bz[:k])))
+    assert np.array_equal(got, ref[0])
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 128, 256), (7, 1024, 512), (32, 4096, 4096), (33, 256, 256), (64, 256, 256), (100, 384, 512),
@@ -1181,6 +1204,11 @@ def test_matmul_any_shape_on_the_matrix_cores(m, k, n, dt, tb):
     got = f(ops.matmul(ad, bd, cd, False, tb, 0.5, 2.0))
     mag = 0.5 * _absprod(f(ad), f(bd), False, tb) + 2.0 * np.abs(f(cd))
     _matmul_check(got, ref, mag, 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    if not tb:
+        # B from an address that is no multiple of 4: same values, the aligned words around it are the buffer's own
+        flat = torch.cat([torch.zeros(1, dtype=dt, device="cuda"), bd.reshape(-1)])
+        got_odd = f(ops.matmul(ad, flat[1:].view(bd.shape), cd, False, tb, 0.5, 2.0))
+        assert np.array_equal(got_odd, got)
 
 
 def test_matmul_any_shape_exact_on_small_integers():
