@@ -461,6 +461,8 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 // rows and columns beyond the matrix are not stored.  Where rows of B as [k, n] are not 16-byte aligned, eight
 // elements come from five aligned words.
 constexpr int HT = 128, HK = 64, HP = 72, HF = 2;
+constexpr size_t kSmallGrid = 384;  // workgroups up to which these tiles replace the 256 x 256 ones
+constexpr size_t kSkinnyPassesSmall = 13000, kRowsKnPassesSmall = 11500;
 
 template <class T, bool TRANS_B, bool B_VEC>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
 __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
@@ -1416,10 +1418,18 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool short_ok = narrow && !trans_a && m < BM && n >= BN && n % 8 == 0 && k % BK == 0 && k > 0 && aligned16(a) &&
                           aligned16(b) && aligned16(y_) && !(n % BN != 0 && bias.ptr == y_) &&
                           k < (1u << 22);  // a lane's offset into A (up to 255 rows) stays below 2^31
+    // FP16 / BF16 shapes that none of the kernels above takes, more than 8 rows: 128 x 128 tiles, any m and n.
+    // They also take the shapes of the 256 x 256 tiles when those are few: a workgroup's walk through k is a chain
+    // of dependent steps (1.33 us per 64 of k on the large tile, 0.83 us on the small one), so while the small tiles
+    // find a CU each, or nearly, the launch ends earlier (k = 4096: 85 -> 53 us up to 64 large tiles, 85 -> 78 at 86,
+    // level at 128)
+    const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && m > 8 && aligned16(a) && (!trans_b || aligned16(b));
+    const bool small_grid = tiles16 && ((m + HT - 1) / HT) * ((n + HT - 1) / HT) * (a_index || b_index ? 1 : batch) <= kSmallGrid;
     bool short_tile = false;
     if (short_ok) {
-        if (trans_b) short_tile = rows ? false : skinny ? ((m + 63) / 64) * n > 23000 : !gemv;
-        else short_tile = rows_kn ? ((m + 31) / 32) * n > 17000 : gemv_kn ? m > 16 : true;
+        // (the tile launch that the passes of the few-rows kernels are weighed against is cheaper on the small tiles)
+        if (trans_b) short_tile = rows ? false : skinny ? ((m + 63) / 64) * n > (small_grid ? kSkinnyPassesSmall : 23000u) : !gemv;
+        else short_tile = rows_kn ? ((m + 31) / 32) * n > (small_grid ? kRowsKnPassesSmall : 17000u) : gemv_kn ? m > 16 : true;
     }
 
     // F32 on the matrix cores.  A launch of the 128 x 128 tiles walks all of k in every workgroup and takes about
@@ -1442,11 +1452,23 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool rows_kn_f32 = rows_kn_f32_ok && f32_passes * (3.0 + 33.0 * kn4096) <= f32_cost_tiles;
     const bool f32_tiles = f32_tiles_ok && m > 8;
 
-    // FP16 / BF16 shapes that none of the kernels above takes, more than 8 rows: 128 x 128 tiles, any m and n
-    const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && m > 8 && aligned16(a) && (!trans_b || aligned16(b));
+    auto launch_tiles16 = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if constexpr (narrow) {
+            const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + HT - 1) / HT), count);
+            if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
+            const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+            if (trans_b) mm_tiles16<T, true, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+            else if (n % 8 == 0 && n >= 8 && aligned16(b)) mm_tiles16<T, false, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+            else mm_tiles16<T, false, false><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+            return launch_status();
+        } else {
+            return RG_HIP_E_UNSUPPORTED;
+        }
+    };
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            if (small_grid && (short_tile || fast)) return launch_tiles16(am0, bm0, ym0, count);
             if (short_tile) {
                 const dim3 grid(static_cast<unsigned>((n + BN - 1) / BN), 1, count);
                 if (trans_b)
@@ -1532,15 +1554,7 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
             }
         }
         if constexpr (narrow) {
-            if (tiles16) {
-                const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + HT - 1) / HT), count);
-                if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
-                const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
-                if (trans_b) mm_tiles16<T, true, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
-                else if (n % 8 == 0 && n >= 8 && aligned16(b)) mm_tiles16<T, false, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
-                else mm_tiles16<T, false, false><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
-                return launch_status();
-            }
+            if (tiles16) return launch_tiles16(am0, bm0, ym0, count);
         }
         if constexpr (std::is_same<T, float>::value) {
             if (rows_f32) {

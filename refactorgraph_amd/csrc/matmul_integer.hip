@@ -908,7 +908,40 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         return launch_status();
     };
 
+    // The 128 x 128 tiles instead of the 256 x 256 ones where the launch is expected to end earlier: a workgroup's
+    // walk through k is a chain of dependent steps (1.6 us per 128 of k on the large tile, 1.12 us on the small one),
+    // and sharing k between workgroups costs a zeroing pass and one atomic per output and range (measured: 9 us and
+    // 4.3 us per million outputs), so few large tiles with a short k lose to four times as many small ones
+    // (2048^3: 40 -> 24 us; 1024 x 4096 x 4096: 52 -> 39 us; 256 x 4096 x 4096 stays: 27 against 37 us).
+    auto small_tiles_pay = [&](bool short_m, uint32_t count) {
+        const double large = static_cast<double>(((m + BM - 1) / BM) * ((n + BN - 1) / BN)) * count;
+        const double small = static_cast<double>(((m + GT - 1) / GT) * ((n + GT - 1) / GT)) * count;
+        const uint32_t k_tiles = static_cast<uint32_t>(k / BK);
+        uint32_t splits = static_cast<uint32_t>(kSplitFill / large);
+        splits = splits > kSplitMax ? kSplitMax : splits;
+        splits = splits > k_tiles / 2 ? k_tiles / 2 : splits;
+        if ((!short_m && m % BM != 0) || n % BN != 0 || splits < 1) splits = 1;
+        const double outputs = 1e-6 * static_cast<double>(m) * static_cast<double>(n) * count;
+        const double steps = (k_tiles + splits - 1) / splits;
+        const double large_us = splits > 1 ? 1.6 * steps + 9 + 4.3 * outputs + (DEQ ? 2 + 2.5 * outputs : 0)
+                                           : 1.6 * steps * static_cast<double>((static_cast<uint64_t>(large) + 255) / 256) + 3;
+        const double small_us = 6 + 1.12 * k_tiles * (small > 256 ? small / 256 : 1.0);
+        return small_us < large_us;
+    };
+    auto launch_small_tiles = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        const dim3 grid(static_cast<unsigned>((n + GT - 1) / GT), static_cast<unsigned>((m + GT - 1) / GT), count);
+        const auto *a8 = static_cast<const uint8_t *>(a);
+        const auto *b8 = static_cast<const uint8_t *>(b);
+        const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
+        if (n % 16 == 0 && aligned16(b)) mmi_tiles<DEQ, true><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
+        else mmi_tiles<DEQ, false><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
+        return launch_status();
+    };
+    const bool small_tiles_ok = k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && (m + GT - 1) / GT <= 65535;
+
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
+        if (small_tiles_ok && (short_tile || (fast && !gemv && !skinny)) && small_tiles_pay(short_tile, count))
+            return launch_small_tiles(am0, bm0, ym0, count);
         if (short_tile) return launch_tiles(std::true_type{}, am0, bm0, ym0, count);
         if (gemv) {
             const auto *a8 = static_cast<const uint8_t *>(a);
@@ -964,13 +997,8 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         }
         if (fast) {
             return launch_tiles(std::false_type{}, am0, bm0, ym0, count);
-        } else if (k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && (m + GT - 1) / GT <= 65535) {
-            const dim3 grid(static_cast<unsigned>((n + GT - 1) / GT), static_cast<unsigned>((m + GT - 1) / GT), count);
-            const auto *a8 = static_cast<const uint8_t *>(a);
-            const auto *b8 = static_cast<const uint8_t *>(b);
-            const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
-            if (n % 16 == 0 && aligned16(b)) mmi_tiles<DEQ, true><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
-            else mmi_tiles<DEQ, false><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
+        } else if (small_tiles_ok) {
+            return launch_small_tiles(am0, bm0, ym0, count);
         } else {
             const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 15) / 16), count);
             mmi_generic<DEQ><<<grid, 256, 0, s>>>(
