@@ -454,37 +454,43 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
 // What the kernels above do not take (fewer than 256 columns, column counts that are no multiple of 8, k that is
 // no multiple of 64, ...) as long as A is not transposed and k is a multiple of 8: 128 x 128 outputs per workgroup
 // of four wavefronts (64 x 64 each, 2 x 2 blocks of v_mfma_f32_32x32x16), k in tiles of 64 through two LDS
-// buffers filled from registers that are loaded two tiles ahead.  Both tiles are kept as [row or column][k] with a
+// buffers filled from registers that are loaded three tiles ahead.  Both tiles are kept as [row or column][k] with a
 // pitch of 72 elements, so every fragment is one 128-bit read; B as [k, n] is turned on its way into LDS (two k-rows
 // of eight columns become eight 32-bit writes).  Loads are unconditional, from addresses clamped into the matrix,
 // so that the wait for a tile does not wait for the later ones as well; what lies beyond k is replaced by zeros,
 // rows and columns beyond the matrix are not stored.  Where rows of B as [k, n] are not 16-byte aligned, eight
 // elements come from five aligned words.
-constexpr int HT = 128, HK = 64, HP = 72, HF = 2;
+constexpr int HT = 128, HK = 64, HP = 72, HF = 3;
+constexpr size_t kHalfTiles = 128;   // tiles of 128 rows up to which tiles of 64 rows are launched instead
 constexpr size_t kSmallGrid = 384;  // workgroups up to which these tiles replace the 256 x 256 ones
-constexpr size_t kSkinnyPassesSmall = 13000, kRowsKnPassesSmall = 11500;
+constexpr size_t kSkinnyPassesSmall = 12000, kRowsKnPassesSmall = 10500;
 
-template <class T, bool TRANS_B, bool B_VEC>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
+// TM: rows of a tile, 128 or 64 (a wavefront then has 32 rows of 64 columns: twice the workgroups for few tiles)
+template <class T, bool TRANS_B, bool B_VEC, int TM>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
 __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
                                                   uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
                                                   uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
-    __shared__ __align__(16) uint16_t As[2][HT * HP];
+    constexpr int MI = TM / 64, AI = TM / 32;  // row blocks of a wavefront, loads of A per thread and tile
+    __shared__ __align__(16) uint16_t As[2][TM * HP];
     __shared__ __align__(16) uint16_t Bs[2][HT * HP];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
-    const uint32_t row0 = blockIdx.y * HT, col0 = blockIdx.x * HT;
+    const uint32_t row0 = blockIdx.y * TM, col0 = blockIdx.x * HT;
     const uint16_t *A = reinterpret_cast<const uint16_t *>(a) + am * m * static_cast<uint64_t>(k);
     const uint16_t *B = reinterpret_cast<const uint16_t *>(b) + bm * static_cast<uint64_t>(k) * n;
 
     // [row][k] tiles: rows tid / 8 + 32 i, k 8 (tid % 8) .. + 7 (a row of a tile is one 128-byte line).
     // B as [k, n]: k-rows 2 (tid / 16) + 32 (i / 2) + i % 2, columns 8 (tid % 16) .. + 7
     const uint32_t pr = tid >> 3, pk = 8 * (tid & 7);
-    const uint16_t *a_src[4], *b_src[4];
+    const uint16_t *a_src[AI], *b_src[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < AI; ++i) {
         const uint32_t r = row0 + pr + 32 * i;
         a_src[i] = A + static_cast<uint64_t>(r < m ? r : m - 1) * k;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
         const uint32_t c = col0 + pr + 32 * i;
         b_src[i] = B + static_cast<uint64_t>(c < n ? c : n - 1) * k;  // (B as [n, k] only)
     }
@@ -492,13 +498,14 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
     const uint32_t bc_load = bc + 8 <= n ? bc : (n >= 8 ? n - 8 : 0);  // (vector loads only)
     const uint16_t *b_last = reinterpret_cast<const uint16_t *>((reinterpret_cast<uint64_t>(B + static_cast<uint64_t>(k) * n) - 1) & ~3ull);
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    u32x4 ra[HF][4], rb[HF][4];  // HF tiles in flight
+    u32x4 ra[HF][AI], rb[HF][4];  // HF tiles in flight
     auto fetch = [&](auto set, uint32_t k0) {
         constexpr int P = decltype(set)::value;
         const uint32_t kq = k0 + pk < k ? k0 + pk : k - 8;  // k is a multiple of 8
 #pragma unroll
+        for (int i = 0; i < AI; ++i) ra[P][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kq);
+#pragma unroll
         for (int i = 0; i < 4; ++i) {
-            ra[P][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kq);
             if constexpr (TRANS_B) {
                 rb[P][i] = *reinterpret_cast<const u32x4 *>(b_src[i] + kq);
             } else {
@@ -516,9 +523,10 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
         constexpr int P = decltype(set)::value;
         const bool k_in = k0 + pk < k;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4 *>(&As[buf][(pr + 32 * i) * HP + pk]) = k_in ? ra[P][i] : zero4;
-            if constexpr (TRANS_B) *reinterpret_cast<u32x4 *>(&Bs[buf][(pr + 32 * i) * HP + pk]) = k_in ? rb[P][i] : zero4;
+        for (int i = 0; i < AI; ++i) *reinterpret_cast<u32x4 *>(&As[buf][(pr + 32 * i) * HP + pk]) = k_in ? ra[P][i] : zero4;
+        if constexpr (TRANS_B) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4 *>(&Bs[buf][(pr + 32 * i) * HP + pk]) = k_in ? rb[P][i] : zero4;
         }
         if constexpr (!TRANS_B) {
             // the two k-rows of a lane's eight columns as one 32-bit word per column.  The eight 16-byte pieces of a
@@ -540,9 +548,9 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
         }
     };
 
-    f16v acc[2][2];
+    f16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -550,42 +558,55 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
 
     const uint32_t l32 = lane & 31, kh = lane >> 5;
     const uint32_t tiles = (k + HK - 1) / HK;
-    auto step = [&](auto set, uint32_t t) {
+    // Step t: (barrier) request tile t + 3 into the registers tile t has left, write tile t + 1 into the buffer
+    // tile t - 1 was read from, multiply tile t.  The barrier says both that tile t is complete in its buffer and
+    // that everybody has finished reading tile t - 1; the LDS writes ride along with the products instead of
+    // standing between two of them.
+    auto step = [&](auto set_free, auto set_next, uint32_t t) {
         const int buf = t & 1;
-        stash(set, buf, t * HK);
-        __syncthreads();  // the tile is complete; the other buffer's readers of two tiles ago have passed this point
-        fetch(set, (t + HF) * HK);
+        __syncthreads();
+        fetch(set_free, (t + HF) * HK);
+        stash(set_next, buf ^ 1, (t + 1) * HK);
 #pragma unroll
         for (int ks = 0; ks < HK / 16; ++ks) {
-            u32x4 fa[2], fb[2];
+            u32x4 fa[MI], fb[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const u32x4 *>(&As[buf][(wm * 64 + 32 * i + l32) * HP + 16 * ks + 8 * kh]);
+            for (int i = 0; i < MI; ++i) fa[i] = *reinterpret_cast<const u32x4 *>(&As[buf][(wm * (TM / 2) + 32 * i + l32) * HP + 16 * ks + 8 * kh]);
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const uint32_t piece = TRANS_B ? 2 * ks + kh : (2 * ks + kh) ^ ((4 * wn + 2 * j + (l32 >> 4)) & 7);
                 fb[j] = *reinterpret_cast<const u32x4 *>(&Bs[buf][(wn * 64 + 32 * j + l32) * HP + 8 * piece]);
             }
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
         }
     };
-    fetch(std::integral_constant<int, 0>{}, 0);
-    fetch(std::integral_constant<int, 1>{}, HK);
-    for (uint32_t t = 0; t < tiles; t += HF) {  // no branch inside: an odd count's last step multiplies zeros
-        step(std::integral_constant<int, 0>{}, t);
-        step(std::integral_constant<int, 1>{}, t + 1);
+    const std::integral_constant<int, 0> s0;
+    const std::integral_constant<int, 1> s1;
+    const std::integral_constant<int, 2> s2;
+    fetch(s0, 0);
+    fetch(s1, HK);
+    fetch(s2, 2 * HK);
+    stash(s0, 0, 0);
+    uint32_t t = 0;
+    for (; t + HF <= tiles; t += HF) {  // no branch inside: the waits count the loads of the later tiles exactly
+        step(s0, s1, t);
+        step(s1, s2, t + 1);
+        step(s2, s0, t + 2);
     }
+    if (t < tiles) step(s0, s1, t);
+    if (t + 1 < tiles) step(s1, s2, t + 1);
     // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
     const T *C = static_cast<const T *>(bias.ptr);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const uint32_t row = row0 + wm * 64 + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
+                const uint32_t row = row0 + wm * (TM / 2) + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
                 const uint32_t col = col0 + wn * 64 + 32 * j + l32;
                 if (row < m && col < n) {
                     float v = alpha * acc[i][j][e];
@@ -1454,12 +1475,20 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 
     auto launch_tiles16 = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
-            const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + HT - 1) / HT), count);
+            // tiles of 64 rows while those of 128 would leave half of the CUs without one
+            const bool half = ((m + HT - 1) / HT) * ((n + HT - 1) / HT) * count <= kHalfTiles;
+            const size_t tm = half ? HT / 2 : HT;
+            const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + tm - 1) / tm), count);
             if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
             const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
-            if (trans_b) mm_tiles16<T, true, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
-            else if (n % 8 == 0 && n >= 8 && aligned16(b)) mm_tiles16<T, false, true><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
-            else mm_tiles16<T, false, false><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0);
+            const bool vec = n % 8 == 0 && n >= 8 && aligned16(b);
+#define RG_TILES16(TB, VEC)                                                                                              \
+    (half ? mm_tiles16<T, TB, VEC, HT / 2><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0)      \
+          : mm_tiles16<T, TB, VEC, HT><<<grid, 256, 0, s>>>(y, a, b, bias, m32, k32, n32, al, be, am0, bm0, ym0))
+            if (trans_b) RG_TILES16(true, true);
+            else if (vec) RG_TILES16(false, true);
+            else RG_TILES16(false, false);
+#undef RG_TILES16
             return launch_status();
         } else {
             return RG_HIP_E_UNSUPPORTED;
