@@ -467,7 +467,7 @@ constexpr size_t kSkinnyPassesSmall = 12000, kRowsKnPassesSmall = 10500;
 
 // TM: rows of a tile, 128 or 64 (a wavefront then has 32 rows of 64 columns: twice the workgroups for few tiles)
 template <class T, bool TRANS_B, bool B_VEC, int TM>  // B_VEC: rows of B as [k, n] start on 16-byte boundaries, n >= 8
-__global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
+__global__ __launch_bounds__(256, 2) void mm_tiles16(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
                                                   uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
                                                   uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
     constexpr int MI = TM / 64, AI = TM / 32;  // row blocks of a wavefront, loads of A per thread and tile
@@ -519,9 +519,12 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
             }
         }
     };
-    auto stash = [&](auto set, int buf, uint32_t k0) {
+    // (the tile that reaches beyond k takes a branch of its own: selects in the common path were scheduled ahead of
+    // the barrier before them, where they waited for loads a step early)
+    auto stash_part = [&](auto set, auto whole, int buf, uint32_t k0) {
         constexpr int P = decltype(set)::value;
-        const bool k_in = k0 + pk < k;
+        constexpr bool WHOLE = decltype(whole)::value;
+        const bool k_in = WHOLE || k0 + pk < k;
 #pragma unroll
         for (int i = 0; i < AI; ++i) *reinterpret_cast<u32x4 *>(&As[buf][(pr + 32 * i) * HP + pk]) = k_in ? ra[P][i] : zero4;
         if constexpr (TRANS_B) {
@@ -534,18 +537,22 @@ __global__ __launch_bounds__(256) void mm_tiles16(T *__restrict__ y, const T *__
             // a wavefront then fall into 64 different LDS banks
 #pragma unroll
             for (int ii = 0; ii < 2; ++ii) {
-                const uint32_t kr = k0 + 2 * bk + 32 * ii;  // (k is even: both rows of the pair are in or out)
+                const bool rows_in = WHOLE || k0 + 2 * bk + 32 * ii < k;  // (k is even: both rows of the pair are in or out)
                 const uint32_t word = (bk + 16 * ii) ^ (((tid >> 1) & 7) << 2);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t col = 8 * (tid & 15) + 2 * j;
                     const uint32_t even = __builtin_amdgcn_perm(rb[P][2 * ii + 1][j], rb[P][2 * ii][j], 0x05040100u);
                     const uint32_t odd = __builtin_amdgcn_perm(rb[P][2 * ii + 1][j], rb[P][2 * ii][j], 0x07060302u);
-                    *reinterpret_cast<uint32_t *>(&Bs[buf][col * HP + 2 * word]) = kr < k ? even : 0u;
-                    *reinterpret_cast<uint32_t *>(&Bs[buf][(col + 1) * HP + 2 * word]) = kr < k ? odd : 0u;
+                    *reinterpret_cast<uint32_t *>(&Bs[buf][col * HP + 2 * word]) = rows_in ? even : 0u;
+                    *reinterpret_cast<uint32_t *>(&Bs[buf][(col + 1) * HP + 2 * word]) = rows_in ? odd : 0u;
                 }
             }
         }
+    };
+    auto stash = [&](auto set, int buf, uint32_t k0) {
+        if (k0 + HK <= k) stash_part(set, std::true_type{}, buf, k0);
+        else stash_part(set, std::false_type{}, buf, k0);
     };
 
     f16v acc[MI][2];
