@@ -138,7 +138,7 @@ template <int A_MODE, bool B_ZP, bool SHORT_M>
 __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, uint8_t *lds1,
                                               const uint8_t *A, const uint8_t *B, uint32_t k, uint32_t lda, uint32_t n,
                                               uint32_t a_xor, const uint32_t (&za_f)[4], ZeroPoint zb,
-                                              uint64_t zb_row0, uint32_t a_rows) {
+                                              uint64_t zb_row0, uint32_t a_rows, uint8_t *zlds) {
     // k: length of the range of k walked here (A, B and zb_row0 point at its start); lda: bytes per row of A
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -211,14 +211,38 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
             else f[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(f[e]), za_f[i]));
         }
     };
-    auto fix_b = [&](v4i &f, uint32_t k0, int ks) {
+    // B's zero points (one per k-row) of the sixteen k of a fragment, held in registers a k-step ahead like the
+    // fragments.  No global load may stand in the loop: its wait would be a wait for every copy in flight (the
+    // counter is shared), which doubled the time of a launch.  A scalar zero point is read once; per-row ones
+    // travel with their tile, one more copy per wavefront and tile (128 bytes into a slot of the wavefront's own),
+    // when their address is a multiple of 4; otherwise they are loaded from memory as before.
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int z_mode = !B_ZP ? 1 : !zb.per_row ? 1 : (reinterpret_cast<uintptr_t>(zb.ptr) & 3u) == 0 ? 2 : 0;
+    const uint32_t z_lds = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t *)zlds));
+    u32x4 zr[2];
+    if (B_ZP && !zb.per_row) {
+        const uint32_t z = splat(zb.ptr[0]);
+        zr[0] = zr[1] = u32x4{z, z, z, z};
+    } else {
+        zr[0] = zr[1] = u32x4{0u, 0u, 0u, 0u};
+    }
+    auto copy_z = [&](int stage, uint32_t k0) {  // 128 zero points of the k-rows k0 .. k0 + 127 into this wavefront's slot
+        const uint8_t *src = scalar_pointer(zb.ptr + zb_row0 + k0);
+        const uint32_t dst = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(z_lds + (stage * 4 + wave) * 256));
+        const uint32_t lane_off = 4 * (lane & 31);  // (the upper half of the wavefront fetches the same bytes again)
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                     :
+                     : "v"(lane_off), "s"(src), "s"(dst)
+                     : "memory", "m0");
+    };
+    auto read_z = [&](int stage, uint32_t k0, int ks, u32x4 &z) {
         if constexpr (B_ZP) {
-            uint32_t z[4];
-            if (zb.per_row) {
-                __builtin_memcpy(z, zb.ptr + zb_row0 + k0 + 16 * (2 * ks + h), 16);
-            } else {
-                z[0] = z[1] = z[2] = z[3] = splat(zb.ptr[0]);
-            }
+            if (z_mode == 2) z = *reinterpret_cast<const u32x4 *>(zlds + (stage * 4 + wave) * 256 + 16 * (2 * ks + h));
+            else if (z_mode == 0) __builtin_memcpy(&z, zb.ptr + zb_row0 + k0 + 16 * (2 * ks + h), 16);
+        }
+    };
+    auto fix_b = [&](v4i &f, const u32x4 &z) {
+        if constexpr (B_ZP) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) f[e] = static_cast<int>(sub_bytes(static_cast<uint32_t>(f[e]), z[e]));
         }
@@ -228,10 +252,17 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
     v4i fa[2][4], fb[2][4];
 #pragma unroll
     for (int q = 0; q < 16; ++q) copy(lds0, 0, q);
+    if (z_mode == 2) copy_z(0, 0);
 #pragma unroll
     for (int q = 0; q < 16; ++q) copy(lds1, k_tiles > 1 ? BK : 0, q);  // k_tiles == 1: tile 0 again, never multiplied
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 (the 16 older copies)
+    if (z_mode == 2) {
+        copy_z(1, k_tiles > 1 ? BK : 0);
+        asm volatile("s_waitcnt vmcnt(17)" ::: "memory");  // tile 0 (the 17 older copies)
+    } else {
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 (the 16 older copies)
+    }
     __syncthreads();
+    read_z(0, 0, 0, zr[0]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) fa[0][i] = read_a(lds0, 0, i);
 #pragma unroll
@@ -253,13 +284,17 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
                 __syncthreads();                                  // tile kt+1 complete, RB no longer read
             }
             if constexpr (o % 4 == 0) fix_a(fa[cur][row], row);
-            if constexpr (row == 0) fix_b(fb[cur][col], kt_ * BK, ks);
+            if constexpr (row == 0) fix_b(fb[cur][col], zr[cur]);
             acc[row][col] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[cur][row], fb[cur][col], acc[row][col], 0, 0, 0);
             const uint8_t *src = ks == 3 ? WB : RB;
             constexpr int nks = (ks + 1) % 4;
             if constexpr (o < 4) fa[nxt][o] = read_a(src, nks, o);
             else if constexpr (o < 12) read_b(src, nks, (o - 4) / 2, (o - 4) % 2, fb[nxt][(o - 4) / 2]);
+            else if constexpr (o == 12) read_z(src == lds0 ? 0 : 1, (ks == 3 ? kt_ + 1 : kt_) * BK, nks, zr[nxt]);
             if constexpr (s >= 48) copy(RB, k_cp, s - 48);
+            if constexpr (s == 63 && B_ZP) {
+                if (z_mode == 2) copy_z(RB == lds0 ? 0 : 1, k_cp);
+            }
             __builtin_amdgcn_sched_barrier(0);
         };
         [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) {
@@ -286,6 +321,7 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     static_assert(!(DEQ && SPLIT), "partial sums cannot be dequantised");
     __shared__ __align__(1024) uint8_t lds0[D_STAGE];
     __shared__ __align__(1024) uint8_t lds1[D_STAGE];
+    __shared__ __align__(256) uint8_t zlds[2 * 4 * 256];  // B's zero points of a tile: a slot per buffer and wavefront
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t bz = blockIdx.z;
@@ -353,11 +389,11 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     const uint64_t zb_row0 = bm * k + k_begin;
 
     if (a_simple) {
-        if (!b_zp) mmi_tile_loop<0, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
-        else mmi_tile_loop<0, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
+        if (!b_zp) mmi_tile_loop<0, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
+        else mmi_tile_loop<0, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
     } else {
-        if (!b_zp) mmi_tile_loop<1, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
-        else mmi_tile_loop<1, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m);
+        if (!b_zp) mmi_tile_loop<1, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
+        else mmi_tile_loop<1, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
     }
 
     int32_t *Y = y + (ym * m + row0 + wm * 128) * n + col0 + wn * 128;
@@ -428,7 +464,7 @@ constexpr uint64_t kSkinnyWorkgroups = 256;  // per launch: one per CU (512 and 
 constexpr int GT = 128, GK = 128, GP = 144;
 
 template <bool DEQ, bool B_VEC>  // B_VEC: rows of B start on 16-byte boundaries, n >= 16
-__global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+__global__ __launch_bounds__(256, 2) void mmi_tiles(int32_t *__restrict__ y, const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
                                                  ZeroPoint za, ZeroPoint zb, Dequant dq, uint32_t m, uint32_t k, uint32_t n,
                                                  uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
     __shared__ __align__(16) uint8_t As[2][GT * GP];
@@ -454,8 +490,12 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
     const uint32_t bq = tid >> 3, bc = col0 + 16 * (tid & 7);
     const uint32_t bc_load = bc + 16 <= n ? bc : (n >= 16 ? n - 16 : 0);  // (vector loads only)
     const uint8_t *b_last = reinterpret_cast<const uint8_t *>((reinterpret_cast<uint64_t>(B) + static_cast<uint64_t>(k) * n - 1) & ~3ull);
+    // B's zero points are loaded with the tiles, without a branch (a load under a branch makes the wait for one tile
+    // a wait for all): without zero points the loads read some byte of B and are masked away
+    const uint8_t *zb_base = zb.ptr ? zb.ptr + (zb.per_row ? bm * k : 0) : B;
+    const uint32_t zb_step = zb.ptr && zb.per_row ? 1u : 0u, zb_keep = zb.ptr ? 0xffffffffu : 0u;
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    u32x4 ra[2][4], rb[2][4];  // two tiles in flight
+    u32x4 ra[2][4], rb[2][4];  // two tiles in flight (a third set of registers spills)
     uint32_t b_zero[2][4];
     auto fetch = [&](auto set, uint32_t k0) {
         constexpr int P = decltype(set)::value;
@@ -465,7 +505,7 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
             ra[P][i] = *reinterpret_cast<const u32x4 *>(a_src[i] + kq);
             const uint32_t kr0 = k0 + 4 * bq + i, kr = kr0 < k ? kr0 : k - 1;
             const uint8_t *src = B + static_cast<uint64_t>(kr) * n;
-            b_zero[P][i] = splat(zp_byte(zb, bm * k + kr));
+            b_zero[P][i] = splat(zb_base[static_cast<uint64_t>(kr) * zb_step]) & zb_keep;
             if constexpr (B_VEC) {
                 rb[P][i] = *reinterpret_cast<const u32x4 *>(src + bc_load);
             } else {
@@ -473,9 +513,12 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
             }
         }
     };
-    auto stash = [&](auto set, int buf, uint32_t k0) {
+    // (the tile that reaches beyond k takes a branch of its own: selects in the common path get scheduled ahead of
+    // the barrier before them, where they wait for loads a step early)
+    auto stash_part = [&](auto set, auto whole, int buf, uint32_t k0) {
         constexpr int P = decltype(set)::value;
-        const bool k_in = k0 + pk < k;
+        constexpr bool WHOLE = decltype(whole)::value;
+        const bool k_in = WHOLE || k0 + pk < k;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             u32x4 v;
@@ -486,7 +529,7 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
         // four k-rows of sixteen columns -> per column one word of four consecutive k.  The eight 16-byte pieces
         // of a column's k are kept in an order that depends on the column (piece ^ (column / 16) % 8), which
         // spreads the eight column groups of a wavefront over the LDS banks
-        const bool rows_in = k0 + 4 * bq < k;  // (k is a multiple of 4: all four rows are in or out)
+        const bool rows_in = WHOLE || k0 + 4 * bq < k;  // (k is a multiple of 4: all four rows are in or out)
         const uint32_t word = bq ^ ((tid & 7) << 2);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -504,6 +547,10 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
             }
         }
     };
+    auto stash = [&](auto set, int buf, uint32_t k0) {
+        if (k0 + GK <= k) stash_part(set, std::true_type{}, buf, k0);
+        else stash_part(set, std::false_type{}, buf, k0);
+    };
 
     v16i acc[2][2];
 #pragma unroll
@@ -515,11 +562,14 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
 
     const uint32_t l32 = lane & 31, kh = lane >> 5;
     const uint32_t tiles = (k + GK - 1) / GK;
-    auto step = [&](auto set, uint32_t t) {
+    // Step t: (barrier) request tile t + 2 into the registers tile t has left, write tile t + 1 into the buffer
+    // tile t - 1 was read from, multiply tile t.  The barrier says both that tile t is complete in its buffer and
+    // that everybody has finished reading tile t - 1.
+    auto step = [&](auto set_free, auto set_next, uint32_t t) {
         const int buf = t & 1;
-        stash(set, buf, t * GK);
-        __syncthreads();  // the tile is complete; the other buffer's readers of two tiles ago have passed this point
-        fetch(set, (t + 2) * GK);
+        __syncthreads();
+        fetch(set_free, (t + 2) * GK);
+        stash(set_next, buf ^ 1, (t + 1) * GK);
 #pragma unroll
         for (int ks = 0; ks < GK / 32; ++ks) {
             v4i fa[2], fb[2];
@@ -536,12 +586,17 @@ __global__ __launch_bounds__(256) void mmi_tiles(int32_t *__restrict__ y, const 
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
     };
-    fetch(std::integral_constant<int, 0>{}, 0);
-    fetch(std::integral_constant<int, 1>{}, GK);
-    for (uint32_t t = 0; t < tiles; t += 2) {  // no branch inside: an odd count's last step multiplies zeros
-        step(std::integral_constant<int, 0>{}, t);
-        step(std::integral_constant<int, 1>{}, t + 1);
+    const std::integral_constant<int, 0> s0;
+    const std::integral_constant<int, 1> s1;
+    fetch(s0, 0);
+    fetch(s1, GK);
+    stash(s0, 0, 0);
+    uint32_t t = 0;
+    for (; t + 2 <= tiles; t += 2) {  // no branch inside: the waits count the loads of the later tile exactly
+        step(s0, s1, t);
+        step(s1, s0, t + 1);
     }
+    if (t < tiles) step(s0, s1, t);
     // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
 #pragma unroll
     for (int j = 0; j < 2; ++j) {

@@ -370,7 +370,7 @@ def test_matmul_integer_bit_exact_config_zero_points(m, k, n):
     assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
 
 
-@pytest.mark.parametrize("m,k,n", [(20, 33, 17), (256, 128, 256), (256, 384, 512)])
+@pytest.mark.parametrize("m,k,n", [(20, 33, 17), (256, 128, 256), (256, 384, 512), (512, 1024, 256), (200, 512, 512)])
 def test_matmul_integer_zero_point_variants_and_broadcast(m, k, n):
     rng = np.random.default_rng(6)
     a = rng.integers(0, 256, (2, 1, m, k), dtype=np.uint8)
@@ -385,6 +385,13 @@ def test_matmul_integer_zero_point_variants_and_broadcast(m, k, n):
         y = host(ops.matmul_integer(dev(a), dev(b), None if az is None else dev(az), None if bz is None else dev(bz)))
         assert y.shape == (2, 3, m, n)
         assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
+    # B's per-row zero points from an address that is no multiple of 4 (the tile kernel then loads them from memory
+    # instead of copying them along with the tiles)
+    az, bz = rng.integers(0, 256, (2 * m,), dtype=np.uint8), rng.integers(-128, 128, (3 * k,), dtype=np.int8)
+    bz_odd = dev(np.concatenate([np.zeros(1, np.int8), bz]))[1:]
+    assert bz_odd.data_ptr() % 4 != 0
+    y = host(ops.matmul_integer(dev(a), dev(b), dev(az), bz_odd))
+    assert np.array_equal(y, oracle.matmul_integer(a, b, az, bz, threads=8))
     # equal batch shapes: the strided (grid.z) path
     a2 = rng.integers(0, 256, (3, m, k), dtype=np.uint8)
     b2 = rng.integers(-128, 128, (3, k, n), dtype=np.int8)
