@@ -902,6 +902,24 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     if (batch == 0 || m == 0 || n == 0) return 0;
     if (m > 0x7fffffffu || n > 0x7fffffffu || k > 0x7fffffffu || batch > 0xffffffffu)
         return RG_HIP_E_UNSUPPORTED;
+    // One B for consecutive matrices of A (activations [batch, m, k] against weights): the batch is more rows of one
+    // product, not `batch` launches that each read B again.  The zero points per (matrix, row) follow: A's are
+    // consecutive like its rows, B's are those of the one matrix.
+    if (batch > 1 && b_index && batch * m <= 0x7fffffffu) {
+        bool fold = true;
+        for (size_t i = 0; i < batch && fold; ++i)
+            fold = b_index[i] == b_index[0] && (a_index ? a_index[i] == a_index[0] + i : true);
+        if (fold) {
+            const size_t a0 = a_index ? a_index[0] : 0, b0 = b_index[0];
+            a = static_cast<const uint8_t *>(a) + a0 * m * k;
+            b = static_cast<const uint8_t *>(b) + b0 * k * n;
+            if (a_zp && !(flags & RG_MMI_A_ZP_SCALAR)) a_zp = static_cast<const uint8_t *>(a_zp) + a0 * m;
+            if (b_zp && !(flags & RG_MMI_B_ZP_SCALAR)) b_zp = static_cast<const uint8_t *>(b_zp) + b0 * k;
+            m *= batch;
+            batch = 1;
+            a_index = b_index = nullptr;
+        }
+    }
     hipStream_t s = as_stream(stream);
     const ZeroPoint za{static_cast<const uint8_t *>(a_zp), (flags & RG_MMI_A_ZP_SCALAR) ? 0u : 1u};
     const ZeroPoint zb{static_cast<const uint8_t *>(b_zp), (flags & RG_MMI_B_ZP_SCALAR) ? 0u : 1u};

@@ -1230,6 +1230,39 @@ def test_matmul_any_shape_exact_on_small_integers():
     assert np.array_equal(host(ops.matmul(dev(a).half(), dev(np.ascontiguousarray(b.T)).half(), trans_b=True).float()), want)
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 256, 512), (16, 128, 256), (100, 64, 264), (300, 192, 512)])
+def test_matmul_one_b_for_the_whole_batch(m, k, n):
+    # activations [batch, m, k] against one weight matrix: the C ABI turns the batch into rows of one product; every
+    # bias form the reference expands (per column, per output element, and one [m, n] for all, which keeps the
+    # per-matrix launches), a batch whose A matrices are not consecutive, and MatMulInteger with zero points per row
+    rng = np.random.default_rng(51)
+    B = 5
+    a = rng.integers(-2, 3, (B, m, k)).astype(np.float32)
+    b = rng.integers(-2, 3, (1, k, n)).astype(np.float32)
+    want = (a.astype(np.int64) @ b[0].astype(np.int64)).astype(np.float32)
+    assert np.max(np.abs(want)) < 1024
+    for bias in (None, rng.integers(-3, 4, (n,)).astype(np.float32), rng.integers(-3, 4, (B, m, n)).astype(np.float32),
+                 rng.integers(-3, 4, (m, n)).astype(np.float32)):
+        got = host(ops.matmul(dev(a).half(), dev(b).half(), None if bias is None else dev(bias).half()).float())
+        assert np.array_equal(got, want if bias is None else want + bias), None if bias is None else bias.shape
+        bt = dev(np.ascontiguousarray(np.swapaxes(b, -1, -2))).half()
+        got = host(ops.matmul(dev(a).half(), bt, None if bias is None else dev(bias).half(), trans_b=True).float())
+        assert np.array_equal(got, want if bias is None else want + bias)
+    # A broadcast as well ([2, 1, m, k] against [1, 3, k, n]: B differs within the batch, nothing to fold)
+    a4 = rng.integers(-2, 3, (2, 1, m, k)).astype(np.float32)
+    b4 = rng.integers(-2, 3, (1, 3, k, n)).astype(np.float32)
+    got = host(ops.matmul(dev(a4).half(), dev(b4).half()).float())
+    assert np.array_equal(got, (a4.astype(np.int64) @ b4.astype(np.int64)).astype(np.float32))
+    ai = rng.integers(0, 256, (B, m, k), dtype=np.uint8)
+    bi = rng.integers(-128, 128, (1, k, n), dtype=np.int8)
+    az, bz = rng.integers(0, 256, (B * m,), dtype=np.uint8), rng.integers(-128, 128, (k,), dtype=np.int8)
+    ref = oracle.matmul_integer(ai, bi, az, bz, threads=8)
+    assert np.array_equal(host(ops.matmul_integer(dev(ai), dev(bi), dev(az), dev(bz))), ref)
+    scale = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    y = host(ops.matmul_integer(dev(ai), dev(bi), dev(az), dev(bz), dequant_scale=dev(scale)))
+    assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
