@@ -409,19 +409,38 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
     uint8_t *stage = (wave & 2 ? lds1 : lds0) + (wave & 1) * 32768;
     const bool odd = lane & 1;
     const uint32_t col_pair = (lane & 31) & ~1u;  // first of the two columns this lane writes
+    // a bias per column (the usual one of a linear layer) is the same for every row: four loads per lane instead
+    // of one per output (4096^3: 133 -> 118 us)
+    const bool column_bias = C && bias.sm == 0;
+    float cb[4] = {0.f, 0.f, 0.f, 0.f};
+    if (column_bias) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cb[j] = beta * up(C[ym * bias.sb + (col0 + j * 32 + (lane & 31)) * bias.sn]);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j) {
+            // any other bias: the sixteen values of a block are requested together, ahead of their use (one at a
+            // time each addition waited for its own load: 4096^3 with a bias per output 160 us)
+            T bv[16];
+            const bool other_bias = C && !column_bias;
+            if (other_bias) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    uint32_t row = row0 + i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + e % 4;
+                    if (SHORT_M && row >= m) row = m - 1;
+                    bv[e] = C[ym * bias.sb + row * bias.sm + (col0 + j * 32 + (lane & 31)) * bias.sn];
+                }
+            }
 #pragma unroll
             for (int eg = 0; eg < 4; ++eg) {
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const uint32_t row = i * 32 + 8 * eg + 4 * (lane >> 5) + e, col = j * 32 + (lane & 31);
                     v[e] = alpha * acc[i][j][4 * eg + e];
-                    if (C && (!SHORT_M || row0 + row < m))
-                        v[e] += beta * up(C[ym * bias.sb + (row0 + row) * bias.sm + (col0 + col) * bias.sn]);
+                    if (column_bias) v[e] += cb[j];
+                    else if (other_bias) v[e] += beta * up(bv[4 * eg + e]);
                 }
                 // even lanes keep rows 0 and 1, odd lanes rows 2 and 3 of the group of four
                 const float give0 = odd ? v[0] : v[2], give1 = odd ? v[1] : v[3];
@@ -438,6 +457,7 @@ __global__ __launch_bounds__(256, 1) void mm_mfma_256x256(T *__restrict__ y, con
                 put(r_first, lo0, hi0);
                 put(r_first + 1, lo1, hi1);
             }
+        }
     // (each wavefront reads back only what it wrote itself: no barrier)
     T *Y = y + (ym * m + row0) * n + col0;
 #pragma unroll
@@ -607,18 +627,51 @@ __global__ __launch_bounds__(256, 2) void mm_tiles16(T *__restrict__ y, const T 
     if (t + 1 < tiles) step(s1, s2, t + 1);
     // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 (lane / 32) + e % 4
     const T *C = static_cast<const T *>(bias.ptr);
+    // (a bias per column is the same for every row: one load per column block instead of one per output)
+    const bool column_bias = C && bias.sm == 0;
+    float cb[2] = {0.f, 0.f};
+    if (column_bias) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t col = col0 + wn * 64 + 32 * j + l32;
+            cb[j] = beta * up(C[ym * bias.sb + (col < n ? col : n - 1) * bias.sn]);
+        }
+    }
+    // with an even n (and Y on a 4-byte boundary) neighbouring lanes exchange two of their four rows, so that a lane
+    // stores two adjacent columns of two rows with 32-bit stores; otherwise element by element
+    const bool pairs = n % 2 == 0 && (reinterpret_cast<uintptr_t>(y) & 3u) == 0;
+    const bool odd = lane & 1;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const uint32_t row = row0 + wm * (TM / 2) + 32 * i + 8 * (e / 4) + 4 * kh + (e % 4);
+            for (int eg = 0; eg < 4; ++eg) {
+                const uint32_t row_eg = row0 + wm * (TM / 2) + 32 * i + 8 * eg + 4 * kh;
                 const uint32_t col = col0 + wn * 64 + 32 * j + l32;
-                if (row < m && col < n) {
-                    float v = alpha * acc[i][j][e];
-                    if (C) v += beta * up(C[ym * bias.sb + row * bias.sm + col * bias.sn]);
-                    y[(ym * m + row) * n + col] = down<T>(v);
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = alpha * acc[i][j][4 * eg + e];
+                    if (column_bias) v[e] += cb[j];
+                    else if (C && row_eg + e < m && col < n) v[e] += beta * up(C[ym * bias.sb + (row_eg + e) * bias.sm + col * bias.sn]);
+                }
+                if (pairs) {
+                    // even lanes keep rows 0 and 1, odd lanes rows 2 and 3 of the group of four
+                    const float give0 = odd ? v[0] : v[2], give1 = odd ? v[1] : v[3];
+                    const float got0 = __shfl_xor(give0, 1, kWave), got1 = __shfl_xor(give1, 1, kWave);
+                    const float lo0 = odd ? got0 : v[0], hi0 = odd ? v[2] : got0;
+                    const float lo1 = odd ? got1 : v[1], hi1 = odd ? v[3] : got1;
+                    const uint32_t row = row_eg + (odd ? 2 : 0), col_pair = col & ~1u;
+                    if (col_pair < n) {  // (n is even: both columns are in or out)
+                        const T p0[2] = {down<T>(lo0), down<T>(hi0)}, p1[2] = {down<T>(lo1), down<T>(hi1)};
+                        if (row < m) *reinterpret_cast<uint32_t *>(y + (ym * m + row) * n + col_pair) = __builtin_bit_cast(uint32_t, p0);
+                        if (row + 1 < m) *reinterpret_cast<uint32_t *>(y + (ym * m + row + 1) * n + col_pair) = __builtin_bit_cast(uint32_t, p1);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (row_eg + e < m && col < n) y[(ym * m + row_eg + e) * n + col] = down<T>(v[e]);
                 }
             }
 }
