@@ -264,7 +264,8 @@ int rg_hip_matmul_integer_dequantize(float *y, const void *a, const void *b, con
  *   history shortened accordingly); nothing is ever read or written outside the caches.
  * k_cache == v_cache == NULL: no cache (past = 0, attends k/v directly).  past_lens == NULL: 0.
  * n_head % n_kv_head == 0; D in {64, 80, 96, 128}; dtype FP16 or BF16; fp32 softmax / accumulation.
- * workspace: rg_hip_attention_kvcache_workspace() bytes (split-KV partials), contents irrelevant.
+ * workspace: rg_hip_attention_kvcache_workspace() bytes (partial results of key ranges, of either
+ *   kernel: up to 35 MiB at D = 128), contents irrelevant.
  * sync_state: NULL, or rg_hip_attention_kvcache_state_bytes() bytes of device memory that the
  *   caller zeroed once and keeps for this purpose (a runtime::Resource of the stream, like the
  *   reference's library handles, src/04kernel/src/utilities/cuda/cublas_context.cu:18-31); the
@@ -293,7 +294,8 @@ int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *
  * every call (not a memset, so the call can be captured).  Limits: those of
  * rg_hip_attention_kvcache (D in {64, 128}; a larger D is refused with RG_HIP_E_WORKSPACE, the
  * partial slots being sized for D <= 128); the launch uses at most 512 workgroups, which is what
- * the array holds partials for.  All calls on one GPU share the array: calls that overlap on one
+ * the array holds partials for (the tiled kernel shares an item's keys between workgroups only
+ * as far as 2 MiB of records reach).  All calls on one GPU share the array: calls that overlap on one
  * GPU (two streams, two threads) race and must be serialised by the caller.  Same kernels as
  * rg_hip_attention_kvcache: the caches come out bit-identical, the output within the rounding of
  * the summation order (which work a wavefront pulls is decided at run time in either entry). */

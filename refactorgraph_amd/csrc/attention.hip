@@ -857,7 +857,7 @@ constexpr uint32_t kMaxWorkgroups = 4096;  // bound used by the workspace query
 // h = 4000: 4 rows 109 us tiled against 318 us split, 2 rows 108 against 159; at N = 1: 4 rows 84 against 20.
 constexpr size_t kPrefillAlways = 32;  // query rows from which the tiled kernel is used whatever the batch
 
-bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq) {
+bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq, size_t cap, size_t D, bool ranges_fit) {
     if (seq >= kPrefillAlways) return true;
     const size_t group = n_head / n_kv_head, heads_per_item = group == 1 ? 1 : group == 2 ? 2 : 4;
     // the split kernel takes at most four heads of a group per launch and reads K/V again in every launch
@@ -867,6 +867,15 @@ bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq) {
     if (seq < 2 && split_launches < 2) return false;
     const size_t rows_per_item = 32 * (4 / heads_per_item);
     const size_t items = N * n_kv_head * ((group + heads_per_item - 1) / heads_per_item) * ((seq + rows_per_item - 1) / rows_per_item);
+    // Few items: the tiled kernel shares an item's keys between workgroups (head dims 64 and 128, records in the
+    // workspace), and then costs about 17.5 us + 9.4e-5 us per kv head and key, against 8 us + 7.3e-5 us per
+    // kv head, key and query row on the split kernel (N = 1, 8 kv heads, 8 new rows: history 1000 13.9 us split
+    // against 18.1 tiled, 4000 26.1 against 22.7, 32768 154 against 46).  The history is device data: half of the
+    // capacity stands for it.
+    if (ranges_fit && seq >= 2 && items * 2 <= 512 && cap >= 1024 && (D == 64 || D == 128)) {
+        const double keys = static_cast<double>(N * n_kv_head) * static_cast<double>(cap) / 2;
+        return 9.5 < keys * (7.3e-5 * static_cast<double>(seq * split_launches) - 9.4e-5);
+    }
     const size_t rounds = (items + 511) / 512;
     return N * n_kv_head * seq * split_launches >= 280 * rounds;
 }
@@ -909,7 +918,10 @@ constexpr size_t kCounterBytes = kMaxWorkgroups * sizeof(uint32_t);
 size_t workspace_bytes(size_t D) {
     // ticket counters (used when the caller passes no persistent ones), then two partial slots
     // per workgroup sized for the widest head group (4)
-    return kCounterBytes + static_cast<size_t>(kMaxWorkgroups) * 2 * 4 * (D + 2) * sizeof(float);
+    // (the tiled kernel's records of key ranges use the same area, never in the same call)
+    const size_t split = static_cast<size_t>(kMaxWorkgroups) * 2 * 4 * (D + 2) * sizeof(float);
+    const size_t tiled = prefill_part_bytes(static_cast<uint32_t>(D));
+    return kCounterBytes + (split > tiled ? split : tiled);
 }
 
 // ---------------------------------------------------------------- library-owned scratch
@@ -951,8 +963,8 @@ int static_scratch(void **out) {
 // zero on entry unless `clear_counters` asks for the clearing launch.
 int attention_call(void *o, const void *q, const void *k, const void *v, void *k_cache, void *v_cache,
                    const int64_t *past_lens, int past_per_row, size_t N, size_t n_head, size_t n_kv_head,
-                   size_t seq, size_t cap, size_t D, float scale, int dtype, float *part, uint32_t *counters,
-                   uint32_t max_workgroups, bool clear_counters, hipStream_t s) {
+                   size_t seq, size_t cap, size_t D, float scale, int dtype, float *part, size_t part_bytes,
+                   uint32_t *counters, uint32_t max_workgroups, bool clear_counters, hipStream_t s) {
     if (!o || !q || !k || !v) return RG_HIP_E_ARGUMENT;
     if ((k_cache == nullptr) != (v_cache == nullptr)) return RG_HIP_E_ARGUMENT;
     if (N == 0 || n_head == 0 || seq == 0) return 0;
@@ -971,7 +983,7 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
 
     // many query rows per batch row: the tiled MFMA kernel (K/V staged once per query tile)
     if (prefill_supported(static_cast<uint32_t>(n_head), static_cast<uint32_t>(n_kv_head), static_cast<uint32_t>(D)) &&
-        (!split_ok || prefill_pays(N, n_head, n_kv_head, seq))) {
+        (!split_ok || prefill_pays(N, n_head, n_kv_head, seq, cap, D, part_bytes >= prefill_part_bytes(static_cast<uint32_t>(D))))) {
         PrefillArgs a{};
         a.q = q; a.k = k; a.v = v; a.o = o; a.kc = k_cache; a.vc = v_cache;
         a.past = past_lens;
@@ -984,6 +996,8 @@ int attention_call(void *o, const void *q, const void *k, const void *v, void *k
         a.D = static_cast<uint32_t>(D);
         a.scale = scale;
         a.dtype = dtype;
+        a.part = part;
+        a.part_bytes = part_bytes;
         return launch_prefill(a, s);
     }
 
@@ -1033,7 +1047,8 @@ extern "C" int rg_hip_attention_kvcache(void *o, const void *q, const void *k, c
     float *part = usable ? reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes) : nullptr;
     uint32_t *counters = static_cast<uint32_t *>(sync_state ? sync_state : workspace);
     return attention_call(o, q, k, v, k_cache, v_cache, past_lens, past_per_row, N, n_head, n_kv_head, seq, cap, D,
-                          scale, dtype, part, counters, kMaxWorkgroups, sync_state == nullptr, as_stream(stream));
+                          scale, dtype, part, usable ? workspace_bytes - kCounterBytes : 0, counters, kMaxWorkgroups,
+                          sync_state == nullptr, as_stream(stream));
 }
 
 extern "C" size_t rg_hip_attention_kvcache_static_scratch_bytes(void) { return rg::kStaticBytes; }
@@ -1054,5 +1069,5 @@ extern "C" int rg_hip_attention_kvcache_static(void *o, const void *q, const voi
     // The counters are cleared by a small fill kernel on every call (no memset: the call may be
     // under stream capture), so that whatever an earlier call left there cannot matter.
     return attention_call(o, q, k, v, k_cache, v_cache, past_lens, past_per_row, N, n_head, n_kv_head, seq, cap, D,
-                          scale, dtype, part, counters, kStaticWorkgroups, true, as_stream(stream));
+                          scale, dtype, part, kStaticPartBytes, counters, kStaticWorkgroups, true, as_stream(stream));
 }

@@ -50,6 +50,8 @@ constexpr int TILE = BN * ROWB;        // 16384: one K or V tile
 constexpr int BUF_BYTES = 2 * TILE;    // K tile + V tile; two such buffers, reused for the output transposition
 constexpr float kSlack = 6.0f;
 constexpr float kMinusBig = -1e30f;
+constexpr uint64_t kSplitMinTiles = 8;  // key tiles of the capacity per range of a SPLIT launch, at least
+constexpr uint64_t kSplitMax = 32;      // ranges per item, at most
 
 // LDS layout of a tile: the 16-byte chunk c of K row r sits at chunk position c ^ (r & 15), which
 // puts the 128-bit fragment reads of 8 or 16 consecutive rows on distinct banks; chunk c of V row r
@@ -135,7 +137,13 @@ struct PrefillPlan {
     // floor(2^32 / d) + 1 for d = head_chunks and d = Hkv: x / d = mulhi(x, magic) for every x with
     // x * d < 2^32, which the host checks (0 stands for d = 1)
     uint32_t magic_chunks, magic_hkv;
+    // key ranges per item (SPLIT instances): the streams above are then (stream, range) pairs, range fastest
+    uint32_t splits, magic_splits;
+    float *part;  // partial results of the ranges, kPartFloats(DH) per item and range
 };
+
+// Partial result of one key range of one item: per thread its accumulator registers of O^T, then m and l.
+__host__ __device__ constexpr uint32_t part_floats(uint32_t dh) { return 256u * (((dh + 31) / 32) * 16 + 2); }
 
 // One item: query tile qt of stream (kv head `kvhead` = b * Hkv + kvh of the batch, head chunk hc).
 // Kept to four scalars: the workgroup holds two of them across its whole life.
@@ -144,6 +152,7 @@ struct Item {
     uint32_t kvhead, hc;
     uint32_t qt;    // kNoItem: there is no such item
     uint32_t base;  // history length of the batch row, moved into [0, cap - seq]
+    uint32_t ks;    // key range of the item this workgroup walks (SPLIT instances; else 0)
     __device__ bool valid() const { return qt != kNoItem; }
 };
 
@@ -171,7 +180,11 @@ __device__ __forceinline__ void copy16(const void *sbase, uint32_t voffset, uint
 
 // HW: query heads per workgroup (1, 2 or 4); the other 4 / HW wavefronts take further 32-row
 // query sub-tiles of the same heads.
-template <class T, int HW, int DH>
+// SPLIT: an item's keys are shared between plan.splits workgroups (few items with a long history: chunked prefill,
+// a new turn of a conversation); each leaves its unnormalised O^T, m and l in plan.part and attn_prefill_merge
+// finishes the item.  The tiles of an item are dealt in equal counts; a range beyond the item's last tile walks
+// tile 0 with every key masked (history lengths are device data: the host sizes the ranges by the capacity).
+template <class T, int HW, int DH, bool SPLIT>
 __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, const PrefillPlan plan) {
     constexpr int QS = 4 / HW;      // query sub-tiles per workgroup
     constexpr int ROWS = 32 * QS;   // query rows per item
@@ -199,13 +212,18 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     // The history length of an item's batch row is read when the item is enumerated and clamped
     // when the item becomes the current one (an item later), so that nobody waits for the load.
     auto next_item = [&](uint64_t &raw_past) __attribute__((always_inline)) -> Item {
-        Item it{0, 0, kNoItem, 0};
+        Item it{0, 0, kNoItem, 0, 0};
         raw_past = 0;
         while (en_k < plan.spx) {
             const uint32_t heavy = plan.q_tiles - 1 - pj;
             const uint32_t qt = en_sub == 0 ? heavy : pj;
             const bool ok = en_sub == 0 || pj != heavy;
-            const uint32_t stream = en_k * plan.xcds + xcd;
+            uint32_t stream = en_k * plan.xcds + xcd;
+            if constexpr (SPLIT) {
+                const uint32_t whole = div_magic(stream, plan.magic_splits);
+                it.ks = stream - whole * plan.splits;
+                stream = whole;
+            }
             if (en_sub == 0) {
                 en_sub = 1;
             } else {
@@ -362,19 +380,42 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     f16v o[DBLK];
     float m = 0.f, l = 0.f;
     bool fresh = true;
-    Item cur{0, 0, kNoItem, 0};
+    Item cur{0, 0, kNoItem, 0, 0};
     uint64_t nxt_raw = 0, nn_raw = 0;
     Item nxt = next_item(nxt_raw);
     if (!nxt.valid()) return;
     nxt.base = clamp_past(nxt_raw);
-    uint32_t r0 = 0, n_tiles = 0, wave_tiles = 0, qpos = 0;
+    // n_tiles: the tile after the last one this workgroup walks for the item, t_first the first one (0 and the
+    // item's tile count unless SPLIT); qlim: the first key this lane's query row does not see
+    uint32_t r0 = 0, n_tiles = 0, wave_tiles = 0, qlim = 0, t_first = 0;
+    bool mask_all = false, last_range = true;
+    auto key_range = [&](const Item &it, uint32_t &first, uint32_t &end, bool &dummy) __attribute__((always_inline)) {
+        const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
+        const uint32_t tiles = uni((it.base + rows_end - 1) / BN + 1);
+        first = 0;
+        end = tiles;
+        dummy = false;
+        if constexpr (SPLIT) {
+            const uint32_t share = div_magic(tiles + plan.splits - 1, plan.magic_splits);  // tiles per range, rounded up
+            first = it.ks * share;
+            if (first >= tiles) {
+                first = 0;
+                end = 1;
+                dummy = true;
+            } else {
+                end = first + share < tiles ? first + share : tiles;
+            }
+        }
+    };
     auto begin_item = [&]() __attribute__((always_inline)) {
         r0 = cur.qt * ROWS + 32 * (wave_u / HW);
         const uint32_t rows_end = (cur.qt + 1) * ROWS < a.seq ? (cur.qt + 1) * ROWS : a.seq;
-        n_tiles = uni((cur.base + rows_end - 1) / BN + 1);
+        const uint32_t all_tiles = uni((cur.base + rows_end - 1) / BN + 1);
+        key_range(cur, t_first, n_tiles, mask_all);
+        last_range = !mask_all && n_tiles == all_tiles;
         const uint32_t wave_last_row = r0 + 31 < a.seq ? r0 + 31 : a.seq - 1;
         wave_tiles = uni(r0 < a.seq ? (cur.base + wave_last_row) / BN + 1 : 0);
-        qpos = cur.base + r0 + l32;  // absolute position of this lane's query row
+        qlim = mask_all ? 0u : cur.base + r0 + l32 + 1;  // absolute position of this lane's query row, plus one
 #pragma unroll
         for (int db = 0; db < DBLK; ++db)
 #pragma unroll
@@ -390,6 +431,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     // (then they are loaded from the inputs again), and stored when the item goes out.
     auto load_own_rows = [&](const Item &it, uint32_t buf, u32x4 (&ak)[ROWS / 16], u32x4 (&av)[ROWS / 16]) __attribute__((always_inline)) {
         if (!(Kc && it.hc == 0)) return;
+        if (SPLIT && !last_range) return;  // (the range that ends with the item's last tile appends)
         const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
         const uint32_t lo = it.qt * ROWS;
         const uint32_t tile_first = (n_tiles - 1) * BN;  // first key of the last tile
@@ -431,14 +473,27 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         const bool head_ok = it.hc * HW + wave_u % HW < plan.group;  // else a repeated head: nothing to store
         const uint32_t fr0 = it.qt * ROWS + 32 * (wave_u / HW);
         const uint32_t rows_end = (it.qt + 1) * ROWS < a.seq ? (it.qt + 1) * ROWS : a.seq;
-        const bool do_append = Kc && it.hc == 0;
+        const bool do_append = Kc && it.hc == 0 && (!SPLIT || last_range);
         const uint32_t own_lo = it.base + it.qt * ROWS, own_hi = it.base + rows_end;
         // (lane indices from an opaque copy: the addresses below are then formed here, once per item, and
         // not ahead of the loops, where they would occupy registers all the time)
         uint32_t tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
         const uint32_t lane = tid & 63, l32 = tid & 31, half = (tid >> 5) & 1;
-        if (fr0 < a.seq && head_ok) {
+        if constexpr (SPLIT) {
+            if (fr0 < a.seq && head_ok) {
+                // record of (item, range): register r of thread t at r * 256 + t.  A wavefront that met no tile of
+                // its own in the range (or only masked keys) leaves a maximum far below any real one.
+                const uint32_t stream = it.kvhead * plan.head_chunks + it.hc;
+                float *rec = plan.part + (static_cast<uint64_t>(stream * plan.q_tiles + it.qt) * plan.splits + it.ks) * part_floats(DH);
+#pragma unroll
+                for (int db = 0; db < DBLK; ++db)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) rec[(db * 16 + e) * 256 + tid] = o[db][e];
+                rec[(DBLK * 16) * 256 + tid] = fresh ? kMinusBig : m;
+                rec[(DBLK * 16 + 1) * 256 + tid] = l;
+            }
+        } else if (fr0 < a.seq && head_ok) {
             const float inv = 1.f / half_sum(l);
 #pragma unroll
             for (int db = 0; db < DBLK; ++db)
@@ -602,13 +657,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
             for (int i = 0; i < 4; ++i) vf[i] = read_v(i);
             RG_SCHED_FENCE();
             // scale, causal mask (only blocks that reach past the wavefront's first query position)
-            const bool need_mask = kt * BN + 32 * kb + 31 > cur.base + r0;
+            const bool need_mask = kt * BN + 32 * kb + 31 > cur.base + r0 || (SPLIT && mask_all);
             float over = -__builtin_inff();
             if (need_mask) {  // wave-uniform: only the blocks on the diagonal pay for the comparisons
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const uint32_t key = kt * BN + 32 * kb + 8 * (e / 4) + 4 * half + (e % 4);
-                    const float t = key > qpos ? -__builtin_inff() : fmaf(sc[e], c_log2e, -m);
+                    const float t = key >= qlim ? -__builtin_inff() : fmaf(sc[e], c_log2e, -m);
                     sc[e] = t;
                     over = fmaxf(over, t);
                 }
@@ -661,7 +716,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     // into the buffer thus freed, and the finished item goes out while it travels
     bool have_cur = false;
     auto q_slot = [&](uint32_t buf) __attribute__((always_inline)) -> bool {
-        Item nn{0, 0, kNoItem, 0};
+        Item nn{0, 0, kNoItem, 0, 0};
         u32x4 ak[ROWS / 16], av[ROWS / 16];
         if (have_cur) load_own_rows(cur, buf ^ BUF_BYTES, ak, av);
         if (nxt.valid()) {
@@ -672,7 +727,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_s_barrier();
             }
-            copy_tile(nxt, 0, buf ^ BUF_BYTES);
+            uint32_t first = 0, end = 0;
+            bool dummy = false;
+            key_range(nxt, first, end, dummy);
+            copy_tile(nxt, first, buf ^ BUF_BYTES);
             nn = next_item(nn_raw);  // its history length is on its way while the output goes out
         }
         if (have_cur) finish_item(cur, ak, av, lds + buf + wave_u * (32 * ROWB));
@@ -699,7 +757,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
         if (!q_slot(buf)) break;
         end_slot();
         buf ^= BUF_BYTES;
-        for (uint32_t kt = 0; kt < n_tiles; ++kt) {
+        for (uint32_t kt = t_first; kt < n_tiles; ++kt) {
             tile(buf, kt);
             end_slot();
             buf ^= BUF_BYTES;
@@ -707,11 +765,54 @@ __global__ __launch_bounds__(256, 2) void attn_prefill(const PrefillArgs a, cons
     }
 }
 
+// Finishes the items of a SPLIT launch: workgroups with the threads of attn_prefill (wavefront = head and query
+// sub-tile, lane = query row and half of the keys), each taking eight of a thread's accumulator registers
+// (blockIdx.y: two groups of four consecutive d), add the ranges' records weighted by 2^(m_range - m_max), normalise
+// and store four consecutive d per instruction.
+constexpr int kMergeRegs = 8;
+template <class T, int HW, int DH>
+__global__ __launch_bounds__(256) void attn_prefill_merge(const PrefillArgs a, const PrefillPlan plan) {
+    constexpr int QS = 4 / HW, ROWS = 32 * QS, DBLK = (DH + 31) / 32;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const uint32_t qt = blockIdx.x % plan.q_tiles, stream = blockIdx.x / plan.q_tiles;
+    const uint32_t kvhead = stream / plan.head_chunks, hc = stream % plan.head_chunks;
+    const uint32_t h = hc * HW + wave % HW;
+    const uint32_t fr0 = qt * ROWS + 32 * (wave / HW);
+    if (h >= plan.group || fr0 >= a.seq) return;  // (whole wavefronts)
+    const float *rec = plan.part + static_cast<uint64_t>(blockIdx.x) * plan.splits * part_floats(DH);
+    const uint32_t e0 = blockIdx.y * kMergeRegs;
+    float m_max = kMinusBig;
+    for (uint32_t r = 0; r < plan.splits; ++r) m_max = fmaxf(m_max, rec[r * part_floats(DH) + (DBLK * 16) * 256 + tid]);
+    float o[kMergeRegs], l = 0.f;
+#pragma unroll
+    for (int e = 0; e < kMergeRegs; ++e) o[e] = 0.f;
+#pragma unroll 4
+    for (uint32_t r = 0; r < plan.splits; ++r) {
+        const float *p = rec + r * part_floats(DH);
+        const float w = __builtin_amdgcn_exp2f(p[(DBLK * 16) * 256 + tid] - m_max);
+        l += w * p[(DBLK * 16 + 1) * 256 + tid];
+#pragma unroll
+        for (int e = 0; e < kMergeRegs; ++e) o[e] += w * p[(e0 + e) * 256 + tid];
+    }
+    const float inv = 1.f / half_sum(l);
+    const uint32_t row = fr0 + l32;
+    if (row >= a.seq) return;
+    T *out = static_cast<T *>(a.o) + (static_cast<uint64_t>(kvhead * plan.group + h) * a.seq + row) * DH;
+#pragma unroll
+    for (int gg = 0; gg < kMergeRegs / 4; ++gg) {
+        // registers 4 g .. 4 g + 3 of block db: d = 32 db + 8 g + 4 half + 0..3
+        const uint32_t e = e0 + 4 * gg, db = e / 16, g = (e % 16) / 4, d = 32 * db + 8 * g + 4 * half;
+        if (d >= DH) continue;  // (head dim 80: the second half of the last block)
+        const uint2 w = make_uint2(Ops<T>::pack2(o[4 * gg] * inv, o[4 * gg + 1] * inv), Ops<T>::pack2(o[4 * gg + 2] * inv, o[4 * gg + 3] * inv));
+        *reinterpret_cast<uint2 *>(out + d) = w;
+    }
+}
+
 template <class T, int HW, int DH>
 uint32_t resident_prefill_workgroups() {
     static uint32_t cached = [] {
         int per_cu = 0, dev = 0, cus = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_prefill<T, HW, DH>, 256, 0) != hipSuccess || per_cu <= 0)
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_prefill<T, HW, DH, false>, 256, 0) != hipSuccess || per_cu <= 0)
             per_cu = 2;
         hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
@@ -729,8 +830,27 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
     plan.head_chunks = (plan.group + HW - 1) / HW;
     plan.q_tiles = (a.seq + ROWS - 1) / ROWS;
     plan.pairs = (plan.q_tiles + 1) / 2;
-    const uint64_t streams = static_cast<uint64_t>(a.N) * a.Hkv * plan.head_chunks;
+    uint64_t streams = static_cast<uint64_t>(a.N) * a.Hkv * plan.head_chunks;
     if (streams * plan.pairs > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+    // Few items and room for a long history: the keys of an item are shared between workgroups, as many as bring
+    // the launch to the workgroups that are resident together, each with at least kSplitMinTiles tiles of the
+    // capacity, while the records fit the workspace (head dims 64 and 128)
+    plan.splits = 1;
+    const uint64_t items = streams * plan.q_tiles;
+    if constexpr (DH == 64 || DH == 128) {
+        const uint64_t resident = resident_prefill_workgroups<T, HW, DH>();
+        const uint64_t cap_tiles = (static_cast<uint64_t>(a.cap) + BN - 1) / BN;
+        uint64_t splits = items ? resident / items : 1;
+        if (splits > cap_tiles / kSplitMinTiles) splits = cap_tiles / kSplitMinTiles;
+        if (splits > kSplitMax) splits = kSplitMax;
+        const uint64_t room = a.part ? a.part_bytes / (items * part_floats(DH) * sizeof(float)) : 0;
+        if (splits > room) splits = room;
+        if (splits >= 2 && streams * splits * plan.pairs <= 0x7fffffffu) plan.splits = static_cast<uint32_t>(splits);
+    }
+    plan.magic_splits = plan.splits > 1 ? static_cast<uint32_t>((1ull << 32) / plan.splits + 1) : 0;
+    plan.part = a.part;
+    const uint64_t whole_streams = streams;
+    streams *= plan.splits;
     plan.xcds = streams % 8 == 0 ? 8 : 1;
     plan.spx = static_cast<uint32_t>(streams / plan.xcds);
     // as many sets of `pairs` workgroups per XCD as stay resident together (at least one)
@@ -739,12 +859,24 @@ int launch_hw(const PrefillArgs &a, hipStream_t s) {
     if (groups < 1) groups = 1;
     if (groups > plan.spx) groups = plan.spx;
     plan.groups = groups;
-    const uint64_t widest = plan.head_chunks > a.Hkv ? plan.head_chunks : a.Hkv;
+    uint64_t widest = plan.head_chunks > a.Hkv ? plan.head_chunks : a.Hkv;
+    if (plan.splits > widest) widest = plan.splits;
     if (streams * widest >= (1ull << 32)) return RG_HIP_E_UNSUPPORTED;
     plan.magic_chunks = plan.head_chunks > 1 ? static_cast<uint32_t>((1ull << 32) / plan.head_chunks + 1) : 0;
     plan.magic_hkv = a.Hkv > 1 ? static_cast<uint32_t>((1ull << 32) / a.Hkv + 1) : 0;
     const uint32_t grid = plan.xcds * plan.groups * plan.pairs;
-    attn_prefill<T, HW, DH><<<grid, 256, 0, s>>>(a, plan);
+    if constexpr (DH == 64 || DH == 128) {
+        if (plan.splits > 1) {
+            attn_prefill<T, HW, DH, true><<<grid, 256, 0, s>>>(a, plan);
+            const int rc = launch_status();
+            if (rc) return rc;
+            constexpr unsigned parts = ((DH + 31) / 32) * 16 / kMergeRegs;
+            attn_prefill_merge<T, HW, DH><<<dim3(static_cast<unsigned>(whole_streams * plan.q_tiles), parts), 256, 0, s>>>(a, plan);
+            return launch_status();
+        }
+    }
+    (void)whole_streams;
+    attn_prefill<T, HW, DH, false><<<grid, 256, 0, s>>>(a, plan);
     return launch_status();
 }
 
@@ -768,6 +900,11 @@ int launch_t(const PrefillArgs &a, hipStream_t s) {
 }
 
 }  // namespace
+
+size_t prefill_part_bytes(uint32_t D_) {
+    // a launch shares keys only while (items x ranges) stay within the workgroups resident together: two per CU
+    return D_ == 64 || D_ == 128 ? static_cast<size_t>(512) * part_floats(D_) * sizeof(float) : 0;
+}
 
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D_) {
     return (D_ == 128 || D_ == 96 || D_ == 80 || D_ == 64) && Hkv != 0 && H % Hkv == 0;

@@ -13,7 +13,12 @@ struct PrefillArgs {
     uint32_t N, H, Hkv, seq, cap, D;
     float scale;
     int dtype;  // RG_FP16 or RG_BF16
+    float *part;        // workspace for the partial results of key ranges (may be null: no ranges then)
+    size_t part_bytes;
 };
+
+// Bytes of `part` with which every launch that shares keys between workgroups finds room.
+size_t prefill_part_bytes(uint32_t D);
 
 // True when launch_prefill handles the shape (head dim 128 or 64, any group size).
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D);

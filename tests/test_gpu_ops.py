@@ -943,6 +943,26 @@ def test_attention_few_new_rows_either_kernel(N, H, Hkv, seq, cap, D, dt):
     assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
 
 
+@pytest.mark.parametrize("N,H,Hkv,seq,cap,D,past,dt", [
+    (1, 32, 8, 128, 4128, 128, [4000], torch.float16),      # a chunk of a long prompt: 32 items, 16 key ranges each
+    (1, 32, 8, 33, 4033, 128, [4000], torch.float16),       # ragged query rows
+    (1, 32, 8, 128, 8128, 128, [10], torch.float16),        # a long cache with a short history: ranges beyond the keys
+    (1, 32, 8, 200, 3200, 128, [0], torch.float16),         # no history at all
+    (2, 8, 8, 100, 2600, 128, [2500, 17], torch.float16),   # one head per kv head, histories that differ
+    (1, 16, 2, 77, 3077, 64, [2999], torch.bfloat16),       # head dim 64, group of 8 (two chunks of four heads)
+    (1, 12, 4, 64, 5064, 128, [4321], torch.bfloat16),      # group of 3
+    (3, 4, 2, 8, 1508, 64, [1500, 0, 700], torch.float16),  # eight new rows: the tiled kernel by the cost rule
+    (1, 32, 8, 16, 6016, 128, [6000], torch.float16),       # sixteen new rows
+])
+def test_attention_long_history_keys_shared_between_workgroups(N, H, Hkv, seq, cap, D, past, dt):
+    # few items (one sequence, a chunk of a prompt or a new turn of a conversation) against a long cache: the tiled
+    # kernel shares an item's keys between workgroups and a second launch merges their partial results
+    o, ref_o, kc, ref_kc, vc, ref_vc = _attention_case(N, H, Hkv, seq, cap, D, past, dt=dt, seed=61)
+    assert not np.isnan(o).any()
+    assert np.max(np.abs(o - ref_o)) <= (ABS_F16 if dt == torch.float16 else 2e-2)
+    assert np.array_equal(kc, ref_kc) and np.array_equal(vc, ref_vc)
+
+
 def test_attention_prefill_no_cache_tiled():
     rng = np.random.default_rng(21)
     mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).half()
