@@ -860,10 +860,10 @@ constexpr size_t kPrefillAlways = 32;  // query rows from which the tiled kernel
 bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq, size_t cap, size_t D, bool ranges_fit) {
     if (seq >= kPrefillAlways) return true;
     const size_t group = n_head / n_kv_head, heads_per_item = group == 1 ? 1 : group == 2 ? 2 : 4;
-    // the split kernel takes at most four heads of a group per launch and reads K/V again in every launch
-    // (a group of 8: twice), while the chunks of a group on the tiled kernel find them in L2
+    // the split kernel takes eight, four, two or one heads of a group per launch and reads K/V again in every launch
+    // (a group of 7: three times), while the chunks of a group on the tiled kernel find them in L2
     size_t split_launches = 0;
-    for (size_t left = group; left > 0; left -= left >= 4 ? 4 : left >= 2 ? 2 : 1) ++split_launches;
+    for (size_t left = group; left > 0; left -= left >= 8 ? 8 : left >= 4 ? 4 : left >= 2 ? 2 : 1) ++split_launches;
     if (seq < 2 && split_launches < 2) return false;
     const size_t rows_per_item = 32 * (4 / heads_per_item);
     const size_t items = N * n_kv_head * ((group + heads_per_item - 1) / heads_per_item) * ((seq + rows_per_item - 1) / rows_per_item);
@@ -872,6 +872,7 @@ bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq, size_t 
     // kv head, key and query row on the split kernel (N = 1, 8 kv heads, 8 new rows: history 1000 13.9 us split
     // against 18.1 tiled, 4000 26.1 against 22.7, 32768 154 against 46).  The history is device data: half of the
     // capacity stands for it.
+    if (ranges_fit && seq == 1 && split_launches >= 2 && (D == 64 || D == 128)) return true;  // (16 x 28/4 heads, history 4000: 80 -> 52 us)
     if (ranges_fit && seq >= 2 && items * 2 <= 512 && cap >= 1024 && (D == 64 || D == 128)) {
         const double keys = static_cast<double>(N * n_kv_head) * static_cast<double>(cap) / 2;
         return 9.5 < keys * (7.3e-5 * static_cast<double>(seq * split_launches) - 9.4e-5);
@@ -891,14 +892,20 @@ int launch(AttnParams p, hipStream_t s) {
 
 template <class T, int D>
 int dispatch_group(AttnParams p, hipStream_t s) {
-    // heads of a kv group are processed G at a time (G in {4, 2, 1})
+    // heads of a kv group are processed G at a time (G in {8, 4, 2, 1})
     uint32_t done = 0;
     while (done < p.group) {
         const uint32_t left = p.group - done;
         p.head0 = done;
         p.append = done == 0;
         int rc;
-        if (left >= 4) {
+        if (left >= 8) {
+            // eight heads read their K/V once instead of twice (64/8 heads, 64 sequences, history 4096: 337 -> 238 us)
+            AttnParams p8 = p;
+            p8.n_workgroups = p.n_workgroups / 2;  // (the partial slots are sized for groups of four)
+            rc = launch<T, D, 8>(p8, s);
+            done += 8;
+        } else if (left >= 4) {
             rc = launch<T, D, 4>(p, s);
             done += 4;
         } else if (left >= 2) {
