@@ -946,6 +946,53 @@ def main():
                  mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
         ops_out["attention_prefill_d64"] = e
 
+    if want("attention_chunk_long_history"):
+        # a chunk of a long prompt (or a new turn of a conversation): one sequence, 128 new rows against a history
+        # of 16384: the tiled kernel shares an item's keys between workgroups, a second launch merges
+        Np, seq, past, Dc = 1, 128, 16384, 128
+        capc = past + seq
+        q = torch.randn((Np, H, seq, Dc), device=dev).half()
+        k = torch.randn((Np, Hkv, seq, Dc), device=dev).half()
+        v = torch.randn((Np, Hkv, seq, Dc), device=dev).half()
+        kc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        vc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        o = torch.empty_like(q)
+        pl = torch.full((Np,), past, device=dev, dtype=torch.int64)
+        wsp = ops.attention_workspace(Np, H, Hkv, seq, capc, Dc, dev)
+        wall, dms, mode = time_steps(
+            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, pl, 1.0 / math.sqrt(Dc), out=o, workspace=wsp,
+                                                   sync_state=state),
+            max(steps // 10, 20), max(warmup // 80, 2), 1)
+        kv_bytes = 2 * Np * Hkv * capc * Dc * 2 + 2 * Np * H * seq * Dc * 2 + 2 * Np * Hkv * seq * Dc * 2
+        e = hbm_entry(kv_bytes, dms)
+        flops = 4 * Np * H * Dc * (seq * past + seq * (seq + 1) // 2)
+        e.update(workload="AttentionKVCache fp16 N=1 H=32 Hkv=8 D=128, 128 new rows against a history of 16384 (both launches)",
+                 device_ms_per_launch=round(dms, 5), timing=mode,
+                 mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
+                 mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
+        ops_out["attention_chunk_long_history"] = e
+
+    if want("attention_decode_group8"):
+        # a decode step of a model with eight query heads per kv head (64/8): one launch reads K/V once for all eight
+        Np, H8, past, Dc = 64, 64, 4096, 128
+        capc = past + 1
+        q = torch.randn((Np, H8, 1, Dc), device=dev).half()
+        k = torch.randn((Np, Hkv, 1, Dc), device=dev).half()
+        v = torch.randn((Np, Hkv, 1, Dc), device=dev).half()
+        kc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        vc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        o = torch.empty_like(q)
+        pl = torch.full((Np,), past, device=dev, dtype=torch.int64)
+        wsp = ops.attention_workspace(Np, H8, Hkv, 1, capc, Dc, dev)
+        wall, dms, mode = time_steps(
+            torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, pl, 1.0 / math.sqrt(Dc), out=o, workspace=wsp,
+                                                   sync_state=state),
+            max(steps // 10, 20), max(warmup // 80, 2), 1)
+        e = hbm_entry(2 * Np * Hkv * capc * Dc * 2 + 2 * Np * H8 * Dc * 2 + 2 * Np * Hkv * Dc * 2, dms)
+        e.update(workload="AttentionKVCache decode fp16 N=64 H=64 Hkv=8 D=128 history 4096",
+                 device_ms_per_launch=round(dms, 5), timing=mode)
+        ops_out["attention_decode_group8"] = e
+
     if ops_out:
         result["ops"] = ops_out
     print(json.dumps(result))
