@@ -212,3 +212,35 @@ def test_attention_on_random_shapes(seed):
         what = (case, N, H, Hkv, seq, cap, D, past.tolist(), str(dt), bool(one_length))
         assert np.max(np.abs(f(o) - ref_o)) <= (2e-3 if dt == torch.float16 else 2e-2), what
         assert np.array_equal(f(kc), ref_kc) and np.array_equal(f(vc), ref_vc), what
+
+
+@pytest.mark.parametrize("seed", [611])
+def test_attention_long_caches_on_random_shapes(seed):
+    # few sequences against long caches: the tiled kernel with an item's keys shared between workgroups (ranges that
+    # lie beyond a short history included), the decode kernel with eight heads of a group per launch
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        N = int(rng.integers(1, 4))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        H = Hkv * int(rng.choice([1, 2, 4, 7, 8, 16]))
+        D = int(rng.choice([64, 128]))
+        seq = int(rng.choice([1, 2, 5, 16, 31, 32, 33, 70, 128, 200]))
+        room = int(rng.choice([1000, 2500, 4000, 9000]))
+        cap = seq + room
+        past = rng.integers(0, room + 1, N)
+        if rng.integers(0, 3) == 0:
+            past[:] = room
+        if rng.integers(0, 5) == 0:
+            past[:] = rng.integers(0, 40)
+        dt = torch.float16 if rng.integers(0, 4) else torch.bfloat16
+        mk = lambda shape: dev(rng.standard_normal(shape).astype(np.float32)).to(dt)
+        q, k, v = mk((N, H, seq, D)), mk((N, Hkv, seq, D)), mk((N, Hkv, seq, D))
+        kc, vc = mk((N, Hkv, cap, D)), mk((N, Hkv, cap, D))
+        kc0, vc0 = kc.clone(), vc.clone()
+        o = ops.attention_kvcache(q, k, v, kc, vc, dev(past.astype(np.int64)), 1 / math.sqrt(D))
+        f = lambda t: host(t.float())
+        ref_o, ref_kc, ref_vc = oracle.attention_kvcache(f(q), f(k), f(v), f(kc0), f(vc0), past, 1 / math.sqrt(D))
+        what = (case, N, H, Hkv, seq, cap, D, past.tolist(), str(dt))
+        assert not np.isnan(f(o)).any(), what
+        assert np.max(np.abs(f(o) - ref_o)) <= (2e-3 if dt == torch.float16 else 2e-2), what
+        assert np.array_equal(f(kc), ref_kc) and np.array_equal(f(vc), ref_vc), what
