@@ -963,14 +963,16 @@ def main():
             torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, pl, 1.0 / math.sqrt(Dc), out=o, workspace=wsp,
                                                    sync_state=state),
             max(steps // 10, 20), max(warmup // 80, 2), 1)
+        # 128 rows x 4 heads share every key: priced on the matrix cores (34 GFLOP against 68 MB)
         kv_bytes = 2 * Np * Hkv * capc * Dc * 2 + 2 * Np * H * seq * Dc * 2 + 2 * Np * Hkv * seq * Dc * 2
-        e = hbm_entry(kv_bytes, dms)
         flops = 4 * Np * H * Dc * (seq * past + seq * (seq + 1) // 2)
-        e.update(workload="AttentionKVCache fp16 N=1 H=32 Hkv=8 D=128, 128 new rows against a history of 16384 (both launches)",
-                 device_ms_per_launch=round(dms, 5), timing=mode,
-                 mfma_tflops=round(flops / (dms * 1e-3) / 1e12, 2),
-                 mfma_frac=round(flops / (dms * 1e-3) / 1e12 / FP16_PEAK_TFLOPS, 4))
-        ops_out["attention_chunk_long_history"] = e
+        tf = flops / (dms * 1e-3) / 1e12
+        ops_out["attention_chunk_long_history"] = {
+            "bound": "mfma", "achieved": round(tf, 1), "peak": FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tf / FP16_PEAK_TFLOPS, 4), "traffic": None,
+            "workload": "AttentionKVCache fp16 N=1 H=32 Hkv=8 D=128, 128 new rows against a history of 16384 (both launches)",
+            "device_ms_per_launch": round(dms, 5), "timing": mode, "hbm_gbs": round(kv_bytes / (dms * 1e-3) / 1e9, 1),
+            "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
 
     if want("attention_decode_group8"):
         # a decode step of a model with eight query heads per kv head (64/8): one launch reads K/V once for all eight
