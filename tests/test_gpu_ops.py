@@ -671,6 +671,26 @@ def test_transpose_bit_exact(shape, perm, dt):
     assert tuple(y.shape) == ref.shape and np.array_equal(host(y), ref) and np.array_equal(ref, np.transpose(x, perm))
 
 
+@pytest.mark.parametrize("shape,perm", [
+    ((200, 136), (1, 0)), ((208, 144), (1, 0)), ((2, 4, 72, 64), (0, 1, 3, 2)), ((3, 80, 5, 48), (0, 3, 2, 1)),
+    ((2, 3, 160, 256), (1, 3, 0, 2)), ((16, 4096), (1, 0)), ((4096, 16), (1, 0)), ((5, 128, 128), (2, 0, 1))])
+@pytest.mark.parametrize("dt", [np.uint8, np.float16])
+def test_transpose_of_8_and_16_bit_elements_with_aligned_rows(shape, perm, dt):
+    # the innermost dimension moves and every row of either tensor starts on a 16-byte boundary: tiles of 128-byte
+    # rows turned in registers and LDS (whole tiles, tiles that reach beyond either extent, outer dimensions on both
+    # sides); the same from addresses 16 bytes into a buffer
+    x = np.random.default_rng(len(shape) + shape[0]).integers(0, 250, shape).astype(dt)
+    y = ops.transpose(dev(x), perm)
+    assert tuple(y.shape) == tuple(x.shape[p] for p in perm) and np.array_equal(host(y), np.transpose(x, perm))
+    n = x.size
+    elems = 16 // x.itemsize
+    src = torch.empty(n + elems, device=DEV, dtype=dev(x).dtype)
+    src[elems:] = dev(x).reshape(-1)
+    dst = torch.empty(n + elems, device=DEV, dtype=src.dtype)
+    y2 = ops.transpose(src[elems:].view(*shape), perm, out=dst[elems:].view(*[shape[p] for p in perm]))
+    assert np.array_equal(host(y2), np.transpose(x, perm))
+
+
 def test_transpose_unaligned_views_and_involution():
     x = torch.arange(3 * 37 * 11, device=DEV, dtype=torch.int16).reshape(3, 37, 11)
     buf = torch.empty(3 * 37 * 11 + 1, device=DEV, dtype=torch.int16)
