@@ -21,6 +21,7 @@
 namespace rg {
 namespace {
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kMaxDims = 8;
 constexpr int UNROLL = 4;  // words a thread has in flight
 constexpr uint32_t TILE_H = 8, TILE_S = 8;   // blocks of a tile along the two dimensions that change places
@@ -72,6 +73,36 @@ __global__ __launch_bounds__(256) void transpose_words(Word *__restrict__ y, con
     for (int j = 0; j < UNROLL; ++j) {
         const uint64_t g = base + j * 256;
         if (g < p.words) __builtin_nontemporal_store(v[j], y + g);
+    }
+}
+
+// Expand whose innermost output dimension is broadcast from single elements (a column [n, 1] spread over rows, a scalar
+// over a vector): a row of the output is one element repeated, so the output goes out in 16-byte words of copies of
+// that element instead of one element per store (1.6 TB/s for 16-bit elements).  The plan's blocks are the rows (its
+// dimensions those in front of the innermost one, output strides in rows), words_per_block their 16-byte words.
+template <class Elem>
+__global__ __launch_bounds__(256) void expand_splat(u32x4_t *__restrict__ y, const Elem *__restrict__ x, const Plan p) {
+    const uint64_t base = (static_cast<uint64_t>(blockIdx.x) * UNROLL) * 256 + threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+        const uint64_t g = base + j * 256;
+        if (g < p.words) {
+            const uint32_t row = p.words_per_block.div(static_cast<uint32_t>(g));
+            uint32_t from = 0, rem = row;
+            for (uint32_t d = 0; d < p.dims; ++d) {
+                const uint32_t q = p.stride_o[d].div(rem);
+                from += q * p.stride_i[d];
+                rem -= q * p.stride_o[d].d;
+            }
+            const uint64_t e = x[from];
+            uint64_t lo = e;
+            if constexpr (sizeof(Elem) < 8) {
+#pragma unroll
+                for (unsigned bits = 8 * sizeof(Elem); bits < 64; bits *= 2) lo |= lo << bits;
+            }
+            u32x4_t v = {static_cast<uint32_t>(lo), static_cast<uint32_t>(lo >> 32), static_cast<uint32_t>(lo), static_cast<uint32_t>(lo >> 32)};
+            __builtin_nontemporal_store(v, y + g);
+        }
     }
 }
 
@@ -351,6 +382,35 @@ extern "C" int rg_hip_expand(void *y, const void *x, const uint32_t *stride_i, c
     if (block_count > 0xffffffffull) return RG_HIP_E_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
     if (dims == 0) return static_cast<int>(hipMemcpyAsync(y, x, bytes, hipMemcpyDeviceToDevice, s));  // nothing is broadcast
+    // single elements repeated along the innermost output dimension, rows of whole 16-byte words
+    if (stride_i[dims - 1] == 0 && stride_o[dims - 1] == 1 && (block_size == 1 || block_size == 2 || block_size == 4 || block_size == 8) &&
+        aligned16(y) && (reinterpret_cast<uintptr_t>(x) & (block_size - 1)) == 0) {
+        const uint64_t row = dims >= 2 ? stride_o[dims - 2] : block_count;  // elements of a row
+        bool ok = row > 0 && (row * block_size) % 16 == 0 && bytes / 16 <= 0xffffffffull;
+        for (size_t d = 0; d + 1 < dims && ok; ++d) ok = stride_o[d] != 0 && stride_o[d] % row == 0;
+        if (ok) {
+            Plan p{};
+            p.dims = static_cast<uint32_t>(dims - 1);
+            p.words = bytes / 16;
+            p.words_per_block = make_divisor(static_cast<uint32_t>(row * block_size / 16));
+            for (size_t d = 0; d + 1 < dims; ++d) {
+                p.stride_o[d] = make_divisor(static_cast<uint32_t>(stride_o[d] / row));
+                p.stride_i[d] = stride_i[d];
+            }
+            const uint64_t grid = (p.words + 256ull * UNROLL - 1) / (256ull * UNROLL);
+            if (grid <= 0x7fffffffull) {
+                const unsigned g = static_cast<unsigned>(grid);
+                u32x4_t *out = static_cast<u32x4_t *>(y);
+                switch (block_size) {
+                    case 1: expand_splat<uint8_t><<<g, 256, 0, s>>>(out, static_cast<const uint8_t *>(x), p); break;
+                    case 2: expand_splat<uint16_t><<<g, 256, 0, s>>>(out, static_cast<const uint16_t *>(x), p); break;
+                    case 4: expand_splat<uint32_t><<<g, 256, 0, s>>>(out, static_cast<const uint32_t *>(x), p); break;
+                    default: expand_splat<uint64_t><<<g, 256, 0, s>>>(out, static_cast<const uint64_t *>(x), p); break;
+                }
+                return launch_status();
+            }
+        }
+    }
     const uintptr_t misalign = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(x) | block_size;
     uint32_t w = 16;
     while (misalign & (w - 1)) w >>= 1;

@@ -757,6 +757,8 @@ def test_split_concat_misaligned_views():
     ((1,), (9, 11)),
     ((2, 3, 4), (2, 3, 4)),                           # nothing to do: a copy
     ((), (4, 5)),
+    ((300, 1), (300, 64)),                            # single elements along rows of whole 16-byte words
+    ((1,), (4096,)), ((3, 1, 5, 1), (3, 2, 5, 16)), ((2, 7, 1), (3, 2, 7, 48)), ((), (2, 3, 32)),
 ])
 def test_expand_bit_exact(inp, out):
     rng = np.random.default_rng(sum(out))
