@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void rms_norm_rows(T *__restrict__ y, const T 
 
     const uint32_t t = threadIdx.x % GROUP;
     const size_t row = static_cast<size_t>(blockIdx.x) * ROWS_PER_BLOCK + threadIdx.x / GROUP;
-    const bool live = row < rows;  // only ever false for GROUP == 64 (no block barrier there)
+    const bool live = row < rows;  // only ever false for GROUP <= 64 (no block barrier there)
     const uint32_t nvec = cols / VEC;
     const T *xr = x + row * cols;
     T *yr = y + row * cols;
@@ -42,7 +42,10 @@ __global__ __launch_bounds__(256) void rms_norm_rows(T *__restrict__ y, const T 
             }
         }
     }
-    if constexpr (GROUP == kWave) {
+    if constexpr (GROUP < kWave) {  // short rows (a head's 128 elements): several to a wavefront
+#pragma unroll
+        for (int o = GROUP / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+    } else if constexpr (GROUP == kWave) {
         acc = wave_sum(acc);
     } else {
         acc = block_allreduce<GROUP / kWave>(
@@ -101,7 +104,13 @@ int dispatch(void *y_, const void *x_, const void *w_, size_t rows, size_t cols,
     constexpr size_t VEC = Vec16<T>::N;
     const bool vec_ok = cols % VEC == 0 && aligned16(y) && aligned16(x) && aligned16(w);
     const size_t nvec = cols / VEC;
-    if (vec_ok && nvec <= 64 * 16) {
+    if (vec_ok && nvec <= 32) {
+        // rows of a few vectors (normalisation per head: 128 elements): 4 to 32 lanes per row instead of 64
+        if (nvec <= 4) launch_rows<T, 4, 1>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 8) launch_rows<T, 8, 1>(y, x, w, rows, cols, eps, s);
+        else if (nvec <= 16) launch_rows<T, 16, 1>(y, x, w, rows, cols, eps, s);
+        else launch_rows<T, 32, 1>(y, x, w, rows, cols, eps, s);
+    } else if (vec_ok && nvec <= 64 * 16) {
         // one wavefront per row: no workgroup barrier, up to 16 loads in flight per lane
         if (nvec <= 64) launch_rows<T, 64, 1>(y, x, w, rows, cols, eps, s);
         else if (nvec <= 128) launch_rows<T, 64, 2>(y, x, w, rows, cols, eps, s);

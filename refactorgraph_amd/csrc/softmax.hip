@@ -88,7 +88,13 @@ __global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *
     }
     auto wmax = [](CT v) { return wave_max(v); };
     auto wsum = [](CT v) { return wave_sum(v); };
-    if constexpr (GROUP == kWave) mx = wave_max(mx);
+    if constexpr (GROUP < kWave) {  // short rows: several to a wavefront, reduced among GROUP neighbouring lanes
+#pragma unroll
+        for (int o = GROUP / 2; o > 0; o >>= 1) {
+            const CT other = __shfl_xor(mx, o, kWave);
+            mx = mx < other ? other : mx;
+        }
+    } else if constexpr (GROUP == kWave) mx = wave_max(mx);
     else mx = block_allreduce<GROUP / kWave>(mx, smem, wmax, [](CT a, CT b) { return a < b ? b : a; });
 
     CT sum = 0;
@@ -100,7 +106,10 @@ __global__ __launch_bounds__(256) void softmax_rows(T *__restrict__ y, const T *
             f[i][e] = Exp<T>::eval(f[i][e] - mx);
             sum += f[i][e];
         }
-    if constexpr (GROUP == kWave) sum = wave_sum(sum);
+    if constexpr (GROUP < kWave) {
+#pragma unroll
+        for (int o = GROUP / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    } else if constexpr (GROUP == kWave) sum = wave_sum(sum);
     else sum = block_allreduce<GROUP / kWave>(sum, smem, wsum, [](CT a, CT b) { return a + b; });
 
     const Normalise<T> norm(sum);
@@ -291,6 +300,36 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_ragged(
     }
 }
 
+// Contiguous rows of up to 32 elements that fit no vectors (two classes, seven experts): one thread per row, the row in
+// registers (64 threads per row left 62 of them idle: 4 M rows of two fp16 elements 732 us).
+template <class T>
+__global__ __launch_bounds__(256) void softmax_tiny(T *__restrict__ y, const T *__restrict__ x, uint64_t rows, uint32_t mid,
+                                                    uint32_t causal_rows) {
+    using CT = typename Compute<T>::type;
+    const uint64_t row = static_cast<uint64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (row >= rows) return;
+    uint32_t keep = mid;
+    if (causal_rows) keep = static_cast<uint32_t>(row % causal_rows) + (mid - causal_rows) + 1;
+    const T *xr = x + row * mid;
+    T *yr = y + row * mid;
+    CT f[32], mx = neg_inf<CT>();
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+        f[e] = static_cast<uint32_t>(e) < keep ? to_compute(xr[e]) : neg_inf<CT>();
+        mx = mx < f[e] ? f[e] : mx;
+    }
+    CT sum = 0;
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+        f[e] = Exp<T>::eval(f[e] - mx);  // (slots beyond the row hold -inf: exactly 0)
+        sum += f[e];
+    }
+    const Normalise<T> norm(sum);
+#pragma unroll
+    for (int e = 0; e < 32; ++e)
+        if (static_cast<uint32_t>(e) < mid) yr[e] = from_compute<T>(static_cast<uint32_t>(e) < keep ? norm(f[e]) : CT(0));
+}
+
 // Any mid / post / alignment: one thread per (pre, post) slice, three passes, neighbouring
 // threads touch neighbouring `post` positions.
 template <class T>
@@ -315,6 +354,47 @@ __global__ __launch_bounds__(256) void softmax_generic(T *__restrict__ y, const 
     for (uint32_t j = keep; j < mid; ++j) y[base + j * post] = from_compute<T>(CT(0));
 }
 
+// An axis that is not the innermost one (post > 1) with a mid worth sharing: a workgroup takes 32 neighbouring
+// (pre, post) slices and SEG threads per slice, which walk mid in steps of SEG (the 32 lanes of a step read
+// neighbouring addresses), keep a running maximum and a sum relative to it (one exponential per element), meet in LDS
+// and walk their elements once more to write.  One thread per slice, as above, left a [4096, 4096] tensor along axis 0
+// to 16 workgroups and 3.7 ms.
+template <class T, int SEG>
+__global__ __launch_bounds__(32 * SEG) void softmax_columns(T *__restrict__ y, const T *__restrict__ x, uint64_t slices,
+                                                            uint32_t mid, uint64_t post) {
+    using CT = typename Compute<T>::type;
+    __shared__ CT sh_m[SEG][32], sh_s[SEG][32];
+    const uint32_t col = threadIdx.x % 32, seg = threadIdx.x / 32;
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 32 + col;
+    const bool live = i < slices;
+    const uint64_t base = live ? (i - i % post) * mid + i % post : 0;
+    CT m = neg_inf<CT>(), sum = 0;
+    if (live) {
+        for (uint32_t j = seg; j < mid; j += SEG) {
+            const CT v = to_compute(x[base + j * post]);
+            if (v > m) {  // (the first finite value lands here: the old sum is 0 and exp(-inf) is 0)
+                sum = sum * Exp<T>::eval(m - v) + CT(1);
+                m = v;
+            } else if (v > neg_inf<CT>()) {
+                sum += Exp<T>::eval(v - m);
+            }
+        }
+    }
+    sh_m[seg][col] = m;
+    sh_s[seg][col] = sum;
+    __syncthreads();
+    CT all_m = neg_inf<CT>(), all_s = 0;
+#pragma unroll
+    for (int k = 0; k < SEG; ++k) all_m = sh_m[k][col] > all_m ? sh_m[k][col] : all_m;
+#pragma unroll
+    for (int k = 0; k < SEG; ++k)
+        if (sh_m[k][col] > neg_inf<CT>()) all_s += sh_s[k][col] * Exp<T>::eval(sh_m[k][col] - all_m);
+    if (!live) return;
+    const Normalise<T> norm(all_s);
+    for (uint32_t j = seg; j < mid; j += SEG)
+        y[base + j * post] = from_compute<T>(norm(Exp<T>::eval(to_compute(x[base + j * post]) - all_m)));
+}
+
 template <class T, int GROUP, int NV>
 void launch_rows(T *y, const T *x, size_t rows, size_t mid, size_t causal_rows, hipStream_t s) {
     constexpr int ROWS_PER_BLOCK = 256 / GROUP;
@@ -332,7 +412,14 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
     const size_t nvec = mid / VEC;
     const bool rows_ok = post == 1 && mid % VEC == 0 && aligned16(y) && aligned16(x) &&
                          (pre + 3) / 4 <= 0x7fffffffu;
-    if (rows_ok && nvec <= 64 * 4) {
+    if (rows_ok && nvec <= 16 && (pre + 15) / 16 <= 0x7fffffffu) {
+        // rows of a few vectors (scores over a handful of experts or classes): 1 to 16 lanes per row instead of 64
+        if (nvec <= 1) launch_rows<T, 1, 1>(y, x, pre, mid, causal_rows, s);
+        else if (nvec <= 2) launch_rows<T, 2, 1>(y, x, pre, mid, causal_rows, s);
+        else if (nvec <= 4) launch_rows<T, 4, 1>(y, x, pre, mid, causal_rows, s);
+        else if (nvec <= 8) launch_rows<T, 8, 1>(y, x, pre, mid, causal_rows, s);
+        else launch_rows<T, 16, 1>(y, x, pre, mid, causal_rows, s);
+    } else if (rows_ok && nvec <= 64 * 4) {
         if (nvec <= 64) launch_rows<T, 64, 1>(y, x, pre, mid, causal_rows, s);
         else if (nvec <= 128) launch_rows<T, 64, 2>(y, x, pre, mid, causal_rows, s);
         else launch_rows<T, 64, 4>(y, x, pre, mid, causal_rows, s);
@@ -349,9 +436,15 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
                                                                              static_cast<uint32_t>(causal_rows));
     } else if (post == 1 && pre <= 0x7fffffffu) {
         const uint32_t m32 = static_cast<uint32_t>(mid), c32 = static_cast<uint32_t>(causal_rows);
-        if (mid <= 2048) softmax_ragged<T, 64><<<static_cast<unsigned>((pre + 3) / 4), 256, 0, s>>>(y, x, pre, m32, c32);
+        if (mid <= 32) softmax_tiny<T><<<static_cast<unsigned>((pre + 255) / 256), 256, 0, s>>>(y, x, pre, m32, c32);
+        else if (mid <= 2048) softmax_ragged<T, 64><<<static_cast<unsigned>((pre + 3) / 4), 256, 0, s>>>(y, x, pre, m32, c32);
         else if (mid <= 32768) softmax_ragged<T, 256><<<static_cast<unsigned>(pre), 256, 0, s>>>(y, x, pre, m32, c32);
         else softmax_ragged<T, 1024><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, pre, m32, c32);
+    } else if (post > 1 && mid >= 32 && causal_rows == 0 && (static_cast<uint64_t>(pre) * post + 31) / 32 <= 0x7fffffffu) {
+        const uint64_t slices = static_cast<uint64_t>(pre) * post;
+        const unsigned grid = static_cast<unsigned>((slices + 31) / 32);
+        if (mid >= 1024) softmax_columns<T, 32><<<grid, 1024, 0, s>>>(y, x, slices, static_cast<uint32_t>(mid), post);
+        else softmax_columns<T, 8><<<grid, 256, 0, s>>>(y, x, slices, static_cast<uint32_t>(mid), post);
     } else {
         const uint64_t slices = static_cast<uint64_t>(pre) * post;
         const uint64_t grid = (slices + 255) / 256;

@@ -52,6 +52,20 @@ def test_rms_norm_f32(shape):
     assert_rel(y, oracle.rms_norm(x, w, 1e-5, threads=8), REL_F32)
 
 
+@pytest.mark.parametrize("rows,cols", [(300, 128), (101, 16), (50, 64), (17, 256), (1000, 8), (7, 32)])
+def test_rms_norm_short_rows_several_to_a_wavefront(rows, cols):
+    # a head's 128 elements (normalisation of queries and keys per head) and shorter rows: 4 to 32 lanes per row
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+    assert_rel(host(ops.rms_norm(dev(x), dev(w), 1e-5)), oracle.rms_norm(x, w, 1e-5, threads=8), REL_F32)
+    xt, wt = dev(x).half(), dev(w).half()
+    ref = oracle.rms_norm(host(xt.float()), host(wt.float()), 1e-5)
+    assert np.max(np.abs(host(ops.rms_norm(xt, wt, 1e-5).float()) - ref)) <= ABS_F16 * max(1.0, np.abs(ref).max() / 2)
+    xd = x.astype(np.float64)
+    assert_rel(host(ops.rms_norm(dev(xd), dev(w.astype(np.float64)), 1e-5)), oracle.rms_norm(xd, w.astype(np.float64), 1e-5), 1e-12)
+
+
 def test_rms_norm_reference_kats():
     # reference tests: iota [2,3,4] with eps 0; x=2, w=3 on [2,3,4096] -> exactly 3
     x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
@@ -102,6 +116,39 @@ def test_softmax_f32(shape, axis):
     x = (3 * rng.standard_normal(shape)).astype(np.float32)
     y = host(ops.softmax(dev(x), axis))
     assert_rel(y, oracle.softmax(x, axis, threads=8), REL_F32)
+
+
+@pytest.mark.parametrize("shape,axis", [((300, 70), 0), ((3, 1100, 40), 1), ((2, 64, 3, 5), 1), ((1500, 2), 0), ((4, 33, 33), 1)])
+def test_softmax_along_an_axis_that_is_not_the_innermost(shape, axis):
+    # 32 slices and 8 or 32 threads per slice to a workgroup; running maximum and sum, -inf among the inputs, a slice
+    # count that is no multiple of 32; float, double and fp16
+    rng = np.random.default_rng(7)
+    x = (3 * rng.standard_normal(shape)).astype(np.float32)
+    x[rng.random(shape) < 0.05] = -np.inf
+    assert_rel(host(ops.softmax(dev(x), axis)), oracle.softmax(x, axis, threads=8), 2 * REL_F32)
+    xd = x.astype(np.float64)
+    assert_rel(host(ops.softmax(dev(xd), axis)), oracle.softmax(xd, axis), 1e-12)
+    x16 = dev(x).half()
+    got = host(ops.softmax(x16, axis).float())
+    assert np.max(np.abs(got - oracle.softmax(host(x16.float()), axis, threads=8))) <= ABS_F16
+
+
+@pytest.mark.parametrize("rows,mid", [(1000, 8), (513, 2), (300, 7), (64, 24), (70, 128), (33, 1), (257, 31), (90, 32), (41, 12)])
+def test_softmax_short_rows(rows, mid):
+    # scores over a handful of experts or classes: 1 to 16 lanes per row where the row is whole vectors, one thread per
+    # row where it is not; plain and causal, float, double and fp16
+    rng = np.random.default_rng(rows + mid)
+    x = (3 * rng.standard_normal((rows, mid))).astype(np.float32)
+    assert_rel(host(ops.softmax(dev(x))), oracle.softmax(x, threads=8), REL_F32)
+    xd = x.astype(np.float64)
+    assert_rel(host(ops.softmax(dev(xd))), oracle.softmax(xd), 1e-12)
+    x16 = dev(x).half()
+    x32 = host(x16.float())
+    assert np.max(np.abs(host(ops.softmax(x16).float()) - oracle.softmax(x32, threads=8))) <= ABS_F16
+    if mid > 1 and rows % mid == 0:
+        sq = x32[:rows // mid * mid].reshape(-1, mid, mid)
+        got = host(ops.softmax(dev(sq).half(), causal=True).float())
+        assert np.max(np.abs(got - oracle.softmax_causal(sq, threads=8))) <= ABS_F16
 
 
 def test_softmax_reference_kat_and_f64():
