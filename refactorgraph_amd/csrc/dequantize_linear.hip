@@ -26,11 +26,13 @@ template <> __device__ __forceinline__ int widen<int8_t>(uint8_t raw) { return s
 // 8-bit input, groups of 4 consecutive elements that share (scalar) or vector-load (per-axis,
 // inner == 1) their scale.  UNROLL groups per thread, 256 lanes apart, so each load/store
 // instruction of a wavefront is contiguous.
-template <class TI, bool PER_AXIS, int UNROLL>
+// PER_AXIS: 0 one scale; 1 the innermost axis carries the scales (a group of 4 takes 4 of them); 2 an axis in front of
+// `inner4` groups of 4 carries them (a group takes one: rows of a weight matrix with a scale each)
+template <class TI, int PER_AXIS, int UNROLL>
 __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const TI *__restrict__ x,
                                                     const float *__restrict__ scale,
                                                     const TI *__restrict__ zp, uint64_t groups,
-                                                    uint32_t axis_len) {
+                                                    uint32_t axis_len, uint32_t inner4) {
     const uint64_t g0 = static_cast<uint64_t>(blockIdx.x) * (256 * UNROLL) + threadIdx.x;
     Bytes4 in[UNROLL];
 #pragma unroll
@@ -41,7 +43,7 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
     }
     float s_scalar = 0.f;
     int z_scalar = 0;
-    if constexpr (!PER_AXIS) {
+    if constexpr (PER_AXIS == 0) {
         s_scalar = scale[0];
         z_scalar = zp ? static_cast<int>(zp[0]) : 0;
     }
@@ -50,7 +52,13 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
         const uint64_t g = g0 + u * 256;
         if (g < groups) {
             Float4 out;
-            if constexpr (PER_AXIS) {
+            if constexpr (PER_AXIS == 2) {
+                const uint32_t a = (static_cast<uint32_t>(g) / inner4) % axis_len;  // (the host keeps groups below 2^32)
+                const float sa = scale[a];
+                const int za = zp ? widen<TI>(reinterpret_cast<const uint8_t *>(zp)[a]) : 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(widen<TI>(in[u].b[e]) - za) * sa;
+            } else if constexpr (PER_AXIS == 1) {
                 const uint32_t a0 = static_cast<uint32_t>((g * 4) % axis_len);
                 const Float4 s = *reinterpret_cast<const Float4 *>(scale + a0);
                 int z[4] = {0, 0, 0, 0};
@@ -75,10 +83,10 @@ __global__ __launch_bounds__(256) void dequant8_vec(float *__restrict__ y, const
 // 32-bit input (the sums of a MatMulInteger), groups of 4 consecutive elements: 16 bytes in, 16 bytes out per lane,
 // UNROLL groups per thread 256 lanes apart.  Same arithmetic, same sharing of the scale as above.
 typedef int i32x4 __attribute__((ext_vector_type(4)));
-template <bool PER_AXIS, int UNROLL>
+template <int PER_AXIS, int UNROLL>
 __global__ __launch_bounds__(256) void dequant32_vec(float *__restrict__ y, const int32_t *__restrict__ x,
                                                      const float *__restrict__ scale, const int32_t *__restrict__ zp,
-                                                     uint64_t groups, uint32_t axis_len) {
+                                                     uint64_t groups, uint32_t axis_len, uint32_t inner4) {
     const uint64_t g0 = static_cast<uint64_t>(blockIdx.x) * (256 * UNROLL) + threadIdx.x;
     i32x4 in[UNROLL];
 #pragma unroll
@@ -88,7 +96,7 @@ __global__ __launch_bounds__(256) void dequant32_vec(float *__restrict__ y, cons
     }
     float s_scalar = 0.f;
     int z_scalar = 0;
-    if constexpr (!PER_AXIS) {
+    if constexpr (PER_AXIS == 0) {
         s_scalar = scale[0];
         z_scalar = zp ? zp[0] : 0;
     }
@@ -97,7 +105,13 @@ __global__ __launch_bounds__(256) void dequant32_vec(float *__restrict__ y, cons
         const uint64_t g = g0 + u * 256;
         if (g < groups) {
             Float4 out;
-            if constexpr (PER_AXIS) {
+            if constexpr (PER_AXIS == 2) {
+                const uint32_t a = (static_cast<uint32_t>(g) / inner4) % axis_len;
+                const float sa = scale[a];
+                const int za = zp ? zp[a] : 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(in[u][e] - za) * sa;
+            } else if constexpr (PER_AXIS == 1) {
                 const uint32_t a0 = static_cast<uint32_t>((g * 4) % axis_len);
                 const Float4 s = *reinterpret_cast<const Float4 *>(scale + a0);
                 i32x4 z = {0, 0, 0, 0};
@@ -139,14 +153,20 @@ int dispatch8(float *y, const void *x_, const float *scale, const void *zp_, siz
     const uint64_t grid = (groups + 256 * UNROLL - 1) / (256 * UNROLL);
     if (base_ok && grid <= 0x7fffffffu) {
         if (!per_axis) {
-            dequant8_vec<TI, false, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
-                y, x, scale, zp, groups, 1);
+            dequant8_vec<TI, 0, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+                y, x, scale, zp, groups, 1, 1);
             return launch_status();
         }
         if (inner == 1 && axis_len % 4 == 0 && aligned16(scale) &&
             (!zp || (reinterpret_cast<uintptr_t>(zp) & 3u) == 0) && axis_len <= 0xffffffffu) {
-            dequant8_vec<TI, true, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
-                y, x, scale, zp, groups, static_cast<uint32_t>(axis_len));
+            dequant8_vec<TI, 1, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+                y, x, scale, zp, groups, static_cast<uint32_t>(axis_len), 1);
+            return launch_status();
+        }
+        // the scales belong to an axis in front of runs of whole groups (per-row scales of a weight matrix)
+        if (inner % 4 == 0 && groups <= 0xffffffffu && axis_len <= 0xffffffffu && inner / 4 <= 0xffffffffu) {
+            dequant8_vec<TI, 2, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+                y, x, scale, zp, groups, static_cast<uint32_t>(axis_len), static_cast<uint32_t>(inner / 4));
             return launch_status();
         }
     }
@@ -168,12 +188,17 @@ int dispatch_wide(float *y, const void *x, const float *scale, const void *zp, s
             auto *xi = static_cast<const int32_t *>(x);
             auto *zi = static_cast<const int32_t *>(zp);
             if (!per_axis) {
-                dequant32_vec<false, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups, 1);
+                dequant32_vec<0, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups, 1, 1);
                 return launch_status();
             }
             if (inner == 1 && axis_len % 4 == 0 && aligned16(scale) && (!zp || aligned16(zp)) && axis_len <= 0xffffffffu) {
-                dequant32_vec<true, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups,
-                                                                                         static_cast<uint32_t>(axis_len));
+                dequant32_vec<1, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups,
+                                                                                      static_cast<uint32_t>(axis_len), 1);
+                return launch_status();
+            }
+            if (inner % 4 == 0 && groups <= 0xffffffffu && axis_len <= 0xffffffffu && inner / 4 <= 0xffffffffu) {
+                dequant32_vec<2, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+                    y, xi, scale, zi, groups, static_cast<uint32_t>(axis_len), static_cast<uint32_t>(inner / 4));
                 return launch_status();
             }
         }

@@ -363,7 +363,7 @@ def test_dequantize_reference_kat():
 
 @pytest.mark.parametrize("dt", [np.uint8, np.int8, np.int16, np.int32])
 @pytest.mark.parametrize("shape,axis", [((4096,), 0), ((3, 5, 4), 1), ((16, 64), 1), ((7, 33), 1), ((8, 12, 6), 0),
-                                        ((256, 1024), 1)])
+                                        ((256, 1024), 1), ((300, 1024), 0), ((5, 7, 128), 1), ((6, 40, 10), 0)])
 def test_dequantize_bit_exact(dt, shape, axis):
     rng = np.random.default_rng(7)
     info = np.iinfo(dt)
