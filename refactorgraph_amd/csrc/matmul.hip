@@ -768,16 +768,28 @@ __global__ __launch_bounds__(256) void mm_skinny(T *__restrict__ y, const T *__r
         }
     };
 
+    // No branch around a load while the ring is full: with loads under a branch the compiler's wait for one tile
+    // becomes a wait for every tile in flight.  The first loads take the last tile again where the wavefront has
+    // fewer than SK_DEPTH of them; the branches are left to the last two rounds.
     Tile tile[SK_DEPTH];
+    if (t0 < t1) {
 #pragma unroll
-    for (int i = 0; i < SK_DEPTH; ++i)
-        if (t0 + i < t1) load(tile[i], t0 + i);
-    for (uint32_t t = t0; t < t1; t += SK_DEPTH) {
+        for (int i = 0; i < SK_DEPTH; ++i) load(tile[i], t0 + i < t1 ? t0 + i : t1 - 1);
+        uint32_t t = t0;
+        for (; t + 2 * SK_DEPTH <= t1; t += SK_DEPTH) {
 #pragma unroll
-        for (int i = 0; i < SK_DEPTH; ++i) {
-            if (t + i < t1) {
+            for (int i = 0; i < SK_DEPTH; ++i) {
                 multiply(tile[i]);
-                if (t + i + SK_DEPTH < t1) load(tile[i], t + i + SK_DEPTH);
+                load(tile[i], t + i + SK_DEPTH);
+            }
+        }
+        for (; t < t1; t += SK_DEPTH) {
+#pragma unroll
+            for (int i = 0; i < SK_DEPTH; ++i) {
+                if (t + i < t1) {
+                    multiply(tile[i]);
+                    if (t + i + SK_DEPTH < t1) load(tile[i], t + i + SK_DEPTH);
+                }
             }
         }
     }

@@ -669,10 +669,20 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[sl][j][e] = 0;
 
+    // B's zero points of a tile's k-steps are loaded with its A fragments, without a branch (a load under a branch
+    // turns the compiler's wait for it into a wait for everything in flight): without zero points the loads read
+    // bytes of B and are masked away; a scalar one is read once
+    const uint8_t *zb_base = b_zp && zb.per_row ? zb.ptr + bm * k : B;
+    const uint32_t zb_keep = b_zp && zb.per_row ? 0xffffffffu : 0u;
+    const uint32_t zb_scalar = b_zp && !zb.per_row ? splat(zb.ptr[0]) : 0u;
     load_b(t_first);
-    for (uint32_t t = t_first; t < t_end; ++t) {
+    // (the next tile's load has no branch around it either: the last tile takes a body of its own)
+    auto tile_step = [&](uint32_t t, auto more) {
         const uint32_t k0 = t * BK;
         v4i fa[SLABS][4];
+        u32x4 zk[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) __builtin_memcpy(&zk[ks], zb_base + k0 + 32 * ks + 16 * h, 16);  // (any alignment)
 #pragma unroll
         for (int sl = 0; sl < SLABS; ++sl)
 #pragma unroll
@@ -682,7 +692,7 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
         for (int i = 0; i < 8; ++i)
             *reinterpret_cast<u32x4 *>(tile + (16 * i + (tid >> 4)) * SK_PITCH + 16 * (tid & 15)) = w[i];
         __syncthreads();
-        if (t + 1 < t_end) load_b(t + 1);  // in flight while this tile is multiplied
+        if constexpr (decltype(more)::value) load_b(t + 1);  // in flight while this tile is multiplied
         if (za.ptr) {
 #pragma unroll
             for (int sl = 0; sl < SLABS; ++sl)
@@ -696,11 +706,9 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
         // transposing reads of 8 k each; lane a of a group of 16 addresses k-row a / 2, columns 8 (a % 2) .. + 7
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            uint32_t z[4] = {0, 0, 0, 0};
-            if (b_zp) {
-                if (zb.per_row) __builtin_memcpy(z, zb.ptr + bm * k + k0 + 32 * ks + 16 * h, 16);
-                else z[0] = z[1] = z[2] = z[3] = splat(zb.ptr[0]);
-            }
+            uint32_t z[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) z[e] = (zk[ks][e] & zb_keep) | zb_scalar;
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const uint32_t cols = 64 * wave + 32 * j + 16 * ((lane >> 4) & 1);
@@ -718,7 +726,9 @@ __global__ __launch_bounds__(256) void mmi_skinny(int32_t *__restrict__ y, const
             }
         }
         __syncthreads();  // the tile is rewritten
-    }
+    };
+    for (uint32_t t = t_first; t + 1 < t_end; ++t) tile_step(t, std::true_type{});
+    tile_step(t_end - 1, std::false_type{});
     // accumulator: column lane % 32 of the block, register e holds row 8 (e / 4) + 4 h + e % 4
     int32_t *Y = y + (ym * m + row_first) * n + col0 + 64 * wave;
 #pragma unroll
