@@ -127,6 +127,55 @@ __global__ __launch_bounds__(256) void dequant32_vec(float *__restrict__ y, cons
     }
 }
 
+// 16-bit input, groups of 4 consecutive elements: 8 bytes in, 16 bytes out per lane.  Same arithmetic, same sharing of the
+// scale (PER_AXIS as above).
+template <class TI, int PER_AXIS, int UNROLL>
+__global__ __launch_bounds__(256) void dequant16_vec(float *__restrict__ y, const TI *__restrict__ x,
+                                                     const float *__restrict__ scale, const TI *__restrict__ zp,
+                                                     uint64_t groups, uint32_t axis_len, uint32_t inner4) {
+    struct alignas(8) Elems4 {
+        TI v[4];
+    };
+    const uint64_t g0 = static_cast<uint64_t>(blockIdx.x) * (256 * UNROLL) + threadIdx.x;
+    Elems4 in[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g = g0 + u * 256;
+        if (g < groups) in[u] = __builtin_bit_cast(Elems4, __builtin_nontemporal_load(reinterpret_cast<const uint64_t *>(x + g * 4)));
+    }
+    float s_scalar = 0.f;
+    int z_scalar = 0;
+    if constexpr (PER_AXIS == 0) {
+        s_scalar = scale[0];
+        z_scalar = zp ? static_cast<int>(zp[0]) : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t g = g0 + u * 256;
+        if (g < groups) {
+            Float4 out;
+            if constexpr (PER_AXIS == 2) {
+                const uint32_t a = (static_cast<uint32_t>(g) / inner4) % axis_len;  // (the host keeps groups below 2^32)
+                const float sa = scale[a];
+                const int za = zp ? static_cast<int>(zp[a]) : 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(static_cast<int>(in[u].v[e]) - za) * sa;
+            } else if constexpr (PER_AXIS == 1) {
+                const uint32_t a0 = static_cast<uint32_t>((g * 4) % axis_len);
+                const Float4 s = *reinterpret_cast<const Float4 *>(scale + a0);
+                Elems4 z = {};
+                if (zp) z = *reinterpret_cast<const Elems4 *>(zp + a0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(static_cast<int>(in[u].v[e]) - static_cast<int>(z.v[e])) * s.v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out.v[e] = static_cast<float>(static_cast<int>(in[u].v[e]) - z_scalar) * s_scalar;
+            }
+            __builtin_nontemporal_store(__builtin_bit_cast(f32x4, out), reinterpret_cast<f32x4 *>(y + g * 4));
+        }
+    }
+}
+
 // Every other case: one element per thread-iteration.
 template <class TI>
 __global__ __launch_bounds__(256) void dequant_generic(float *__restrict__ y, const TI *__restrict__ x,
@@ -198,6 +247,30 @@ int dispatch_wide(float *y, const void *x, const float *scale, const void *zp, s
             }
             if (inner % 4 == 0 && groups <= 0xffffffffu && axis_len <= 0xffffffffu && inner / 4 <= 0xffffffffu) {
                 dequant32_vec<2, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
+                    y, xi, scale, zi, groups, static_cast<uint32_t>(axis_len), static_cast<uint32_t>(inner / 4));
+                return launch_status();
+            }
+        }
+    }
+    if constexpr (sizeof(TI) == 2) {
+        constexpr int UNROLL = 4;
+        const uint64_t groups = n / 4;
+        const uint64_t grid = (groups + 256 * UNROLL - 1) / (256 * UNROLL);
+        auto *xi = static_cast<const TI *>(x);
+        auto *zi = static_cast<const TI *>(zp);
+        if (n % 4 == 0 && aligned16(y) && (reinterpret_cast<uintptr_t>(x) & 7u) == 0 && grid <= 0x7fffffffu) {
+            if (!per_axis) {
+                dequant16_vec<TI, 0, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups, 1, 1);
+                return launch_status();
+            }
+            if (inner == 1 && axis_len % 4 == 0 && aligned16(scale) && (!zp || (reinterpret_cast<uintptr_t>(zp) & 7u) == 0) &&
+                axis_len <= 0xffffffffu) {
+                dequant16_vec<TI, 1, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(y, xi, scale, zi, groups,
+                                                                                          static_cast<uint32_t>(axis_len), 1);
+                return launch_status();
+            }
+            if (inner % 4 == 0 && groups <= 0xffffffffu && axis_len <= 0xffffffffu && inner / 4 <= 0xffffffffu) {
+                dequant16_vec<TI, 2, UNROLL><<<static_cast<unsigned>(grid), 256, 0, s>>>(
                     y, xi, scale, zi, groups, static_cast<uint32_t>(axis_len), static_cast<uint32_t>(inner / 4));
                 return launch_status();
             }
