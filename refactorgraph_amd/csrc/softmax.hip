@@ -330,6 +330,77 @@ __global__ __launch_bounds__(256) void softmax_tiny(T *__restrict__ y, const T *
         if (static_cast<uint32_t>(e) < mid) yr[e] = from_compute<T>(static_cast<uint32_t>(e) < keep ? norm(f[e]) : CT(0));
 }
 
+// A few very long contiguous rows (logits over a vocabulary): one workgroup per row leaves the chip idle (a row of
+// 128256 floats 47 us).  The row is cut into chunks, one workgroup each, in three launches that need no workspace:
+// (1) a chunk's maximum and its sum relative to it go, as two floats, into the first 8 bytes of the chunk's place in
+// y; (2) one workgroup per row combines them and writes the row's maximum and sum into every chunk's first 8 bytes;
+// (3) a chunk reads its 8 bytes, then its elements of x, and writes its outputs over them.  Only for y and x that
+// do not overlap (in place, step 1 would destroy inputs).  CT is float for every T but double.
+constexpr int kChunkThreads = 1024;
+
+template <class T>
+__global__ __launch_bounds__(kChunkThreads) void softmax_chunk_stats(T *__restrict__ y, const T *__restrict__ x, uint32_t mid,
+                                                                     uint32_t chunk) {
+    using CT = typename Compute<T>::type;
+    __shared__ CT smem[kChunkThreads / kWave];
+    const uint64_t row = blockIdx.y;
+    const uint32_t c0 = blockIdx.x * chunk, c1 = blockIdx.x + 1 == gridDim.x ? mid : c0 + chunk;  // (the last chunk takes the rest)
+    const T *xr = x + row * mid;
+    CT m = neg_inf<CT>();
+    for (uint32_t j = c0 + threadIdx.x; j < c1; j += kChunkThreads) {
+        const CT v = to_compute(xr[j]);
+        m = m < v ? v : m;
+    }
+    m = block_allreduce<kChunkThreads / kWave>(m, smem, [](CT v) { return wave_max(v); }, [](CT a, CT b) { return a < b ? b : a; });
+    CT sum = 0;
+    if (m > neg_inf<CT>())
+        for (uint32_t j = c0 + threadIdx.x; j < c1; j += kChunkThreads) sum += Exp<T>::eval(to_compute(xr[j]) - m);
+    sum = block_allreduce<kChunkThreads / kWave>(sum, smem, [](CT v) { return wave_sum(v); }, [](CT a, CT b) { return a + b; });
+    if (threadIdx.x == 0) {
+        const float pair[2] = {static_cast<float>(m), static_cast<float>(sum)};
+        __builtin_memcpy(reinterpret_cast<char *>(y + row * mid + c0), pair, 8);  // (any alignment)
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void softmax_chunk_combine(T *__restrict__ y, uint32_t mid, uint32_t chunk, uint32_t chunks) {
+    __shared__ float smem[4];
+    const uint64_t row = blockIdx.x;
+    char *yr = reinterpret_cast<char *>(y + row * mid);
+    float m = -__builtin_inff();
+    for (uint32_t c = threadIdx.x; c < chunks; c += 256) {
+        float pair[2];
+        __builtin_memcpy(pair, yr + static_cast<uint64_t>(c) * chunk * sizeof(T), 8);
+        m = fmaxf(m, pair[0]);
+    }
+    m = block_allreduce<4>(m, smem, [](float v) { return wave_max(v); }, [](float a, float b) { return fmaxf(a, b); });
+    float sum = 0.f;
+    for (uint32_t c = threadIdx.x; c < chunks; c += 256) {
+        float pair[2];
+        __builtin_memcpy(pair, yr + static_cast<uint64_t>(c) * chunk * sizeof(T), 8);
+        if (pair[0] > -__builtin_inff()) sum += pair[1] * expf(pair[0] - m);
+    }
+    sum = block_allreduce<4>(sum, smem, [](float v) { return wave_sum(v); }, [](float a, float b) { return a + b; });
+    const float pair[2] = {m, sum};
+    for (uint32_t c = threadIdx.x; c < chunks; c += 256) __builtin_memcpy(yr + static_cast<uint64_t>(c) * chunk * sizeof(T), pair, 8);
+}
+
+template <class T>
+__global__ __launch_bounds__(kChunkThreads) void softmax_chunk_write(T *__restrict__ y, const T *__restrict__ x, uint32_t mid,
+                                                                     uint32_t chunk) {
+    using CT = typename Compute<T>::type;
+    const uint64_t row = blockIdx.y;
+    const uint32_t c0 = blockIdx.x * chunk, c1 = blockIdx.x + 1 == gridDim.x ? mid : c0 + chunk;  // (the last chunk takes the rest)
+    const T *xr = x + row * mid;
+    T *yr = y + row * mid;
+    float pair[2];
+    __builtin_memcpy(pair, reinterpret_cast<const char *>(yr + c0), 8);
+    __syncthreads();  // everybody has the row's maximum and sum before the first output lands on them
+    const CT m = static_cast<CT>(pair[0]);
+    const Normalise<T> norm(static_cast<CT>(pair[1]));
+    for (uint32_t j = c0 + threadIdx.x; j < c1; j += kChunkThreads) yr[j] = from_compute<T>(norm(Exp<T>::eval(to_compute(xr[j]) - m)));
+}
+
 // Any mid / post / alignment: one thread per (pre, post) slice, three passes, neighbouring
 // threads touch neighbouring `post` positions.
 template <class T>
@@ -410,6 +481,29 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
     auto *x = static_cast<const T *>(x_);
     constexpr size_t VEC = Vec16<T>::N;
     const size_t nvec = mid / VEC;
+    // a few very long rows: chunks of a row to a workgroup each (not for double: the chunk results travel as floats)
+    if (post == 1 && causal_rows == 0 && sizeof(T) <= 4 && mid >= 32768 && mid <= 0xffffffffu && pre * (mid / 8192) <= 2048 && pre <= 65535) {
+        const char *xb = reinterpret_cast<const char *>(x), *yb = reinterpret_cast<const char *>(y);
+        const size_t bytes = pre * mid * sizeof(T);
+        const bool apart = xb + bytes <= yb || yb + bytes <= xb;
+        size_t chunks = 512 / pre;
+        if (chunks > mid / 4096) chunks = mid / 4096;
+        if (apart && chunks >= 4) {
+            // chunks of a multiple of 8 elements; the last one takes what is left (never less than a chunk, so that
+            // its first 8 bytes are its own)
+            const uint32_t chunk = static_cast<uint32_t>(mid / chunks) / 8 * 8;
+            const uint32_t n_chunks = static_cast<uint32_t>(mid / chunk);
+            const dim3 grid(n_chunks, static_cast<unsigned>(pre));
+            softmax_chunk_stats<T><<<grid, kChunkThreads, 0, s>>>(y, x, static_cast<uint32_t>(mid), chunk);
+            int rc = launch_status();
+            if (rc) return rc;
+            softmax_chunk_combine<T><<<static_cast<unsigned>(pre), 256, 0, s>>>(y, static_cast<uint32_t>(mid), chunk, n_chunks);
+            rc = launch_status();
+            if (rc) return rc;
+            softmax_chunk_write<T><<<grid, kChunkThreads, 0, s>>>(y, x, static_cast<uint32_t>(mid), chunk);
+            return launch_status();
+        }
+    }
     const bool rows_ok = post == 1 && mid % VEC == 0 && aligned16(y) && aligned16(x) &&
                          (pre + 3) / 4 <= 0x7fffffffu;
     if (rows_ok && nvec <= 16 && (pre + 15) / 16 <= 0x7fffffffu) {

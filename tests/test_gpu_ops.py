@@ -151,6 +151,25 @@ def test_softmax_short_rows(rows, mid):
         assert np.max(np.abs(got - oracle.softmax_causal(sq, threads=8))) <= ABS_F16
 
 
+@pytest.mark.parametrize("shape", [(1, 70001), (3, 32768), (2, 1, 40001), (16, 50257)])
+def test_softmax_few_very_long_rows_in_chunks(shape):
+    # logits over a vocabulary: the rows are cut into chunks, a workgroup each, whose maxima and sums travel through the
+    # first bytes of the chunks' places in the output (three launches); in place the one-workgroup kernel stays
+    rng = np.random.default_rng(shape[-1])
+    x = (3 * rng.standard_normal(shape)).astype(np.float32)
+    x.reshape(-1)[7] = -np.inf
+    ref = oracle.softmax(x.astype(np.float64), threads=8)
+    y = host(ops.softmax(dev(x)))
+    assert not np.isnan(y).any()
+    assert_rel(y, ref, 2 * REL_F32)
+    z = dev(x)
+    assert_rel(host(ops.softmax(z, out=z)), ref, 2 * REL_F32)
+    for dt, tol in ((torch.float16, ABS_F16), (torch.bfloat16, 2e-2)):
+        xt = dev(x).to(dt)
+        got = host(ops.softmax(xt).float())
+        assert np.max(np.abs(got - oracle.softmax(host(xt.float()), threads=8))) <= tol
+
+
 def test_softmax_reference_kat_and_f64():
     x = np.zeros((2, 3, 2, 4), np.float64)
     assert np.all(host(ops.softmax(dev(x), 1)) == 1.0 / 3)
