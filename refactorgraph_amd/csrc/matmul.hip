@@ -496,7 +496,12 @@ __global__ __launch_bounds__(256, 2) void mm_tiles16(T *__restrict__ y, const T 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
-    const uint32_t row0 = blockIdx.y * TM, col0 = blockIdx.x * HT;
+    // Tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so each XCD gets a contiguous run of tiles,
+    // walked down the rows of one column panel after the other: the workgroups of an XCD share a panel of B in its L2.
+    const uint32_t row_tiles = (m + TM - 1) / TM, n_tiles = row_tiles * ((n + HT - 1) / HT);
+    uint32_t tile = blockIdx.x;
+    if (n_tiles % 8 == 0) tile = (tile % 8) * (n_tiles / 8) + tile / 8;
+    const uint32_t row0 = (tile % row_tiles) * TM, col0 = (tile / row_tiles) * HT;
     const uint16_t *A = reinterpret_cast<const uint16_t *>(a) + am * m * static_cast<uint64_t>(k);
     const uint16_t *B = reinterpret_cast<const uint16_t *>(b) + bm * static_cast<uint64_t>(k) * n;
 
@@ -1550,8 +1555,9 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
             // tiles of 64 rows while those of 128 would leave half of the CUs without one
             const bool half = ((m + HT - 1) / HT) * ((n + HT - 1) / HT) * count <= kHalfTiles;
             const size_t tm = half ? HT / 2 : HT;
-            const dim3 grid(static_cast<unsigned>((n + HT - 1) / HT), static_cast<unsigned>((m + tm - 1) / tm), count);
-            if (grid.y > 65535) return RG_HIP_E_UNSUPPORTED;
+            const uint64_t tiles = ((m + tm - 1) / tm) * ((n + HT - 1) / HT);
+            if (tiles > 0x7fffffffu) return RG_HIP_E_UNSUPPORTED;
+            const dim3 grid(static_cast<unsigned>(tiles), 1, count);
             const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
             const bool vec = n % 8 == 0 && n >= 8 && aligned16(b);
 #define RG_TILES16(TB, VEC)                                                                                              \
@@ -1736,7 +1742,8 @@ extern "C" int rg_hip_matmul(void *y, const void *a, const void *b, const void *
     Bias bias{c, c_stride_batch, c_stride_m, c_stride_n};
     // One B for consecutive matrices of A (activations [batch, m, k] against weights): the batch is more rows of one
     // product, not `batch` launches that each read B again (64 x [1,4096] against [4096,4096]: 337 -> 12 us).
-    if (batch > 1 && b_index && !trans_a && batch * m <= 0x7fffffffu && (!c || c_stride_batch == m * c_stride_m)) {
+    // (up to 2^20 rows: every kernel's grid takes that many)
+    if (batch > 1 && b_index && !trans_a && batch * m <= (1u << 20) && (!c || c_stride_batch == m * c_stride_m)) {
         bool fold = true;
         for (size_t i = 0; i < batch && fold; ++i)
             fold = b_index[i] == b_index[0] && (a_index ? a_index[i] == a_index[0] + i : true);

@@ -472,7 +472,12 @@ __global__ __launch_bounds__(256, 2) void mmi_tiles(int32_t *__restrict__ y, con
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
-    const uint32_t row0 = blockIdx.y * GT, col0 = blockIdx.x * GT;
+    // Tile order: consecutive workgroup ids go round-robin to the 8 XCDs, so each XCD gets a contiguous run of tiles,
+    // walked down the rows of one column panel after the other: the workgroups of an XCD share a panel of B in its L2.
+    const uint32_t row_tiles = (m + GT - 1) / GT, n_tiles = row_tiles * ((n + GT - 1) / GT);
+    uint32_t tile_id = blockIdx.x;
+    if (n_tiles % 8 == 0) tile_id = (tile_id % 8) * (n_tiles / 8) + tile_id / 8;
+    const uint32_t row0 = (tile_id % row_tiles) * GT, col0 = (tile_id / row_tiles) * GT;
     const uint8_t *A = a + am * m * static_cast<uint64_t>(k);
     const uint8_t *B = b + bm * static_cast<uint64_t>(k) * n;
 
@@ -915,7 +920,8 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
     // One B for consecutive matrices of A (activations [batch, m, k] against weights): the batch is more rows of one
     // product, not `batch` launches that each read B again.  The zero points per (matrix, row) follow: A's are
     // consecutive like its rows, B's are those of the one matrix.
-    if (batch > 1 && b_index && batch * m <= 0x7fffffffu) {
+    // (up to 2^20 rows: every kernel's grid takes that many)
+    if (batch > 1 && b_index && batch * m <= (1u << 20)) {
         bool fold = true;
         for (size_t i = 0; i < batch && fold; ++i)
             fold = b_index[i] == b_index[0] && (a_index ? a_index[i] == a_index[0] + i : true);
@@ -1012,7 +1018,7 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         return small_us < large_us;
     };
     auto launch_small_tiles = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
-        const dim3 grid(static_cast<unsigned>((n + GT - 1) / GT), static_cast<unsigned>((m + GT - 1) / GT), count);
+        const dim3 grid(static_cast<unsigned>(((m + GT - 1) / GT) * ((n + GT - 1) / GT)), 1, count);
         const auto *a8 = static_cast<const uint8_t *>(a);
         const auto *b8 = static_cast<const uint8_t *>(b);
         const uint32_t m32 = static_cast<uint32_t>(m), k32 = static_cast<uint32_t>(k), n32 = static_cast<uint32_t>(n);
@@ -1020,7 +1026,7 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         else mmi_tiles<DEQ, false><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
         return launch_status();
     };
-    const bool small_tiles_ok = k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && (m + GT - 1) / GT <= 65535;
+    const bool small_tiles_ok = k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && ((m + GT - 1) / GT) * ((n + GT - 1) / GT) <= 0x7fffffffu;
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if (small_tiles_ok && (short_tile || (fast && !gemv && !skinny)) && small_tiles_pay(short_tile, count))
