@@ -1371,6 +1371,19 @@ def test_matmul_one_b_for_the_whole_batch(m, k, n):
     assert np.array_equal(y, oracle.dequantize_linear(ref, scale, None, axis=2))
 
 
+def test_matmul_one_b_for_a_batch_of_many_small_matrices():
+    # 3000 matrices of 24 rows against one [64, 40] matrix: 72000 rows of one product (1125 tiles of 64 rows)
+    rng = np.random.default_rng(52)
+    a = rng.integers(-2, 3, (3000, 24, 64)).astype(np.float32)
+    b = rng.integers(-2, 3, (1, 64, 40)).astype(np.float32)
+    want = (a.astype(np.int64) @ b[0].astype(np.int64)).astype(np.float32)
+    assert np.array_equal(host(ops.matmul(dev(a).half(), dev(b).half()).float()), want)
+    ai = rng.integers(0, 256, (3000, 24, 64), dtype=np.uint8)
+    bi = rng.integers(-128, 128, (1, 64, 40), dtype=np.int8)
+    az = rng.integers(0, 256, (3000 * 24,), dtype=np.uint8)
+    assert np.array_equal(host(ops.matmul_integer(dev(ai), dev(bi), dev(az), None)), oracle.matmul_integer(ai, bi, az, None, threads=8))
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
