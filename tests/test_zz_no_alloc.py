@@ -67,6 +67,19 @@ def test_static_scratch_entry_matches_the_workspace_entry_twice():
         assert float((o.float() - ro.float()).abs().max()) <= ABS_F16
 
 
+def test_static_scratch_entry_with_a_long_cache_and_few_query_tiles():
+    # a prompt chunk against a long cache: the tiled kernel shares an item's keys between workgroups as far as the
+    # library's 2 MiB of scratch hold their records (fewer ranges than with the caller's workspace), then a call
+    # whose records do not fit at all; same results either way
+    scale = 1 / math.sqrt(128)
+    for t in (_inputs(1, 32, 8, 64, 4160, 128, [4000], seed=3), _inputs(2, 32, 8, 100, 3100, 128, [3000, 5], seed=4),
+              _inputs(1, 8, 2, 16, 2064, 128, [2048], seed=5)):
+        o, kc, vc = _static(t, scale)
+        ro, rkc, rvc = _existing(t, scale)
+        assert torch.equal(kc, rkc) and torch.equal(vc, rvc)
+        assert float((o.float() - ro.float()).abs().max()) <= ABS_F16
+
+
 def test_static_scratch_entry_refuses_what_the_workspace_entry_refuses():
     d = torch.zeros(4096, device=DEV, dtype=torch.float16)
     p = d.data_ptr()
