@@ -1164,7 +1164,13 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
     const uint32_t bz = blockIdx.z;
     const uint64_t am = a_matrix0 + bz, bm = b_matrix0 + bz, ym = y_matrix0 + bz;
     const uint32_t pieces = k / 8;  // 16-byte pieces of a row
-    const uint32_t row0 = (blockIdx.x * (blockDim.x / 64) + wave) * R;
+    // A workgroup walks several blocks of rows of W when there are more blocks than the launch has workgroups (a
+    // vocabulary's worth of rows): A is copied into LDS once, not once per 16 rows (the short-lived workgroups of
+    // one block each left [1,4096] x [32000,4096]^T at 2.7 TB/s).
+    const uint32_t row_blocks = (n + (blockDim.x / 64) * R - 1) / ((blockDim.x / 64) * R);
+    bool a_in_lds = false;
+    for (uint32_t rb = blockIdx.x; rb < row_blocks; rb += gridDim.x) {
+    const uint32_t row0 = (rb * (blockDim.x / 64) + wave) * R;
 
     const u32x4 *W[R];
 #pragma unroll
@@ -1187,45 +1193,66 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
         const uint32_t len = !LONG ? pieces : pieces - p0 < segment ? pieces - p0 : segment;
         const uint32_t steps = (len + 63) / 64;  // a wavefront covers 64 pieces per step
         u32x4 buf[DEPTH][R];
+        // No branch around a load (with one, the compiler's wait for one step becomes a wait for every step in flight):
+        // lanes and steps beyond the row's end fetch its last piece again and are left out of the products.
         auto load = [&](int slot, uint32_t step) {
-            const uint32_t c = step * 64 + lane;
+            step = step < steps ? step : steps - 1;
+            uint32_t c = step * 64 + lane;
+            c = c < len ? c : len - 1;
 #pragma unroll
-            for (int j = 0; j < R; ++j)
-                if (c < len) buf[slot][j] = __builtin_nontemporal_load(W[j] + p0 + c);
+            for (int j = 0; j < R; ++j) buf[slot][j] = __builtin_nontemporal_load(W[j] + p0 + c);
         };
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d)
-            if (static_cast<uint32_t>(d) < steps) load(d, d);
+        for (int d = 0; d < DEPTH; ++d) load(d, d);
 
         // A into LDS while the first pieces of W are on their way; rows beyond m are zero
-        if (LONG && p0) __syncthreads();  // everybody has finished with the segment before
+        if (LONG || !a_in_lds) {
+            if (LONG && (p0 || a_in_lds)) __syncthreads();  // everybody has finished with the segment before
 #pragma unroll
-        for (int i = 0; i < M; ++i)
-            for (uint32_t c = tid; c < len; c += blockDim.x) {
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (static_cast<uint32_t>(i) < m) v = A[static_cast<uint64_t>(i) * pieces + p0 + c];
-                sa[i * len + c] = v;
-            }
-        __syncthreads();
+            for (int i = 0; i < M; ++i)
+                for (uint32_t c = tid; c < len; c += blockDim.x) {
+                    u32x4 v = {0u, 0u, 0u, 0u};
+                    if (static_cast<uint32_t>(i) < m) v = A[static_cast<uint64_t>(i) * pieces + p0 + c];
+                    sa[i * len + c] = v;
+                }
+            __syncthreads();
+            a_in_lds = true;
+        }
 
-        for (uint32_t s = 0; s < steps; s += DEPTH) {
+        auto multiply = [&](int d, uint32_t step) {
+            const uint32_t c = step * 64 + lane;
+            if (step < steps && c < len) {
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
-                if (s + d < steps) {
-                    const uint32_t c = (s + d) * 64 + lane;
-                    if (c < len) {
+                for (int i = 0; i < M; ++i) {
+                    const u32x4 av = sa[i * len + c];
 #pragma unroll
-                        for (int i = 0; i < M; ++i) {
-                            const u32x4 av = sa[i * len + c];
+                    for (int j = 0; j < R; ++j)
 #pragma unroll
-                            for (int j = 0; j < R; ++j)
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) acc[j][i] = dot2<T>(buf[d][j][e], av[e], acc[j][i]);
-                        }
-                    }
-                    if (s + d + DEPTH < steps) load(d, s + d + DEPTH);
+                        for (int e = 0; e < 4; ++e) acc[j][i] = dot2<T>(buf[d][j][e], av[e], acc[j][i]);
                 }
             }
+        };
+        auto last_round = [&](uint32_t s) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) multiply(d, s + d);
+        };
+        uint32_t s = 0;
+        for (; s + 2 * DEPTH <= steps; s += DEPTH) {  // the ring stays full
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                multiply(d, s + d);
+                load(d, s + d + DEPTH);
+            }
+        }
+        if (s + DEPTH < steps) {  // one more round with loads (some of them beyond the end), then the last one
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                multiply(d, s + d);
+                load(d, s + d + DEPTH);
+            }
+            last_round(s + DEPTH);
+        } else {
+            last_round(s);
         }
     } while (LONG && (p0 += segment) < pieces);
 
@@ -1249,6 +1276,7 @@ __global__ __launch_bounds__(1024) void mm_gemv(T *__restrict__ y, const T *__re
             y[(ym * m + i) * n + col] = down<T>(v);
         }
     }
+    }  // row blocks
 }
 
 // ---------------------------------------------------------------- one to four rows of A, B as [k, n]
@@ -1450,6 +1478,7 @@ int launch_rows_kn(T *y, const T *a, const T *b, Bias bias, uint32_t rows, uint3
 }
 
 constexpr uint32_t GV_LDS_BYTES = 64 * 1024;  // of A per workgroup at most
+constexpr uint32_t kGemvMaxGrid = 512;     // workgroups of a launch: two per CU
 
 template <class T, int M>
 int launch_gemv(T *y, const T *a, const T *w, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
@@ -1461,7 +1490,9 @@ int launch_gemv(T *y, const T *a, const T *w, Bias bias, uint32_t m, uint32_t k,
     // the wavefronts of a workgroup share one copy of A: as many as still leave a workgroup for every CU
     uint32_t waves = 16;
     while (waves > 4 && static_cast<uint64_t>((n + waves * R - 1) / (waves * R)) * count < 256) waves /= 2;
-    const dim3 grid((n + waves * R - 1) / (waves * R), 1, count);
+    uint32_t blocks = (n + waves * R - 1) / (waves * R);
+    if (blocks > kGemvMaxGrid) blocks = kGemvMaxGrid;  // (the rest of the row blocks in turns)
+    const dim3 grid(blocks, 1, count);
     if (segment == k / 8) mm_gemv<T, M, R, false><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, segment, alpha, beta, am0, bm0, ym0);
     else mm_gemv<T, M, R, true><<<grid, 64 * waves, lds, s>>>(y, a, w, bias, m, k, n, segment, alpha, beta, am0, bm0, ym0);
     return launch_status();
@@ -1500,8 +1531,9 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 
     // two to sixteen rows, weights as [n, k]: operands straight from global memory into 4x4x4 block products
     // (a single row too when k is long: the matrix-vector kernel keeps a whole row of W per wavefront in flight,
-    // which stops paying beyond 16 KiB)
-    const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
+    // which stops paying beyond 16 KiB; and against a vocabulary's worth of short rows, where a wavefront of that
+    // kernel ends a row after few loads: [1, 1024] x [65536, 1024]^T 40 -> 28 us, at k = 2048 and n = 32000 level)
+    const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192 || (k <= 2048 && n >= 32000)) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
                       k > 0 && k < (1u << 26) && aligned16(a) && aligned16(b);
 
     // fewer than 256 rows, weights as [k, n]: the same block products behind a transposition in registers, 32 rows a
@@ -1526,7 +1558,8 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     bool short_tile = false;
     if (short_ok) {
         // (the tile launch that the passes of the few-rows kernels are weighed against is cheaper on the small tiles)
-        if (trans_b) short_tile = rows ? false : skinny ? ((m + 63) / 64) * n > (small_grid ? kSkinnyPassesSmall : 23000u) : !gemv;
+        // (one to four rows against W as [n, k] read W once at the speed of the memory whatever n is: never a tile)
+        if (trans_b) short_tile = rows || gemv ? false : skinny ? ((m + 63) / 64) * n > (small_grid ? kSkinnyPassesSmall : 23000u) : true;
         else short_tile = rows_kn ? ((m + 31) / 32) * n > (small_grid ? kRowsKnPassesSmall : 17000u) : gemv_kn ? m > 16 : true;
     }
 

@@ -1384,6 +1384,25 @@ def test_matmul_one_b_for_a_batch_of_many_small_matrices():
     assert np.array_equal(host(ops.matmul_integer(dev(ai), dev(bi), dev(az), None)), oracle.matmul_integer(ai, bi, az, None, threads=8))
 
 
+@pytest.mark.parametrize("m, k, n", [(1, 128, 24576), (1, 136, 24584), (3, 128, 24592), (4, 72, 25000), (1, 256, 32000),
+                                     (1, 1024, 32768), (2, 128, 24577)])
+def test_matmul_few_rows_against_a_vocabulary_of_rows(m, k, n):
+    # one to four rows against W as [n, k] with more than 23000 rows: the kernels that read W once, whatever n
+    # is (a workgroup of the one-row kernel walks several blocks of rows); exact on small integers, with a bias
+    rng = np.random.default_rng(m * 1000 + k)
+    a = rng.integers(-2, 3, (m, k)).astype(np.float32)
+    w = rng.integers(-2, 3, (n, k)).astype(np.float32)
+    c = rng.integers(-8, 9, (n,)).astype(np.float32)
+    want = (a.astype(np.int64) @ w.T.astype(np.int64)).astype(np.float32)
+    for dt in (torch.float16, torch.bfloat16):
+        if dt == torch.bfloat16 and np.max(np.abs(want)) + 8 >= 256:
+            continue
+        got = host(ops.matmul(dev(a).to(dt), dev(w).to(dt), trans_b=True).float())
+        assert np.array_equal(got, want)
+        got = host(ops.matmul(dev(a).to(dt), dev(w).to(dt), dev(c).to(dt), trans_b=True).float())
+        assert np.array_equal(got, want + c)
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
