@@ -1553,7 +1553,10 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     // of dependent steps (1.33 us per 64 of k on the large tile, 0.83 us on the small one), so while the small tiles
     // find a CU each, or nearly, the launch ends earlier (k = 4096: 85 -> 53 us up to 64 large tiles, 85 -> 78 at 86,
     // level at 128)
-    const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && m > 8 && aligned16(a) && (!trans_b || aligned16(b));
+    // Up to 8 rows only where the plain kernel is expected to take longer (it needs 2.9 ns per thousand elements of B,
+    // 596 us for [8, 4096] x [4096, 50257]; a tile launch about 4 us and 0.83 us per 64 of k).
+    const bool tiles16_rows = m > 8 || static_cast<uint64_t>(n) * k > 1400000u + 4500u * static_cast<uint64_t>(k);
+    const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && tiles16_rows && aligned16(a) && (!trans_b || aligned16(b));
     const bool small_grid = tiles16 && ((m + HT - 1) / HT) * ((n + HT - 1) / HT) * (a_index || b_index ? 1 : batch) <= kSmallGrid;
     bool short_tile = false;
     if (short_ok) {

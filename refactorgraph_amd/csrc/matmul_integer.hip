@@ -1026,7 +1026,10 @@ int mmi_launch(int32_t *y, const void *a, const void *b, const void *a_zp, const
         else mmi_tiles<DEQ, false><<<grid, 256, 0, s>>>(y, a8, b8, za, zb, dq, m32, k32, n32, am0, bm0, ym0);
         return launch_status();
     };
-    const bool small_tiles_ok = k % 16 == 0 && k > 0 && m > 8 && aligned16(a) && ((m + GT - 1) / GT) * ((n + GT - 1) / GT) <= 0x7fffffffu;
+    // (up to 8 rows only where the plain kernel is expected to take longer: it needs 3.3 ns per thousand elements of B,
+    // 675 us for [8, 4096] x [4096, 50257]; a launch of these tiles about 6 us and 1.12 us per 128 of k)
+    const bool small_tiles_rows = m > 8 || static_cast<uint64_t>(n) * k > 1800000u + 2650u * static_cast<uint64_t>(k);
+    const bool small_tiles_ok = k % 16 == 0 && k > 0 && small_tiles_rows && aligned16(a) && ((m + GT - 1) / GT) * ((n + GT - 1) / GT) <= 0x7fffffffu;
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if (small_tiles_ok && (short_tile || (fast && !gemv && !skinny)) && small_tiles_pay(short_tile, count))

@@ -1403,6 +1403,28 @@ def test_matmul_few_rows_against_a_vocabulary_of_rows(m, k, n):
         assert np.array_equal(got, want + c)
 
 
+@pytest.mark.parametrize("m, k, n", [(1, 64, 50257), (5, 80, 50257), (8, 64, 40001), (7, 4096, 5003)])
+def test_matmul_up_to_8_rows_against_an_odd_vocabulary(m, k, n):
+    # n odd (no kernel with 16-byte loads along n takes it) and so large that the 128 x 128 tiles with most of
+    # their rows masked beat the plain kernel: both layouts of B, and MatMulInteger with every kind of zero point
+    rng = np.random.default_rng(m * 100 + k)
+    a = rng.integers(-1, 2, (m, k)).astype(np.float32)
+    b = rng.integers(-1, 2, (k, n)).astype(np.float32)
+    c = rng.integers(-8, 9, (n,)).astype(np.float32)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.max(np.abs(want)) + 8 < 256
+    for dt in (torch.float16, torch.bfloat16):
+        assert np.array_equal(host(ops.matmul(dev(a).to(dt), dev(b).to(dt), dev(c).to(dt)).float()), want + c)
+        bt = dev(np.ascontiguousarray(b.T)).to(dt)
+        assert np.array_equal(host(ops.matmul(dev(a).to(dt), bt, trans_b=True).float()), want)
+    ai = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    bi = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    az, bz = rng.integers(0, 256, (m,), dtype=np.uint8), rng.integers(-128, 128, (k,), dtype=np.int8)
+    for za, zb in ((None, None), (az[:1], bz[:1]), (az, bz)):
+        got = host(ops.matmul_integer(dev(ai), dev(bi), None if za is None else dev(za), None if zb is None else dev(zb)))
+        assert np.array_equal(got, oracle.matmul_integer(ai, bi, za, zb, threads=8))
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
