@@ -1531,9 +1531,10 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 
     // two to sixteen rows, weights as [n, k]: operands straight from global memory into 4x4x4 block products
     // (a single row too when k is long: the matrix-vector kernel keeps a whole row of W per wavefront in flight,
-    // which stops paying beyond 16 KiB; and against a vocabulary's worth of short rows, where a wavefront of that
-    // kernel ends a row after few loads: [1, 1024] x [65536, 1024]^T 40 -> 28 us, at k = 2048 and n = 32000 level)
-    const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192 || (k <= 2048 && n >= 32000)) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
+    // which stops paying beyond 16 KiB; and when k is short, where a wavefront of that kernel ends a row after few
+    // loads, at k = 128 with 16 of its lanes: [1, 1024] x [65536, 1024]^T 40 -> 28 us, 32 products of
+    // [1, 128] x [4096, 128]^T 67 -> 24 us, [1, 2048] x [4096, 2048]^T 4.8 -> 4.3 us)
+    const bool rows = narrow && !trans_a && trans_b && (m >= 2 || k > 8192 || k <= 2048) && m <= 16 && n % 16 == 0 && k % 128 == 0 &&
                       k > 0 && k < (1u << 26) && aligned16(a) && aligned16(b);
 
     // fewer than 256 rows, weights as [k, n]: the same block products behind a transposition in registers, 32 rows a
@@ -1559,12 +1560,25 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
     const bool tiles16 = narrow && !trans_a && k % 8 == 0 && k > 0 && tiles16_rows && aligned16(a) && (!trans_b || aligned16(b));
     const bool small_grid = tiles16 && ((m + HT - 1) / HT) * ((n + HT - 1) / HT) * (a_index || b_index ? 1 : batch) <= kSmallGrid;
     bool short_tile = false;
-    if (short_ok) {
-        // (the tile launch that the passes of the few-rows kernels are weighed against is cheaper on the small tiles)
+    if (short_ok || small_grid) {
+        // (the tile launch that the passes of the few-rows kernels are weighed against is cheaper on the small tiles;
+        // there the matrices of a batch count too, all of them being tiles of one launch that find a CU each)
         // (one to four rows against W as [n, k] read W once at the speed of the memory whatever n is: never a tile)
-        if (trans_b) short_tile = rows || gemv ? false : skinny ? ((m + 63) / 64) * n > (small_grid ? kSkinnyPassesSmall : 23000u) : true;
-        else short_tile = rows_kn ? ((m + 31) / 32) * n > (small_grid ? kRowsKnPassesSmall : 17000u) : gemv_kn ? m > 16 : true;
+        const uint64_t columns = small_grid ? n * (a_index || b_index ? 1 : batch) : n;
+        // passes of four rows over B as [k, n] against one launch of small tiles (a pass: 4.3 us or B at 5 TB/s)
+        const double b_us = 2.0 * static_cast<double>(k) * static_cast<double>(columns) / 5.0e6;
+        const double gemv_kn_us = static_cast<double>((m + 3) / 4) * (b_us > 4.3 ? b_us : 4.3);
+        const bool gemv_kn_slow = small_grid && m > 4 && 4.0 + 0.83 * static_cast<double>((k + HK - 1) / HK) < gemv_kn_us;
+        if (trans_b) short_tile = rows || gemv ? false : skinny ? ((m + 63) / 64) * columns > (small_grid ? kSkinnyPassesSmall : 23000u) : true;
+        else short_tile = rows_kn ? ((m + 31) / 32) * columns > (small_grid ? kRowsKnPassesSmall : 17000u)
+                                  : gemv_kn ? (short_ok && m > 16) || gemv_kn_slow : true;
     }
+    // A short k leaves a tile little to do between fetching its operands and storing its results, and two small tiles
+    // per CU overlap the one's stores with the other's loads: with k <= 128 the small tiles take a full grid too
+    // ([4096, 128] x [128, 4096] 24.7 -> 22.9 us, [8192, 128] x [128, 8192] 93 -> 76 us, 32 products of
+    // [512, 128] x [512, 128]^T 21 -> 13.5 us; at k = 256 they lose, 28 -> 31 us), and with k <= 512 every short tile
+    // is a small one and taken before the few-rows kernels (32 products [128, 128] x [4096, 128]^T 110 -> 25 us)
+    const bool short_k = tiles16 && m > 16 && ((fast && k <= 128) || (short_ok && k <= 512));
 
     // F32 on the matrix cores.  A launch of the 128 x 128 tiles walks all of k in every workgroup and takes about
     // 300 us at k = 4096 however few tiles there are; up to that cost few rows go through the block products of
@@ -1611,7 +1625,7 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
-            if (small_grid && (short_tile || fast)) return launch_tiles16(am0, bm0, ym0, count);
+            if ((small_grid && (short_tile || fast)) || short_k) return launch_tiles16(am0, bm0, ym0, count);
             if (short_tile) {
                 const dim3 grid(static_cast<unsigned>((n + BN - 1) / BN), 1, count);
                 if (trans_b)

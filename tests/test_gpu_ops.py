@@ -1425,6 +1425,24 @@ def test_matmul_up_to_8_rows_against_an_odd_vocabulary(m, k, n):
         assert np.array_equal(got, oracle.matmul_integer(ai, bi, za, zb, threads=8))
 
 
+@pytest.mark.parametrize("B, S, T, D", [(32, 32, 32, 128), (32, 128, 128, 128), (32, 128, 512, 128), (6, 40, 264, 64),
+                                        (32, 1, 512, 128), (5, 3, 300, 128), (4, 512, 512, 128), (3, 20, 48, 128)])
+def test_matmul_batches_of_attention_products(B, S, T, D):
+    # scores Q K^T (short k) and their product with V (few columns), one pair of matrices per head: batches whose
+    # matrices together decide between the few-rows kernels and one launch of small tiles; exact on small integers
+    rng = np.random.default_rng(B * 1000 + S)
+    q = rng.integers(-1, 2, (B, S, D)).astype(np.float32)
+    kk = rng.integers(-1, 2, (B, T, D)).astype(np.float32)
+    p = rng.integers(-1, 2, (B, S, T)).astype(np.float32)
+    v = rng.integers(-1, 2, (B, T, D)).astype(np.float32)
+    want_s = np.einsum("bsd,btd->bst", q, kk)
+    want_o = np.einsum("bst,btd->bsd", p, v)
+    assert max(np.max(np.abs(want_s)), np.max(np.abs(want_o))) < 256
+    for dt in (torch.float16, torch.bfloat16):
+        assert np.array_equal(host(ops.matmul(dev(q).to(dt), dev(kk).to(dt), trans_b=True).float()), want_s)
+        assert np.array_equal(host(ops.matmul(dev(p).to(dt), dev(v).to(dt)).float()), want_o)
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
