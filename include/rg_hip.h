@@ -156,7 +156,8 @@ int rg_hip_cast(void *y, const void *x, size_t size, int from_dtype, int to_dtyp
  * y [batch, m, n], row-major.  alpha and beta are converted to dtype first, like the reference;
  * sums are accumulated in float (double for F64).
  * a_index / b_index: as for rg_hip_matmul_integer (HOST arrays of `batch` matrix indices, or NULL
- * for matrix i; one B for consecutive matrices of A runs as one product of batch * m rows).  c may be NULL (then beta is ignored); otherwise the bias element of
+ * for matrix i; one B for consecutive matrices of A runs as one product of batch * m rows, groups of consecutive
+ * matrices of A with one B each as one product per group).  c may be NULL (then beta is ignored); otherwise the bias element of
  * Y[batch b, row i, column j] is c[b * c_stride_batch + i * c_stride_m + j * c_stride_n] (strides
  * in elements, 0 broadcasts), which covers every bias the reference expands when its batch
  * dimensions are all 1 or equal to the output's. */

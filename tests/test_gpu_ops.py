@@ -1443,6 +1443,33 @@ def test_matmul_batches_of_attention_products(B, S, T, D):
         assert np.array_equal(host(ops.matmul(dev(p).to(dt), dev(v).to(dt)).float()), want_o)
 
 
+@pytest.mark.parametrize("S, T, D", [(1, 300, 128), (4, 264, 64), (40, 136, 128), (130, 96, 72)])
+def test_matmul_groups_of_matrices_that_share_one_b(S, T, D):
+    # the query heads of a key / value head: [2, 3, 4, S, D] against [2, 3, 1, T, D] is six products of 4 S rows;
+    # a bias over the whole output; then shapes whose matrices only partly follow each other in both operands
+    rng = np.random.default_rng(S * 10 + D)
+    q = rng.integers(-1, 2, (2, 3, 4, S, D)).astype(np.float32)
+    kk = rng.integers(-1, 2, (2, 3, 1, T, D)).astype(np.float32)
+    p = rng.integers(-1, 2, (2, 3, 4, S, T)).astype(np.float32)
+    v = rng.integers(-1, 2, (2, 3, 1, T, D)).astype(np.float32)
+    c = rng.integers(-8, 9, (2, 3, 4, S, T)).astype(np.float32)
+    want_s = np.einsum("abgsd,abtd->abgst", q, kk[:, :, 0])
+    want_o = np.einsum("abgst,abtd->abgsd", p, v[:, :, 0])
+    assert max(np.max(np.abs(want_s)) + 8, np.max(np.abs(want_o))) < 256
+    for dt in (torch.float16, torch.bfloat16):
+        assert np.array_equal(host(ops.matmul(dev(q).to(dt), dev(kk).to(dt), trans_b=True).float()), want_s)
+        assert np.array_equal(host(ops.matmul(dev(q).to(dt), dev(kk).to(dt), dev(c).to(dt), trans_b=True).float()), want_s + c)
+        assert np.array_equal(host(ops.matmul(dev(p).to(dt), dev(v).to(dt)).float()), want_o)
+    a = rng.integers(-1, 2, (3, 1, S, D)).astype(np.float32)
+    b = rng.integers(-1, 2, (1, 5, D, T)).astype(np.float32)
+    assert np.array_equal(host(ops.matmul(dev(a).half(), dev(b).half()).float()), np.einsum("asd,bdt->abst", a[:, 0], b[0]))
+    a = rng.integers(-1, 2, (1, 5, S, D)).astype(np.float32)
+    b = rng.integers(-1, 2, (3, 5, D, T)).astype(np.float32)
+    assert np.array_equal(host(ops.matmul(dev(a).half(), dev(b).half()).float()), np.einsum("bsd,abdt->abst", a[0], b))
+    got = host(ops.matmul(dev(q).float(), dev(kk).float(), trans_b=True))
+    assert np.array_equal(got, want_s)
+
+
 def test_matmul_fp16_exact_on_small_integers_full_tile_grid():
     # integer-valued operands with |sum| < 2048: every fp16 result is exact, so the MFMA path must
     # reproduce numpy's integer product bit for bit over a 3 x 2 grid of tiles and 5 k-tiles
