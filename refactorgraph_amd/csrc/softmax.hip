@@ -220,7 +220,7 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_ragged(
     using CT = typename Compute<T>::type;
     constexpr int VEC = Vec16<T>::N;
     constexpr int BLOCK = THREADS < 256 ? 256 : THREADS, RPB = BLOCK / THREADS;
-    static_assert(THREADS == kWave || THREADS == BLOCK, "a row belongs to one wavefront or to the whole workgroup");
+    static_assert((THREADS <= kWave && kWave % THREADS == 0) || THREADS == BLOCK, "a row belongs to a part of a wavefront or to the whole workgroup");
     __shared__ CT smem[BLOCK / kWave];
     const uint32_t t = threadIdx.x % THREADS;
     const uint64_t row = static_cast<uint64_t>(blockIdx.x) * RPB + threadIdx.x / THREADS;
@@ -270,9 +270,16 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_ragged(
     auto wmax = [](CT v) { return wave_max(v); };
     auto wsum = [](CT v) { return wave_sum(v); };
     CT row_max, total;
-    if constexpr (THREADS == kWave) {
-        row_max = wave_max(mx);
-        total = wave_sum(sum * Exp<T>::eval(mx - row_max));
+    if constexpr (THREADS <= kWave) {  // (short rows: several to a wavefront, so that it has several rows' loads in flight)
+        row_max = mx;
+#pragma unroll
+        for (int off = THREADS / 2; off > 0; off >>= 1) {
+            const CT other = __shfl_xor(row_max, off, kWave);
+            row_max = row_max < other ? other : row_max;
+        }
+        total = sum * Exp<T>::eval(mx - row_max);
+#pragma unroll
+        for (int off = THREADS / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, kWave);
     } else {
         row_max = block_allreduce<THREADS / kWave>(mx, smem, wmax, [](CT a, CT b) { return a < b ? b : a; });
         total = block_allreduce<THREADS / kWave>(sum * Exp<T>::eval(mx - row_max), smem, wsum, [](CT a, CT b) { return a + b; });
@@ -531,6 +538,8 @@ int dispatch(void *y_, const void *x_, size_t pre, size_t mid, size_t post, size
     } else if (post == 1 && pre <= 0x7fffffffu) {
         const uint32_t m32 = static_cast<uint32_t>(mid), c32 = static_cast<uint32_t>(causal_rows);
         if (mid <= 32) softmax_tiny<T><<<static_cast<unsigned>((pre + 255) / 256), 256, 0, s>>>(y, x, pre, m32, c32);
+        else if (mid / Vec16<T>::N <= 48) softmax_ragged<T, 16><<<static_cast<unsigned>((pre + 15) / 16), 256, 0, s>>>(y, x, pre, m32, c32);
+        else if (mid / Vec16<T>::N <= 96) softmax_ragged<T, 32><<<static_cast<unsigned>((pre + 7) / 8), 256, 0, s>>>(y, x, pre, m32, c32);
         else if (mid <= 2048) softmax_ragged<T, 64><<<static_cast<unsigned>((pre + 3) / 4), 256, 0, s>>>(y, x, pre, m32, c32);
         else if (mid <= 32768) softmax_ragged<T, 256><<<static_cast<unsigned>(pre), 256, 0, s>>>(y, x, pre, m32, c32);
         else softmax_ragged<T, 1024><<<static_cast<unsigned>(pre), 1024, 0, s>>>(y, x, pre, m32, c32);

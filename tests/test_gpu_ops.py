@@ -151,6 +151,25 @@ def test_softmax_short_rows(rows, mid):
         assert np.max(np.abs(got - oracle.softmax_causal(sq, threads=8))) <= ABS_F16
 
 
+@pytest.mark.parametrize("heads, seq, mid", [(3, 37, 300), (2, 45, 301), (5, 33, 33), (1, 99, 700), (2, 150, 150), (3, 7, 390)])
+def test_softmax_rows_that_start_anywhere_within_a_vector(heads, seq, mid):
+    # rows of a length that is no whole number of 16-byte vectors, 16, 32 or 64 lanes each (several rows to a
+    # wavefront, a last workgroup with rows to spare): plain and causal, fp16, bf16 and float
+    rng = np.random.default_rng(seq * 1000 + mid)
+    x = (3 * rng.standard_normal((heads, seq, mid))).astype(np.float32)
+    x[0, -1, :5] = -np.inf  # (the last row keeps every column under the causal mask too)
+    for dt, tol in ((torch.float16, ABS_F16), (torch.bfloat16, 8 * ABS_F16)):
+        xh = dev(x).to(dt)
+        x32 = host(xh.float())
+        assert np.max(np.abs(host(ops.softmax(xh).float()) - oracle.softmax(x32, threads=8))) <= tol
+        if mid >= seq:
+            assert np.max(np.abs(host(ops.softmax(xh, causal=True).float()) - oracle.softmax_causal(x32, threads=8))) <= tol
+    if mid % 4:
+        assert_rel(host(ops.softmax(dev(x))), oracle.softmax(x, threads=8), REL_F32)
+        if mid >= seq:
+            assert_rel(host(ops.softmax(dev(x), causal=True)), oracle.softmax_causal(x, threads=8), REL_F32)
+
+
 @pytest.mark.parametrize("shape", [(1, 70001), (3, 32768), (2, 1, 40001), (16, 50257)])
 def test_softmax_few_very_long_rows_in_chunks(shape):
     # logits over a vocabulary: the rows are cut into chunks, a workgroup each, whose maxima and sums travel through the
