@@ -110,8 +110,11 @@ int dispatch(void *y_, const void *x_, const void *w_, size_t rows, size_t cols,
         else if (nvec <= 8) launch_rows<T, 8, 1>(y, x, w, rows, cols, eps, s);
         else if (nvec <= 16) launch_rows<T, 16, 1>(y, x, w, rows, cols, eps, s);
         else launch_rows<T, 32, 1>(y, x, w, rows, cols, eps, s);
-    } else if (vec_ok && nvec <= 64 * 16) {
-        // one wavefront per row: no workgroup barrier, up to 16 loads in flight per lane
+    } else if (vec_ok && nvec <= (rows < 1024 ? 64 * 4 : sizeof(T) == 2 ? 64 * 8 : 64 * 16)) {
+        // one wavefront per row: no workgroup barrier, up to 16 loads in flight per lane.  Long rows go to a workgroup
+        // each where that ends earlier: few rows (8 rows of 4096 floats 6.1 -> 2.8 us) and 16-bit rows of more than 512
+        // vectors, whose 16 vectors per lane as floats cost the occupancy (4096 rows of 8192 halves from HBM
+        // 34 -> 26 us, of 5120 22 -> 17 us; rows of floats are level: 4096 x 4096 24.0 and 24.1 us)
         if (nvec <= 64) launch_rows<T, 64, 1>(y, x, w, rows, cols, eps, s);
         else if (nvec <= 128) launch_rows<T, 64, 2>(y, x, w, rows, cols, eps, s);
         else if (nvec <= 256) launch_rows<T, 64, 4>(y, x, w, rows, cols, eps, s);

@@ -77,6 +77,20 @@ def test_rms_norm_reference_kats():
     assert np.all(host(ops.rms_norm(dev(x), dev(w), 0.0)) == 3.0)
 
 
+@pytest.mark.parametrize("rows,cols", [(8, 4096), (3, 8192), (5, 2048), (1100, 5120), (1030, 8192), (1024, 4104), (1, 16384)])
+def test_rms_norm_long_rows_a_wavefront_or_a_workgroup_each(rows, cols):
+    # few rows, and many 16-bit rows of more than 4096 elements, take a workgroup per row; the others a wavefront
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+    assert_rel(host(ops.rms_norm(dev(x), dev(w), 1e-5)), oracle.rms_norm(x, w, 1e-5, threads=8), REL_F32)
+    for dt in (torch.float16, torch.bfloat16):
+        xt, wt = dev(x).to(dt), dev(w).to(dt)
+        ref = oracle.rms_norm(host(xt.float()), host(wt.float()), 1e-5, threads=8)
+        tol = ABS_F16 if dt == torch.float16 else 4e-2
+        assert np.max(np.abs(host(ops.rms_norm(xt, wt, 1e-5).float()) - ref)) <= tol * max(1.0, np.abs(ref).max() / 2)
+
+
 def test_rms_norm_f64_and_halves():
     rng = np.random.default_rng(3)
     x = rng.standard_normal((33, 1024))
