@@ -73,15 +73,6 @@ int rg_hip_graph_end(void *stream, void **graph_exec);
 int rg_hip_graph_launch(void *graph_exec, void *stream);
 int rg_hip_graph_destroy(void *graph_exec);
 
-/* ---- measurement aid ------------------------------------------------------------------------
- * No counterpart in the reference and not an operator: `workgroups` workgroups of four wavefronts
- * (one per SIMD) each run `iterations` x 16 v_mfma_i32_32x32x32_i8 on operands that stay in
- * registers (2 * 32^3 integer operations per product and wavefront) and write one int32 per thread
- * to out [workgroups * 256].  operands: 8 KiB (64 lanes x 8 fragments x 16 bytes, 16-byte aligned)
- * whose values set how many bits toggle.  bench.py times it to quote MatMulInteger against what
- * the matrix pipe sustains on the same kind of data (the part lowers its clock under this load). */
-int rg_hip_probe_mfma_i8(int32_t *out, const void *operands, size_t workgroups, size_t iterations, void *stream);
-
 /* ---- RmsNormalization --------------------------------------------------------------------
  * replaces the NVRTC kernel + launch of
  * src/04kernel/src/kernels/rms_normalization/cuda_kernel.cc:53-88,128-130;

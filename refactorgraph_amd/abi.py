@@ -38,7 +38,6 @@ SIGNATURES = {
     "rg_hip_graph_launch": (_i, [_vp, _vp]),
     "rg_hip_graph_destroy": (_i, [_vp]),
     "rg_hip_error_string": (C.c_char_p, [_i]),
-    "rg_hip_probe_mfma_i8": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "rg_hip_rms_norm": (_i, [_vp, _vp, _vp, _sz, _sz, _f, _i, _vp]),
     "rg_hip_softmax": (_i, [_vp, _vp, _sz, _sz, _sz, _i, _sz, _vp]),
     "rg_hip_rope": (_i, [_vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _f, _i, _vp]),

@@ -4,6 +4,8 @@
     librg_host.so    C++ host layer mirroring the reference's plugin surface
                      (hardware::Device, runtime::Resources/Routine, kernel::Kernel,
                      collectors); links librg_hip.so
+    librg_probe.so   measurement aids of bench.py (bench_probes/): ceilings of the matrix pipe
+                     and of HBM; not part of the boundary, loaded by the benchmark only
 
 hipcc cross-compiles for gfx950 without a GPU, so this runs anywhere the ROCm toolchain is
 installed.  Usage: ``python -m refactorgraph_amd.build [--jobs N]``.
@@ -81,10 +83,18 @@ def build_host(jobs=8):
     return out
 
 
+def build_probes():
+    os.makedirs(OBJ, exist_ok=True)
+    out = os.path.join(LIB, "librg_probe.so")
+    _run([HIPCC, *HIP_FLAGS, "-shared", os.path.join(PKG, "bench_probes", "probes.hip"), "-o", out])
+    return out
+
+
 def build_all(jobs=8):
     hip = build_hip(jobs)
     host = build_host(jobs)
-    return hip, host
+    probes = build_probes()
+    return hip, host, probes
 
 
 if __name__ == "__main__":

@@ -310,6 +310,154 @@ __device__ __forceinline__ void mmi_tile_loop(v16i (&acc)[4][4], uint8_t *lds0, 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
 }
 
+// The walk through k for the common case (a scalar zero point of 0 or 128 for A, none for B, full tiles), laid out
+// for a wavefront that is alone on its SIMD: whatever it issues besides its products has to fit behind them.
+// Measured on this part: a product occupies the matrix pipe for 32 clocks, in which the wavefront issues up to six
+// more vector or scalar instructions (or two LDS reads) without delaying the next product; a seventh costs its own
+// four clocks, dependent scalar arithmetic eight clocks an instruction, and the four wavefronts' copies share one
+// address unit (16 clocks per 1 KiB copy), so a burst of sixteen copies per wavefront in sixteen consecutive slots
+// queues up there and holds the wavefronts.  Hence:
+//   * a copy is one scalar add into M0 and the copy itself: its source is one scalar base per operand and tile plus
+//     a per-copy lane offset that stays in a register;
+//   * the XOR of an A fragment's four words is dealt to four consecutive slots, ahead of the fragment's first use;
+//   * fragment reads are issued in pairs in the first six slots of a k-step;
+//   * the copies of a tile are dealt over a whole tile's worth of slots, one every fourth slot, through a ring of
+//     four 32 KiB stages of 64 k each (A 256 x 64 at +0, B 64 x 256 at +16384).
+// Tile t lives in stage t % 4; its stage is free again after the barrier in the middle of tile t (all its fragment
+// reads are issued in the first half of the tile), from where the A part of tile t + 4 is copied into it (slots 16,
+// 20, 24, 28) and then the B part (slots 0, 4, 8, 12 of tile t + 1).  The same barrier, behind a wait for all but the
+// 16 newest copies, makes tile t + 1 visible to every wavefront.
+//   A stage: row r at r * 64, chunk c of it at position c ^ ((r >> 2) & 3)
+//   B stage: k-row r at r * 256, chunk c at position c ^ b_swizzle(r & 7)
+// (2,630 clocks per 128 of k against 3,030 for the two-buffer loop below, which the other cases keep.  On uniform
+// random bytes the part is power-limited and gives the clocks back as a lower frequency, 1.61 against 1.77 GHz inside
+// the loop; operands that toggle fewer bits keep the gain: all-zero operands 52.5 -> 46.1 us at 4096^3.)
+__device__ __forceinline__ void mmi_tile_loop_ring(v16i (&acc)[4][4], uint8_t *lds, const uint8_t *A, const uint8_t *B,
+                                                   uint32_t k, uint32_t lda, uint32_t n, uint32_t a_xor) {
+    constexpr uint32_t RK = 64, R_STAGE = 32768, R_B = 16384;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave >> 1, wn = wave & 1, h = lane >> 5;
+    const uint8_t *a_wave = scalar_pointer(A + static_cast<uint64_t>(wave * 64) * lda);
+    const uint8_t *b_wave = scalar_pointer(B + static_cast<uint64_t>(wave * 16) * n);
+    // copy q < 4: A rows 16 (4 wave + q) .. + 15, this lane row + lane / 4, chunk position lane % 4;
+    // copy 4 + p: B k-rows 4 (4 wave + p) .. + 3, this lane k-row + lane / 16, chunk position lane % 16
+    uint32_t voff[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        voff[q] = (16 * q + (lane >> 2)) * lda + 16 * ((lane & 3) ^ ((lane >> 4) & 3));
+        voff[4 + q] = (4 * q + (lane >> 4)) * n + 16 * ((lane & 15) ^ b_swizzle(4 * (q & 1) + (lane >> 4)));
+    }
+    const uint32_t lds_wave = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t *)lds)) + wave * 4096));
+    const uint32_t k_tiles = k / RK;
+    // copy Q (0..7) of tile `tile` (clamped to tile 0 behind the end: copied, never multiplied) into stage ST
+    auto tile_a = [&](uint32_t tile) { return scalar_pointer(a_wave + (tile < k_tiles ? tile * RK : 0)); };
+    auto tile_b = [&](uint32_t tile) { return scalar_pointer(b_wave + static_cast<uint64_t>(tile < k_tiles ? tile * RK : 0) * n); };
+    auto copy = [&]<int Q, int ST>(const uint8_t *from) __attribute__((always_inline)) {
+        constexpr uint32_t to = ST * R_STAGE + (Q < 4 ? Q * 1024 : R_B + (Q - 4) * 1024);
+        const uint32_t lane_off = voff[Q], lds_to = lds_wave;
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(lane_off), "s"(from), "s"(lds_to), "n"(to)
+                     : "memory", "m0", "scc");
+    };
+    const uint32_t a_off = (wm * 128 + (lane & 31)) * 64 + 16 * (h ^ ((lane >> 2) & 3));
+    auto read_a = [&](int stage, int ks, int i) -> v4i {
+        return *reinterpret_cast<const v4i *>(lds + stage * R_STAGE + (a_off ^ (32 * ks)) + i * 2048);
+    };
+    uint32_t b_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t a16 = lane & 15, chunk = wn * 8 + 2 * j + ((lane >> 4) & 1);
+        b_off[j] = R_B + (16 * h + (a16 >> 1)) * 256 + 16 * (chunk ^ b_swizzle(a16 >> 1)) + 8 * (a16 & 1);
+    }
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    auto read_b = [&](int stage, int ks, int j, int half, v4i &f) {
+        const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (__attribute__((address_space(3))) v2i *)(lds + stage * R_STAGE + b_off[j] + (32 * ks + 8 * half) * 256));
+        f[2 * half] = r[0];
+        f[2 * half + 1] = r[1];
+    };
+
+    v4i fa[2][4], fb[2][4];
+    // tiles 0, 1, 2 and the A part of tile 3 (its B part follows in the first half of tile 0)
+    {
+        const uint8_t *a0 = tile_a(0), *b0 = tile_b(0), *a1 = tile_a(1), *b1 = tile_b(1), *a2 = tile_a(2), *b2 = tile_b(2),
+                      *a3 = tile_a(3);
+        [&]<int... Q>(std::integer_sequence<int, Q...>) __attribute__((always_inline)) {
+            (copy.template operator()<Q, 0>(Q < 4 ? a0 : b0), ...);
+            (copy.template operator()<Q, 1>(Q < 4 ? a1 : b1), ...);
+            (copy.template operator()<Q, 2>(Q < 4 ? a2 : b2), ...);
+        }(std::make_integer_sequence<int, 8>{});
+        [&]<int... Q>(std::integer_sequence<int, Q...>) __attribute__((always_inline)) {
+            (copy.template operator()<Q, 3>(a3), ...);
+        }(std::make_integer_sequence<int, 4>{});
+    }
+    asm volatile("s_waitcnt vmcnt(20)" ::: "memory");  // tile 0 (the 8 oldest of 28 copies)
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[0][i] = read_a(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        read_b(0, 0, j, 0, fb[0][j]);
+        read_b(0, 0, j, 1, fb[0][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fa[0][i][e] ^= static_cast<int>(a_xor);
+
+    // tile `t` is in stage ST
+    auto step = [&]<int ST>(uint32_t t) __attribute__((always_inline)) {
+        const uint8_t *b_cp = tile_b(t + 3), *a_cp = tile_a(t + 4);
+        auto slot = [&]<int s>() __attribute__((always_inline)) {
+            // rows walk the columns back and forth, so that only one operand changes between MFMAs
+            constexpr int ks = s / 16, o = s % 16, row = o / 4, col = (row & 1) ? 3 - o % 4 : o % 4;
+            constexpr int cur = ks & 1, nxt = cur ^ 1;
+            if constexpr (s == 16) {
+                // tile t + 1 has landed (all but the 16 newest copies) and this wavefront's reads of stage ST are done
+                asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+                __syncthreads();  // tile t + 1 complete for everybody, stage ST no longer read
+            }
+            acc[row][col] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[cur][row], fb[cur][col], acc[row][col], 0, 0, 0);
+            constexpr int src = ks == 1 ? (ST + 1) % 4 : ST;
+            constexpr int nks = ks ^ 1;
+            if constexpr (o < 2) {
+                fa[nxt][2 * o] = read_a(src, nks, 2 * o);
+                fa[nxt][2 * o + 1] = read_a(src, nks, 2 * o + 1);
+            } else if constexpr (o < 6) {
+                read_b(src, nks, o - 2, 0, fb[nxt][o - 2]);
+                read_b(src, nks, o - 2, 1, fb[nxt][o - 2]);
+            }
+            // the XOR of A's zero point, one word per slot: fragments 2 and 3 of this k-step (first used in slots 8
+            // and 12), then fragments 0 and 1 of the next
+            if constexpr (o < 8) fa[cur][2 + o / 4][o % 4] ^= static_cast<int>(a_xor);
+            else fa[nxt][(o - 8) / 4][o % 4] ^= static_cast<int>(a_xor);
+            if constexpr (s % 4 == 0) {
+                if constexpr (s < 16) copy.template operator()<4 + s / 4, (ST + 3) % 4>(b_cp);   // B part of tile t + 3
+                else copy.template operator()<(s - 16) / 4, ST>(a_cp);                           // A part of tile t + 4
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        [&]<int... I>(std::integer_sequence<int, I...>) __attribute__((always_inline)) {
+            (slot.template operator()<I>(), ...);
+        }(std::make_integer_sequence<int, 32>{});
+    };
+    uint32_t t = 0;
+    for (; t + 4 <= k_tiles; t += 4) {
+        step.template operator()<0>(t);
+        step.template operator()<1>(t + 1);
+        step.template operator()<2>(t + 2);
+        step.template operator()<3>(t + 3);
+    }
+    if (t < k_tiles) {  // k is a multiple of 128: two tiles are left
+        step.template operator()<0>(t);
+        step.template operator()<1>(t + 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the workgroup's LDS is released
+}
+
 // SPLIT: blockIdx.y picks a range of `split_tiles` k-tiles and the sums are added to a zeroed Y with integer atomics
 // (exact in any order): for products with too few output tiles to occupy the chip.
 // SHORT_M: fewer than 256 rows of A, one row of tiles.
@@ -319,8 +467,8 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
                                                            Dequant dq, uint32_t m, uint32_t k, uint32_t n, uint32_t split_tiles,
                                                            uint32_t a_matrix0, uint32_t b_matrix0, uint32_t y_matrix0) {
     static_assert(!(DEQ && SPLIT), "partial sums cannot be dequantised");
-    __shared__ __align__(1024) uint8_t lds0[D_STAGE];
-    __shared__ __align__(1024) uint8_t lds1[D_STAGE];
+    __shared__ __align__(1024) uint8_t lds_all[2 * D_STAGE];
+    uint8_t *const lds0 = lds_all, *const lds1 = lds_all + D_STAGE;
     __shared__ __align__(256) uint8_t zlds[2 * 4 * 256];  // B's zero points of a tile: a slot per buffer and wavefront
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -388,7 +536,9 @@ __global__ __launch_bounds__(256, 1) void mmi_mfma_256x256(int32_t *__restrict__
     if (b_zp && !zb.per_row && zb.ptr[0] == 0) b_zp = false;
     const uint64_t zb_row0 = bm * k + k_begin;
 
-    if (a_simple) {
+    if (a_simple && !b_zp && !SHORT_M && k < (1u << 26)) {  // (63 rows of A stay below 2^32 bytes: lane offsets of the copies)
+        mmi_tile_loop_ring(acc, lds_all, A, B, k_len, k, n, a_xor);
+    } else if (a_simple) {
         if (!b_zp) mmi_tile_loop<0, false, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
         else mmi_tile_loop<0, true, SHORT_M>(acc, lds0, lds1, A, B, k_len, k, n, a_xor, za_f, zb, zb_row0, m, zlds);
     } else {
