@@ -82,6 +82,21 @@ int rg_hip_graph_destroy(void *graph_exec);
 int rg_hip_rms_norm(void *y, const void *x, const void *w,
                     size_t rows, size_t cols, float eps, int dtype, void *stream);
 
+/* RmsNormalization whose output goes on into DynamicQuantizeLinear (the head of a quantised linear layer):
+ * y as rg_hip_rms_norm writes it for F32, and yq / scale / zero_point as rg_hip_dynamic_quantize_linear
+ * computes them from y, bit for bit (contracts: src/04kernel/src/kernels/rms_normalization/cpu_kernel.cc:47-65
+ * and src/04kernel/src/kernels/dynamic_quantize_linear/cpu_kernel.cc:25-70).  No counterpart in the reference,
+ * which runs the two operators one after the other: here the normalising launch leaves the least and the
+ * greatest value of every workgroup's rows in the workspace, so the quantising launch is the only one that reads
+ * y (two launches instead of three; y read once instead of twice).
+ * rg_hip_rms_norm_quantize_workspace returns 0 for shapes the pair is not fused for (rows that are no whole
+ * 16-byte vectors, fewer than 132 or more than 8192 columns, more than 4096 workgroups): run the two
+ * operators then.  Pointers 16-byte aligned. */
+size_t rg_hip_rms_norm_quantize_workspace(size_t rows, size_t cols);
+int rg_hip_rms_norm_quantize(uint8_t *yq, float *scale, uint8_t *zero_point, float *y, const float *x,
+                             const float *w, size_t rows, size_t cols, float eps,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- Softmax -----------------------------------------------------------------------------
  * replaces src/04kernel/src/kernels/softmax/cuda_kernel.cu:21-125 (and the cuDNN path
  * cudnn_kernel.cc:37-76); shape digest as SoftmaxInfo
@@ -284,7 +299,8 @@ int rg_hip_attention_kvcache(void *o, const void *q, const void *k, const void *
  * library's device image, one copy per GPU, held until the process ends; the call allocates
  * nothing and frees nothing, and the counters are cleared by a small fill kernel at the start of
  * every call (not a memset, so the call can be captured).  Limits: those of
- * rg_hip_attention_kvcache (D in {64, 128}; a larger D is refused with RG_HIP_E_WORKSPACE, the
+ * rg_hip_attention_kvcache (D in {64, 80, 96, 128}, the head dims 80 and 96 on the tiled kernel only
+ * and without key ranges shared between workgroups; a larger D is refused with RG_HIP_E_WORKSPACE, the
  * partial slots being sized for D <= 128); the launch uses at most 512 workgroups, which is what
  * the array holds partials for (the tiled kernel shares an item's keys between workgroups only
  * as far as 2 MiB of records reach).  All calls on one GPU share the array: calls that overlap on one

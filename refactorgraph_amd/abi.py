@@ -39,6 +39,8 @@ SIGNATURES = {
     "rg_hip_graph_destroy": (_i, [_vp]),
     "rg_hip_error_string": (C.c_char_p, [_i]),
     "rg_hip_rms_norm": (_i, [_vp, _vp, _vp, _sz, _sz, _f, _i, _vp]),
+    "rg_hip_rms_norm_quantize_workspace": (_sz, [_sz, _sz]),
+    "rg_hip_rms_norm_quantize": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _f, _vp, _sz, _vp]),
     "rg_hip_softmax": (_i, [_vp, _vp, _sz, _sz, _sz, _i, _sz, _vp]),
     "rg_hip_rope": (_i, [_vp, _vp, _vp, _i, _sz, _sz, _sz, _sz, _f, _i, _vp]),
     "rg_hip_dequantize_linear": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _i, _i, _vp]),

@@ -20,7 +20,7 @@ struct PrefillArgs {
 // Bytes of `part` with which every launch that shares keys between workgroups finds room.
 size_t prefill_part_bytes(uint32_t D);
 
-// True when launch_prefill handles the shape (head dim 128 or 64, any group size).
+// True when launch_prefill handles the shape (head dim 64, 80, 96 or 128, any group size).
 bool prefill_supported(uint32_t H, uint32_t Hkv, uint32_t D);
 
 // Enqueues the kernel; returns a hipError_t as int.

@@ -184,6 +184,20 @@ __global__ __launch_bounds__(256) void dql_quantize(uint8_t *__restrict__ y, flo
 }
 
 }  // namespace
+
+// The quantising launch on extrema that another kernel has left (RmsNormalization with its output's least and
+// greatest value per workgroup): x is read once here.
+int quantize_with_partials(uint8_t *y, float *scale, uint8_t *zero_point, const float *x, size_t size, const float *partials,
+                           size_t n_partials, hipStream_t s) {
+    const int vec = aligned16(x) && (reinterpret_cast<uintptr_t>(y) & 3u) == 0;
+    uint64_t grid = (size + 4 * kTile - 1) / (4 * kTile);
+    if (grid > 8192) grid = 8192;
+    if (grid == 0) grid = 1;
+    dql_quantize<<<static_cast<unsigned>(grid), 256, 0, s>>>(y, scale, zero_point, x, partials,
+                                                             static_cast<uint32_t>(n_partials), size, vec);
+    return launch_status();
+}
+
 }  // namespace rg
 
 extern "C" size_t rg_hip_dynamic_quantize_linear_workspace(size_t) {

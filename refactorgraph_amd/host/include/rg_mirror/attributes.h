@@ -43,6 +43,10 @@ namespace refactor::kernel {
         dim_t m, k, n;
         bool hasBias, biasSupported;
         size_t biasStrideBatch, biasStrideM, biasStrideN;
+        // a bias whose batch dimensions are neither all 1 nor the output's is laid out over [batch..., m, n] first,
+        // as the reference does with every bias (src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:26-39):
+        // its shape and the output's, for an ExpandInfo; empty when the strides above describe the bias
+        std::vector<dim_t> biasExpandFrom, biasExpandTo;
         Broadcaster broadcaster;
 
         MatMulInfo(Tensor const &, Tensor const &, std::optional<std::reference_wrapper<Tensor const>>,

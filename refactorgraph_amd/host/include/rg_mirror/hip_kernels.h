@@ -21,6 +21,22 @@ namespace refactor::kernel {
         RoutineWorkspace lower(Resources &) const final;
     };
 
+    // RmsNormalization (float) whose output a DynamicQuantizeLinear reads: both operators' outputs, bit for
+    // bit, from two launches instead of three (the normalising launch leaves its output's extrema per
+    // workgroup, so its output is read once).  No counterpart in the reference; computation::Graph::lower puts
+    // it in place of such a pair.  Inputs: x, w.  Outputs: y (float), yq (uint8), scale, zero point.
+    struct RmsNormalizationQuantizeHip final : public Kernel {
+        float epsilon;
+        dim_t blockCount, blockSize;
+
+        RmsNormalizationQuantizeHip(float, dim_t, dim_t) noexcept;
+        static KernelBox build(float epsilon, dim_t blockCount, dim_t blockSize) noexcept;
+        static size_t typeId() noexcept;
+        size_t kernelTypeId() const noexcept final;
+        std::string_view description() const noexcept final;
+        RoutineWorkspace lower(Resources &) const final;
+    };
+
     struct SoftmaxHip final : public Kernel {
         SoftmaxInfo info;
         dim_t causalRows;// 0: plain softmax

@@ -140,7 +140,21 @@ namespace refactor::kernel {
         } else if (same) {
             biasStrideBatch = static_cast<size_t>(cm) * cn;
         } else {
-            biasSupported = false;
+            // some batch dimensions broadcast and others do not: expanded into a workspace first, if the shapes
+            // broadcast at all
+            for (size_t i = 2; i < cs.size(); ++i) {
+                if (at(i) != 1 && at(i) != out[out.size() + 1 - i]) {
+                    biasSupported = false;
+                    return;
+                }
+            }
+            biasExpandFrom.assign(cs.begin(), cs.end());
+            biasExpandTo = out;
+            biasExpandTo.push_back(m);
+            biasExpandTo.push_back(n);
+            biasStrideN = 1;
+            biasStrideM = n;
+            biasStrideBatch = static_cast<size_t>(m) * n;
         }
     }
 

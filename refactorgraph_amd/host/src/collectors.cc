@@ -194,11 +194,20 @@ namespace refactor::kernel {
         switch (_target) {
             case Target::Cpu:
                 break;
-            case Target::Amd:
-                if (inputs[0].get().shape.size() <= outputs[0].get().shape.size()) {
-                    ADD(ExpandHip::build(ExpandInfo(inputs[0], outputs[0])))
+            case Target::Amd: {
+                // a collector reports "no kernel" for what it cannot take; ExpandInfo's constructor asserts, so the
+                // shapes are checked here: right-aligned, every input extent is 1 or the output's
+                if (inputs.empty() || outputs.empty()) { break; }
+                auto const &in = inputs[0].get().shape;
+                auto const &out = outputs[0].get().shape;
+                if (in.size() > out.size() || inputs[0].get().dataType != outputs[0].get().dataType) { break; }
+                bool broadcasts = true;
+                for (size_t i = 0; i < in.size() && broadcasts; ++i) {
+                    auto const i_ = in[in.size() - 1 - i], o_ = out[out.size() - 1 - i];
+                    broadcasts = i_ == o_ || i_ == 1;
                 }
-                break;
+                if (broadcasts) { ADD(ExpandHip::build(ExpandInfo(inputs[0], outputs[0]))) }
+            } break;
             default:
                 UNREACHABLEX(void, "Unknown target");
         }

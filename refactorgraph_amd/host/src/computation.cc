@@ -102,6 +102,56 @@ namespace refactor::computation {
     }
     std::string RotaryEmbedding::serialize() const { return detail::cat(name(), '(', theta, ')'); }
 
+    // RmsNormalizationHip (float) -> DynamicQuantizeLinearHip  ==>  RmsNormalizationQuantizeHip, which keeps the
+    // normalised tensor as its first output (it may have further readers) and takes over the three outputs of the
+    // quantising node.  Rebuilt from keys like the fusion below.
+    struct Lowered {
+        graph_topo::GraphTopo topology;
+        std::vector<kernel::Node> nodes;
+        std::vector<kernel::Edge> edges;
+    };
+    static Lowered fuseQuantize(Lowered g) {
+        using kernel::DynamicQuantizeLinearHip;
+        using kernel::RmsNormalizationHip;
+        auto &[topology, nodes, edges] = g;
+        std::vector<count_t> producer(edges.size(), count_t(-1));
+        for (auto [idx, inputs, outputs] : topology)
+            for (auto e : outputs) producer[e] = idx;
+        std::unordered_map<count_t, count_t> fusedInto;// consumer node -> producer node
+        std::unordered_map<count_t, count_t> consumerOf;// producer node -> consumer node
+        for (auto [idx, inputs, outputs] : topology) {
+            auto const &k = nodes[idx].kernel;
+            if (!k || !k->is<DynamicQuantizeLinearHip>() || inputs.size() != 1 || outputs.size() != 3) continue;
+            auto const p = producer[inputs[0]];
+            if (p == count_t(-1) || consumerOf.count(p) || !nodes[p].kernel || !nodes[p].kernel->is<RmsNormalizationHip>()) continue;
+            auto const &rn = static_cast<RmsNormalizationHip const &>(*nodes[p].kernel);
+            if (rn.dataType != DataType::F32 || topology.node(p).outputs.size() != 1) continue;
+            auto fused = kernel::RmsNormalizationQuantizeHip::build(rn.epsilon, rn.blockCount, rn.blockSize);
+            if (!fused) continue;
+            nodes[p].kernel = std::move(fused);
+            nodes[p].name += "+" + nodes[idx].name;
+            fusedInto.emplace(idx, p);
+            consumerOf.emplace(p, idx);
+        }
+        if (fusedInto.empty()) return g;
+        graph_topo::Builder<count_t, kernel::Node, count_t, kernel::Edge> builder;
+        for (auto [idx, inputs, outputs] : topology) {
+            if (fusedInto.count(idx)) continue;
+            graph_topo::BuilderNode<count_t> n{{inputs.begin(), inputs.end()}, {outputs.begin(), outputs.end()}};
+            if (auto it = consumerOf.find(idx); it != consumerOf.end()) {
+                auto const consumer = topology.node(it->second);
+                n.outputs.insert(n.outputs.end(), consumer.outputs.begin(), consumer.outputs.end());
+            }
+            builder.topology.emplace(idx, std::move(n));
+            builder.nodes.emplace(idx, std::move(nodes[idx]));
+        }
+        for (auto e : topology.globalInputs()) builder.globalInputs.push_back(e);
+        for (auto e : topology.globalOutputs()) builder.globalOutputs.push_back(e);
+        for (count_t e = 0; e < edges.size(); ++e) builder.edges.emplace(e, std::move(edges[e]));
+        auto built = builder.build();
+        return {std::move(built.topology), std::move(built.nodes), std::move(built.edges)};
+    }
+
     // MatMulIntegerHip -> (int32 edge read once) -> DequantizeLinearHip  ==>  MatMulIntegerDequantizeHip.
     // The graph is rebuilt from keys (old indices) so that the edge numbering stays what GraphTopo
     // promises whatever the position of the scale's producer.
@@ -204,7 +254,10 @@ namespace refactor::computation {
         }
         auto topology = graph.topology;
         topology.reconnect(identities);
-        if (target == Target::Amd) return fuseDequantize(std::move(topology), std::move(nodes), std::move(edges));
+        if (target == Target::Amd) {
+            auto g = fuseQuantize({std::move(topology), std::move(nodes), std::move(edges)});
+            return fuseDequantize(std::move(g.topology), std::move(g.nodes), std::move(g.edges));
+        }
         return kernel::Graph(std::move(topology), std::move(nodes), std::move(edges));
     }
 

@@ -48,6 +48,30 @@ namespace refactor::kernel {
             };
     }
 
+    using RNQ = RmsNormalizationQuantizeHip;
+    RNQ::RmsNormalizationQuantizeHip(float epsilon_, dim_t blockCount_, dim_t blockSize_) noexcept
+        : Kernel(), epsilon(epsilon_), blockCount(blockCount_), blockSize(blockSize_) {}
+    KernelBox RNQ::build(float epsilon, dim_t blockCount, dim_t blockSize) noexcept {
+        if (rg_hip_rms_norm_quantize_workspace(blockCount, blockSize) == 0) { return nullptr; }
+        return std::make_unique<RNQ>(epsilon, blockCount, blockSize);
+    }
+    size_t RNQ::typeId() noexcept { return idOf<RNQ>(); }
+    size_t RNQ::kernelTypeId() const noexcept { return typeId(); }
+    std::string_view RNQ::description() const noexcept {
+        return "Performing rms normalization with dynamic quantization of its output on AMD gfx950";
+    }
+    RoutineWorkspace RNQ::lower(Resources &) const {
+        auto const bytes = rg_hip_rms_norm_quantize_workspace(blockCount, blockSize);
+        auto routine = [epsilon = epsilon, rows = blockCount, cols = blockSize, bytes]//
+            (Resources &res, void *workspace, void const *const *inputs, void *const *outputs) {
+                HIP_CALL(rg_hip_rms_norm_quantize(static_cast<uint8_t *>(outputs[1]), static_cast<float *>(outputs[2]),
+                                                  static_cast<uint8_t *>(outputs[3]), static_cast<float *>(outputs[0]),
+                                                  static_cast<float const *>(inputs[0]), static_cast<float const *>(inputs[1]),
+                                                  rows, cols, epsilon, workspace, bytes, streamOf(res)));
+            };
+        return RoutineWorkspace(std::move(routine), bytes);
+    }
+
     // ------------------------------------------------------------------ Softmax
 
     using SM = SoftmaxHip;
@@ -330,6 +354,30 @@ namespace refactor::kernel {
                 aIndex[i] = at[0];
                 bIndex[i] = at[1];
             }
+        }
+        if (!info.biasExpandFrom.empty()) {
+            // The bias broadcasts over some batch dimensions only: Expand lays it out over [batch..., m, n] in the
+            // workspace and the product reads it from there, one element per output.  (The reference expands into Y
+            // and lets the library update Y in place; here tiles of ragged shapes overlap, so Y cannot be both.)
+            ExpandInfo const e(info.dataType, info.biasExpandFrom, info.biasExpandTo);
+            std::vector<uint32_t> strideI, strideO;
+            for (auto [i, o] : e.strides) {
+                strideI.push_back(i);
+                strideO.push_back(o);
+            }
+            auto const bytes = static_cast<size_t>(e.blockSize) * e.blockCount;
+            auto routine = [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex), strideI = std::move(strideI),
+                            strideO = std::move(strideO), blockSize = e.blockSize, blockCount = e.blockCount]//
+                (Resources &res, void *workspace, void const *const *inputs, void *const *outputs) {
+                    HIP_CALL(rg_hip_expand(workspace, inputs[2], strideI.data(), strideO.data(), strideI.size(), blockSize,
+                                           blockCount, streamOf(res)));
+                    HIP_CALL(rg_hip_matmul(outputs[0], inputs[0], inputs[1], workspace,
+                                           static_cast<int>(info.dataType.internal), info.transA, info.transB, info.alpha,
+                                           info.beta, info.batch(), info.m, info.k, info.n,
+                                           aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
+                                           info.biasStrideBatch, info.biasStrideM, info.biasStrideN, streamOf(res)));
+                };
+            return RoutineWorkspace(std::move(routine), bytes);
         }
         return [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
             (Resources &res, void *, void const *const *inputs, void *const *outputs) {

@@ -49,6 +49,25 @@ def rms_norm(x, w, eps=1e-5, out=None):
     return y
 
 
+def rms_norm_quantize(x, w, eps=1e-5):
+    """RmsNormalization followed by DynamicQuantizeLinear of its output, fused: returns (y, yq, scale, zero_point)."""
+    _need_gpu(x, w)
+    assert x.dtype == torch.float32
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    nbytes = lib().rg_hip_rms_norm_quantize_workspace(rows, cols)
+    if nbytes == 0:
+        raise ValueError("rg_hip_rms_norm_quantize does not take this shape")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    y = torch.empty_like(x)
+    yq = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    scale = torch.empty((), dtype=torch.float32, device=x.device)
+    zp = torch.empty((), dtype=torch.uint8, device=x.device)
+    check(lib().rg_hip_rms_norm_quantize(_ptr(yq), _ptr(scale), _ptr(zp), _ptr(y), _ptr(x), _ptr(w), rows, cols, float(eps),
+                                         _ptr(ws), nbytes, _stream()), "rg_hip_rms_norm_quantize")
+    return y, yq, scale, zp
+
+
 def softmax(x, axis=-1, causal=False, out=None):
     _need_gpu(x)
     axis = axis % x.dim()

@@ -245,9 +245,20 @@ static void collectorsSelectOrDecline() {
         EXPECT(info.biasStrideM == 1 && info.biasStrideN == 0 && info.biasStrideBatch == 0);
         MatMulInfo full(*a, *bt, std::cref(*cFull), false, true, 1.f, 1.f);
         EXPECT(full.biasStrideBatch == 20 && full.biasStrideM == 4 && full.biasStrideN == 1);
-        EXPECT(!MatMulInfo(*a, *bt, std::cref(*cOdd), false, true, 1.f, 1.f).biasSupported);
+        // a bias that broadcasts over one batch dimension only is expanded into a workspace first
+        MatMulInfo odd(*a, *bt, std::cref(*cOdd), false, true, 1.f, 1.f);
+        EXPECT(odd.biasSupported && (odd.biasExpandFrom == std::vector<dim_t>{2, 1, 5, 4}) &&
+               (odd.biasExpandTo == std::vector<dim_t>{2, 3, 5, 4}) && odd.biasStrideBatch == 20 && odd.biasStrideM == 4);
         EXPECT(MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cRow}, {*cFull}).size() == 1);
-        EXPECT(MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cOdd}, {*cFull}).empty());
+        {
+            auto ks = MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cOdd}, {*cFull});
+            runtime::Resources res_;
+            EXPECT(ks.size() == 1 && ks[0]->lower(res_).workspaceOffset == 2 * 3 * 5 * 4 * 4);
+        }
+        // one that does not broadcast at all is declined
+        auto cBad = Tensor::share(DataType::F32, Shape{3, 1, 5, 4});
+        EXPECT(!MatMulInfo(*a, *bt, std::cref(*cBad), false, true, 1.f, 1.f).biasSupported);
+        EXPECT(MatMulCollector(T::Amd, 1, 1, false, true).filter({*a, *bt, *cBad}, {*cFull}).empty());
         EXPECT(MatMulCollector(T::Cpu, 1, 1, false, true).filter({*a, *bt}, {*cFull}).empty());
         auto ai = Tensor::share(DataType::I32, Shape{5, 7});
         auto bi = Tensor::share(DataType::I32, Shape{7, 4});
@@ -765,6 +776,16 @@ static void dataMoverDigests() {
     EXPECT(SplitCollector(T::Cpu, 3).filter({*joined}, refs).empty() && ConcatCollector(T::Cpu, 3).filter(refs, {*joined}).empty());
     EXPECT(SplitCollector(T::Amd, 9).filter({*joined}, refs).empty());// no such axis
     EXPECT(ExpandCollector(T::Amd).filter({*in}, {*out}).size() == 1 && ExpandCollector(T::Amd).filter({*out}, {*in}).empty());
+    {// shapes that do not broadcast, a type change and missing tensors give no kernel and throw nothing
+        auto odd = Tensor::share(DataType::F32, Shape{3, 4, 2, 6}), other = Tensor::share(DataType::I32, Shape{2, 3, 4, 5, 6});
+        bool threw = false;
+        try {
+            EXPECT(ExpandCollector(T::Amd).filter({*odd}, {*out}).empty());
+            EXPECT(ExpandCollector(T::Amd).filter({*in}, {*other}).empty());
+            EXPECT(ExpandCollector(T::Amd).filter({}, {*out}).empty() && ExpandCollector(T::Amd).filter({*in}, {}).empty());
+        } catch (...) { threw = true; }
+        EXPECT(!threw);
+    }
     auto c = Tensor::share(DataType::Bool, Shape{2, 5});
     auto x = Tensor::share(DataType::F32, Shape{2, 3, 2, 5}), y = Tensor::share(DataType::F32, Shape{3, 2, 5});
     auto wh = WhereCollector(T::Amd).filter({*c, *x, *y}, {*x});
@@ -974,15 +995,15 @@ static void matMulHip() {
         auto kernels = C ? MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({A, B, *C}, {Y})
                          : MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({A, B}, {Y});
         EXPECT(kernels.size() == 1);
-        auto routine = kernels[0]->lower(res).routine;
+        auto [routine, workspace] = kernels[0]->lower(res);
         auto ma = dev.malloc(a.size() * 4), mb = dev.malloc(b.size() * 4), mc = dev.malloc(std::max<size_t>(c.size(), 1) * 4),
-             my = dev.malloc(Y.elementsSize() * 4);
+             my = dev.malloc(Y.elementsSize() * 4), ws = dev.malloc(workspace ? workspace : 1);
         ma->copyFromHost(a.data());
         mb->copyFromHost(b.data());
         if (!c.empty()) mc->copyFromHost(c.data());
         void const *inputs[]{*ma, *mb, *mc};
         void *outputs[]{*my};
-        routine(res, nullptr, inputs, outputs);
+        routine(res, *ws, inputs, outputs);
         std::vector<float> y(Y.elementsSize());
         my->copyToHost(y.data());
         return y;
@@ -1003,6 +1024,37 @@ static void matMulHip() {
         auto y = run(*A, *B, C.get(), *Y, {1.0, 2.0, 0.0, 0.5, 1.0, 0.0, 0.0, 1.0}, {1.0, 2.0, 0.0, 0.5, 1.0, 0.0, 0.0, 1.0},
                      {1.0, 0.0});
         EXPECT((y == std::vector<float>{2.0, 4.0, 0.0, 0.25, 2.0, 3.0, 0.0, 0.5, 2.0, 3.0, 0.0, 0.5, 2.0, 1.0, 0.0, 1.0}));
+    }
+    {// a bias that broadcasts over one batch dimension and not the other ([3, 1, m, 1] under [3, 2, m, n]): the
+     // reference expands every bias into Y first (src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:26-39); here this
+     // one goes through Expand into the workspace.  Shapes of test_cpu.cpp:57-79 with a third matrix; integers: exact
+        std::mt19937 rng(13);
+        std::uniform_int_distribution<int> g(-3, 3);
+        dim_t const m = 5, k = 7, n = 6;
+        std::vector<float> a(3 * m * k), b(2 * k * n), c(3 * m);
+        for (auto &v : a) v = static_cast<float>(g(rng));
+        for (auto &v : b) v = static_cast<float>(g(rng));
+        for (auto &v : c) v = static_cast<float>(g(rng));
+        auto A = Tensor::share(DataType::F32, Shape{3, 1, m, k});
+        auto B = Tensor::share(DataType::F32, Shape{1, 2, k, n});
+        auto C = Tensor::share(DataType::F32, Shape{3, 1, m, 1});
+        auto Y = Tensor::share(DataType::F32, Shape{3, 2, m, n});
+        MatMulInfo info(*A, *B, std::make_optional(std::cref(*C)), false, false, 1, 1);
+        EXPECT(info.biasSupported && !info.biasExpandFrom.empty());
+        auto y = run(*A, *B, C.get(), *Y, a, b, c);
+        bool same = true;
+        for (dim_t i = 0; i < 3; ++i)
+            for (dim_t j = 0; j < 2; ++j)
+                for (dim_t r = 0; r < m; ++r)
+                    for (dim_t q = 0; q < n; ++q) {
+                        float sum = c[i * m + r];
+                        for (dim_t t = 0; t < k; ++t) sum += a[(i * m + r) * k + t] * b[(j * k + t) * n + q];
+                        same = same && y[((i * 2 + j) * m + r) * n + q] == sum;
+                    }
+        EXPECT(same);
+        // what does not broadcast is still declined
+        auto bad = Tensor::share(DataType::F32, Shape{2, 1, m, 1});
+        EXPECT(MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({*A, *B, *bad}, {*Y}).empty());
     }
     {// against the oracle's serial loop, float, odd sizes, no bias
         std::mt19937 rng(9);

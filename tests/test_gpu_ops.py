@@ -975,6 +975,29 @@ def test_attention_decode_full_config():
     assert np.isfinite(o).all()
 
 
+def test_attention_decode_run_to_run_difference_is_bounded():
+    # Which blocks a wavefront pulls is decided at run time (a counter in LDS), so the order in which the pieces of a
+    # segment are summed may change from run to run: the caches must come out bit for bit the same, the outputs
+    # within two units in the last place of the 16-bit result (each run rounds a float that differs by reordering)
+    N, H, Hkv, cap, D = 32, 32, 8, 4096, 128
+    g = torch.Generator(device=DEV).manual_seed(21)
+    rnd = lambda shape: torch.randn(shape, generator=g, device=DEV).half()
+    q, k, v = rnd((N, H, 1, D)), rnd((N, Hkv, 1, D)), rnd((N, Hkv, 1, D))
+    kc0, vc0 = rnd((N, Hkv, cap, D)), rnd((N, Hkv, cap, D))
+    past = torch.from_numpy(np.random.default_rng(14).integers(1024, 4096, N)).to(DEV)
+    runs = []
+    for _ in range(3):
+        kc, vc = kc0.clone(), vc0.clone()
+        o = ops.attention_kvcache(q, k, v, kc, vc, past)
+        torch.cuda.synchronize()
+        runs.append((o, kc, vc))
+    o0, kc_a, vc_a = runs[0]
+    ulp = torch.maximum(o0.float().abs(), torch.tensor(2.0 ** -14, device=DEV)).log2().floor().exp2() * 2.0 ** -10
+    for o, kc, vc in runs[1:]:
+        assert torch.equal(kc, kc_a) and torch.equal(vc, vc_a)
+        assert bool(((o.float() - o0.float()).abs() <= 2 * ulp).all())
+
+
 def test_attention_persistent_sync_state_is_left_zero():
     # with caller-owned ticket counters the call is one launch; the counters must come back zero
     # so that consecutive calls (different shapes) can share them

@@ -80,6 +80,24 @@ def test_static_scratch_entry_with_a_long_cache_and_few_query_tiles():
         assert float((o.float() - ro.float()).abs().max()) <= ABS_F16
 
 
+def test_static_scratch_entry_on_the_other_head_groups_and_head_dims():
+    # eight query heads per kv head against a long history (the launch of half as many workgroups), groups of 3 and 5
+    # with one new row (the tiled kernel with key ranges, as far as the scratch holds their records), head dims 80
+    # and 96 (tiled kernel only, no key ranges)
+    cases = [(_inputs(2, 64, 8, 1, 4097, 128, [4096, 1500], seed=6), 1 / math.sqrt(128)),
+             (_inputs(3, 24, 8, 1, 2100, 128, [2099, 40, 1024], seed=7), 1 / math.sqrt(128)),
+             (_inputs(2, 20, 4, 1, 1500, 64, [1499, 700], seed=8), 0.125),
+             (_inputs(2, 16, 4, 1, 600, 80, [599, 100], seed=9), 0.11),
+             (_inputs(1, 12, 4, 40, 300, 96, [200], seed=10), 0.1),
+             (_inputs(2, 16, 2, 1, 90, 128, [3, 89], seed=11), 0.09)]
+    for t, scale in cases:
+        o, kc, vc = _static(t, scale)
+        ro, rkc, rvc = _existing(t, scale)
+        assert torch.equal(kc, rkc) and torch.equal(vc, rvc)
+        assert float((o.float() - ro.float()).abs().max()) <= ABS_F16
+        assert bool(torch.isfinite(o).all())
+
+
 def test_static_scratch_entry_refuses_what_the_workspace_entry_refuses():
     d = torch.zeros(4096, device=DEV, dtype=torch.float16)
     p = d.data_ptr()
