@@ -558,6 +558,40 @@ def main():
         ops_out["dynamic_quantize_linear"] = e
         del xs, ys
 
+    if want("rms_norm_quantize"):
+        # the head of a quantised layer: RmsNormalization then DynamicQuantizeLinear of its output, as the fused pair
+        # (two launches, the normalised tensor read once) and as the two operators one after the other (three
+        # launches, read twice).  Algorithmic bytes of the pair: x in, y out, y in, yq out.
+        nb = 4
+        xs = [torch.randn((4096, 4096), device=dev) for _ in range(nb)]
+        wg = torch.rand(4096, device=dev) + 0.5
+        yn = [torch.empty((4096, 4096), device=dev) for _ in range(nb)]
+        yq = [torch.empty((4096, 4096), device=dev, dtype=torch.uint8) for _ in range(nb)]
+        sc_, zp_ = torch.empty((), device=dev), torch.empty((), device=dev, dtype=torch.uint8)
+        L = ops.lib()
+        wsf = torch.empty(L.rg_hip_rms_norm_quantize_workspace(4096, 4096), dtype=torch.uint8, device=dev)
+        wsq = torch.empty(L.rg_hip_dynamic_quantize_linear_workspace(4096 * 4096), dtype=torch.uint8, device=dev)
+        st = lambda: torch.cuda.current_stream().cuda_stream
+
+        def fused(i):
+            rc = L.rg_hip_rms_norm_quantize(yq[i].data_ptr(), sc_.data_ptr(), zp_.data_ptr(), yn[i].data_ptr(), xs[i].data_ptr(),
+                                            wg.data_ptr(), 4096, 4096, 1e-5, wsf.data_ptr(), wsf.numel(), st())
+            assert rc == 0, rc
+
+        def apart(i):
+            ops.rms_norm(xs[i], wg, 1e-5, out=yn[i])
+            ops.dynamic_quantize_linear(yn[i], out=yq[i], workspace=wsq)
+
+        wall, dms_f, mode = time_steps(torch, fused, steps, warmup, nb)
+        wall, dms_a, mode = time_steps(torch, apart, steps, warmup, nb)
+        pair_bytes = 4096 * 4096 * (4 + 4 + 4 + 1) + 4096 * 4
+        e = hbm_entry(pair_bytes, dms_f, None, (4 + 1) / 13)
+        e.update(workload="RmsNormalization f32 [4096,4096] -> DynamicQuantizeLinear, fused pair (2 launches)",
+                 device_ms_per_launch=round(dms_f, 5), timing=mode, two_operators_device_ms=round(dms_a, 5),
+                 two_operators_gbs=round(pair_bytes / (dms_a * 1e-3) / 1e9, 1))
+        ops_out["rms_norm_quantize"] = e
+        del xs, yn, yq
+
     if want("cast"):
         # the Cast either side of the fp16 operators: f32 -> fp16 of an activation tensor (6 B per element)
         nb = 6  # 6 x 100 MB

@@ -1360,6 +1360,102 @@ static void quantisedLinearStream() {
         }
 }
 
+// The head of a quantised layer as a graph: RmsNormalization -> DynamicQuantizeLinear -> MatMulInteger ->
+// DequantizeLinear.  On the AMD target lower() joins the first two (the normalising launch leaves its output's
+// extrema, so the normalised tensor is read once) and the last two; the normalised tensor stays an output of the
+// joined node (here it is a result of the graph as well).  Checked against the oracle chain: the normalised
+// tensor within 1e-5 relative of the reference's serial sum, everything behind it bit for bit on that tensor.
+static void normQuantisedLinearStream() {
+    constexpr dim_t M = 64, K = 1024, N = 256;
+    auto x = Tensor::share(DataType::F32, Shape{M, K});
+    auto wn = Tensor::share(DataType::F32, Shape{K});
+    auto xn = Tensor::share(DataType::F32, Shape{M, K});
+    auto xq = Tensor::share(DataType::U8, Shape{M, K});
+    auto scale = Tensor::share(DataType::F32, Shape{});
+    auto zp = Tensor::share(DataType::U8, Shape{});
+    auto [wBlob, wPtr] = kernel::Blob::share(K * N);
+    auto w = Tensor::share(DataType::I8, Shape{K, N}, LayoutType::Others, wBlob);
+    auto acc = Tensor::share(DataType::I32, Shape{M, N});
+    auto y = Tensor::share(DataType::F32, Shape{M, N});
+    std::mt19937 rng(27);
+    std::vector<int8_t> w_(K * N);
+    for (auto &v : w_) v = static_cast<int8_t>(rng());
+    std::memcpy(wPtr, w_.data(), w_.size());
+    std::vector<float> x_(M * K), g_(K);
+    std::normal_distribution<float> g(0.1f, 1.5f);
+    std::uniform_real_distribution<float> u(0.5f, 1.5f);
+    for (auto &v : x_) v = g(rng);
+    for (auto &v : g_) v = u(rng);
+
+    // edges: 0 x 1 gain | 2 xn | 3 xq 4 scale 5 zp | 6 W (local) 7 acc | 8 y
+    graph_topo::GraphTopo topo(2, 2);
+    topo.pushNode({0, 1}, 0, 1);
+    topo.pushNode({2}, 0, 3);
+    topo.pushNode({3, 6, 5}, 1, 1);
+    topo.pushNode({7, 4}, 0, 1);
+    topo.setGlobalOutput(0, 8);
+    topo.setGlobalOutput(1, 2);
+    std::vector<computation::Node> ops;
+    ops.push_back({std::make_unique<computation::RmsNormalization>(1e-5f), "norm"});
+    ops.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
+    ops.push_back({std::make_unique<computation::MatMulInteger>(), "matmul"});
+    ops.push_back({std::make_unique<computation::DequantizeLinear>(), "dequantise"});
+    auto lowered = computation::Graph(std::move(topo), std::move(ops),
+                                      {{x, "x"}, {wn, "gain"}, {xn, "xn"}, {xq, "xq"}, {scale, "scale"}, {zp, "zp"},
+                                       {w, "W"}, {acc, "acc"}, {y, "y"}})
+                       .lower(computation::Target::Amd);
+    EXPECT(lowered._internal.nodes.size() == 2);
+    EXPECT(lowered._internal.nodes[0].name == "norm+quantise" && lowered._internal.nodes[0].kernel->is<RmsNormalizationQuantizeHip>());
+    EXPECT(lowered._internal.nodes[1].name == "matmul+dequantise" && lowered._internal.nodes[1].kernel->is<MatMulIntegerDequantizeHip>());
+    {
+        auto node = lowered._internal.topology.node(0);
+        EXPECT(node.inputs.size() == 2 && node.outputs.size() == 4);
+    }
+
+    auto dev = device::init(Device::Type::Amd, 0, "pool=4294967296");
+    for (auto allocator : {flatAllocate, reusableAllocate}) {
+        auto stream = lowered.lower(dev, allocator);
+        stream.setData(0, x_.data(), x->bytesSize());
+        stream.setData(1, g_.data(), wn->bytesSize());
+        stream.run();
+        device::sync(Device::Type::Amd);
+        std::vector<float> out(M * N), norm(M * K), normRef(M * K);
+        EXPECT(stream.copyData(stream.graph().topology.globalOutputs()[0], out.data(), out.size() * 4));
+        EXPECT(stream.copyData(stream.graph().topology.globalOutputs()[1], norm.data(), norm.size() * 4));
+        oracle_rms_norm_f32(normRef.data(), x_.data(), g_.data(), M, K, 1e-5f, 1);
+        bool close = true;
+        for (size_t i = 0; i < norm.size(); ++i) close &= std::fabs(norm[i] - normRef[i]) <= 1e-5f * std::fabs(normRef[i]) + 1e-30f;
+        EXPECT(close);
+        // the chain behind the normalised tensor, on the tensor the device produced
+        std::vector<uint8_t> q(M * K);
+        float s;
+        uint8_t z;
+        oracle_dynamic_quantize_linear(q.data(), &s, &z, norm.data(), norm.size());
+        std::vector<int32_t> accRef(M * N);
+        oracle_matmul_integer(accRef.data(), q.data(), w_.data(), &z, 0, 1, nullptr, 1, 1, 1, M, K, N, nullptr, nullptr, 1, 1, 8);
+        std::vector<float> ref(M * N);
+        oracle_dequantize_linear(ref.data(), accRef.data(), &s, nullptr, 1, 1, M * N, ORACLE_I32, 1, 1);
+        EXPECT(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0);
+    }
+    // shapes the pair is not joined for keep their two kernels (rows that are no whole vectors)
+    {
+        auto xo = Tensor::share(DataType::F32, Shape{8, 130});
+        auto wo = Tensor::share(DataType::F32, Shape{130});
+        auto qo = Tensor::share(DataType::U8, Shape{8, 130});
+        graph_topo::GraphTopo t2(2, 3);
+        t2.pushNode({0, 1}, 0, 1);
+        t2.pushNode({2}, 0, 3);
+        for (count_t i = 0; i < 3; ++i) t2.setGlobalOutput(i, 3 + i);
+        std::vector<computation::Node> ops2;
+        ops2.push_back({std::make_unique<computation::RmsNormalization>(1e-5f), "norm"});
+        ops2.push_back({std::make_unique<computation::DynamicQuantizeLinear>(), "quantise"});
+        auto apart = computation::Graph(std::move(t2), std::move(ops2),
+                                        {{xo, "x"}, {wo, "gain"}, {xo, "xn"}, {qo, "xq"}, {scale, "scale"}, {zp, "zp"}})
+                         .lower(computation::Target::Amd);
+        EXPECT(apart._internal.nodes.size() == 2 && apart._internal.nodes[0].kernel->is<RmsNormalizationHip>());
+    }
+}
+
 // One decode step of an attention block as a graph: RotaryEmbedding on q and k ([N, 1, heads, D]),
 // Reshape to the attention layout ([N, heads, 1, D]: the same bytes, no kernel), Attention with the
 // caches as persistent global outputs.  Two steps enqueued routine by routine, then the graph is
@@ -1974,6 +2070,7 @@ int main(int argc, char **argv) {
         RUN(dataMoversHip);
         RUN(fusedQkvDecodeStream);
         RUN(quantisedLinearStream);
+        RUN(normQuantisedLinearStream);
         RUN(executorOnGpu);
         RUN(decodeAttentionStream);
         RUN(prefillAttentionStream);

@@ -368,6 +368,26 @@ def _dql_check(x):
     return host(y), host(scale)[0], host(zp)[0]
 
 
+def test_rms_norm_quantize_fused_pair():
+    # the fused pair against its two operators: the normalised tensor bit for bit what rg_hip_rms_norm writes, the
+    # quantised tensor, scale and zero point bit for bit what the CPU kernel computes from that tensor
+    rng = np.random.default_rng(31)
+    for rows, cols in ((4096, 4096), (7, 4096), (1024, 132), (300, 8192), (3, 1024), (2048, 512)):
+        x = torch.from_numpy(rng.standard_normal((rows, cols)).astype(np.float32) * 2 + 0.25).to(DEV)
+        w = torch.from_numpy(rng.uniform(0.5, 1.5, cols).astype(np.float32)).to(DEV)
+        y, yq, scale, zp = ops.rms_norm_quantize(x, w, 1e-5)
+        torch.cuda.synchronize()
+        assert torch.equal(y, ops.rms_norm(x, w, 1e-5))
+        ry, rs, rz = oracle.dynamic_quantize_linear(y.cpu().numpy().reshape(-1))
+        assert np.array_equal(yq.cpu().numpy().reshape(-1), ry) and scale.item() == rs and zp.item() == rz
+        ref = oracle.rms_norm(x.cpu().numpy(), w.cpu().numpy(), 1e-5)
+        assert np.all(np.abs(y.cpu().numpy() - ref) <= 1e-5 * np.abs(ref) + 1e-30)
+    # shapes the pair is not fused for are reported as such
+    assert ops.lib().rg_hip_rms_norm_quantize_workspace(16, 130) == 0
+    assert ops.lib().rg_hip_rms_norm_quantize_workspace(1 << 20, 256) == 0
+    assert ops.lib().rg_hip_rms_norm_quantize_workspace(4096, 4096) == 1024 * 8
+
+
 def test_dynamic_quantize_reference_kats():
     # src/04kernel/test/kernels/dynamic_quantize_linear/test_cpu.cpp:21-38 and test_cuda.cpp:36-39
     y, scale, zp = _dql_check(np.array([0, 2, -3, -2.5, 1.34, 0.5], np.float32))
