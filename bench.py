@@ -84,6 +84,9 @@ def parse():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a reference point for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters into bytes)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="print the issue and copy-rate probes of librg_probe.so (shader clocks per matrix product with "
+                         "other instructions behind it; bytes per clock a CU takes from L2) as one JSON line, and exit")
     return ap.parse_args()
 
 
@@ -233,7 +236,9 @@ def probes():
         lib = C.CDLL(path)
         vp, sz = C.c_void_p, C.c_size_t
         for name, args in (("rg_probe_mfma_i8", [vp, vp, sz, sz, vp]), ("rg_probe_hbm_read", [vp, vp, sz, sz, vp]),
-                           ("rg_probe_hbm_write", [vp, sz, sz, vp]), ("rg_probe_hbm_copy", [vp, vp, sz, sz, vp])):
+                           ("rg_probe_hbm_write", [vp, sz, sz, vp]), ("rg_probe_hbm_copy", [vp, vp, sz, sz, vp]),
+                           ("rg_probe_issue_shadow", [vp, C.c_int, C.c_int, sz, sz, vp]),
+                           ("rg_probe_copy_rate", [vp, vp, C.c_int, sz, sz, sz, sz, vp])):
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = C.c_int, args
         _PROBES.append(lib)
@@ -247,6 +252,46 @@ def pooled(fn_piece, pieces):
         from concurrent.futures import ThreadPoolExecutor
         _POOL.append(ThreadPoolExecutor(CPU_THREADS))
     return lambda: list(_POOL[0].map(fn_piece, pieces))
+
+
+def calibrate(torch):
+    """The probes behind the issue budgets that the matrix kernels are written to: clocks per
+    v_mfma_i32_32x32x32_i8 (32 when nothing delays it) with `count` instructions of one kind issued behind every
+    product by a wavefront alone on its SIMD, and the bytes per clock one CU takes from L2."""
+    pr = probes()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.zeros(8192, dtype=torch.int64, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    kinds = ["v_xor_b32", "s_nop", "ds_read_b128", "s_add_u32 (dependent)", "v_exp_f32", "v_cvt_pk_f16_f32",
+             "v_dot2c_f32_f16", "v_max3_f32", "v_fma_f32", "ds_read_b64_tr_b16"]
+    shadow = {}
+    iters = 64
+    for kind, name in enumerate(kinds):
+        row = {}
+        for count in (0, 1, 2, 3, 4, 6, 8, 12):
+            for _ in range(2):
+                rc = pr.rg_probe_issue_shadow(out.data_ptr(), kind, count, cus, iters, st)
+                if rc != 0:
+                    raise RuntimeError(f"rg_probe_issue_shadow -> {rc}")
+                torch.cuda.synchronize()
+            row[str(count)] = round(out[:cus].double().mean().item() / (iters * 16), 1)
+        shadow[name] = row
+    src = torch.zeros(32 << 20, dtype=torch.uint8, device="cuda")
+    copy = {}
+    iters = 256
+    for to_lds in (1, 0):
+        for waves in (4, 8):
+            for depth in (4, 8, 16, 32):
+                for _ in range(2):
+                    rc = pr.rg_probe_copy_rate(out.data_ptr(), src.data_ptr(), to_lds, waves, depth, cus, iters, st)
+                    if rc != 0:
+                        raise RuntimeError(f"rg_probe_copy_rate -> {rc}")
+                    torch.cuda.synchronize()
+                clocks = out[:cus].double().mean().item()
+                copy[f"{'lds' if to_lds else 'regs'}_{waves}w_x{depth}"] = round(iters * depth * waves * 1024 / clocks, 1)
+    return {"clocks_per_mfma_i8_32x32x32_with_n_behind_it": shadow, "l2_bytes_per_clock_per_cu": copy,
+            "note": "zero operands and a constant source: the clock stays up, clocks are what is measured; "
+                    "key of the copy table: destination, wavefronts, 1 KiB transfers in flight per wavefront"}
 
 
 CEILINGS = {}   # hbm_read / hbm_write / hbm_copy entries of this run (filled before the first operator)
@@ -288,6 +333,10 @@ def main():
 
     def want(name):
         return args.ops == "all" and (not only or name in only)
+
+    if args.calibrate:
+        print(json.dumps(calibrate(torch)))
+        return
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
