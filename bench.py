@@ -48,7 +48,7 @@ MEASURED_TRAFFIC = {
     "softmax_causal": (2 * 540713 + 2097158) * 1024,
     "rope": (2 * 131646 + 262167) * 1024,
     "dequantize_linear": (2 * 8292 + 65569) * 1024,
-    "matmul_integer": (2 * 50834 + 65647) * 1024,
+    "matmul_integer": (2 * 50313 + 65560) * 1024,
     "attention_prefill": (2 * 110058 + 196608) * 1024,
     "cast": (2 * 32784 + 32768) * 1024,
     "matmul": (2 * 98778 + 33024) * 1024,
@@ -56,7 +56,8 @@ MEASURED_TRAFFIC = {
     "matmul_eight_rows": (2 * 16661 + 64) * 1024,
     "dequantize_linear_i32": (2 * 32869 + 65611) * 1024,
     "transpose": (2 * 65552 + 131217) * 1024,
-    "matmul_integer_dequantize": (2 * 49361 + 65582) * 1024,
+    "matmul_integer_dequantize": (2 * 50363 + 65581) * 1024,
+    "rms_norm_quantize": (2 * 32883 + 65568 + 2 * 32889 + 16384) * 1024,
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
     "matmul_one_row": (2 * 16444 + 8) * 1024,
     "matmul_one_row_kn": (2 * 16499 + 20) * 1024,
@@ -634,7 +635,7 @@ def main():
         wall, dms_f, mode = time_steps(torch, fused, steps, warmup, nb)
         wall, dms_a, mode = time_steps(torch, apart, steps, warmup, nb)
         pair_bytes = 4096 * 4096 * (4 + 4 + 4 + 1) + 4096 * 4
-        e = hbm_entry(pair_bytes, dms_f, None, (4 + 1) / 13)
+        e = hbm_entry(pair_bytes, dms_f, "rms_norm_quantize", (4 + 1) / 13)
         e.update(workload="RmsNormalization f32 [4096,4096] -> DynamicQuantizeLinear, fused pair (2 launches)",
                  device_ms_per_launch=round(dms_f, 5), timing=mode, two_operators_device_ms=round(dms_a, 5),
                  two_operators_gbs=round(pair_bytes / (dms_a * 1e-3) / 1e9, 1))
