@@ -171,6 +171,19 @@ int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtyp
                   float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
                   const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
                   size_t c_stride_m, size_t c_stride_n, void *stream);
+/* The same product with a workspace, as the reference's routine receives one from its lowering
+ * (src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:12,38: `lower` returns a RoutineWorkspace and the routine is
+ * handed `void *workspace`).  rg_hip_matmul_workspace() says how many bytes help for a shape (0: none do, and
+ * rg_hip_matmul_ws then runs exactly what rg_hip_matmul runs).  With at least that many bytes (8-byte aligned,
+ * contents arbitrary, nothing to clear; not to be shared by calls that may overlap), one to four rows of A
+ * against FP16 / BF16 weights kept as [k, n] - a decode step on the layout ONNX MatMul stores - run with k shared
+ * between workgroups that each read 512 contiguous bytes of a k-row; their float sums meet in the workspace and
+ * are added in a fixed order, so results do not depend on timing.  A smaller or NULL workspace is not an error. */
+size_t rg_hip_matmul_workspace(int dtype, int trans_a, int trans_b, size_t batch, size_t m, size_t k, size_t n);
+int rg_hip_matmul_ws(void *y, const void *a, const void *b, const void *c, int dtype, int trans_a, int trans_b,
+                     float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
+                     const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
+                     size_t c_stride_m, size_t c_stride_n, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- Transpose ----------------------------------------------------------------------------
  * replaces src/04kernel/cuda/src/transpose.cu + src/04kernel/src/kernels/transpose/cuda_kernel.cu:8-30;

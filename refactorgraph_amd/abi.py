@@ -49,6 +49,8 @@ SIGNATURES = {
     "rg_hip_cast": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rg_hip_transpose": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_matmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "rg_hip_matmul_workspace": (_sz, [_i, _i, _i, _sz, _sz, _sz, _sz]),
+    "rg_hip_matmul_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _sz, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp, _sz, _vp]),
     "rg_hip_split": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_concat": (_i, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "rg_hip_expand": (_i, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),

@@ -870,8 +870,12 @@ bool prefill_pays(size_t N, size_t n_head, size_t n_kv_head, size_t seq, size_t 
     // Few items: the tiled kernel shares an item's keys between workgroups (head dims 64 and 128, records in the
     // workspace), and then costs about 17.5 us + 9.4e-5 us per kv head and key, against 8 us + 7.3e-5 us per
     // kv head, key and query row on the split kernel (N = 1, 8 kv heads, 8 new rows: history 1000 13.9 us split
-    // against 18.1 tiled, 4000 26.1 against 22.7, 32768 154 against 46).  The history is device data: half of the
-    // capacity stands for it.
+    // against 18.1 tiled, 4000 26.1 against 22.7, 32768 154 against 46).  The history is device data and the host
+    // may not read it, so half of the capacity stands for it.  Both costs are linear in the history with the
+    // tiled kernel's slope the smaller one, so the wrong choice costs most at the ends: with a history near
+    // nothing where the rule chose tiled (about 10 us lost, the difference of the constant terms), with a full
+    // cache where it chose split (the slopes' difference times the capacity).  Half the capacity makes these two
+    // worst cases meet as closely as one fixed value can.
     if (ranges_fit && seq == 1 && split_launches >= 2 && (D == 64 || D == 128)) return true;  // (16 x 28/4 heads, history 4000: 80 -> 52 us)
     if (ranges_fit && seq >= 2 && items * 2 <= 512 && cap >= 1024 && (D == 64 || D == 128)) {
         const double keys = static_cast<double>(N * n_kv_head) * static_cast<double>(cap) / 2;

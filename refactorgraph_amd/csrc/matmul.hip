@@ -34,6 +34,9 @@
 
 #include "common.hpp"
 
+#include <atomic>
+#include <chrono>
+
 namespace rg {
 namespace {
 
@@ -1441,6 +1444,454 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
     }
 }
 
+// ---------------------------------------------------------------- one to four rows of A, B as [k, n], k shared between workgroups
+//
+// The kernel above walks all of k in one workgroup, so its strips must be narrow for the launch to cover the chip:
+// at n = 4096 a workgroup reads 32 to 128 bytes of every k-row, and runs that short cost DRAM and L2 efficiency
+// (one row against [4096, 4096]: 15.5 us where W as [n, k] takes 7).  With a workspace the strip can be wide
+// instead: a workgroup takes 256 columns (512 contiguous bytes of a k-row, two k-rows per wavefront load) and a
+// share of k, keeps its whole share in flight at once when that is at most 256 k-rows (8 loads per lane), and
+// leaves its float sums in the workspace; the workgroup that finds every share of its strip delivered adds the shares
+// in their fixed order and stores.  The result therefore does not depend on which workgroup that is.
+// (the hand-off is described where it happens; it uses no atomic operation and needs nothing cleared)
+constexpr int KSP_COLS = 256;   // columns of a strip
+constexpr int KSP_ROWS = 32;    // k-rows a workgroup's 16 wavefronts load per instruction
+constexpr int KSP_DEPTH = 8;    // loads per lane in flight
+constexpr int KSP_MAX_KR = 2048;  // k-rows of a share
+
+__device__ __forceinline__ void store_through(float *p, float v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_through(const float *p) {
+    return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+template <class T, int M>
+__global__ __launch_bounds__(1024) void mm_kn_split(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
+                                                   uint32_t m, uint32_t k, uint32_t n, float alpha, float beta, uint32_t kr,
+                                                   uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ flags,
+                                                   unsigned long long launch_no) {
+    // kr: k-rows per share, a multiple of KSP_ROWS * KSP_DEPTH; k is even
+    __shared__ __align__(16) float sums[16 * M * KSP_COLS];  // [wavefront][row of A][column of the strip]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t strip = blockIdx.x, share = blockIdx.y;
+    const uint32_t col0 = strip * KSP_COLS, k0 = share * kr;
+    const uint32_t k_here = k - k0 < kr ? k - k0 : kr;           // k-rows of this share that exist (even)
+    const bool live = col0 + 8 * l32 < n;
+    const T *bcol = b + (live ? col0 + 8 * l32 : 0);
+    const uint32_t my_row = 2 * wave + half;                     // + KSP_ROWS * j
+
+    float acc[M][8];
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
+
+    // The wavefront's two k-rows of a load are neighbours, so their elements of a row of A are one aligned 32-bit
+    // word at a wave-uniform address: scalar loads, which neither wait for the loads of B nor make them wait.
+    struct Round {
+        u32x4 v[KSP_DEPTH];
+        uint32_t pa[M][KSP_DEPTH];
+    };
+    auto load = [&](Round &t, uint32_t base) {
+#pragma unroll
+        for (int i = 0; i < M; ++i)
+#pragma unroll
+            for (int j = 0; j < KSP_DEPTH; ++j) {
+                const uint32_t r = base + KSP_ROWS * j + 2 * wave;
+                const bool have = static_cast<uint32_t>(i) < m && r < k_here;
+                const uint32_t word = *reinterpret_cast<const uint32_t *>(a + static_cast<uint64_t>(have ? i : 0) * k + k0 + (have ? r : 0));
+                t.pa[i][j] = have ? word : 0u;
+            }
+#pragma unroll
+        for (int j = 0; j < KSP_DEPTH; ++j) {
+            // rows beyond the share repeat its last row; their factor from A is zero
+            const uint32_t r = base + KSP_ROWS * j + my_row, rr = r < k_here ? r : k_here - 1;
+            t.v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(bcol + static_cast<uint64_t>(k0 + rr) * n));
+        }
+    };
+    auto multiply = [&](const Round &t) {
+#pragma unroll
+        for (int j = 0; j < KSP_DEPTH; ++j) {
+            float f[8];
+            widen8<T>(t.v[j], f);
+#pragma unroll
+            for (int i = 0; i < M; ++i) {
+                const uint16_t bits = static_cast<uint16_t>(half ? t.pa[i][j] >> 16 : t.pa[i][j] & 0xffffu);
+                const float av = up(__builtin_bit_cast(T, bits));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(av, f[e], acc[i][e]);
+            }
+        }
+    };
+
+    constexpr uint32_t STEP = KSP_ROWS * KSP_DEPTH;
+    Round r0, r1;
+    load(r0, 0);
+    for (uint32_t base = 0; base < kr; base += 2 * STEP) {
+        const bool more = base + STEP < kr;
+        if (more) load(r1, base + STEP);
+        multiply(r0);
+        if (more) {
+            if (base + 2 * STEP < kr) load(r0, base + 2 * STEP);
+            multiply(r1);
+        }
+    }
+
+    // the two halves of a wavefront hold different k-rows of the same columns
+#pragma unroll
+    for (int i = 0; i < M; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            const float t = swap32_sum(acc[i][e], acc[i][e + 1]);  // lower half: column e, upper half: column e + 1
+            sums[(wave * M + i) * KSP_COLS + 8 * l32 + e + half] = t;
+        }
+    __syncthreads();
+    const T *C = static_cast<const T *>(bias.ptr);
+    auto finish = [&](uint32_t i, uint32_t col, float v) {
+        v *= alpha;
+        if (C) v += beta * up(C[i * bias.sm + col * bias.sn]);
+        y[static_cast<uint64_t>(i) * n + col] = down<T>(v);
+    };
+#pragma unroll
+    for (int q = 0; q < (M * KSP_COLS + 1023) / 1024; ++q) {
+        const uint32_t t = tid + 1024 * q, i = t / KSP_COLS, cc = t % KSP_COLS;
+        float v = 0.f;
+        if (t < M * KSP_COLS) {
+#pragma unroll
+            for (int wv = 0; wv < 16; ++wv) v += sums[(wv * M + i) * KSP_COLS + cc];
+            if (shares == 1) {
+                if (i < m && col0 + cc < n) finish(i, col0 + cc, v);
+            } else {
+                store_through(part + (static_cast<uint64_t>(strip) * shares + share) * (M * KSP_COLS) + t, v);
+            }
+        }
+    }
+    if (shares == 1) return;
+    // Hand-off without a counter: the sums are written through; every wavefront waits until its stores have been
+    // acknowledged and the barrier collects the wavefronts; then one thread writes this share's flag, the launch's
+    // number, waits for that store's acknowledgement as well, and after a second barrier every thread reads one flag
+    // of the strip (loads that bypass the XCD's L2).  A workgroup that finds all flags set adds the shares up.  The
+    // workgroup whose flag reached memory last is certain to find them all; another one that arrived at almost the
+    // same time may too, and then both store the same values (same sums, same order).  Flags that hold anything
+    // else than this launch's number - whatever the workspace held before - count as not set, so nothing has to be
+    // cleared beforehand; whoever adds up clears the strip's flags afterwards (every share has arrived by then), so
+    // that a replay of a captured launch, which carries the same number, starts like the first run.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    unsigned long long *strip_flags = flags + static_cast<uint64_t>(strip) * shares;
+    if (tid == 0) {
+        __hip_atomic_store(strip_flags + share, launch_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    int set = 1;
+    if (tid < shares) set = __hip_atomic_load(strip_flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch_no;
+    if (!__syncthreads_and(set)) return;
+    const float *strip_part = part + static_cast<uint64_t>(strip) * shares * (M * KSP_COLS);
+#pragma unroll
+    for (int q = 0; q < (M * KSP_COLS + 1023) / 1024; ++q) {
+        const uint32_t t = tid + 1024 * q, i = t / KSP_COLS, cc = t % KSP_COLS;
+        if (t < M * KSP_COLS) {
+            // eight shares' sums are requested by one piece of assembly that also waits for them (as separate
+            // device-scope loads each would be followed by a wait of its own), then added in the shares' order
+            float v = 0.f;
+            if constexpr (M == 1) {
+                // one row of A: the shares' sums are 1 KiB apart, so sixteen of them are four addresses with four
+                // immediate offsets each - one request, one wait (a strip's last group may reach into the next
+                // strip's sums or the padding behind the last one; those values are not used)
+                for (uint32_t sh = 0; sh < shares; sh += 16) {
+                    float g[16];
+                    const uint32_t o0 = (sh * KSP_COLS + t) * 4, o1 = o0 + 4096, o2 = o0 + 8192, o3 = o0 + 12288;
+                    asm volatile("global_load_dword %0, %16, %20 sc1\n\t"
+                                 "global_load_dword %1, %16, %20 offset:1024 sc1\n\t"
+                                 "global_load_dword %2, %16, %20 offset:2048 sc1\n\t"
+                                 "global_load_dword %3, %16, %20 offset:3072 sc1\n\t"
+                                 "global_load_dword %4, %17, %20 sc1\n\t"
+                                 "global_load_dword %5, %17, %20 offset:1024 sc1\n\t"
+                                 "global_load_dword %6, %17, %20 offset:2048 sc1\n\t"
+                                 "global_load_dword %7, %17, %20 offset:3072 sc1\n\t"
+                                 "global_load_dword %8, %18, %20 sc1\n\t"
+                                 "global_load_dword %9, %18, %20 offset:1024 sc1\n\t"
+                                 "global_load_dword %10, %18, %20 offset:2048 sc1\n\t"
+                                 "global_load_dword %11, %18, %20 offset:3072 sc1\n\t"
+                                 "global_load_dword %12, %19, %20 sc1\n\t"
+                                 "global_load_dword %13, %19, %20 offset:1024 sc1\n\t"
+                                 "global_load_dword %14, %19, %20 offset:2048 sc1\n\t"
+                                 "global_load_dword %15, %19, %20 offset:3072 sc1\n\t"
+                                 "s_waitcnt vmcnt(0)"
+                                 : "=&v"(g[0]), "=&v"(g[1]), "=&v"(g[2]), "=&v"(g[3]), "=&v"(g[4]), "=&v"(g[5]), "=&v"(g[6]), "=&v"(g[7]),
+                                   "=&v"(g[8]), "=&v"(g[9]), "=&v"(g[10]), "=&v"(g[11]), "=&v"(g[12]), "=&v"(g[13]), "=&v"(g[14]), "=&v"(g[15])
+                                 : "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(strip_part)
+                                 : "memory");
+#pragma unroll
+                    for (int j = 0; j < 16; ++j)
+                        if (sh + j < shares) v += g[j];
+                }
+            } else
+            for (uint32_t sh = 0; sh < shares; sh += 8) {
+                uint32_t off[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) off[j] = ((sh + j < shares ? sh + j : shares - 1) * (M * KSP_COLS) + t) * 4;
+                float g0, g1, g2, g3, g4, g5, g6, g7;
+                asm volatile("global_load_dword %0, %8, %16 sc1\n\t"
+                             "global_load_dword %1, %9, %16 sc1\n\t"
+                             "global_load_dword %2, %10, %16 sc1\n\t"
+                             "global_load_dword %3, %11, %16 sc1\n\t"
+                             "global_load_dword %4, %12, %16 sc1\n\t"
+                             "global_load_dword %5, %13, %16 sc1\n\t"
+                             "global_load_dword %6, %14, %16 sc1\n\t"
+                             "global_load_dword %7, %15, %16 sc1\n\t"
+                             "s_waitcnt vmcnt(0)"
+                             : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3), "=&v"(g4), "=&v"(g5), "=&v"(g6), "=&v"(g7)
+                             : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]),
+                               "s"(strip_part)
+                             : "memory");
+                const float got[8] = {g0, g1, g2, g3, g4, g5, g6, g7};
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (sh + j < shares) v += got[j];
+            }
+            if (i < m && col0 + cc < n) finish(i, col0 + cc, v);
+        }
+    }
+    if (tid < shares) __hip_atomic_store(strip_flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Shares of k for the kernel above: about one workgroup per CU, shares of whole load rounds, at most 255.
+struct KnSplitPlan {
+    uint32_t strips, shares, kr;
+    size_t ticket_bytes, bytes;
+};
+inline KnSplitPlan kn_split_plan(size_t k, size_t n, uint32_t rows_padded) {
+    KnSplitPlan p{};
+    p.strips = static_cast<uint32_t>((n + KSP_COLS - 1) / KSP_COLS);
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, c = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && c > 0) cus = c;
+        else cus = 256;
+    }
+    constexpr uint32_t STEP = KSP_ROWS * KSP_DEPTH;
+    uint32_t shares = (static_cast<uint32_t>(cus) + p.strips / 2) / p.strips;
+    if (shares < 1) shares = 1;
+    uint32_t kr = static_cast<uint32_t>((k + shares - 1) / shares);
+    kr = (kr + STEP - 1) / STEP * STEP;
+    if (kr > KSP_MAX_KR) kr = KSP_MAX_KR;
+    shares = static_cast<uint32_t>((k + kr - 1) / kr);
+    p.shares = shares;
+    p.kr = kr;
+    p.ticket_bytes = (static_cast<size_t>(p.strips) * shares * 8 + 255) / 256 * 256;  // one flag per share
+    p.bytes = p.ticket_bytes + static_cast<size_t>(p.strips) * shares * rows_padded * KSP_COLS * sizeof(float) + 16384;  // (padding: see the kernel)
+    return p;
+}
+
+// ---------------------------------------------------------------- up to 32 rows of A, B as [k, n], k shared between workgroups
+//
+// The same sharing for the matrix cores.  A workgroup takes a strip of 128 columns and at most 512 k-rows: that part
+// of B (128 KiB) is requested in one go, straight into LDS (16 wavefronts x 8 copies of four 256-byte rows, so every
+// byte the workgroup will ever read is in flight from its first microsecond), laid out like the B tile of the large
+// kernel: chunk c of k-row r at chunk position c ^ n_swizzle(r & 3), which makes the transposing 64-bit reads that
+// turn [k, n] into operand layout conflict free.  Wavefront w copies and multiplies k-rows 32 w .. 32 w + 31 for all
+// four column blocks of the strip, so it waits for its own copies only: eight v_mfma_f32_32x32x16 whose first
+// operand comes from two transposing reads (k-rows 8 h .. 8 h + 7 of the step for half h of the wavefront) and whose
+// second operand is one 128-bit load of A from global memory (row lane % 32, the same eight k; two such loads per
+// wavefront, issued before the copies so that they arrive before them - with every wavefront loading operands for
+// a quarter of the share instead, the 32-byte pieces of A's rows cost more than all of B: 15.7 us).  The sixteen
+// wavefronts' sums meet in LDS, the shares of k in the workspace as above.
+constexpr int KM_COLS = 128;      // columns of a strip (256 bytes of a k-row)
+constexpr int KM_ROWB = 256;      // bytes of a k-row of the strip in LDS
+constexpr int KM_MAX_KR = 512;    // k-rows of a share: 128 KiB of LDS
+constexpr int KM_PART = 4096;     // floats a workgroup leaves: 32 rows of A x 128 columns
+
+template <class T>
+__global__ __launch_bounds__(1024) void mm_kn_mfma_split(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
+                                                        uint32_t m, uint32_t k, uint32_t n, float alpha, float beta, uint32_t kr,
+                                                        uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ flags,
+                                                        unsigned long long launch_no) {
+    // kr: k-rows per share, a multiple of 128, at most KM_MAX_KR; k a multiple of 8, n of 128
+    __shared__ __align__(1024) uint8_t lds[KM_MAX_KR * KM_ROWB];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t strip = blockIdx.x, share = blockIdx.y;
+    const uint32_t col0 = strip * KM_COLS, k0 = share * kr;
+    const uint32_t k_here = k - k0 < kr ? k - k0 : kr;  // k-rows of this share that exist (a multiple of 8)
+
+    // the operand from A first: row l32 (rows beyond m repeat the last one, their results are not stored), k-rows
+    // 32 wave + 16 ks + 8 half .. + 7; beyond the share's last k-row the operand is zero
+    u32x4 af[2];
+    {
+        const T *arow = a + static_cast<uint64_t>(l32 < m ? l32 : m - 1) * k + k0;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const uint32_t kk = 32 * wave + 16 * ks + 8 * half;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(arow + (kk < k_here ? kk : 0));
+            af[ks] = kk < k_here ? v : u32x4{0, 0, 0, 0};
+        }
+    }
+    // the copies: instruction i of this wavefront brings k-rows 32 wave + 4 i .. + 3, the rows it multiplies itself;
+    // lane L fills chunk position L % 16 of row L / 16 of them, which holds chunk (L % 16) ^ n_swizzle(L / 16).
+    // Rows beyond the share's last one repeat it (A's operand is zero there).
+    const bool busy = 32 * wave < kr;
+    if (busy) {
+        const uint32_t cp_r = lane >> 4, chunk = (lane & 15) ^ n_swizzle(cp_r);
+        const T *src0 = b + col0 + 8 * chunk;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t r0 = 32 * wave + 4 * i, r = r0 + cp_r, rr = r < k_here ? r : k_here - 1;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src0 + static_cast<uint64_t>(k0 + rr) * n),
+                                             (__attribute__((address_space(3))) void *)(lds + r0 * KM_ROWB), 16, 0, 0);
+        }
+    }
+    f16v acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // a wavefront reads only what it has copied itself: no barrier
+    if (busy) {
+        // transposing read: lane s of a group of 16 addresses k-row s / 4, columns 4 (s % 4) .. + 3 of the group's 16;
+        // column block j of the strip is reached by XOR with 64 j (the swizzle leaves bits 6-7 of the offset alone)
+        const uint32_t s16 = lane & 15, v_r = s16 >> 2;
+        const uint32_t chunk = 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1);
+        const uint8_t *fp = lds + (32 * wave + 8 * half + v_r) * KM_ROWB + 16 * (chunk ^ n_swizzle(v_r)) + 8 * (s16 & 1);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint8_t *q = fp + 16 * ks * KM_ROWB;
+                const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (s4 __attribute__((address_space(3))) *)(lds + ((q - lds) ^ (64 * j))));
+                const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (s4 __attribute__((address_space(3))) *)(lds + (((q - lds) + 4 * KM_ROWB) ^ (64 * j))));
+                const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                acc[j] = Mfma<T>::run(u32x4{l2[0], l2[1], h2[0], h2[1]}, af[ks], acc[j]);
+            }
+    }
+    // lane holds row l32 of A; register e column 8 (e / 4) + 4 half + e % 4 of column block j.  The sixteen
+    // wavefronts' sums meet in the tile's memory, one column block at a time (64 KiB each).
+    float *sums = reinterpret_cast<float *>(lds);  // [wavefront][register][lane]
+    const T *C = static_cast<const T *>(bias.ptr);
+    auto finish = [&](uint32_t x, float v) {  // x: column block, register, lane as laid out above
+        const uint32_t e = (x >> 6) & 15, i = x & 31, col = col0 + 32 * (x >> 10) + 8 * (e >> 2) + 4 * ((x >> 5) & 1) + (e & 3);
+        if (i < m) {
+            v *= alpha;
+            if (C) v += beta * up(C[i * bias.sm + col * bias.sn]);
+            y[static_cast<uint64_t>(i) * n + col] = down<T>(v);
+        }
+    };
+    f4v mine;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        __syncthreads();  // the fragments, or the sums of the block before, have been read
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sums[wave * 1024 + e * 64 + lane] = acc[u][e];
+        __syncthreads();
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) v += sums[w * 1024 + tid];
+        if (shares == 1) finish(u * 1024 + tid, v);
+        mine[u] = v;
+    }
+    if (shares == 1) return;
+    // hand-off as in mm_kn_split; a thread's four sums are one 128-bit piece of the workspace, so that the workgroup
+    // that adds up gets eight shares with one request per thread
+    const float *strip_part = part + static_cast<uint64_t>(strip) * shares * KM_PART;
+    asm volatile("global_store_dwordx4 %0, %1, %2 sc1" : : "v"((share * KM_PART + 4 * tid) * 4), "v"(mine), "s"(strip_part) : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    unsigned long long *strip_flags = flags + static_cast<uint64_t>(strip) * shares;
+    if (tid == 0) {
+        __hip_atomic_store(strip_flags + share, launch_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    int set = 1;
+    if (tid < shares) set = __hip_atomic_load(strip_flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch_no;
+    if (!__syncthreads_and(set)) return;
+    f4v total = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t sh = 0; sh < shares; sh += 8) {
+        uint32_t off[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) off[j] = ((sh + j < shares ? sh + j : shares - 1) * KM_PART + 4 * tid) * 4;
+        f4v g0, g1, g2, g3, g4, g5, g6, g7;
+        asm volatile("global_load_dwordx4 %0, %8, %16 sc1\n\t"
+                     "global_load_dwordx4 %1, %9, %16 sc1\n\t"
+                     "global_load_dwordx4 %2, %10, %16 sc1\n\t"
+                     "global_load_dwordx4 %3, %11, %16 sc1\n\t"
+                     "global_load_dwordx4 %4, %12, %16 sc1\n\t"
+                     "global_load_dwordx4 %5, %13, %16 sc1\n\t"
+                     "global_load_dwordx4 %6, %14, %16 sc1\n\t"
+                     "global_load_dwordx4 %7, %15, %16 sc1\n\t"
+                     "s_waitcnt vmcnt(0)"
+                     : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3), "=&v"(g4), "=&v"(g5), "=&v"(g6), "=&v"(g7)
+                     : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]),
+                       "s"(strip_part)
+                     : "memory");
+        const f4v got[8] = {g0, g1, g2, g3, g4, g5, g6, g7};
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (sh + j < shares) total += got[j];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) finish(u * 1024 + tid, total[u]);
+    if (tid < shares) __hip_atomic_store(strip_flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+inline KnSplitPlan kn_mfma_split_plan(size_t k, size_t n) {
+    KnSplitPlan p{};
+    p.strips = static_cast<uint32_t>(n / KM_COLS);
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    uint32_t shares = (static_cast<uint32_t>(cus) + p.strips / 2) / p.strips;
+    if (shares < 1) shares = 1;
+    uint32_t kr = static_cast<uint32_t>((k + shares - 1) / shares);
+    kr = (kr + 127) / 128 * 128;
+    if (kr > KM_MAX_KR) kr = KM_MAX_KR;
+    p.shares = static_cast<uint32_t>((k + kr - 1) / kr);
+    p.kr = kr;
+    p.ticket_bytes = (static_cast<size_t>(p.strips) * p.shares * 8 + 255) / 256 * 256;  // one flag per share
+    p.bytes = p.ticket_bytes + static_cast<size_t>(p.strips) * p.shares * KM_PART * sizeof(float);
+    return p;
+}
+
+// A number no other launch of this process carries (started from the clock so that what an earlier process
+// left in a reused allocation does not match either).
+inline unsigned long long next_launch_number() {
+    static std::atomic<unsigned long long> counter{
+        static_cast<unsigned long long>(std::chrono::steady_clock::now().time_since_epoch().count()) * 0x9E3779B97F4A7C15ull};
+    return counter.fetch_add(1, std::memory_order_relaxed) | (1ull << 63);  // never 0, which stands for a cleared flag
+}
+
+template <class T>
+int launch_kn_split(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                    void *workspace, const KnSplitPlan &plan, hipStream_t s) {
+    auto *flags = static_cast<unsigned long long *>(workspace);
+    float *part = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + plan.ticket_bytes);
+    const dim3 grid(plan.strips, plan.shares, 1);
+    const unsigned long long no = next_launch_number();
+    if (m <= 1) mm_kn_split<T, 1><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares, part, flags, no);
+    else if (m <= 2) mm_kn_split<T, 2><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares, part, flags, no);
+    else mm_kn_split<T, 4><<<grid, 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares, part, flags, no);
+    return launch_status();
+}
+
+template <class T>
+int launch_kn_mfma_split(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
+                         void *workspace, const KnSplitPlan &plan, hipStream_t s) {
+    if constexpr (sizeof(T) == 2) {
+        auto *flags = static_cast<unsigned long long *>(workspace);
+        float *part = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + plan.ticket_bytes);
+        mm_kn_mfma_split<T><<<dim3(plan.strips, plan.shares, 1), 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares,
+                                                                                 part, flags, next_launch_number());
+        return launch_status();
+    } else {
+        return RG_HIP_E_UNSUPPORTED;
+    }
+}
+
 template <class T, int M, int L>
 int launch_gemv_kn_l(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
                      uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count, uint32_t row0, uint32_t rows, hipStream_t s) {
@@ -1501,7 +1952,7 @@ int launch_gemv(T *y, const T *a, const T *w, Bias bias, uint32_t m, uint32_t k,
 template <class T>
 int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_a, int trans_b, float alpha, float beta,
                  size_t batch, size_t m, size_t k, size_t n, const uint32_t *a_index, const uint32_t *b_index,
-                 hipStream_t s) {
+                 hipStream_t s, void *workspace = nullptr, size_t workspace_bytes = 0) {
     auto *y = static_cast<T *>(y_);
     auto *a = static_cast<const T *>(a_);
     auto *b = static_cast<const T *>(b_);
@@ -1625,6 +2076,27 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 
     auto launch = [&](uint32_t am0, uint32_t bm0, uint32_t ym0, uint32_t count) -> int {
         if constexpr (narrow) {
+            // five to 32 rows against weights as [k, n] with a workspace at hand: the same sharing on the matrix cores
+            if (workspace && !trans_a && !trans_b && m > 4 && m <= 32 && batch == 1 && count == 1 && n % KM_COLS == 0 && k > 0 &&
+                k % 8 == 0 && static_cast<uint64_t>(k) * n >= (1u << 20) && aligned16(b) && aligned16(a) &&
+                reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
+                const KnSplitPlan plan = kn_mfma_split_plan(k, n);
+                if (plan.shares <= 255 && plan.bytes <= workspace_bytes)
+                    return launch_kn_mfma_split<T>(y + static_cast<uint64_t>(ym0) * m * n, a + static_cast<uint64_t>(am0) * m * k,
+                                                   b + static_cast<uint64_t>(bm0) * k * n, bias, static_cast<uint32_t>(m),
+                                                   static_cast<uint32_t>(k), static_cast<uint32_t>(n), al, be, workspace, plan, s);
+            }
+            // one to four rows against weights as [k, n] with a workspace at hand: wide strips, k shared between
+            // workgroups (from 2 MB of weights on; below that the launch is all there is to either kernel)
+            if (workspace && !trans_a && !trans_b && m <= 4 && batch == 1 && count == 1 && n % 8 == 0 && k > 0 && k % 2 == 0 &&
+                static_cast<uint64_t>(k) * n >= (1u << 20) && aligned16(b) && reinterpret_cast<uintptr_t>(a) % 4 == 0 &&
+                reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
+                const KnSplitPlan plan = kn_split_plan(k, n, m <= 1 ? 1 : m <= 2 ? 2 : 4);
+                if (plan.shares <= 255 && plan.bytes <= workspace_bytes)
+                    return launch_kn_split<T>(y + static_cast<uint64_t>(ym0) * m * n, a + static_cast<uint64_t>(am0) * m * k,
+                                              b + static_cast<uint64_t>(bm0) * k * n, bias, static_cast<uint32_t>(m),
+                                              static_cast<uint32_t>(k), static_cast<uint32_t>(n), al, be, workspace, plan, s);
+            }
             if ((small_grid && (short_tile || fast)) || short_k) return launch_tiles16(am0, bm0, ym0, count);
             if (short_tile) {
                 const dim3 grid(static_cast<unsigned>((n + BN - 1) / BN), 1, count);
@@ -1786,10 +2258,33 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
 }  // namespace
 }  // namespace rg
 
+extern "C" size_t rg_hip_matmul_workspace(int dtype, int trans_a, int trans_b, size_t batch, size_t m, size_t k, size_t n) {
+    using namespace rg;
+    if ((dtype != RG_FP16 && dtype != RG_BF16) || trans_a || trans_b || batch != 1 || m == 0 || m > 32 || k == 0 ||
+        k > 0x7fffffffu || n > 0x7fffffffu || static_cast<uint64_t>(k) * n < (1u << 20))
+        return 0;
+    if (m > 4) {
+        if (n % KM_COLS != 0 || k % 8 != 0) return 0;
+        const KnSplitPlan plan = kn_mfma_split_plan(k, n);
+        return plan.shares <= 255 ? plan.bytes : 0;
+    }
+    if (n % 8 != 0 || k % 2 != 0) return 0;
+    const KnSplitPlan plan = kn_split_plan(k, n, m <= 1 ? 1 : m <= 2 ? 2 : 4);
+    return plan.shares <= 255 ? plan.bytes : 0;
+}
+
 extern "C" int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtype, int trans_a, int trans_b,
                              float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
                              const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
                              size_t c_stride_m, size_t c_stride_n, void *stream) {
+    return rg_hip_matmul_ws(y, a, b, c, dtype, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, c_stride_batch,
+                            c_stride_m, c_stride_n, nullptr, 0, stream);
+}
+
+extern "C" int rg_hip_matmul_ws(void *y, const void *a, const void *b, const void *c, int dtype, int trans_a, int trans_b,
+                                float alpha, float beta, size_t batch, size_t m, size_t k, size_t n,
+                                const uint32_t *a_index, const uint32_t *b_index, size_t c_stride_batch,
+                                size_t c_stride_m, size_t c_stride_n, void *workspace, size_t workspace_bytes, void *stream) {
     using namespace rg;
     if (!y || !a || !b) return RG_HIP_E_ARGUMENT;
     if (batch == 0 || m == 0 || n == 0) return 0;
@@ -1822,9 +2317,12 @@ extern "C" int rg_hip_matmul(void *y, const void *a, const void *b, const void *
     switch (dtype) {
         case RG_F32: return launch_typed<float>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
         case RG_F64: return launch_typed<double>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
-        case RG_FP16: return launch_typed<__half>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+        case RG_FP16:
+            return launch_typed<__half>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s, workspace,
+                                        workspace_bytes);
         case RG_BF16:
-            return launch_typed<__hip_bfloat16>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s);
+            return launch_typed<__hip_bfloat16>(y, a, b, bias, trans_a, trans_b, alpha, beta, batch, m, k, n, a_index, b_index, s,
+                                                workspace, workspace_bytes);
         default: return RG_HIP_E_UNSUPPORTED;
     }
 }

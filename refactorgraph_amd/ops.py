@@ -134,7 +134,7 @@ def cast(x, dtype, out=None):
     return y
 
 
-def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=None):
+def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=None, workspace=None):
     """Y = alpha * op(A) @ op(B) + beta * C.  a [..., m, k] ([..., k, m] when trans_a), b [..., k, n]
     ([..., n, k] when trans_b), batch dimensions broadcast; c broadcasts to [m, n] (any leading
     dimensions of size 1) or has the output's full shape.  float32/float64/float16/bfloat16."""
@@ -167,12 +167,16 @@ def matmul(a, b, c=None, trans_a=False, trans_b=False, alpha=1.0, beta=1.0, out=
         if cs[-2] == 1:
             sm = 0
     y = torch.empty(ob + (m, n), dtype=a.dtype, device=a.device) if out is None else out
-    check(lib().rg_hip_matmul(
+    if workspace is None:
+        # what the routine's lowering would ask the allocator for (a uint8 tensor passed as `workspace` is used as is)
+        need = lib().rg_hip_matmul_workspace(_T2CODE[a.dtype], int(trans_a), int(trans_b), batch, m, k, n)
+        workspace = torch.empty(need, dtype=torch.uint8, device=a.device) if need else None
+    check(lib().rg_hip_matmul_ws(
         _ptr(y), _ptr(a), _ptr(b), _ptr(c), _T2CODE[a.dtype], int(trans_a), int(trans_b), float(alpha), float(beta),
         batch, m, k, n,
         None if a_idx is None else a_idx.ctypes.data_as(C.c_void_p),
         None if b_idx is None else b_idx.ctypes.data_as(C.c_void_p),
-        sb, sm, sn, _stream()), "rg_hip_matmul")
+        sb, sm, sn, _ptr(workspace), 0 if workspace is None else workspace.numel(), _stream()), "rg_hip_matmul_ws")
     return y
 
 

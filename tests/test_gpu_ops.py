@@ -1646,6 +1646,49 @@ def test_matmul_few_rows_weights_as_k_by_n(m, k, n, dt):
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 4096), (2, 4096, 4096), (3, 1000, 4104), (4, 4096, 11008), (1, 8192, 2048),
+                                   (4, 520, 2056), (1, 33000, 256), (2, 256, 4096), (4, 20000, 1024), (3, 4096, 65536 + 8),
+                                   (8, 4096, 4096), (32, 4096, 4096), (13, 1000, 4224), (32, 520, 2048), (5, 4096, 11008),
+                                   (17, 33000, 256), (32, 256, 4096), (20, 20000, 1024), (31, 136, 32768)])
+def test_matmul_few_rows_k_by_n_with_workspace(m, k, n, dt):
+    # one to four rows against weights as [k, n] through rg_hip_matmul_ws: strips of 256 columns, k shared between
+    # workgroups, their float sums in a workspace that is handed over full of ones (nothing may need clearing) and
+    # reused by the second call; shares that end inside k, a last strip that ends inside its 256 columns, one share
+    # only (k = 256), more strips than CUs (n = 65544: two shares, a share holding at most 2048 k-rows); k beyond 255 shares never
+    # arises below 2^23, so the longest k here has shares of the maximum 2048 rows.  Five to 32 rows: the same sharing
+    # on the matrix cores (strips of 128 columns, shares of at most 512 k-rows copied straight into LDS), k that ends
+    # inside a share and inside a quarter of it, rows of A that the 32-row operand repeats.  Same bar as without
+    # the workspace, the same bits on every call, and exact on integer-valued operands.
+    rng = np.random.default_rng(37)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal((m, n)).astype(np.float32)
+    ad, wd, cd = (dev(t).to(dt) for t in (a, w, bias))
+    name = "fp16" if dt == torch.float16 else "bf16"
+    code = ops._T2CODE[dt]
+    need = ops.lib().rg_hip_matmul_workspace(code, 0, 0, 1, m, k, n)
+    assert need > 0
+    ws = torch.full((need + 64,), 0xff, dtype=torch.uint8, device="cuda")
+    f = lambda t: host(t.float())
+    to_oracle = (lambda t: host(t)) if name == "fp16" else (lambda t: host(t.view(torch.uint16)))
+    ref = oracle.matmul(to_oracle(ad), to_oracle(wd), to_oracle(cd), False, False, 0.5, -1.5, name)
+    ref = ref.astype(np.float32) if name == "fp16" else oracle._bf16_to_f32(ref)
+    first = ops.matmul(ad, wd, cd, False, False, 0.5, -1.5, workspace=ws)
+    _matmul_check(f(first), ref, 0.5 * _absprod(f(ad), f(wd), False, False), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    assert torch.equal(first, ops.matmul(ad, wd, cd, False, False, 0.5, -1.5, workspace=ws))
+    assert torch.equal(first, ops.matmul(ad, wd, cd, False, False, 0.5, -1.5))      # a fresh workspace of the size asked for
+    # a workspace that is too small is not an error: the call runs what rg_hip_matmul runs
+    small = torch.empty(64, dtype=torch.uint8, device="cuda")
+    _matmul_check(f(ops.matmul(ad, wd, cd, False, False, 0.5, -1.5, workspace=small)), ref,
+                  0.5 * _absprod(f(ad), f(wd), False, False), 2.0 ** -10 if name == "fp16" else 2.0 ** -7)
+    ai = rng.integers(-2, 3, (m, k)).astype(np.float32)
+    wi = rng.integers(-2, 3, (k, n)).astype(np.float32)
+    want = ai.astype(np.int64) @ wi.astype(np.int64)
+    if np.max(np.abs(want)) < (2048 if name == "fp16" else 256):
+        assert np.array_equal(f(ops.matmul(dev(ai).to(dt), dev(wi).to(dt), workspace=ws)), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 8, 1), (1, 4096, 4096), (2, 520, 37), (3, 1000, 250), (4, 4096, 1024), (4, 11008, 72),
                                    (1, 32768, 16), (4, 20480, 24), (3, 20488, 8), (1, 40000, 8), (2, 33008, 5), (5, 2048, 33), (7, 1000, 130),
                                    (8, 4096, 512), (6, 11008, 64)])
