@@ -174,7 +174,7 @@ int rg_hip_matmul(void *y, const void *a, const void *b, const void *c, int dtyp
 /* The same product with a workspace, as the reference's routine receives one from its lowering
  * (src/04kernel/src/kernels/mat_mul/cublas_kernel.cu:12,38: `lower` returns a RoutineWorkspace and the routine is
  * handed `void *workspace`).  rg_hip_matmul_workspace() says how many bytes help for a shape (0: none do, and
- * rg_hip_matmul_ws then runs exactly what rg_hip_matmul runs).  With at least that many bytes (8-byte aligned,
+ * rg_hip_matmul_ws then runs exactly what rg_hip_matmul runs).  With at least that many bytes (16-byte aligned,
  * contents arbitrary, nothing to clear; not to be shared by calls that may overlap), one to four rows of A
  * against FP16 / BF16 weights kept as [k, n] - a decode step on the layout ONNX MatMul stores - run with k shared
  * between workgroups that each read 512 contiguous bytes of a k-row; their float sums meet in the workspace and

@@ -1453,7 +1453,7 @@ __global__ __launch_bounds__(1024) void mm_gemv_kn(T *__restrict__ y, const T *_
 // share of k, keeps its whole share in flight at once when that is at most 256 k-rows (8 loads per lane), and
 // leaves its float sums in the workspace; the workgroup that finds every share of its strip delivered adds the shares
 // in their fixed order and stores.  The result therefore does not depend on which workgroup that is.
-// (the hand-off is described where it happens; it uses no atomic operation and needs nothing cleared)
+// (the hand-off, shares_complete below, needs nothing cleared beforehand)
 constexpr int KSP_COLS = 256;   // columns of a strip
 constexpr int KSP_ROWS = 32;    // k-rows a workgroup's 16 wavefronts load per instruction
 constexpr int KSP_DEPTH = 8;    // loads per lane in flight
@@ -1466,10 +1466,49 @@ __device__ __forceinline__ float load_through(const float *p) {
     return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
 
+constexpr unsigned long long kCounterAtRest = 0x5DEECE66D1CE4E5Bull;  // what a strip's arrival counter holds between launches
+
+// The workgroup's sums have been stored (written through).  Returns true in the workgroup that has to add the
+// strip's shares up.  Every wavefront waits until its stores have been acknowledged and the barrier collects them;
+// then one thread counts this share in.  The counter rests at a fixed 64-bit value between launches (the workgroup
+// that counts in last puts it back), so the arrival that reads that value + shares - 1 is the last one: one round
+// trip.  A counter that reads anything else - the workspace is handed over with arbitrary contents - says nothing,
+// and then, for every share of that launch alike, flags decide: this share's flag is set to the launch's number and
+// acknowledged, the strip's flags are read (loads that bypass the XCD's L2), and a workgroup that finds them all
+// set adds up.  The workgroup whose flag reached memory last is certain to; another one that arrived at almost the
+// same time may too, and then both store the same values.  Flags holding anything else than this launch's number
+// count as not set; whoever adds up clears them and puts the counter to rest.  No clearing launch, no dependence
+// of the result on who is last.
+__device__ __forceinline__ bool shares_complete(unsigned long long *counter, unsigned long long *strip_flags, uint32_t share,
+                                                uint32_t shares, unsigned long long launch_no, uint32_t tid) {
+    __shared__ int state;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned long long d = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - kCounterAtRest;
+        state = d < shares ? (d == shares - 1 ? 2 : 1) : 0;
+        if (d == shares - 1) __hip_atomic_store(counter, kCounterAtRest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d >= shares) {
+            __hip_atomic_store(strip_flags + share, launch_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    }
+    __syncthreads();
+    const int st = state;
+    if (st != 0) return st == 2;
+    int set = 1;
+    for (uint32_t f = tid; f < shares; f += blockDim.x)
+        set &= __hip_atomic_load(strip_flags + f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch_no;
+    if (!__syncthreads_and(set)) return false;
+    for (uint32_t f = tid; f < shares; f += blockDim.x) __hip_atomic_store(strip_flags + f, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(counter, kCounterAtRest, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 template <class T, int M>
 __global__ __launch_bounds__(1024) void mm_kn_split(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
                                                    uint32_t m, uint32_t k, uint32_t n, float alpha, float beta, uint32_t kr,
-                                                   uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ flags,
+                                                   uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ sync,
                                                    unsigned long long launch_no) {
     // kr: k-rows per share, a multiple of KSP_ROWS * KSP_DEPTH; k is even
     __shared__ __align__(16) float sums[16 * M * KSP_COLS];  // [wavefront][row of A][column of the strip]
@@ -1569,26 +1608,7 @@ __global__ __launch_bounds__(1024) void mm_kn_split(T *__restrict__ y, const T *
         }
     }
     if (shares == 1) return;
-    // Hand-off without a counter: the sums are written through; every wavefront waits until its stores have been
-    // acknowledged and the barrier collects the wavefronts; then one thread writes this share's flag, the launch's
-    // number, waits for that store's acknowledgement as well, and after a second barrier every thread reads one flag
-    // of the strip (loads that bypass the XCD's L2).  A workgroup that finds all flags set adds the shares up.  The
-    // workgroup whose flag reached memory last is certain to find them all; another one that arrived at almost the
-    // same time may too, and then both store the same values (same sums, same order).  Flags that hold anything
-    // else than this launch's number - whatever the workspace held before - count as not set, so nothing has to be
-    // cleared beforehand; whoever adds up clears the strip's flags afterwards (every share has arrived by then), so
-    // that a replay of a captured launch, which carries the same number, starts like the first run.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    unsigned long long *strip_flags = flags + static_cast<uint64_t>(strip) * shares;
-    if (tid == 0) {
-        __hip_atomic_store(strip_flags + share, launch_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __syncthreads();
-    int set = 1;
-    if (tid < shares) set = __hip_atomic_load(strip_flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch_no;
-    if (!__syncthreads_and(set)) return;
+    if (!shares_complete(sync + strip, sync + gridDim.x + static_cast<uint64_t>(strip) * shares, share, shares, launch_no, tid)) return;
     const float *strip_part = part + static_cast<uint64_t>(strip) * shares * (M * KSP_COLS);
 #pragma unroll
     for (int q = 0; q < (M * KSP_COLS + 1023) / 1024; ++q) {
@@ -1656,7 +1676,6 @@ __global__ __launch_bounds__(1024) void mm_kn_split(T *__restrict__ y, const T *
             if (i < m && col0 + cc < n) finish(i, col0 + cc, v);
         }
     }
-    if (tid < shares) __hip_atomic_store(strip_flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Shares of k for the kernel above: about one workgroup per CU, shares of whole load rounds, at most 255.
@@ -1682,161 +1701,180 @@ inline KnSplitPlan kn_split_plan(size_t k, size_t n, uint32_t rows_padded) {
     shares = static_cast<uint32_t>((k + kr - 1) / kr);
     p.shares = shares;
     p.kr = kr;
-    p.ticket_bytes = (static_cast<size_t>(p.strips) * shares * 8 + 255) / 256 * 256;  // one flag per share
+    p.ticket_bytes = (static_cast<size_t>(p.strips) * (shares + 1) * 8 + 255) / 256 * 256;  // a counter per strip, a flag per share
     p.bytes = p.ticket_bytes + static_cast<size_t>(p.strips) * shares * rows_padded * KSP_COLS * sizeof(float) + 16384;  // (padding: see the kernel)
     return p;
 }
 
 // ---------------------------------------------------------------- up to 32 rows of A, B as [k, n], k shared between workgroups
 //
-// The same sharing for the matrix cores.  A workgroup takes a strip of 128 columns and at most 512 k-rows: that part
-// of B (128 KiB) is requested in one go, straight into LDS (16 wavefronts x 8 copies of four 256-byte rows, so every
-// byte the workgroup will ever read is in flight from its first microsecond), laid out like the B tile of the large
-// kernel: chunk c of k-row r at chunk position c ^ n_swizzle(r & 3), which makes the transposing 64-bit reads that
-// turn [k, n] into operand layout conflict free.  Wavefront w copies and multiplies k-rows 32 w .. 32 w + 31 for all
-// four column blocks of the strip, so it waits for its own copies only: eight v_mfma_f32_32x32x16 whose first
-// operand comes from two transposing reads (k-rows 8 h .. 8 h + 7 of the step for half h of the wavefront) and whose
-// second operand is one 128-bit load of A from global memory (row lane % 32, the same eight k; two such loads per
-// wavefront, issued before the copies so that they arrive before them - with every wavefront loading operands for
-// a quarter of the share instead, the 32-byte pieces of A's rows cost more than all of B: 15.7 us).  The sixteen
-// wavefronts' sums meet in LDS, the shares of k in the workspace as above.
-constexpr int KM_COLS = 128;      // columns of a strip (256 bytes of a k-row)
-constexpr int KM_ROWB = 256;      // bytes of a k-row of the strip in LDS
-constexpr int KM_MAX_KR = 512;    // k-rows of a share: 128 KiB of LDS
-constexpr int KM_PART = 4096;     // floats a workgroup leaves: 32 rows of A x 128 columns
-
+// The same sharing for the matrix cores.  A workgroup of four wavefronts takes a strip of 64 columns and at most 1024
+// k-rows: that part of B (128 KiB) is requested in one go, straight into LDS, so every byte the workgroup will ever
+// read is in flight from its first microsecond.  Wavefront w copies and multiplies a quarter of the k-rows for both
+// column blocks of the strip, so it waits for its own copies only.  LDS layout: k-rows of 128 bytes, chunk c of row r
+// at chunk position c ^ 4 ((r >> 1) & 1): the four rows x 64 bytes that 32 lanes of a transposing 64-bit read touch
+// then lie on 64 different banks.  A product's first operand comes from two such reads (k-rows 8 h .. 8 h + 7 of the
+// step for half h of the wavefront), its second operand is one 128-bit load of A from global memory (row lane % 32,
+// the same eight k), issued before the copies so that it arrives before them.  The four wavefronts' sums meet in
+// LDS, the shares of k in the workspace as above; the finished tile leaves through LDS in whole 128-byte rows.
+// Measured on the way here ([32, 4096] x [4096, 4096], 23.0 us before): with strips of 128 columns, 16 wavefronts
+// and shares of 512 k-rows 15.2 us, of which the copies alone 7.1, the products 0.4, the sixteen wavefronts' sums
+// through LDS 1.8, 4 MB of float sums into the workspace 1.1, the hand-off 1.2 and the one workgroup per strip that
+// adds up 128 KiB and stores 4096 scattered 16-bit values 3.6.  As built now 13.3 us: the copies alone 7.8 (128-byte
+// pieces of B's rows), A's operands 1.4 (32-byte pieces of 32 rows per load, twice as many strips ask for them),
+// the products 1.2, and 3.0 for everything behind them.
+constexpr int KM_COLS = 64;       // columns of a strip (128 bytes of a k-row)
+constexpr int KM_ROWB = 128;      // bytes of a k-row of the strip in LDS
+constexpr int KM_MAX_KR = 1024;   // k-rows of a share: 128 KiB of LDS
+constexpr int KM_PART = 2048;     // floats a workgroup leaves: 32 rows of A x 64 columns
 template <class T>
-__global__ __launch_bounds__(1024) void mm_kn_mfma_split(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
-                                                        uint32_t m, uint32_t k, uint32_t n, float alpha, float beta, uint32_t kr,
-                                                        uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ flags,
-                                                        unsigned long long launch_no) {
-    // kr: k-rows per share, a multiple of 128, at most KM_MAX_KR; k a multiple of 8, n of 128
+__global__ __launch_bounds__(256) void mm_kn_mfma_split(T *__restrict__ y, const T *__restrict__ a, const T *__restrict__ b, Bias bias,
+                                                       uint32_t m, uint32_t k, uint32_t n, float alpha, float beta, uint32_t kr,
+                                                       uint32_t shares, float *__restrict__ part, unsigned long long *__restrict__ sync,
+                                                       unsigned long long launch_no) {
+    // kr: k-rows per share, a multiple of 256, at most KM_MAX_KR; k a multiple of 8, n of 64
+    // sync: one arrival counter per strip, then one flag per strip and share
     __shared__ __align__(1024) uint8_t lds[KM_MAX_KR * KM_ROWB];
     const uint32_t tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, half = lane >> 5;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t strip = blockIdx.x, share = blockIdx.y;
     const uint32_t col0 = strip * KM_COLS, k0 = share * kr;
     const uint32_t k_here = k - k0 < kr ? k - k0 : kr;  // k-rows of this share that exist (a multiple of 8)
+    const uint32_t kq = kr / 4, row0 = wave * kq;        // this wavefront's k-rows of the share: a multiple of 64
 
     // the operand from A first: row l32 (rows beyond m repeat the last one, their results are not stored), k-rows
-    // 32 wave + 16 ks + 8 half .. + 7; beyond the share's last k-row the operand is zero
-    u32x4 af[2];
+    // row0 + 16 ks + 8 half .. + 7; beyond the share's last k-row the operand is zero
+    constexpr int MAX_STEPS = KM_MAX_KR / 4 / 16;
+    u32x4 af[MAX_STEPS];
     {
         const T *arow = a + static_cast<uint64_t>(l32 < m ? l32 : m - 1) * k + k0;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const uint32_t kk = 32 * wave + 16 * ks + 8 * half;
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(arow + (kk < k_here ? kk : 0));
-            af[ks] = kk < k_here ? v : u32x4{0, 0, 0, 0};
+        for (int ks = 0; ks < MAX_STEPS; ++ks) {
+            const uint32_t kk = row0 + 16 * ks + 8 * half;
+            const bool have = 16 * ks < kq && kk < k_here;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(arow + (have ? kk : 0));
+            af[ks] = have ? v : u32x4{0, 0, 0, 0};
         }
     }
-    // the copies: instruction i of this wavefront brings k-rows 32 wave + 4 i .. + 3, the rows it multiplies itself;
-    // lane L fills chunk position L % 16 of row L / 16 of them, which holds chunk (L % 16) ^ n_swizzle(L / 16).
-    // Rows beyond the share's last one repeat it (A's operand is zero there).
-    const bool busy = 32 * wave < kr;
-    if (busy) {
-        const uint32_t cp_r = lane >> 4, chunk = (lane & 15) ^ n_swizzle(cp_r);
+    // the copies: eight k-rows of 128 bytes per instruction; lane L fills chunk position L % 8 of row L / 8 of them,
+    // which holds chunk (L % 8) ^ 4 ((L / 8 >> 1) & 1).  Rows beyond the share's last one repeat it (A's operand is
+    // zero there).
+    {
+        const uint32_t cp_r = lane >> 3, chunk = (lane & 7) ^ (4 * ((cp_r >> 1) & 1));
         const T *src0 = b + col0 + 8 * chunk;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t r0 = 32 * wave + 4 * i, r = r0 + cp_r, rr = r < k_here ? r : k_here - 1;
+#pragma unroll 4
+        for (uint32_t r0 = row0; r0 < row0 + kq; r0 += 8) {
+            const uint32_t r = r0 + cp_r, rr = r < k_here ? r : k_here - 1;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src0 + static_cast<uint64_t>(k0 + rr) * n),
                                              (__attribute__((address_space(3))) void *)(lds + r0 * KM_ROWB), 16, 0, 0);
         }
     }
-    f16v acc[4];
+    f16v acc[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // a wavefront reads only what it has copied itself: no barrier
-    if (busy) {
+    {
         // transposing read: lane s of a group of 16 addresses k-row s / 4, columns 4 (s % 4) .. + 3 of the group's 16;
-        // column block j of the strip is reached by XOR with 64 j (the swizzle leaves bits 6-7 of the offset alone)
+        // the other column block of the strip is reached by XOR with 64 (bit 2 of the chunk position)
         const uint32_t s16 = lane & 15, v_r = s16 >> 2;
         const uint32_t chunk = 2 * ((lane >> 4) & 1) + ((s16 & 3) >> 1);
-        const uint8_t *fp = lds + (32 * wave + 8 * half + v_r) * KM_ROWB + 16 * (chunk ^ n_swizzle(v_r)) + 8 * (s16 & 1);
+        const uint32_t f_off = (row0 + 8 * half + v_r) * KM_ROWB + 16 * (chunk ^ (4 * ((v_r >> 1) & 1))) + 8 * (s16 & 1);
+        // the reads of four k-steps are issued together, ahead of their products: read by read behind its product,
+        // a wavefront that is alone on its SIMD waits out the LDS latency 64 times over (4.5 us instead of 0.5)
+        auto read4 = [&](u32x4 (&bf)[4][2], int ks0) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+            for (int q = 0; q < 4; ++q)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint8_t *q = fp + 16 * ks * KM_ROWB;
-                const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (s4 __attribute__((address_space(3))) *)(lds + ((q - lds) ^ (64 * j))));
-                const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (s4 __attribute__((address_space(3))) *)(lds + (((q - lds) + 4 * KM_ROWB) ^ (64 * j))));
-                const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-                acc[j] = Mfma<T>::run(u32x4{l2[0], l2[1], h2[0], h2[1]}, af[ks], acc[j]);
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t o = f_off + 16 * (ks0 + q) * KM_ROWB;
+                    const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *)(lds + (o ^ (64 * j))));
+                    const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (s4 __attribute__((address_space(3))) *)(lds + ((o + 4 * KM_ROWB) ^ (64 * j))));
+                    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                    bf[q][j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+                }
+        };
+        u32x4 bf[2][4][2];
+        if (kq > 0) read4(bf[0], 0);
+#pragma unroll
+        for (int g = 0; g < MAX_STEPS / 4; ++g) {
+            if (64 * g < kq) {
+                if (64 * (g + 1) < kq && g + 1 < MAX_STEPS / 4) read4(bf[(g + 1) & 1], 4 * (g + 1));
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[j] = Mfma<T>::run(bf[g & 1][q][j], af[4 * g + q], acc[j]);
             }
-    }
-    // lane holds row l32 of A; register e column 8 (e / 4) + 4 half + e % 4 of column block j.  The sixteen
-    // wavefronts' sums meet in the tile's memory, one column block at a time (64 KiB each).
-    float *sums = reinterpret_cast<float *>(lds);  // [wavefront][register][lane]
-    const T *C = static_cast<const T *>(bias.ptr);
-    auto finish = [&](uint32_t x, float v) {  // x: column block, register, lane as laid out above
-        const uint32_t e = (x >> 6) & 15, i = x & 31, col = col0 + 32 * (x >> 10) + 8 * (e >> 2) + 4 * ((x >> 5) & 1) + (e & 3);
-        if (i < m) {
-            v *= alpha;
-            if (C) v += beta * up(C[i * bias.sm + col * bias.sn]);
-            y[static_cast<uint64_t>(i) * n + col] = down<T>(v);
         }
-    };
-    f4v mine;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        __syncthreads();  // the fragments, or the sums of the block before, have been read
-#pragma unroll
-        for (int e = 0; e < 16; ++e) sums[wave * 1024 + e * 64 + lane] = acc[u][e];
-        __syncthreads();
-        float v = 0.f;
-#pragma unroll
-        for (int w = 0; w < 16; ++w) v += sums[w * 1024 + tid];
-        if (shares == 1) finish(u * 1024 + tid, v);
-        mine[u] = v;
     }
-    if (shares == 1) return;
-    // hand-off as in mm_kn_split; a thread's four sums are one 128-bit piece of the workspace, so that the workgroup
-    // that adds up gets eight shares with one request per thread
-    const float *strip_part = part + static_cast<uint64_t>(strip) * shares * KM_PART;
-    asm volatile("global_store_dwordx4 %0, %1, %2 sc1" : : "v"((share * KM_PART + 4 * tid) * 4), "v"(mine), "s"(strip_part) : "memory");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // lane holds row l32 of A; register e column 8 (e / 4) + 4 half + e % 4 of column block j.  The four wavefronts'
+    // sums meet in the tile's memory: element x = 1024 j + 64 e + lane of wavefront w at float 2048 w + x.
+    float *sums = reinterpret_cast<float *>(lds);
+    __syncthreads();  // every wavefront has read its fragments
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sums[wave * KM_PART + j * 1024 + e * 64 + lane] = acc[j][e];
     __syncthreads();
-    unsigned long long *strip_flags = flags + static_cast<uint64_t>(strip) * shares;
-    if (tid == 0) {
-        __hip_atomic_store(strip_flags + share, launch_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // thread t owns elements 8 t .. 8 t + 7
+    f4v mine[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        mine[h] = *reinterpret_cast<const f4v *>(sums + 8 * tid + 4 * h);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) mine[h] += *reinterpret_cast<const f4v *>(sums + w * KM_PART + 8 * tid + 4 * h);
+    }
+    if (shares > 1) {
+        const float *strip_part = part + static_cast<uint64_t>(strip) * shares * KM_PART;
+        const uint32_t my_off = (share * KM_PART + 8 * tid) * 4;
+        asm volatile("global_store_dwordx4 %0, %1, %3 sc1\n\tglobal_store_dwordx4 %0, %2, %3 offset:16 sc1"
+                     : : "v"(my_off), "v"(mine[0]), "v"(mine[1]), "s"(strip_part) : "memory");
+        if (!shares_complete(sync + strip, sync + gridDim.x + static_cast<uint64_t>(strip) * shares, share, shares, launch_no, tid)) return;
+        mine[0] = mine[1] = f4v{0.f, 0.f, 0.f, 0.f};
+        for (uint32_t sh = 0; sh < shares; sh += 4) {
+            uint32_t off[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) off[j] = ((sh + j < shares ? sh + j : shares - 1) * KM_PART + 8 * tid) * 4;
+            f4v g0, g1, g2, g3, g4, g5, g6, g7;
+            asm volatile("global_load_dwordx4 %0, %8, %12 sc1\n\t"
+                         "global_load_dwordx4 %1, %8, %12 offset:16 sc1\n\t"
+                         "global_load_dwordx4 %2, %9, %12 sc1\n\t"
+                         "global_load_dwordx4 %3, %9, %12 offset:16 sc1\n\t"
+                         "global_load_dwordx4 %4, %10, %12 sc1\n\t"
+                         "global_load_dwordx4 %5, %10, %12 offset:16 sc1\n\t"
+                         "global_load_dwordx4 %6, %11, %12 sc1\n\t"
+                         "global_load_dwordx4 %7, %11, %12 offset:16 sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3), "=&v"(g4), "=&v"(g5), "=&v"(g6), "=&v"(g7)
+                         : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(strip_part)
+                         : "memory");
+            const f4v got[8] = {g0, g1, g2, g3, g4, g5, g6, g7};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (sh + j < shares) {
+                    mine[0] += got[2 * j];
+                    mine[1] += got[2 * j + 1];
+                }
+        }
+    }
+    // the tile leaves through LDS: [row of A][64 columns] of T, then 16 bytes per thread
+    __syncthreads();  // the sums in LDS have been read
+    T *tile = reinterpret_cast<T *>(lds);
+    const T *C = static_cast<const T *>(bias.ptr);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+        const uint32_t x = 8 * tid + v, e = (x >> 6) & 15, i = x & 31, c = 32 * (x >> 10) + 8 * (e >> 2) + 4 * ((x >> 5) & 1) + (e & 3);
+        float r = mine[v / 4][v % 4] * alpha;
+        if (C && i < m) r += beta * up(C[i * bias.sm + (col0 + c) * bias.sn]);
+        tile[i * KM_COLS + c] = down<T>(r);
     }
     __syncthreads();
-    int set = 1;
-    if (tid < shares) set = __hip_atomic_load(strip_flags + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == launch_no;
-    if (!__syncthreads_and(set)) return;
-    f4v total = {0.f, 0.f, 0.f, 0.f};
-    for (uint32_t sh = 0; sh < shares; sh += 8) {
-        uint32_t off[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) off[j] = ((sh + j < shares ? sh + j : shares - 1) * KM_PART + 4 * tid) * 4;
-        f4v g0, g1, g2, g3, g4, g5, g6, g7;
-        asm volatile("global_load_dwordx4 %0, %8, %16 sc1\n\t"
-                     "global_load_dwordx4 %1, %9, %16 sc1\n\t"
-                     "global_load_dwordx4 %2, %10, %16 sc1\n\t"
-                     "global_load_dwordx4 %3, %11, %16 sc1\n\t"
-                     "global_load_dwordx4 %4, %12, %16 sc1\n\t"
-                     "global_load_dwordx4 %5, %13, %16 sc1\n\t"
-                     "global_load_dwordx4 %6, %14, %16 sc1\n\t"
-                     "global_load_dwordx4 %7, %15, %16 sc1\n\t"
-                     "s_waitcnt vmcnt(0)"
-                     : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3), "=&v"(g4), "=&v"(g5), "=&v"(g6), "=&v"(g7)
-                     : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]),
-                       "s"(strip_part)
-                     : "memory");
-        const f4v got[8] = {g0, g1, g2, g3, g4, g5, g6, g7};
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            if (sh + j < shares) total += got[j];
+    {
+        const uint32_t i = tid >> 3, c8 = tid & 7;
+        if (i < m) *reinterpret_cast<u32x4 *>(y + static_cast<uint64_t>(i) * n + col0 + 8 * c8) = *reinterpret_cast<const u32x4 *>(tile + i * KM_COLS + 8 * c8);
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) finish(u * 1024 + tid, total[u]);
-    if (tid < shares) __hip_atomic_store(strip_flags + tid, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 inline KnSplitPlan kn_mfma_split_plan(size_t k, size_t n) {
@@ -1848,11 +1886,11 @@ inline KnSplitPlan kn_mfma_split_plan(size_t k, size_t n) {
     uint32_t shares = (static_cast<uint32_t>(cus) + p.strips / 2) / p.strips;
     if (shares < 1) shares = 1;
     uint32_t kr = static_cast<uint32_t>((k + shares - 1) / shares);
-    kr = (kr + 127) / 128 * 128;
+    kr = (kr + 255) / 256 * 256;  // a wavefront's quarter in groups of four k-steps
     if (kr > KM_MAX_KR) kr = KM_MAX_KR;
     p.shares = static_cast<uint32_t>((k + kr - 1) / kr);
     p.kr = kr;
-    p.ticket_bytes = (static_cast<size_t>(p.strips) * p.shares * 8 + 255) / 256 * 256;  // one flag per share
+    p.ticket_bytes = (static_cast<size_t>(p.strips) * (p.shares + 1) * 8 + 255) / 256 * 256;  // a counter per strip, a flag per share
     p.bytes = p.ticket_bytes + static_cast<size_t>(p.strips) * p.shares * KM_PART * sizeof(float);
     return p;
 }
@@ -1882,10 +1920,10 @@ template <class T>
 int launch_kn_mfma_split(T *y, const T *a, const T *b, Bias bias, uint32_t m, uint32_t k, uint32_t n, float alpha, float beta,
                          void *workspace, const KnSplitPlan &plan, hipStream_t s) {
     if constexpr (sizeof(T) == 2) {
-        auto *flags = static_cast<unsigned long long *>(workspace);
+        auto *sync = static_cast<unsigned long long *>(workspace);
         float *part = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + plan.ticket_bytes);
-        mm_kn_mfma_split<T><<<dim3(plan.strips, plan.shares, 1), 1024, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares,
-                                                                                 part, flags, next_launch_number());
+        mm_kn_mfma_split<T><<<dim3(plan.strips, plan.shares, 1), 256, 0, s>>>(y, a, b, bias, m, k, n, alpha, beta, plan.kr, plan.shares,
+                                                                                part, sync, next_launch_number());
         return launch_status();
     } else {
         return RG_HIP_E_UNSUPPORTED;
@@ -2078,8 +2116,8 @@ int launch_typed(void *y_, const void *a_, const void *b_, Bias bias, int trans_
         if constexpr (narrow) {
             // five to 32 rows against weights as [k, n] with a workspace at hand: the same sharing on the matrix cores
             if (workspace && !trans_a && !trans_b && m > 4 && m <= 32 && batch == 1 && count == 1 && n % KM_COLS == 0 && k > 0 &&
-                k % 8 == 0 && static_cast<uint64_t>(k) * n >= (1u << 20) && aligned16(b) && aligned16(a) &&
-                reinterpret_cast<uintptr_t>(workspace) % 8 == 0) {
+                k % 8 == 0 && static_cast<uint64_t>(k) * n >= (1u << 20) && aligned16(b) && aligned16(a) && aligned16(y_) &&
+                reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
                 const KnSplitPlan plan = kn_mfma_split_plan(k, n);
                 if (plan.shares <= 255 && plan.bytes <= workspace_bytes)
                     return launch_kn_mfma_split<T>(y + static_cast<uint64_t>(ym0) * m * n, a + static_cast<uint64_t>(am0) * m * k,
