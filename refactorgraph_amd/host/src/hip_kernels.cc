@@ -379,14 +379,20 @@ namespace refactor::kernel {
                 };
             return RoutineWorkspace(std::move(routine), bytes);
         }
-        return [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex)]//
-            (Resources &res, void *, void const *const *inputs, void *const *outputs) {
-                HIP_CALL(rg_hip_matmul(outputs[0], inputs[0], inputs[1], info.hasBias ? inputs[2] : nullptr,
-                                       static_cast<int>(info.dataType.internal), info.transA, info.transB, info.alpha,
-                                       info.beta, info.batch(), info.m, info.k, info.n,
-                                       aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
-                                       info.biasStrideBatch, info.biasStrideM, info.biasStrideN, streamOf(res)));
+        // A workspace where the library has a use for one (few rows against weights kept as [k, n]: sums of shares
+        // of k meet there); its contents never need preparing, so any range of the stack will do.
+        auto const bytes = rg_hip_matmul_workspace(static_cast<int>(info.dataType.internal), info.transA, info.transB,
+                                                   info.batch(), info.m, info.k, info.n);
+        auto routine = [info = info, aIndex = std::move(aIndex), bIndex = std::move(bIndex), bytes]//
+            (Resources &res, void *workspace, void const *const *inputs, void *const *outputs) {
+                HIP_CALL(rg_hip_matmul_ws(outputs[0], inputs[0], inputs[1], info.hasBias ? inputs[2] : nullptr,
+                                          static_cast<int>(info.dataType.internal), info.transA, info.transB, info.alpha,
+                                          info.beta, info.batch(), info.m, info.k, info.n,
+                                          aIndex.empty() ? nullptr : aIndex.data(), bIndex.empty() ? nullptr : bIndex.data(),
+                                          info.biasStrideBatch, info.biasStrideM, info.biasStrideN, bytes ? workspace : nullptr, bytes,
+                                          streamOf(res)));
             };
+        return RoutineWorkspace(std::move(routine), bytes);
     }
 
     // ------------------------------------------------------------------ Cast

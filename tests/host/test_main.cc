@@ -1056,6 +1056,48 @@ static void matMulHip() {
         auto bad = Tensor::share(DataType::F32, Shape{2, 1, m, 1});
         EXPECT(MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({*A, *B, *bad}, {*Y}).empty());
     }
+    {// few rows of FP16 against weights kept as [k, n]: lower() asks for the library's workspace (shares of k meet
+     // there) and the routine hands it on; operands in {-1, 0, 1}, so every sum is an integer FP16 holds exactly.
+     // The workspace arrives as the allocator left it: nothing in it needs preparing.
+        std::mt19937 rng(17);
+        std::uniform_int_distribution<int> g(-1, 1);
+        dim_t const k = 1024, n = 1024;
+        for (dim_t m : {dim_t(1), dim_t(4), dim_t(20)}) {
+            std::vector<int> a(m * k), b(k * n);
+            for (auto &v : a) v = g(rng);
+            for (auto &v : b) v = g(rng);
+            std::vector<uint16_t> ah(a.size()), bh(b.size());
+            for (size_t i = 0; i < a.size(); ++i) ah[i] = f2h(static_cast<float>(a[i]));
+            for (size_t i = 0; i < b.size(); ++i) bh[i] = f2h(static_cast<float>(b[i]));
+            auto A = Tensor::share(DataType::FP16, Shape{m, k});
+            auto B = Tensor::share(DataType::FP16, Shape{k, n});
+            auto Y = Tensor::share(DataType::FP16, Shape{m, n});
+            auto kernels = MatMulCollector(Device::Type::Amd, 1, 1, false, false).filter({*A, *B}, {*Y});
+            EXPECT(kernels.size() == 1);
+            auto [routine, workspace] = kernels[0]->lower(res);
+            EXPECT(workspace > 0);
+            auto ma = dev.malloc(ah.size() * 2), mb = dev.malloc(bh.size() * 2), my = dev.malloc(m * n * 2), ws = dev.malloc(workspace);
+            std::vector<uint8_t> junk(workspace, 0xa5);
+            ws->copyFromHost(junk.data());
+            ma->copyFromHost(ah.data());
+            mb->copyFromHost(bh.data());
+            void const *inputs[]{*ma, *mb};
+            void *outputs[]{*my};
+            std::vector<uint16_t> y(m * n);
+            bool same = true;
+            for (int round = 0; round < 2; ++round) {  // the second call finds what the first one left
+                routine(res, *ws, inputs, outputs);
+                my->copyToHost(y.data());
+                for (dim_t i = 0; i < m; ++i)
+                    for (dim_t j = 0; j < n; ++j) {
+                        int sum = 0;
+                        for (dim_t t = 0; t < k; ++t) sum += a[i * k + t] * b[t * n + j];
+                        same = same && y[i * n + j] == f2h(static_cast<float>(sum));
+                    }
+            }
+            EXPECT(same);
+        }
+    }
     {// against the oracle's serial loop, float, odd sizes, no bias
         std::mt19937 rng(9);
         std::uniform_int_distribution<int> g(-4, 4);  // integer-valued: every partial sum is exact
