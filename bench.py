@@ -470,6 +470,34 @@ def main():
     ops_out = {}
     steps, warmup = args.steps, args.warmup
 
+    def cpu_all(fn, algorithmic_bytes, sample, unit="GB/s", per=1e9):
+        """The all-cores row: `fn` runs the same arithmetic as the one-core leg with its rows split over
+        CPU_THREADS host threads (the oracle's own `threads=` argument, or pieces dealt to a thread pool)."""
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 1.0:
+                break
+        return {"value": round(algorithmic_bytes * reps / dt / per, 5), "unit": unit, "cores": CPU_THREADS, "kind": "port",
+                "sample": f"{sample} ({reps} repetitions, {dt / reps * 1e3:.1f} ms each)"}
+
+    def cpu_leg(fn, algorithmic_bytes, sample):
+        """Times the oracle on a bounded sample for about a second; the rate is quoted in the algorithmic bytes
+        of that sample so that it compares with `achieved`."""
+        fn()  # page in
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 1.0:
+                break
+        return {"value": round(algorithmic_bytes * reps / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{sample} ({reps} repetitions, {dt / reps * 1e3:.1f} ms each)"}
+
     if want("rms_norm"):
         nb = 5  # 5 x (134 MB in + 134 MB out): beyond the 256 MB MALL
         xs = [torch.randn((32, 128, 4096), device=dev) for _ in range(nb)]

@@ -145,6 +145,39 @@ def test_matmul_on_random_shapes(seed):
         assert np.all(np.abs(y - ref) <= 1.01 * limit), (case, batch, m, k, n, str(dt), trans_b, int(bias_kind))
 
 
+@pytest.mark.parametrize("seed", [451, 452])
+def test_matmul_few_rows_with_workspace_on_random_shapes(seed):
+    # at most 32 rows against weights kept as [k, n], through the workspace (shares of k between workgroups): shapes
+    # whose k ends inside a share, a load round and a quarter of a share; one workspace, full of junk at first, serves
+    # every case of a seed in turn, so each case finds what another shape left there
+    rng = np.random.default_rng(seed)
+    ws = torch.full((24 << 20,), 0x5a, dtype=torch.uint8, device=DEV)
+    for case in range(24):
+        m = int(rng.integers(1, 33))
+        step_k, step_n = (2, 8) if m <= 4 else (8, 64)
+        n = int(rng.integers(1, 5000 // step_n + 1)) * step_n
+        k = max(int(rng.integers(1, 6000 // step_k + 1)) * step_k, -(-(1 << 20) // n // step_k) * step_k)
+        dt = torch.float16 if rng.integers(0, 3) else torch.bfloat16
+        need = ops.lib().rg_hip_matmul_workspace(ops._T2CODE[dt], 0, 0, 1, m, k, n)
+        assert 0 < need <= ws.numel(), (case, m, k, n)
+        a = dev(rng.standard_normal((m, k)).astype(np.float32)).to(dt)
+        b = dev((rng.standard_normal((k, n)) * 0.25).astype(np.float32)).to(dt)
+        bias_kind = rng.integers(0, 3)
+        c = None if bias_kind == 0 else dev(rng.standard_normal((n,) if bias_kind == 1 else (m, n)).astype(np.float32)).to(dt)
+        alpha, beta = (1.0, 1.0) if rng.integers(0, 2) else (0.5, 2.0)
+        got = ops.matmul(a, b, c, alpha=alpha, beta=beta, workspace=ws)
+        assert torch.equal(got, ops.matmul(a, b, c, alpha=alpha, beta=beta, workspace=ws)), (case, m, k, n)
+        y = host(got.float())
+        af, bf = host(a.float()).astype(np.float64), host(b.float()).astype(np.float64)
+        ref, mag = alpha * (af @ bf), alpha * (np.abs(af) @ np.abs(bf))
+        if c is not None:
+            cf = host(c.float()).astype(np.float64)
+            ref, mag = ref + beta * cf, mag + np.abs(beta * cf)
+        eps = 2.0 ** -10 if dt == torch.float16 else 2.0 ** -7
+        limit = eps * np.abs(ref) + mag * 2.0 ** -20 + 1e-6
+        assert np.all(np.abs(y - ref) <= 1.01 * limit), (case, m, k, n, str(dt), int(bias_kind))
+
+
 @pytest.mark.parametrize("seed", [501, 502])
 def test_data_movers_on_random_shapes(seed):
     rng = np.random.default_rng(seed)
