@@ -60,9 +60,10 @@ MEASURED_TRAFFIC = {
     "rms_norm_quantize": (2 * 32883 + 65568 + 2 * 32889 + 16384) * 1024,
     "matmul_integer_few_rows": (2 * 8761 + 8192 + 2 * 10 + 512) * 1024,
     "matmul_one_row": (2 * 16444 + 8) * 1024,
-    "matmul_one_row_kn": (2 * 16499 + 20) * 1024,
+    "matmul_one_row_kn": (2 * 16630 + 273) * 1024,
+    "matmul_four_rows_kn": (2 * 17236 + 1065) * 1024,
     "matmul_f32_one_row": (2 * 35255 + 16) * 1024,
-    "matmul_few_rows_kn": (2 * 17591 + 256) * 1024,
+    "matmul_few_rows_kn": (2 * 18505 + 4362) * 1024,
     "matmul_integer_one_row": (2 * 8242 + 512 + 2 * 10 + 16) * 1024,
     "dynamic_quantize_linear": (2 * 32798 + 32 + 2 * 32889 + 16384) * 1024,
     "softmax_long_rows": (2 * 32828 + 65602) * 1024,
