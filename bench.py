@@ -1137,6 +1137,35 @@ def main():
             "device_ms_per_launch": round(dms, 5), "timing": mode, "hbm_gbs": round(kv_bytes / (dms * 1e-3) / 1e9, 1),
             "warmup_ms": LAST["warmup_ms"], "warmup_steps": LAST["warmup_steps"]}
 
+    if want("attention_short_history_large_cache"):
+        # where the host's choice between the two attention kernels is weakest: the history length is device data, so
+        # half the capacity stands for it; a conversation that has just begun in a cache sized for 32768 positions
+        # (8 new rows, history 100) is sent to the tiled kernel with key ranges and a merging launch, most of whose
+        # ranges hold no key.  The same call with the cache nearly full is where that choice pays.
+        Np, seq, capc, Dc = 1, 8, 32768, 128
+        q = torch.randn((Np, H, seq, Dc), device=dev).half()
+        k = torch.randn((Np, Hkv, seq, Dc), device=dev).half()
+        v = torch.randn((Np, Hkv, seq, Dc), device=dev).half()
+        kc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        vc = torch.randn((Np, Hkv, capc, Dc), device=dev).half()
+        o = torch.empty_like(q)
+        wsp = ops.attention_workspace(Np, H, Hkv, seq, capc, Dc, dev)
+        times = {}
+        for label, past in (("short", 100), ("full", capc - seq - 8)):
+            pl = torch.full((Np,), past, device=dev, dtype=torch.int64)
+            wall, dms, mode = time_steps(
+                torch, lambda i: ops.attention_kvcache(q, k, v, kc, vc, pl, 1.0 / math.sqrt(Dc), out=o, workspace=wsp,
+                                                       sync_state=state),
+                max(steps // 10, 20), max(warmup // 80, 2), 1)
+            times[label] = dms
+        short_bytes = 2 * Np * Hkv * (100 + seq) * Dc * 2 + 2 * Np * H * seq * Dc * 2 + 2 * Np * Hkv * seq * Dc * 2
+        e = hbm_entry(short_bytes, times["short"])
+        e.update(workload="AttentionKVCache fp16 N=1 H=32 Hkv=8 D=128, 8 new rows, cache capacity 32768, history 100 "
+                          "(the kernel is chosen for half the capacity)",
+                 device_ms_per_launch=round(times["short"], 5), timing=mode,
+                 same_call_history_32752_device_ms=round(times["full"], 5))
+        ops_out["attention_short_history_large_cache"] = e
+
     if want("attention_decode_group8"):
         # a decode step of a model with eight query heads per kv head (64/8): one launch reads K/V once for all eight
         Np, H8, past, Dc = 64, 64, 4096, 128
